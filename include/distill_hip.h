@@ -1,0 +1,87 @@
+/*
+ * C ABI of the MI355X (gfx950) distillation-loss library, libdistill_hip.so.
+ *
+ * The reference (golololologol/LLM-Distillery) has no FFI layer: its loss path is
+ * a chain of PyTorch eager ops called from Python.  Each entry point below names
+ * the reference lines whose work it replaces.  Conventions shared by all GPU
+ * entry points:
+ *   - every pointer is a DEVICE pointer on the current HIP device unless the
+ *     parameter comment says "host";
+ *   - nothing is allocated, freed or retained; buffers belong to the caller;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*) and the call
+ *     returns without synchronising;
+ *   - strides are in ELEMENTS of the array's dtype;
+ *   - the return value is DL_OK or a negative dl_status; no exception crosses
+ *     the boundary.
+ */
+#ifndef DISTILL_HIP_H
+#define DISTILL_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { DL_F32 = 0, DL_BF16 = 1, DL_F16 = 2 } dl_dtype;      /* floating storage types */
+typedef enum { DL_I32 = 0, DL_I64 = 1 } dl_itype;                   /* index storage types     */
+typedef enum { DL_FKL = 0, DL_RKL = 1, DL_JSD = 2 } dl_kind;        /* divergence              */
+
+typedef enum {
+  DL_OK = 0,
+  DL_ERR_NULL = -1,     /* a required pointer is NULL                      */
+  DL_ERR_DTYPE = -2,    /* unknown dtype / itype / kind                    */
+  DL_ERR_SHAPE = -3,    /* negative or inconsistent sizes                  */
+  DL_ERR_LIMIT = -4,    /* a size exceeds what the kernels support         */
+  DL_ERR_LAUNCH = -5,   /* the HIP runtime refused the launch              */
+  DL_ERR_ALIGN = -6     /* a pointer/stride breaks a stated alignment rule */
+} dl_status;
+
+#define DL_MAX_TOPK 2048      /* entries per row a sparse teacher may hold        */
+#define DL_MAX_TEACHERS 8     /* teachers merged in one launch                    */
+
+/* Library ABI revision; bumped when a signature changes. */
+int dl_abi_version(void);
+/* Static, NUL-terminated description of a dl_status. */
+const char* dl_status_string(int status);
+
+/*
+ * Forward or reverse KL against a sparse (top-K) teacher, loss and gradient in one sweep.
+ * Replaces, for one launch over all token rows:
+ *   classes/student/model.py:408,420-421   slice + .float() + /T, row select, teacher /T
+ *   utils/finetuning_utils.py:88,91-92     log_softmax (student over V, teacher over K), gather
+ *   utils/finetuning_utils.py:49-56,104-105  F.kl_div(log_target=True).sum(-1)   (kind FKL / RKL)
+ *   classes/losses.py:77-78                the autograd replay of all of the above
+ *
+ * logits     [n_rows, V] (row stride `row_stride`), dtype `logits_dtype`, native model dtype.
+ * row_map    [n_rows] int32: teacher row feeding logits row r; a value outside
+ *            [0, n_teacher_rows) marks a masked/padded row (loss 0, gradient row zero-filled);
+ *            NULL = identity.
+ * t_val      [*, K] stored teacher log-probs (dtype `t_val_dtype`), t_idx [*, K] vocabulary ids
+ *            (`t_idx_itype`); both K-contiguous.  t_cnt: optional int32 per teacher row, only the
+ *            first t_cnt entries count (NULL = all K).  Ids outside [0, V) are ignored.
+ *            The teacher is renormalised over its counted entries: log_softmax(t_val * inv_T_teacher).
+ * row_loss   [n_rows] fp32 per-token divergence (optional, may be NULL).
+ * grad       [n_rows, V] (stride `grad_stride`), same dtype as logits; receives
+ *            d(sum_r row_loss[r]) / d logits * grad_scale (optional, NULL = forward only).
+ * K <= DL_MAX_TOPK.
+ */
+int dl_div_topk(int kind,
+                const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                const int32_t* row_map,
+                const void* t_val, int t_val_dtype, const void* t_idx, int t_idx_itype, int K,
+                int64_t n_teacher_rows, const int32_t* t_cnt,
+                float inv_T_student, float inv_T_teacher, float grad_scale,
+                float* row_loss, void* grad, int64_t grad_stride, void* stream);
+
+/*
+ * Deterministic sum of n fp32 values times `scale` into out[0] (fixed reduction tree,
+ * double accumulation).  Replaces the `.mean()` of utils/finetuning_utils.py:54 /
+ * the `+=` accumulation of classes/losses.py:43-47.
+ */
+int dl_reduce_sum(const float* values, int64_t n, float scale, float* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DISTILL_HIP_H */

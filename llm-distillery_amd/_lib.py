@@ -1,0 +1,64 @@
+"""ctypes binding of libdistill_hip.so (the C ABI declared in include/distill_hip.h).
+
+The library is the only compute path: if it is missing this module raises on
+first use -- there is no PyTorch or CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libdistill_hip.so")
+
+# dtype / kind codes of include/distill_hip.h
+DL_F32, DL_BF16, DL_F16 = 0, 1, 2
+DL_I32, DL_I64 = 0, 1
+DL_FKL, DL_RKL, DL_JSD = 0, 1, 2
+DL_MAX_TOPK = 2048
+DL_MAX_TEACHERS = 8
+
+_P = c_void_p
+_SIGNATURES = {
+    "dl_abi_version": (c_int, []),
+    "dl_status_string": (c_char_p, [c_int]),
+    "dl_div_topk": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, _P, c_int, c_int, c_int64, _P,
+                            c_float, c_float, c_float, _P, _P, c_int64, _P]),
+    "dl_reduce_sum": (c_int, [_P, c_int64, c_float, _P, _P]),
+}
+
+_lib = None
+
+
+class DistillLibraryError(RuntimeError):
+    pass
+
+
+def exported_symbols() -> list[str]:
+    return sorted(_SIGNATURES)
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once and attach the argument types."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise DistillLibraryError(
+            f"{LIB_PATH} is missing: build it with `python llm-distillery_amd/build.py` "
+            "(hipcc, gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)      # AttributeError if the library lacks a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    """Translate a dl_status into the Python error the caller sees."""
+    if status != 0:
+        msg = load().dl_status_string(status).decode()
+        raise RuntimeError(f"{what}: {msg} (dl_status {status})")

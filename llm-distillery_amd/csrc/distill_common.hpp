@@ -1,0 +1,197 @@
+// Shared device helpers for the row-streaming distillation-loss kernels (gfx950).
+//
+// Execution model used by every kernel in this directory: one workgroup owns one
+// token row of the [rows x vocab] logits.  The row is fetched with 16-byte
+// non-temporal loads into registers (it is read from HBM exactly once), reduced
+// with wave64 butterflies plus a cross-wave combine in LDS, and the gradient is
+// written from the same registers with 16-byte non-temporal stores.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dl {
+
+constexpr int WAVE = 64;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// dtype tags mirrored from the C header
+enum : int { F32 = 0, BF16 = 1, F16 = 2 };
+enum : int { I32 = 0, I64 = 1 };
+
+struct TagF32 { static constexpr int id = F32; static constexpr int bytes = 4; static constexpr int epc = 4; };
+struct TagBF16 { static constexpr int id = BF16; static constexpr int bytes = 2; static constexpr int epc = 8; };
+struct TagF16 { static constexpr int id = F16; static constexpr int bytes = 2; static constexpr int epc = 8; };
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// ---- 16-byte chunk <-> floats -------------------------------------------------
+template <class Tag> struct Chunk;
+
+template <> struct Chunk<TagF32> {
+  static constexpr int N = 4;
+  __device__ static __forceinline__ u32x4 neg_inf() { return u32x4{0xff800000u, 0xff800000u, 0xff800000u, 0xff800000u}; }
+  __device__ static __forceinline__ void unpack(const u32x4& c, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(c[i]);
+  }
+  __device__ static __forceinline__ u32x4 pack(const float* f) {
+    return u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+  }
+};
+
+template <> struct Chunk<TagBF16> {
+  static constexpr int N = 8;
+  __device__ static __forceinline__ u32x4 neg_inf() { return u32x4{0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u}; }
+  __device__ static __forceinline__ void unpack(const u32x4& c, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(c[i] << 16);
+      f[2 * i + 1] = __uint_as_float(c[i] & 0xffff0000u);
+    }
+  }
+  __device__ static __forceinline__ u32x4 pack(const float* f) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      bf16x2 b = __builtin_convertvector(f32x2{f[2 * i], f[2 * i + 1]}, bf16x2);   // v_cvt_pk_bf16_f32, RNE
+      r[i] = __builtin_bit_cast(unsigned, b);
+    }
+    return r;
+  }
+};
+
+template <> struct Chunk<TagF16> {
+  static constexpr int N = 8;
+  __device__ static __forceinline__ u32x4 neg_inf() { return u32x4{0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u}; }
+  __device__ static __forceinline__ void unpack(const u32x4& c, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned u = c[i];   // copy first: bit_cast straight from a vector element reads element 0
+      f16x2 h = __builtin_bit_cast(f16x2, u);
+      f[2 * i] = (float)h[0];
+      f[2 * i + 1] = (float)h[1];
+    }
+  }
+  __device__ static __forceinline__ u32x4 pack(const float* f) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f16x2 h = __builtin_convertvector(f32x2{f[2 * i], f[2 * i + 1]}, f16x2);
+      r[i] = __builtin_bit_cast(unsigned, h);
+    }
+    return r;
+  }
+};
+
+// ---- scalar element access by runtime dtype (K-wide side arrays only) ----------
+__device__ __forceinline__ float load_as_float(const void* base, int dtype, int64_t i) {
+  if (dtype == F32) return reinterpret_cast<const float*>(base)[i];
+  unsigned short u = reinterpret_cast<const unsigned short*>(base)[i];
+  if (dtype == BF16) return __uint_as_float(((unsigned)u) << 16);
+  return (float)__builtin_bit_cast(_Float16, u);
+}
+
+__device__ __forceinline__ void store_from_float(void* base, int dtype, int64_t i, float v) {
+  if (dtype == F32) {
+    reinterpret_cast<float*>(base)[i] = v;
+  } else if (dtype == BF16) {
+    __bf16 b = (__bf16)v;
+    reinterpret_cast<unsigned short*>(base)[i] = __builtin_bit_cast(unsigned short, b);
+  } else {
+    _Float16 h = (_Float16)v;
+    reinterpret_cast<unsigned short*>(base)[i] = __builtin_bit_cast(unsigned short, h);
+  }
+}
+
+__device__ __forceinline__ int64_t load_index(const void* base, int itype, int64_t i) {
+  if (itype == I32) return (int64_t)reinterpret_cast<const int32_t*>(base)[i];
+  return reinterpret_cast<const int64_t*>(base)[i];
+}
+
+// ---- streaming 16-byte accesses ------------------------------------------------
+__device__ __forceinline__ u32x4 load16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ void store16_stream(void* p, const u32x4& v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+
+// ---- reductions: fixed butterfly order => bit-reproducible ----------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+
+// All threads of the workgroup receive the result.  `scratch` holds NT/64 floats;
+// two barriers per call so it can be reused immediately.
+template <int NT, bool IS_MAX>
+__device__ __forceinline__ float block_reduce(float v, float* scratch) {
+  constexpr int NW = NT / WAVE;
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  if constexpr (NW == 1) return v;
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  if (lane == 0) scratch[w] = v;
+  __syncthreads();
+  float r = scratch[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) r = IS_MAX ? fmaxf(r, scratch[i]) : (r + scratch[i]);
+  __syncthreads();
+  return r;
+}
+template <int NT> __device__ __forceinline__ float block_max(float v, float* s) { return block_reduce<NT, true>(v, s); }
+template <int NT> __device__ __forceinline__ float block_sum(float v, float* s) { return block_reduce<NT, false>(v, s); }
+
+// Two sums in one pair of barriers.
+template <int NT>
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* scratch) {
+  constexpr int NW = NT / WAVE;
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if constexpr (NW == 1) return;
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  if (lane == 0) { scratch[w] = a; scratch[NW + w] = b; }
+  __syncthreads();
+  float ra = scratch[0], rb = scratch[NW];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) { ra += scratch[i]; rb += scratch[NW + i]; }
+  __syncthreads();
+  a = ra; b = rb;
+}
+
+// Teacher row feeding logits row r: row_map[r] (identity without a map); anything outside
+// [0, n_trows) means "masked row".
+__device__ __forceinline__ int64_t teacher_row(const int32_t* row_map, int64_t r, int64_t n_trows) {
+  const int64_t t = row_map ? (int64_t)row_map[r] : r;
+  return (t >= 0 && t < n_trows) ? t : -1;
+}
+
+// Makes the compiler forget what it knows about a chunk held in registers.  Placed at
+// the head of every sweep over a register-resident row so that the unpacked fp32 copies of
+// one sweep are not kept alive for the next (that would double the register footprint).
+__device__ __forceinline__ void forget(u32x4& c) {
+  asm volatile("" : "+v"(c));
+}
+
+// zero-fill one gradient row (masked / padded token positions)
+template <class Tag, int NT>
+__device__ __forceinline__ void zero_row(void* grad_row, int64_t nchunks) {
+  const u32x4 z{0u, 0u, 0u, 0u};
+  for (int64_t c = threadIdx.x; c < nchunks; c += NT)
+    store16_stream(reinterpret_cast<char*>(grad_row) + c * 16, z);
+}
+
+}  // namespace dl

@@ -1,0 +1,46 @@
+// ABI revision, status strings and the deterministic scalar reduction.
+#include "distill_common.hpp"
+#include "distill_hip.h"
+
+namespace dl {
+
+// One workgroup, fixed association order: thread t adds values t, t+NT, ... in double,
+// then a fixed LDS tree.  Same input => same bits.
+template <int NT>
+__global__ __launch_bounds__(NT) void reduce_sum_kernel(const float* v, int64_t n, float scale, float* out) {
+  __shared__ double sh[NT];
+  double acc = 0.0;
+  for (int64_t i = threadIdx.x; i < n; i += NT) acc += (double)v[i];
+  sh[threadIdx.x] = acc;
+  __syncthreads();
+  for (int o = NT / 2; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = (float)(sh[0] * (double)scale);
+}
+
+}  // namespace dl
+
+extern "C" int dl_abi_version(void) { return 1; }
+
+extern "C" const char* dl_status_string(int status) {
+  switch (status) {
+    case DL_OK: return "ok";
+    case DL_ERR_NULL: return "a required pointer is NULL";
+    case DL_ERR_DTYPE: return "unknown dtype, index type or divergence kind";
+    case DL_ERR_SHAPE: return "negative or inconsistent sizes";
+    case DL_ERR_LIMIT: return "a size exceeds what the kernels support";
+    case DL_ERR_LAUNCH: return "the HIP runtime refused the launch";
+    case DL_ERR_ALIGN: return "a pointer or stride breaks an alignment rule";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int dl_reduce_sum(const float* values, int64_t n, float scale, float* out, void* stream) {
+  if (!out || (n > 0 && !values)) return DL_ERR_NULL;
+  if (n < 0) return DL_ERR_SHAPE;
+  hipLaunchKernelGGL((dl::reduce_sum_kernel<1024>), dim3(1), dim3(1024), 0,
+                     reinterpret_cast<hipStream_t>(stream), values, n, scale, out);
+  return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}

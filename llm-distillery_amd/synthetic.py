@@ -1,0 +1,59 @@
+"""Seeded synthetic inputs for the five benchmark configurations.
+
+Everything is generated in row chunks on the target device so the largest config
+(32768 x 128256 bf16) never needs more than one fp32 chunk of scratch.  The same
+seed on the same device type gives the same tensors.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+CHUNK_ROWS = 1024
+
+
+def _gen(device, seed: int) -> torch.Generator:
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    return g
+
+
+def _gumbel(shape, g, device):
+    u = torch.rand(shape, generator=g, device=device).clamp_(1e-10, 1.0 - 1e-7)
+    return -torch.log(-torch.log(u))
+
+
+def topk_teacher_for(student_chunk: torch.Tensor, K: int, n_hot: int, g, teacher_vocab: int | None = None):
+    """K unique int32 ids per row (the row's `n_hot` largest logits plus uniform
+    draws without replacement) and fp16 log-probs = log-softmax of
+    Gumbel-perturbed scores over those K entries."""
+    R, V = student_chunk.shape
+    dev = student_chunk.device
+    Vt = V if teacher_vocab is None else teacher_vocab
+    sf = student_chunk.float()
+    hot = sf.topk(n_hot, dim=-1).indices if n_hot > 0 else torch.empty((R, 0), dtype=torch.long, device=dev)
+    noise = torch.rand((R, Vt), generator=g, device=dev)
+    if n_hot > 0:
+        noise.scatter_(1, hot, -1.0)
+    rest = noise.topk(K - n_hot, dim=-1).indices
+    ids = torch.cat((hot, rest), dim=1)
+    base = torch.gather(sf, 1, ids.clamp(max=V - 1))
+    scores = base + _gumbel((R, K), g, dev)
+    logp = torch.log_softmax(scores, dim=-1)
+    return logp.to(torch.float16), ids.to(torch.int32)
+
+
+def config3(device, rows: int = 8 * 4096, V: int = 128256, K: int = 200, seed: int = 3, std: float = 3.0,
+            dtype=torch.bfloat16):
+    """Sparse top-K teacher, forward KL: student ~ N(0, 3^2) bf16, K=200 ids per
+    token (argmax-20 of the student row + 180 uniform), fp16 teacher log-probs, T=1."""
+    g = _gen(device, seed)
+    logits = torch.empty((rows, V), dtype=dtype, device=device)
+    t_val = torch.empty((rows, K), dtype=torch.float16, device=device)
+    t_idx = torch.empty((rows, K), dtype=torch.int32, device=device)
+    for a in range(0, rows, CHUNK_ROWS):
+        b = min(rows, a + CHUNK_ROWS)
+        chunk = (torch.randn((b - a, V), generator=g, device=device) * std).to(dtype)
+        logits[a:b] = chunk
+        t_val[a:b], t_idx[a:b] = topk_teacher_for(chunk, K, min(20, K), g)
+    return {"logits": logits, "t_val": t_val, "t_idx": t_idx, "T": 1.0, "kind": "fkl"}

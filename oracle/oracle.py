@@ -202,14 +202,14 @@ def mean_loss_and_grad(kind: str, logits: torch.Tensor, T: float, *,
     before the loss (the reference index_selects content rows) and get a zero
     gradient.  Top-K teacher: `t_vals` [Nv,K] stored log-probs, `t_idx` [Nv,K].
     Dense teacher: `t_logits` [Nv,Vt==V].  Returns (loss, rows[Nv], grad[R,V]
-    in the storage dtype of `logits`).
+    in the compute dtype, i.e. before the cast back to the storage dtype of `logits`).
     """
     R = logits.shape[0]
     if valid is None:
         valid = torch.ones(R, dtype=torch.bool)
     sel = torch.nonzero(valid).squeeze(-1)
-    leaf = logits.detach().clone().requires_grad_(True)
-    z = torch.index_select(leaf, 0, sel).to(dtype) / T
+    leaf = logits.detach().to(dtype).requires_grad_(True)      # the `.float()` of the caller
+    z = torch.index_select(leaf, 0, sel) / T
     if t_T is None:
         t_T = T
     if t_logits is not None:
@@ -219,6 +219,17 @@ def mean_loss_and_grad(kind: str, logits: torch.Tensor, T: float, *,
     loss = rows.mean()
     loss.backward()
     return loss.detach(), rows.detach(), leaf.grad.detach()
+
+
+def storage_tolerance(ref: torch.Tensor, storage_dtype, rtol: float) -> torch.Tensor:
+    """Element-wise bound for comparing a gradient stored in `storage_dtype` with an
+    unrounded reference: `rtol` on the value plus the half-ulp the round-to-nearest
+    store may add (bf16 2^-8, fp16 2^-11 relative; fp16 also its subnormal spacing),
+    plus fp32 epsilon on the scale of the largest entry (entries that should be exactly
+    zero come out of the float64 autograd as ~1e-20 cancellation residue)."""
+    half_ulp = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[storage_dtype]
+    floor = {torch.float32: 1e-30, torch.bfloat16: 1e-30, torch.float16: 2.0 ** -25}[storage_dtype]
+    return ref.abs() * (rtol + half_ulp) + floor + 1.2e-7 * ref.abs().max()
 
 
 # ---------------------------------------------------------------------------

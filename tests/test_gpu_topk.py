@@ -1,0 +1,167 @@
+"""GPU parity of the sparse-teacher kernels (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-3, torch.float16: 2e-3}
+
+
+@pytest.fixture(scope="module")
+def D():
+    import llm_distillery_amd as d
+    d._lib.load()
+    return d
+
+
+def _case(R, V, K, dtype, seed, std=2.0, idx_dtype=torch.int32, val_dtype=torch.float16):
+    g = torch.Generator().manual_seed(seed)
+    logits = (torch.randn(R, V, generator=g) * std).to(dtype)
+    tl = torch.log_softmax(logits.float() + torch.randn(R, V, generator=g), -1)
+    tv, ti = torch.topk(tl, K)
+    return logits, tv.to(val_dtype), ti.to(idx_dtype)
+
+
+def _check(D, kind, logits, tv, ti, T, valid=None, teacher_T=None, **tol_over):
+    R, V = logits.shape
+    n_valid = R if valid is None else int(valid.sum())
+    loss64, rows64, grad64 = O.mean_loss_and_grad(kind, logits, T, t_vals=tv, t_idx=ti, valid=valid, t_T=teacher_T,
+                                             dtype=torch.float64)
+    row_map = None
+    if valid is not None:
+        rm = torch.full((R,), -1, dtype=torch.int32)
+        rm[valid] = torch.arange(n_valid, dtype=torch.int32)
+        row_map = rm.to(DEV)
+    rl, grad = D.div_topk(kind, logits.to(DEV), tv.to(DEV), ti.to(DEV), row_map=row_map, T=T, teacher_T=teacher_T,
+                          grad_scale=1.0 / n_valid)
+    loss = D.reduce_sum(rl, 1.0 / n_valid)
+    torch.cuda.synchronize()
+    rows_gpu = rl.cpu()
+    if valid is not None:
+        assert torch.count_nonzero(rows_gpu[~valid]) == 0
+        assert torch.count_nonzero(grad.cpu()[~valid]) == 0
+        rows_gpu = rows_gpu[valid]
+    # loss: 1e-5 relative against the float64 oracle (fp32 accumulation in the kernel)
+    np.testing.assert_allclose(loss.item(), loss64.item(), rtol=1e-5)
+    np.testing.assert_allclose(rows_gpu.double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+    # gradients: 1e-4 relative (fp32 logits) / 2e-3 (16-bit logits) on the value, plus the half
+    # ulp that storing the gradient in the logits' dtype may add
+    rtol = tol_over.get("rtol", TOL[logits.dtype])
+    err = (grad.cpu().double() - grad64).abs()
+    bound = O.storage_tolerance(grad64, logits.dtype, rtol)
+    bad = err > bound
+    assert not bad.any(), f"{int(bad.sum())} gradient entries off; worst ratio {(err / bound).max().item():.3f}"
+    return grad
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind", ["fkl", "rkl"])
+def test_topk_small(D, dtype, kind):
+    logits, tv, ti = _case(37, 1024, 24, dtype, 1)
+    _check(D, kind, logits, tv, ti, T=1.0)
+
+
+@pytest.mark.parametrize("V,K", [(32000, 200), (128256, 200), (50264, 64), (8192, 400)])
+def test_fkl_topk_register_path_sizes(D, V, K):
+    logits, tv, ti = _case(24, V, K, torch.bfloat16, 2, std=3.0)
+    _check(D, "fkl", logits, tv, ti, T=1.0)
+
+
+def test_fkl_topk_fp32_vocab_32000_temperature_and_mask(D):
+    logits, tv, ti = _case(40, 32000, 100, torch.float32, 3)
+    valid = torch.ones(40, dtype=torch.bool)
+    valid[[3, 4, 17, 39]] = False
+    _check(D, "fkl", logits, tv[:36], ti[:36], T=2.0, valid=valid)
+    _check(D, "rkl", logits, tv[:36], ti[:36], T=0.7, valid=valid)
+
+
+def test_validation_asymmetry_teacher_not_scaled(D):
+    # classes/student/model.py:501-502: the student is divided by T, the teacher is not
+    logits, tv, ti = _case(16, 4096, 32, torch.float32, 4)
+    _check(D, "fkl", logits, tv, ti, T=1.7, teacher_T=1.0)
+
+
+@pytest.mark.parametrize("V", [1000, 32003, 130001])
+def test_streaming_path_odd_vocab_and_int64_fp32_teacher(D, V):
+    # V not a multiple of the 16-byte chunk -> streaming kernel; teacher as the reference loads it (fp32/int64)
+    logits, tv, ti = _case(9, V, 50, torch.bfloat16, 5, idx_dtype=torch.int64, val_dtype=torch.float32)
+    _check(D, "fkl", logits, tv, ti, T=1.3)
+    _check(D, "rkl", logits, tv, ti, T=1.3)
+
+
+def test_streaming_path_rows_larger_than_register_file(D):
+    logits, tv, ti = _case(6, 152064, 200, torch.bfloat16, 6)
+    _check(D, "fkl", logits, tv, ti, T=1.0)
+    logits, tv, ti = _case(4, 100000, 64, torch.float32, 7)
+    _check(D, "fkl", logits, tv, ti, T=1.0)
+
+
+def test_cropped_view_of_wider_model_vocab(D):
+    # classes/student/model.py:408 slices [:, :, :crop] out of the model's vocabulary
+    g = torch.Generator().manual_seed(8)
+    full = (torch.randn(2, 10, 32064, generator=g) * 2).to(torch.bfloat16)
+    crop = full[:, :, :32000]
+    flat = crop.reshape(20, 32000)
+    tl = torch.log_softmax(flat.float() + torch.randn(20, 32000, generator=g), -1)
+    tv, ti = torch.topk(tl, 40)
+    loss64, rows64, grad_ref = O.mean_loss_and_grad("fkl", flat, 1.0, t_vals=tv, t_idx=ti, dtype=torch.float32)
+    dev_full = full.to(DEV)
+    rl, grad = D.div_topk("fkl", dev_full[:, :, :32000], tv.to(DEV), ti.to(torch.int32).to(DEV), grad_scale=1 / 20)
+    assert grad.shape == (2, 10, 32000)
+    np.testing.assert_allclose(rl.cpu().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+    err = (grad.cpu().float().reshape(20, -1) - grad_ref).abs()
+    assert (err <= O.storage_tolerance(grad_ref, torch.bfloat16, 2e-3)).all()
+
+
+def test_duplicate_ids_ragged_counts_and_out_of_range_ids(D):
+    g = torch.Generator().manual_seed(9)
+    R, V, K = 12, 2048, 16
+    logits = (torch.randn(R, V, generator=g) * 2)
+    ti = torch.randint(0, V, (R, K), generator=g)
+    ti[:, 5] = ti[:, 2]                  # duplicates inside a row accumulate
+    tv = torch.randn(R, K, generator=g)
+    _check(D, "fkl", logits, tv, ti.to(torch.int32), T=1.0)
+    _check(D, "rkl", logits, tv, ti.to(torch.int32), T=1.0)
+    # ragged: only the first cnt entries count; ids outside [0, V) are ignored; empty rows give 0
+    cnt = torch.tensor([16, 1, 0, 7, 16, 3, 0, 9, 2, 16, 5, 11], dtype=torch.int32)
+    ti2 = ti.clone()
+    ti2[4, 3] = V + 5
+    ti2[9, 0] = -3
+    rl, grad = D.div_topk("fkl", logits.to(DEV), tv.to(DEV), ti2.to(torch.int32).to(DEV), t_cnt=cnt.to(DEV))
+    rl, grad = rl.cpu(), grad.cpu()
+    for r in range(R):
+        keep = [k for k in range(int(cnt[r])) if 0 <= int(ti2[r, k]) < V]
+        if not keep:
+            assert rl[r] == 0 and torch.count_nonzero(grad[r]) == 0
+            continue
+        z = logits[r:r + 1].double()
+        t = O.teacher_logprobs_topk(tv[r:r + 1, keep], 1.0, torch.float64)
+        ref = O.fwd_kl_topk_rows(z, t, ti2[r:r + 1, keep])
+        np.testing.assert_allclose(rl[r].item(), ref.item(), rtol=2e-5, atol=2e-6)
+
+
+def test_forward_only_and_bit_reproducible(D):
+    logits, tv, ti = _case(64, 32000, 200, torch.bfloat16, 10)
+    a = D.div_topk("fkl", logits.to(DEV), tv.to(DEV), ti.to(DEV), want_grad=False)
+    assert a[1] is None
+    b = D.div_topk("fkl", logits.to(DEV), tv.to(DEV), ti.to(DEV))
+    c = D.div_topk("fkl", logits.to(DEV), tv.to(DEV), ti.to(DEV))
+    assert torch.equal(a[0], b[0]) and torch.equal(b[0], c[0]) and torch.equal(b[1], c[1])
+    assert torch.equal(D.reduce_sum(b[0]), D.reduce_sum(c[0]))
+
+
+def test_errors_are_python_exceptions(D):
+    logits, tv, ti = _case(4, 512, 8, torch.float32, 11)
+    with pytest.raises(RuntimeError):
+        D.div_topk("fkl", logits, tv, ti)                         # CPU tensors: no fallback
+    with pytest.raises(RuntimeError):
+        D.div_topk("fkl", logits.to(DEV), tv.to(DEV), ti.to(DEV)[:, :4])
+    big = torch.zeros(2, 4096, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="exceeds"):
+        D.div_topk("fkl", torch.zeros(2, 8192, device=DEV), big, torch.zeros(2, 4096, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError):
+        D.div_topk("jsd", logits.to(DEV), tv.to(DEV), ti.to(DEV))

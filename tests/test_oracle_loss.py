@@ -223,7 +223,7 @@ def test_alpha_weighted_special_cases():
     torch.testing.assert_close(k.grad, own / 3)
 
 
-def test_mean_loss_and_grad_masks_rows_and_rounds_to_storage_dtype():
+def test_mean_loss_and_grad_masks_rows():
     g = torch.Generator().manual_seed(10)
     R, V, K = 8, 64, 6
     logits = (torch.randn(R, V, generator=g) * 2).to(torch.bfloat16)
@@ -231,8 +231,8 @@ def test_mean_loss_and_grad_masks_rows_and_rounds_to_storage_dtype():
     nv = int(valid.sum())
     tv, ti = torch.topk(torch.log_softmax(torch.randn(nv, V, generator=g), -1), K)
     loss, rows, grad = O.mean_loss_and_grad("fkl", logits, 2.0, t_vals=tv, t_idx=ti, valid=valid)
-    assert grad.dtype == torch.bfloat16 and rows.shape == (nv,)
+    assert grad.dtype == torch.float32 and rows.shape == (nv,)
     assert torch.count_nonzero(grad[~valid]) == 0
     torch.testing.assert_close(loss, rows.mean())
     # every valid row's gradient sums to ~0 (softmax minus a distribution)
-    assert grad[valid].float().sum(-1).abs().max() < 1e-2
+    assert grad[valid].float().sum(-1).abs().max() < 1e-6
