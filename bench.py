@@ -1,0 +1,124 @@
+"""Benchmark of the distillation-loss hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--rows R]
+
+One step = one pass of the fused forward-KL loss + gradient over one batch of
+synthetic input (8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200
+fp16/int32 teacher, T=1) followed by the deterministic mean reduction.  Inputs are
+resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+V, K = 128256, 200
+BYTES_PER_TOKEN = V * 2 + V * 2 + K * (2 + 4)     # logits read + grad write + teacher (fp16 + int32)
+
+
+def cpu_baseline(rows: int, reps: int = 3):
+    """The reference's op sequence (cast -> /T -> log_softmax -> gather -> kl_div -> mean
+    -> backward) in PyTorch eager on the host cores, on a bounded row sample of the same
+    workload (rows are independent, so tokens/s carries over to the full row count)."""
+    import torch
+    from llm_distillery_amd import synthetic as S
+    from oracle import oracle as O
+
+    c = S.config3("cpu", rows=rows, seed=3)
+    O.mean_loss_and_grad("fkl", c["logits"][:64], 1.0, t_vals=c["t_val"][:64], t_idx=c["t_idx"][:64].long())
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        O.mean_loss_and_grad("fkl", c["logits"], 1.0, t_vals=c["t_val"], t_idx=c["t_idx"].long())
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{rows} of 32768 rows at V={V}, K={K}, fp32 eager oracle fwd+bwd, median of {reps} "
+                      f"({med:.2f} s each; os.cpu_count()={os.cpu_count()})"}
+
+
+def measured_traffic():
+    """HBM bytes per launch from the committed rocprofv3 counter summary, if present."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get("fkl_topk_c3_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--rows", type=int, default=8 * 4096)
+    ap.add_argument("--cpu-rows", type=int, default=1024, help="row sample for the CPU baseline (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path is row-parallel and every configuration fits one "
+                 "MI355X; run with --gpus 1")
+
+    import torch
+    import llm_distillery_amd as D
+    from llm_distillery_amd import synthetic as S
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    rows = args.rows
+    c = S.config3(dev, rows=rows, seed=3)
+    logits, t_val, t_idx = c["logits"], c["t_val"], c["t_idx"]
+    grad = torch.empty_like(logits)
+    scale = 1.0 / rows
+
+    def step():
+        row_loss, _ = D.div_topk("fkl", logits, t_val, t_idx, T=1.0, grad_scale=scale, grad_out=grad)
+        return D.reduce_sum(row_loss, scale)
+
+    for _ in range(args.warmup):
+        loss = step()
+    torch.cuda.synchronize()
+
+    # per-launch duration of the dominant kernel: events on the stream the kernel runs on
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        row_loss, _ = D.div_topk("fkl", logits, t_val, t_idx, T=1.0, grad_scale=scale, grad_out=grad)
+        b.record()
+        loss = D.reduce_sum(row_loss, scale)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    ms_per_step = wall * 1e3 / args.steps
+    algo_bytes = rows * BYTES_PER_TOKEN
+    achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "tokens/sec fused KL fwd+bwd @ vocab 128256 bf16; % of HBM peak GB/s",
+        "value": rows / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"C3 forward-KL fwd+bwd, top-K={K} fp16/int32 teacher, {rows} tokens x {V} vocab "
+                               "bf16 logits, T=1, bf16 gradient", "rows": rows, "vocab": V, "topk": K},
+        "loss": loss.item(),
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(),
+                     "kernel": "fkl_topk_reg_kernel<bf16,1024,16>", "kernel_ms": kern_ms,
+                     "algorithmic_bytes": algo_bytes},
+        "cpu_baseline": cpu_baseline(args.cpu_rows) if args.cpu_rows > 0 else None,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
