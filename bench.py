@@ -62,6 +62,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--rows", type=int, default=8 * 4096)
     ap.add_argument("--cpu-rows", type=int, default=1024, help="row sample for the CPU baseline (0 = skip)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch the library's plain copy kernel over the logits buffer (known traffic: "
+                         "rows*V*2 bytes each way), the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is row-parallel and every configuration fits one "
@@ -86,6 +89,10 @@ def main():
     for _ in range(args.warmup):
         loss = step()
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        for _ in range(3):
+            D.copy16(logits, grad)
+        torch.cuda.synchronize()
 
     # per-launch duration of the dominant kernel: events on the stream the kernel runs on
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]

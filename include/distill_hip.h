@@ -46,6 +46,15 @@ int dl_abi_version(void);
 const char* dl_status_string(int status);
 
 /*
+ * Process-wide tuning / test hooks (no reference counterpart).  Names:
+ *   "split_parts"  0 = automatic (default), 1 / 2 / 4 = column parts a wide row is cut into;
+ *   "spin_limit"   polls a part of a split row waits for its partners before it recomputes the
+ *                  row statistics alone (default 20000; 0 = never wait, exercises that path).
+ * Returns DL_ERR_DTYPE for an unknown name, DL_ERR_SHAPE for a value out of range.
+ */
+int dl_set_option(const char* name, int value);
+
+/*
  * Forward or reverse KL against a sparse (top-K) teacher, loss and gradient in one sweep.
  * Replaces, for one launch over all token rows:
  *   classes/student/model.py:408,420-421   slice + .float() + /T, row select, teacher /T
@@ -64,6 +73,11 @@ const char* dl_status_string(int status);
  * row_loss   [n_rows] fp32 per-token divergence (optional, may be NULL).
  * grad       [n_rows, V] (stride `grad_stride`), same dtype as logits; receives
  *            d(sum_r row_loss[r]) / d logits * grad_scale (optional, NULL = forward only).
+ * workspace  optional scratch of at least dl_div_topk_workspace_bytes(...) bytes, 16-byte aligned,
+ *            contents irrelevant on entry and on return.  Rows too wide for one workgroup's share
+ *            of the register file are cut into column parts that meet through it; without a
+ *            workspace (NULL or too small) such rows take a slower one-workgroup-per-row kernel.
+ *            Two launches that may overlap in time must not share a workspace.
  * K <= DL_MAX_TOPK.
  */
 int dl_div_topk(int kind,
@@ -72,7 +86,11 @@ int dl_div_topk(int kind,
                 const void* t_val, int t_val_dtype, const void* t_idx, int t_idx_itype, int K,
                 int64_t n_teacher_rows, const int32_t* t_cnt,
                 float inv_T_student, float inv_T_teacher, float grad_scale,
-                float* row_loss, void* grad, int64_t grad_stride, void* stream);
+                float* row_loss, void* grad, int64_t grad_stride,
+                void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Scratch size dl_div_topk can make use of for this problem (0 = none needed).  Host-only. */
+int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V);
 
 /*
  * Deterministic sum of n fp32 values times `scale` into out[0] (fixed reduction tree,
@@ -80,6 +98,13 @@ int dl_div_topk(int kind,
  * the `+=` accumulation of classes/losses.py:43-47.
  */
 int dl_reduce_sum(const float* values, int64_t n, float scale, float* out, void* stream);
+
+/*
+ * Plain 16-byte streaming copy of n_bytes (a multiple of 16; both pointers 16-byte aligned).
+ * No reference counterpart: it is the calibration kernel of known traffic that the HBM
+ * counters (FETCH_SIZE / WRITE_SIZE) of the loss kernels are scaled by.
+ */
+int dl_copy16(const void* src, void* dst, int64_t n_bytes, void* stream);
 
 #ifdef __cplusplus
 }

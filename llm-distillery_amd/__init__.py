@@ -4,6 +4,6 @@ Hand-written gfx950 HIP kernels behind a C ABI (libdistill_hip.so), exposed
 through the reference's own Python boundary (`calculate_divergence`, `Losses`).
 """
 from . import _lib  # noqa: F401
-from .ops import div_topk, reduce_sum  # noqa: F401
+from .ops import copy16, div_topk, reduce_sum, set_option  # noqa: F401
 
-__all__ = ["div_topk", "reduce_sum"]
+__all__ = ["copy16", "div_topk", "reduce_sum", "set_option"]

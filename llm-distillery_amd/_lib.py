@@ -24,8 +24,11 @@ _SIGNATURES = {
     "dl_abi_version": (c_int, []),
     "dl_status_string": (c_char_p, [c_int]),
     "dl_div_topk": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, _P, c_int, c_int, c_int64, _P,
-                            c_float, c_float, c_float, _P, _P, c_int64, _P]),
+                            c_float, c_float, c_float, _P, _P, c_int64, _P, c_int64, _P]),
+    "dl_div_topk_workspace_bytes": (c_int64, [c_int, c_int, c_int64, c_int64]),
+    "dl_set_option": (c_int, [c_char_p, c_int]),
     "dl_reduce_sum": (c_int, [_P, c_int64, c_float, _P, _P]),
+    "dl_copy16": (c_int, [_P, _P, c_int64, _P]),
 }
 
 _lib = None

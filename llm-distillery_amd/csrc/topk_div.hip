@@ -1,20 +1,27 @@
 // Forward / reverse KL against a sparse (top-K) teacher: loss and gradient in one sweep.
 //
-// One workgroup per token row.  Forward KL needs the full-vocabulary
-// log-sum-exp of the student row, so the row is pulled into registers with
-// 16-byte non-temporal loads (read from HBM once), reduced, and the gradient
+// Forward KL needs the full-vocabulary log-sum-exp of the student row, so the row is pulled
+// into registers with 16-byte non-temporal loads (read from HBM once), reduced, and the gradient
 //     d kl / d logit_j = (softmax(z)_j - sum_k q_k [j == idx_k]) * inv_T * scale
-// is produced from the same registers: a dense softmax sweep, then K sparse
-// corrections after a workgroup barrier.  The K teacher entries (id, log-prob,
-// gathered student logit) live in LDS.
+// is produced from the same registers: a dense softmax sweep, then K sparse corrections after a
+// workgroup barrier.  The K teacher entries (id, log-prob, gathered student logit) live in LDS.
 //
-// Reverse KL (student renormalised over the K ids) touches only the K gathered
-// logits; its gradient row is a zero fill plus K sparse values.
+// A 128256-entry bf16 row is 250 KB, half of a CU's register file, so a workgroup that holds a
+// whole row runs alone on its CU and its load / arithmetic / store phases cannot overlap.  The
+// split kernel therefore cuts a row into P column parts, one workgroup each; several parts of
+// different rows share a CU and hide each other's phases.  The parts of a row exchange their
+// (max, sum-exp, partial loss) through a small workspace in global memory; the wait on the
+// partner is bounded, and a part that gives up recomputes the row statistics on its own.
 //
-// Rows that do not fit the register file (or break the 16-byte alignment rules)
-// take the streaming kernel, which reads the row twice.
+// Reverse KL (student renormalised over the K ids) touches only the K gathered logits; its
+// gradient row is a zero fill plus K sparse values.
+//
+// Rows that do not fit (or break the 16-byte alignment rules) take the streaming kernel, which
+// reads the row twice.
 #include "distill_common.hpp"
 #include "distill_hip.h"
+#include <atomic>
+#include <cstring>
 
 namespace dl {
 
@@ -25,116 +32,223 @@ struct TopkParams {
   int64_t n_trows; const int32_t* t_cnt;
   float inv_T_s, inv_T_t, grad_scale;
   float* row_loss; void* grad; int64_t grad_stride;
+  void* workspace; int parts; int spin_limit;
 };
 
-// LDS carve-up shared by the kernels of this file.
-struct TopkLds {
-  float* red;   // 2 * (NT/64) floats, padded to 64
-  int* idx;     // K   vocabulary id or -1
-  float* t;     // K   scaled teacher logit -> teacher prob q_k
-  float* z;     // K   gathered student logit -> student prob at the id
-  __device__ TopkLds(unsigned char* base, int K) {
-    red = reinterpret_cast<float*>(base);
-    idx = reinterpret_cast<int*>(base + 256);
-    t = reinterpret_cast<float*>(idx + K);
-    z = t + K;
+constexpr int MAX_PARTS = 8;
+
+// What one part of a split row tells the others: three floats and a tag that depends on all of
+// them.  The four words are written and read with relaxed device-scope accesses (they bypass the
+// non-coherent cache levels; no cache-wide flush or invalidate); a reader accepts a record only
+// when the tag matches, so no ordering between the words is needed.  A cleared record is invalid.
+struct PartStats { unsigned m, s, b, tag; };
+__device__ __forceinline__ unsigned part_tag(unsigned m, unsigned s, unsigned b) {
+  return m ^ ((s << 7) | (s >> 25)) ^ ((b << 13) | (b >> 19)) ^ 0x5eed1234u;
+}
+__device__ __forceinline__ void part_publish(PartStats* w, float m, float s, float b) {
+  const unsigned um = __float_as_uint(m), us = __float_as_uint(s), ub = __float_as_uint(b);
+  __hip_atomic_store(&w->m, um, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->s, us, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->b, ub, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->tag, part_tag(um, us, ub), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Bounded wait for a partner's record; false = gave up after `limit` polls.
+__device__ __forceinline__ bool part_collect(PartStats* w, int limit, float& m, float& s, float& b) {
+  for (int spins = 0; spins < limit; ++spins) {
+    const unsigned um = __hip_atomic_load(&w->m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned us = __hip_atomic_load(&w->s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned ub = __hip_atomic_load(&w->b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned ut = __hip_atomic_load(&w->tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (ut == part_tag(um, us, ub)) {
+      m = __uint_as_float(um); s = __uint_as_float(us); b = __uint_as_float(ub);
+      return true;
+    }
+    __builtin_amdgcn_s_sleep(4);
   }
-  static size_t bytes(int K) { return 256 + (size_t)K * 12; }
+  return false;
+}
+
+// LDS carve-up shared by the kernels of this file.  The id array is padded to a multiple of 16
+// with -1 so that it can be scanned four ids per read.
+struct TopkLds {
+  float* red;        // reduction scratch, 64 floats
+  float* xm; float* xs; float* xb; int* xok;    // per-part statistics of a split row, MAX_PARTS each
+  int* idx;          // Kp  vocabulary id or -1
+  float* t;          // Kp  scaled teacher logit -> teacher log-probability over the K entries
+  float* q;          // Kp  teacher probability
+  float* z;          // Kp  gathered student logit
+  int Kp;
+  __device__ TopkLds(unsigned char* base, int K) {
+    Kp = (K + 15) & ~15;
+    red = reinterpret_cast<float*>(base);
+    xm = red + 64; xs = xm + MAX_PARTS; xb = xs + MAX_PARTS; xok = reinterpret_cast<int*>(xb + MAX_PARTS);
+    idx = reinterpret_cast<int*>(base + 512);
+    t = reinterpret_cast<float*>(idx + Kp);
+    q = t + Kp;
+    z = q + Kp;
+  }
+  __host__ __device__ static size_t bytes(int K) { return 512 + (size_t)((K + 15) & ~15) * 16; }
 };
 
-// Stage the teacher row: ids, scaled log-probs and the student logits at those ids.
-// Returns log-sum-exp of the scaled teacher entries (-inf if the row has none).
+// Stage the teacher row: ids, scaled log-probs, and the student logits at the ids that fall into
+// the column range [lo, hi) this workgroup owns.  Returns the log-sum-exp of the scaled teacher
+// entries (-inf if the row has none); afterwards s.t holds the teacher log-probabilities and s.q
+// the probabilities (0 for padding and ignored entries).
 template <class Tag, int NT>
 __device__ __forceinline__ float stage_teacher(const TopkParams& p, const TopkLds& s, int64_t trow,
-                                               const char* row) {
+                                               const char* row, int lo, int hi) {
   const int K = p.K;
   const int cnt = p.t_cnt ? min(p.t_cnt[trow], K) : K;
   float tmax = -INFINITY;
-  for (int k = threadIdx.x; k < K; k += NT) {
+  for (int k = threadIdx.x; k < s.Kp; k += NT) {
     const int64_t at = trow * (int64_t)K + k;
     const int64_t id = k < cnt ? load_index(p.t_idx, p.t_idx_itype, at) : -1;
     const bool ok = id >= 0 && id < p.V;
     const float tv = ok ? load_as_float(p.t_val, p.t_val_dtype, at) * p.inv_T_t : -INFINITY;
     s.idx[k] = ok ? (int)id : -1;
     s.t[k] = tv;
-    s.z[k] = ok ? load_as_float(row, Tag::id, id) : 0.f;
+    s.z[k] = (ok && id >= lo && id < hi) ? load_as_float(row, Tag::id, id) : 0.f;
     tmax = fmaxf(tmax, tv);
   }
   tmax = block_max<NT>(tmax, s.red);     // barrier inside: LDS entries visible afterwards
   if (tmax == -INFINITY) return tmax;
   float part = 0.f;
-  for (int k = threadIdx.x; k < K; k += NT) part += expf(s.t[k] - tmax);
-  const float tsum = block_sum<NT>(part, s.red);
-  return tmax + logf(tsum);
+  for (int k = threadIdx.x; k < s.Kp; k += NT) part += expf(s.t[k] - tmax);
+  const float tlse = tmax + logf(block_sum<NT>(part, s.red));
+  for (int k = threadIdx.x; k < s.Kp; k += NT) {      // own entries only: no barrier needed yet
+    const float lt = s.t[k] - tlse;
+    s.t[k] = lt;
+    s.q[k] = expf(lt);
+  }
+  return tlse;
 }
 
-// Forward-KL row value; leaves q_k in s.t and the student probability at the id in s.z.
+// Partial forward-KL sums over the ids inside [lo, hi):  B = sum q_k (t_k - z_k * inv_T)  and, over
+// all ids, Q = sum q_k.  The row value is  sum over parts of B  +  lse * Q.
 template <int NT>
-__device__ __forceinline__ float fkl_from_staged(const TopkParams& p, const TopkLds& s, float tlse, float lse) {
-  float part = 0.f;
-  for (int k = threadIdx.x; k < p.K; k += NT) {
-    if (s.idx[k] >= 0) {
-      const float tk = s.t[k] - tlse;
-      const float sk = s.z[k] * p.inv_T_s - lse;
-      const float q = expf(tk);
-      part += q * (tk - sk);
-      s.t[k] = q;
-      s.z[k] = expf(sk);
-    } else {
-      s.t[k] = 0.f;
+__device__ __forceinline__ void fkl_partials(const TopkParams& p, const TopkLds& s, float tlse, int lo,
+                                             int hi, float& B, float& Q) {
+  B = 0.f; Q = 0.f;
+  for (int k = threadIdx.x; k < s.Kp; k += NT) {
+    const int id = s.idx[k];
+    if (id >= 0) {
+      const float q = s.q[k];
+      Q += q;
+      if (id >= lo && id < hi) B += q * (s.t[k] - s.z[k] * p.inv_T_s);
     }
   }
-  return block_sum<NT>(part, s.red);
+  block_sum2<NT>(B, Q, s.red);
 }
 
-// K sparse corrections of the dense softmax row already written by this workgroup.
-// Ids that occur more than once receive the summed teacher mass (every duplicate
-// writes the same value).
+// Teacher mass on the id of entry k, summed over every entry that carries the same id.
+__device__ __forceinline__ float mass_on_id(const TopkLds& s, int k, int id) {
+  int same = 0;
+  const int4* ids = reinterpret_cast<const int4*>(s.idx);
+#pragma unroll 4
+  for (int j = 0; j < s.Kp / 4; ++j) {
+    const int4 v = ids[j];
+    same += (v.x == id) + (v.y == id) + (v.z == id) + (v.w == id);
+  }
+  if (same == 1) return s.q[k];
+  float q = 0.f;                        // duplicates inside a row are rare: slow path
+  for (int j = 0; j < s.Kp; ++j) q += (s.idx[j] == id) ? s.q[j] : 0.f;
+  return q;
+}
+
+// Sparse corrections of the dense softmax row already written by this workgroup, for the ids
+// inside [lo, hi).  b is the row's log2-sum-exp2, a = inv_T * log2(e), c = inv_T * scale.
 template <class Tag, int NT>
-__device__ __forceinline__ void fkl_sparse_fix(const TopkParams& p, const TopkLds& s, void* grow, float c) {
-  for (int k = threadIdx.x; k < p.K; k += NT) {
+__device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int lo, int hi,
+                                               float a, float b, float c) {
+  for (int k = threadIdx.x; k < s.Kp; k += NT) {
     const int id = s.idx[k];
-    if (id < 0) continue;
-    float q = 0.f;
-    for (int j = 0; j < p.K; ++j) q += (s.idx[j] == id) ? s.t[j] : 0.f;
-    store_from_float(grow, Tag::id, id, (s.z[k] - q) * c);
+    if (id < lo || id >= hi) continue;
+    const float q = mass_on_id(s, k, id);
+    store_from_float(grow, Tag::id, id, (fast_exp2(fmaf(s.z[k], a, -b)) - q) * c);
   }
 }
 
+// Full-row statistics straight from global memory (two uses: the streaming kernel, and a split
+// part whose partner did not answer in time).  Returns the row maximum and sum 2^((x - max) a).
+template <class Tag, int NT, bool VEC>
+__device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, float a, float* red, float& mx,
+                                                   float& sm) {
+  using C = Chunk<Tag>;
+  float m = -INFINITY;
+  sm = 0.f;
+  if (VEC) {
+    for (int64_t ch = threadIdx.x; ch < V / C::N; ch += NT) {
+      float f[C::N];
+      C::unpack(*reinterpret_cast<const u32x4*>(row + ch * 16), f);
+      float cm = f[0];
+#pragma unroll
+      for (int e = 1; e < C::N; ++e) cm = fmaxf(cm, f[e]);
+      if (cm > m) { sm *= fast_exp2((m - cm) * a); m = cm; }
+      const float mb = m * a;
+#pragma unroll
+      for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[e], a, -mb));
+    }
+  } else {
+    for (int64_t j = threadIdx.x; j < V; j += NT) {
+      const float f = load_as_float(row, Tag::id, j);
+      if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
+      sm += fast_exp2(fmaf(f, a, -m * a));
+    }
+  }
+  mx = block_max<NT>(m, red);
+  sm = (m == -INFINITY) ? 0.f : sm * fast_exp2((m - mx) * a);
+  sm = block_sum<NT>(sm, red);
+}
+
 // ---------------------------------------------------------------------------------------
-// Forward KL, row resident in registers: NT threads x NCH 16-byte chunks per thread.
+// Forward KL, (part of) a row resident in registers: NT threads x NCH 16-byte chunks per thread.
+// SPLIT: P = p.parts workgroups per row.  Consecutive workgroup ids are dealt round-robin to the 8
+// XCDs, each of which dispatches its share in order, so the parts of a row are placed 8 ids apart:
+// they land on the same XCD back to back (partners start together and meet through one L2).
+// Within a group of 8*P ids, id t serves row 8*group + t % 8, part t / 8.
 // ---------------------------------------------------------------------------------------
-template <class Tag, int NT, int NCH>
-__global__ __launch_bounds__(NT) void fkl_topk_reg_kernel(const TopkParams p) {
+template <class Tag, int NT, int NCH, bool SPLIT>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))     // <= 128 VGPRs: 16 waves per CU
+void fkl_topk_reg_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const TopkLds s(smem, p.K);
   using C = Chunk<Tag>;
-  const int64_t r = blockIdx.x;
   const int tid = threadIdx.x;
-  const int64_t nch = p.V / C::N;
+  const int P = SPLIT ? p.parts : 1;
+  const unsigned grp = SPLIT ? blockIdx.x / (8u * P) : 0u, t_in = SPLIT ? blockIdx.x % (8u * P) : 0u;
+  const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : blockIdx.x;
+  const int h = SPLIT ? (int)(t_in >> 3) : 0;
+  if (SPLIT && r >= p.n_rows) return;
+  const int64_t c0 = (int64_t)h * NT * NCH;                       // first chunk of this part
+  const int64_t nch = min((int64_t)NT * NCH, p.V / C::N - c0);    // chunks of this part
+  const int lo = (int)(c0 * C::N), hi = lo + (int)(nch * C::N);   // its column range
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
+  char* gpart = grow ? grow + c0 * 16 : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   if (trow < 0) {
-    if (grow) zero_row<Tag, NT>(grow, nch);
-    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    if (gpart) zero_row<Tag, NT>(gpart, nch);
+    if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  const char* rpart = row + c0 * 16;
 
   u32x4 reg[NCH];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int64_t c = (int64_t)i * NT + tid;
-    reg[i] = c < nch ? load16_stream(row + c * 16) : C::neg_inf();
+    reg[i] = c < nch ? load16_stream(rpart + c * 16) : C::neg_inf();
   }
 
   // teacher side while the row is in flight
-  const float tlse = stage_teacher<Tag, NT>(p, s, trow, row);
+  const float tlse = stage_teacher<Tag, NT>(p, s, trow, row, lo, hi);
   if (tlse == -INFINITY) {            // no usable teacher entry: the row contributes nothing
-    if (grow) zero_row<Tag, NT>(grow, nch);
-    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    if (gpart) zero_row<Tag, NT>(gpart, nch);
+    if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
+  float B, Q;
+  fkl_partials<NT>(p, s, tlse, lo, hi, B, Q);
 
   const float a = p.inv_T_s * LOG2E;
   float mx = -INFINITY;
@@ -147,7 +261,7 @@ __global__ __launch_bounds__(NT) void fkl_topk_reg_kernel(const TopkParams p) {
     for (int e = 0; e < C::N; ++e) mx = fmaxf(mx, f[e]);
   }
   mx = block_max<NT>(mx, s.red);
-  const float mb = mx * a;
+  float mb = mx * a;
   float sm = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
@@ -158,13 +272,42 @@ __global__ __launch_bounds__(NT) void fkl_topk_reg_kernel(const TopkParams p) {
     for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[e], a, -mb));
   }
   sm = block_sum<NT>(sm, s.red);
+
+  if (SPLIT) {
+    // publish this part's statistics, collect the others'
+    PartStats* ws = reinterpret_cast<PartStats*>(p.workspace) + r * P;
+    if (tid == 0) part_publish(ws + h, mx, sm, B);
+    if (tid < P) {
+      float om = mx, os = sm, ob = B;
+      const int ok = (tid == h) || part_collect(ws + tid, p.spin_limit, om, os, ob);
+      s.xm[tid] = om; s.xs[tid] = os; s.xb[tid] = ob; s.xok[tid] = ok;
+    }
+    __syncthreads();
+    bool all_ok = true;
+    for (int j = 0; j < P; ++j) all_ok = all_ok && (s.xok[j] != 0);
+    if (all_ok) {
+      float M = s.xm[0];
+      for (int j = 1; j < P; ++j) M = fmaxf(M, s.xm[j]);
+      float S = 0.f, Bt = 0.f;
+      for (int j = 0; j < P; ++j) { S += s.xs[j] * fast_exp2((s.xm[j] - M) * a); Bt += s.xb[j]; }
+      mb = M * a; sm = S; B = Bt;
+    } else {
+      // a partner did not answer: rebuild the row statistics and the loss sum alone
+      __syncthreads();
+      for (int k = tid; k < s.Kp; k += NT) {
+        const int id = s.idx[k];
+        if (id >= 0 && (id < lo || id >= hi)) s.z[k] = load_as_float(row, Tag::id, id);
+      }
+      __syncthreads();
+      fkl_partials<NT>(p, s, tlse, 0, (int)p.V, B, Q);
+      row_stats_streamed<Tag, NT, true>(row, p.V, a, s.red, mx, sm);
+      mb = mx * a;
+    }
+  }
   const float b = mb + fast_log2(sm);      // log2-sum-exp2 of the scaled row
-  const float lse = b * LN2;
+  if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = B + (b * LN2) * Q;
 
-  const float kl = fkl_from_staged<NT>(p, s, tlse, lse);
-  if (tid == 0 && p.row_loss) p.row_loss[r] = kl;
-
-  if (grow) {
+  if (gpart) {
     const float c = p.inv_T_s * p.grad_scale;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -175,11 +318,11 @@ __global__ __launch_bounds__(NT) void fkl_topk_reg_kernel(const TopkParams p) {
         C::unpack(reg[i], f);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * c;
-        store16_stream(grow + ch * 16, C::pack(f));
+        store16_stream(gpart + ch * 16, C::pack(f));
       }
     }
-    __syncthreads();      // dense row stores are ordered before the sparse corrections
-    fkl_sparse_fix<Tag, NT>(p, s, grow, c);
+    __syncthreads();      // dense stores are ordered before the sparse corrections
+    fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c);
   }
 }
 
@@ -199,7 +342,7 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
   float tlse = -INFINITY;
-  if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row);
+  if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
   if (tlse == -INFINITY) {
     if (grow) {
       if (VEC) zero_row<Tag, NT>(grow, nch);
@@ -208,37 +351,13 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
+  float B, Q;
+  fkl_partials<NT>(p, s, tlse, 0, (int)V, B, Q);
   const float a = p.inv_T_s * LOG2E;
-  // pass 1: per-thread running (max, sum) in the exp2 domain
-  float m = -INFINITY, sm = 0.f;
-  if (VEC) {
-    for (int64_t ch = tid; ch < nch; ch += NT) {
-      float f[C::N];
-      C::unpack(*reinterpret_cast<const u32x4*>(row + ch * 16), f);
-      float cm = f[0];
-#pragma unroll
-      for (int e = 1; e < C::N; ++e) cm = fmaxf(cm, f[e]);
-      if (cm > m) { sm *= fast_exp2((m - cm) * a); m = cm; }
-      const float mb = m * a;
-#pragma unroll
-      for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[e], a, -mb));
-    }
-  } else {
-    for (int64_t j = tid; j < V; j += NT) {
-      const float f = load_as_float(row, Tag::id, j);
-      if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
-      sm += fast_exp2(fmaf(f, a, -m * a));
-    }
-  }
-  const float mx = block_max<NT>(m, s.red);
-  const float mb = mx * a;
-  sm = (m == -INFINITY) ? 0.f : sm * fast_exp2(fmaf(m, a, -mb));
-  sm = block_sum<NT>(sm, s.red);
-  const float b = mb + fast_log2(sm);
-  const float lse = b * LN2;
-
-  const float kl = fkl_from_staged<NT>(p, s, tlse, lse);
-  if (tid == 0 && p.row_loss) p.row_loss[r] = kl;
+  float mx, sm;
+  row_stats_streamed<Tag, NT, VEC>(row, V, a, s.red, mx, sm);
+  const float b = mx * a + fast_log2(sm);
+  if (tid == 0 && p.row_loss) p.row_loss[r] = B + (b * LN2) * Q;
 
   if (grow) {
     const float c = p.inv_T_s * p.grad_scale;
@@ -255,7 +374,7 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
         store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * c);
     }
     __syncthreads();
-    fkl_sparse_fix<Tag, NT>(p, s, grow, c);
+    fkl_sparse_fix<Tag, NT>(s, grow, 0, (int)V, a, b, c);
   }
 }
 
@@ -278,28 +397,28 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
   float tlse = -INFINITY;
-  if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row);
+  if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
   if (tlse == -INFINITY) {
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
   // student renormalised over the staged ids
   float zm = -INFINITY;
-  for (int k = tid; k < p.K; k += NT)
+  for (int k = tid; k < s.Kp; k += NT)
     if (s.idx[k] >= 0) zm = fmaxf(zm, s.z[k] * p.inv_T_s);
   zm = block_max<NT>(zm, s.red);
   float part = 0.f;
-  for (int k = tid; k < p.K; k += NT)
+  for (int k = tid; k < s.Kp; k += NT)
     if (s.idx[k] >= 0) part += expf(s.z[k] * p.inv_T_s - zm);
   const float slse = zm + logf(block_sum<NT>(part, s.red));
   part = 0.f;
-  for (int k = tid; k < p.K; k += NT) {
+  for (int k = tid; k < s.Kp; k += NT) {
     if (s.idx[k] >= 0) {
       const float sp = s.z[k] * p.inv_T_s - slse;
-      const float d = sp - (s.t[k] - tlse);
+      const float d = sp - s.t[k];
       const float rk = expf(sp);
       part += rk * d;
-      s.t[k] = rk;      // student mass on the support
+      s.q[k] = rk;      // student mass on the support
       s.z[k] = d;       // log ratio
     }
   }
@@ -308,14 +427,20 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   if (grow) {
     const float c = p.inv_T_s * p.grad_scale;
     __syncthreads();    // zero fill precedes the sparse values
-    for (int k = tid; k < p.K; k += NT) {
+    for (int k = tid; k < s.Kp; k += NT) {
       const int id = s.idx[k];
       if (id < 0) continue;
       float g = 0.f;
-      for (int j = 0; j < p.K; ++j) g += (s.idx[j] == id) ? s.t[j] * (s.z[j] - rkl) : 0.f;
+      for (int j = 0; j < s.Kp; ++j) g += (s.idx[j] == id) ? s.q[j] * (s.z[j] - rkl) : 0.f;
       store_from_float(grow, Tag::id, id, g * c);
     }
   }
+}
+
+// clears the `ready` words of the split kernel's workspace
+__global__ __launch_bounds__(256) void clear_workspace_kernel(u32x4* ws, int64_t n16) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) ws[i] = u32x4{0u, 0u, 0u, 0u};
 }
 
 // ---------------------------------------------------------------------------------------
@@ -323,20 +448,50 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
 // ---------------------------------------------------------------------------------------
 template <class Tag, int NT, int NCH>
 static hipError_t launch_reg(const TopkParams& p, hipStream_t st) {
-  hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH>), dim3((unsigned)p.n_rows), dim3(NT),
+  hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, false>), dim3((unsigned)p.n_rows), dim3(NT),
                      TopkLds::bytes(p.K), st, p);
   return hipGetLastError();
 }
 
+template <class Tag, int NT, int NCH>
+static hipError_t launch_split(TopkParams p, int parts, hipStream_t st) {
+  p.parts = parts;
+  const int64_t n16 = p.n_rows * parts;          // one 16-byte PartStats per (row, part)
+  hipLaunchKernelGGL(clear_workspace_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
+                     reinterpret_cast<u32x4*>(p.workspace), n16);
+  hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, true>), dim3((unsigned)((p.n_rows + 7) / 8 * 8 * parts)), dim3(NT),
+                     TopkLds::bytes(p.K), st, p);
+  return hipGetLastError();
+}
+
+// Library options (dl_set_option): tuning and test hooks, process-wide.
+static std::atomic<int> g_split_parts{0};       // 0 = automatic, else 1 / 2 / 4
+static std::atomic<int> g_spin_limit{20000};    // polls a part waits for a partner; 0 = never wait
+
+// Number of column parts a row of `nch` 16-byte chunks is cut into (1 = one workgroup per row).
+static int split_parts(int64_t nch) {
+  if (nch <= 512 * 16) return 1;
+  const int forced = g_split_parts.load();
+  if (forced == 1 || forced == 2 || forced == 4) return forced;
+  return 4;
+}
+
 template <class Tag>
-static hipError_t launch_fkl(const TopkParams& p, bool aligned, hipStream_t st) {
+static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipStream_t st) {
   const int64_t nch = p.V / Tag::epc;
   if (aligned) {
     if (nch <= 256 * 4) return launch_reg<Tag, 256, 4>(p, st);
     if (nch <= 256 * 8) return launch_reg<Tag, 256, 8>(p, st);
     if (nch <= 256 * 16) return launch_reg<Tag, 256, 16>(p, st);
     if (nch <= 512 * 16) return launch_reg<Tag, 512, 16>(p, st);
-    if (nch <= 1024 * 16) return launch_reg<Tag, 1024, 16>(p, st);
+    if (nch <= 1024 * 16) {
+      const int parts = split_parts(nch);
+      const bool ws_ok = p.workspace && ws_bytes >= p.n_rows * parts * (int64_t)sizeof(PartStats) &&
+                         p.n_rows * parts <= 0x7fffffffLL;
+      if (parts == 2 && ws_ok) return launch_split<Tag, 512, 16>(p, 2, st);
+      if (parts == 4 && ws_ok) return launch_split<Tag, 256, 16>(p, 4, st);
+      return launch_reg<Tag, 1024, 16>(p, st);
+    }
     hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, true>), dim3((unsigned)p.n_rows), dim3(1024),
                        TopkLds::bytes(p.K), st, p);
   } else {
@@ -357,13 +512,37 @@ static hipError_t launch_rkl(const TopkParams& p, bool aligned, hipStream_t st) 
   return hipGetLastError();
 }
 
+static int spin_limit() { return g_spin_limit.load(); }
+
 }  // namespace dl
+
+extern "C" int dl_set_option(const char* name, int value) {
+  if (!name) return DL_ERR_NULL;
+  if (!strcmp(name, "split_parts")) {
+    if (value != 0 && value != 1 && value != 2 && value != 4) return DL_ERR_SHAPE;
+    dl::g_split_parts.store(value);
+    return DL_OK;
+  }
+  if (!strcmp(name, "spin_limit")) {
+    if (value < 0) return DL_ERR_SHAPE;
+    dl::g_spin_limit.store(value);
+    return DL_OK;
+  }
+  return DL_ERR_DTYPE;
+}
+
+extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V) {
+  if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
+  const int64_t nch = V / (logits_dtype == DL_F32 ? 4 : 8);
+  if (nch <= 512 * 16 || nch > 1024 * 16) return 0;
+  return n_rows * dl::MAX_PARTS * (int64_t)sizeof(dl::PartStats);
+}
 
 extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
                            int64_t V, const int32_t* row_map, const void* t_val, int t_val_dtype,
                            const void* t_idx, int t_idx_itype, int K, int64_t n_teacher_rows,
                            const int32_t* t_cnt, float inv_T_student, float inv_T_teacher, float grad_scale, float* row_loss,
-                           void* grad, int64_t grad_stride, void* stream) {
+                           void* grad, int64_t grad_stride, void* workspace, int64_t workspace_bytes, void* stream) {
   using namespace dl;
   if (!logits || !t_val || !t_idx) return DL_ERR_NULL;
   if (kind != DL_FKL && kind != DL_RKL) return DL_ERR_DTYPE;
@@ -379,13 +558,14 @@ extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64
                        ((row_stride * eb) % 16 == 0) &&
                        (!grad || (reinterpret_cast<uintptr_t>(grad) % 16 == 0 && (grad_stride * eb) % 16 == 0));
   TopkParams p{logits, row_stride, n_rows, V, row_map, t_val, t_val_dtype, t_idx, t_idx_itype, K, n_teacher_rows,
-               t_cnt, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride};
+               t_cnt, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride,
+               (reinterpret_cast<uintptr_t>(workspace) % 16 == 0) ? workspace : nullptr, 1, spin_limit()};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   hipError_t e;
   if (kind == DL_FKL) {
-    e = logits_dtype == DL_F32 ? launch_fkl<TagF32>(p, aligned, st)
-        : logits_dtype == DL_BF16 ? launch_fkl<TagBF16>(p, aligned, st)
-                                  : launch_fkl<TagF16>(p, aligned, st);
+    e = logits_dtype == DL_F32 ? launch_fkl<TagF32>(p, aligned, workspace_bytes, st)
+        : logits_dtype == DL_BF16 ? launch_fkl<TagBF16>(p, aligned, workspace_bytes, st)
+                                  : launch_fkl<TagF16>(p, aligned, workspace_bytes, st);
   } else {
     e = logits_dtype == DL_F32 ? launch_rkl<TagF32>(p, aligned, st)
         : logits_dtype == DL_BF16 ? launch_rkl<TagBF16>(p, aligned, st)

@@ -89,11 +89,14 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
             raise RuntimeError("grad_out must match logits as a [rows, V] tensor")
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
     lib = _lib.load()
+    ws_bytes = lib.dl_div_topk_workspace_bytes(KINDS[kind], _DT[x.dtype], R, V) if want_grad else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     with torch.cuda.device(dev):
         st = lib.dl_div_topk(KINDS[kind], x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr,
                              t_val.data_ptr(), _DT[t_val.dtype], t_idx.data_ptr(), _IT[t_idx.dtype], K, N,
                              cnt_ptr, 1.0 / T, 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
-                             row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
+                             row_loss.data_ptr(), g_ptr, g_stride,
+                             ws.data_ptr() if ws is not None else 0, ws_bytes, _stream_ptr(dev))
     _lib.check(st, "dl_div_topk")
     if grad is not None and logits.dim() != 2 and grad_out is None:
         grad = grad.view(logits.shape)
@@ -111,3 +114,19 @@ def reduce_sum(values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
         st = _lib.load().dl_reduce_sum(v.data_ptr(), v.numel(), scale, out.data_ptr(), _stream_ptr(v.device))
     _lib.check(st, "dl_reduce_sum")
     return out
+
+
+def copy16(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """Streaming copy of src's bytes into dst (the calibration kernel for HBM counters)."""
+    _dev(src, "src"), _dev(dst, "dst")
+    n = src.numel() * src.element_size()
+    if not (src.is_contiguous() and dst.is_contiguous()) or dst.numel() * dst.element_size() != n:
+        raise RuntimeError("copy16 needs two contiguous buffers of the same byte size")
+    with torch.cuda.device(src.device):
+        st = _lib.load().dl_copy16(src.data_ptr(), dst.data_ptr(), n, _stream_ptr(src.device))
+    _lib.check(st, "dl_copy16")
+
+
+def set_option(name: str, value: int) -> None:
+    """Process-wide tuning / test hooks of the library ("split_parts", "spin_limit")."""
+    _lib.check(_lib.load().dl_set_option(name.encode(), int(value)), f"dl_set_option({name!r})")

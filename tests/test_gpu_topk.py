@@ -165,3 +165,25 @@ def test_errors_are_python_exceptions(D):
         D.div_topk("fkl", torch.zeros(2, 8192, device=DEV), big, torch.zeros(2, 4096, dtype=torch.int32, device=DEV))
     with pytest.raises(ValueError):
         D.div_topk("jsd", logits.to(DEV), tv.to(DEV), ti.to(DEV))
+
+
+@pytest.mark.parametrize("parts", [1, 2, 4])
+def test_split_row_parts_agree_and_give_up_path(D, parts):
+    """A 128256-wide row is cut into column parts that exchange statistics through the workspace.
+    Every setting must give the oracle's numbers, also when no part waits for its partners
+    (spin_limit 0: each part then rebuilds the row statistics alone)."""
+    logits, tv, ti = _case(40, 128256, 200, torch.bfloat16, 12, std=3.0)
+    valid = torch.ones(40, dtype=torch.bool)
+    valid[[0, 7, 33]] = False
+    try:
+        D.set_option("split_parts", parts)
+        _check(D, "fkl", logits, tv[:37], ti[:37], T=1.0, valid=valid)
+        D.set_option("spin_limit", 0)
+        _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid)
+    finally:
+        D.set_option("split_parts", 0)
+        D.set_option("spin_limit", 20000)
+    with pytest.raises(RuntimeError):
+        D.set_option("split_parts", 3)
+    with pytest.raises(RuntimeError):
+        D.set_option("no_such_option", 1)
