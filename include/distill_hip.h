@@ -93,6 +93,32 @@ int dl_div_topk(int kind,
 int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V);
 
 /*
+ * Phase 1 of the general (two-phase) path: per valid row r with teacher row t = row_map[r],
+ *   lse[t]   = logsumexp_j(logits[r, j] * inv_T)                       (fp32, natural log)
+ *   zk[t, k] = logits[r, t_idx[t, k]] * inv_T                          (fp32; 0 for ids outside [0, V))
+ * Replaces classes/student/model.py:408,420 (slice, cast, /T, row select) and
+ * utils/finetuning_utils.py:88,92 (full-vocabulary log_softmax + gather): the student log-probs
+ * on the teacher's support are zk - lse.  Rows whose row_map entry is outside
+ * [0, n_teacher_rows) are skipped (their lse / zk entries are not written).
+ */
+int dl_rowstats_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                     const int32_t* row_map, const void* t_idx, int t_idx_itype, int K,
+                     int64_t n_teacher_rows, float inv_T, float* lse, float* zk, void* stream);
+
+/*
+ * Phase 2: the gradient of any scalar L that depends on the logits only through phase 1's
+ * outputs, given coef_lse[t] = dL/d lse[t] and coef_zk[t, k] = dL/d zk[t, k]:
+ *   grad[r, j] = ( coef_lse[t] * softmax(logits[r] * inv_T)_j + sum_k coef_zk[t, k] [j == t_idx[t, k]] ) * inv_T
+ * in the logits' dtype; masked rows are zero-filled.  `lse` is phase 1's output.
+ * Replaces the autograd replay (classes/losses.py:77-78) of log_softmax + gather + index_select
+ * + /T + cast.
+ */
+int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                         const int32_t* row_map, const void* t_idx, int t_idx_itype, int K,
+                         int64_t n_teacher_rows, float inv_T, const float* lse, const float* coef_lse,
+                         const float* coef_zk, void* grad, int64_t grad_stride, void* stream);
+
+/*
  * Deterministic sum of n fp32 values times `scale` into out[0] (fixed reduction tree,
  * double accumulation).  Replaces the `.mean()` of utils/finetuning_utils.py:54 /
  * the `+=` accumulation of classes/losses.py:43-47.

@@ -120,6 +120,8 @@ __device__ __forceinline__ int64_t load_index(const void* base, int itype, int64
 __device__ __forceinline__ u32x4 load16_stream(const void* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
+// Non-temporal stores: a bare copy kernel runs ~4 % faster with the default policy, but in the
+// loss kernels (sparse corrections follow the dense row) the non-temporal hint measured faster.
 __device__ __forceinline__ void store16_stream(void* p, const u32x4& v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }

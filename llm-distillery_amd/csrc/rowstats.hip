@@ -1,0 +1,217 @@
+// Two-phase path for losses whose per-row weights depend on all rows (the reference's
+// alpha-weighted composite): phase 1 returns, per row, the full-vocabulary log-sum-exp and the
+// scaled logits at the teacher's ids; the caller combines them (K-wide work) and asks phase 2 for
+//     grad[r, j] = ( a_r * softmax(z_r)_j + sum_k c_rk [j == idx_rk] ) * inv_T
+// where a_r = dL/d lse_r and c_rk = dL/d zk_rk.  Phase 1 is a read-only streaming reduction,
+// phase 2 an element-wise sweep (read row, write gradient) plus K sparse additions.
+#include "distill_common.hpp"
+#include "distill_hip.h"
+
+namespace dl {
+
+struct StatsParams {
+  const void* logits; int64_t row_stride; int64_t n_rows; int64_t V;
+  const int32_t* row_map; const void* t_idx; int t_idx_itype; int K; int64_t n_trows;
+  float inv_T;
+  float* lse; float* zk;                               // outputs of phase 1 / inputs of phase 2
+  const float* coef_lse; const float* coef_zk;         // phase 2
+  void* grad; int64_t grad_stride;
+};
+
+// ---- phase 1: lse_r = logsumexp_j(x_rj * inv_T),  zk_rk = x[r, idx_rk] * inv_T ------------------
+template <class Tag, int NT, bool VEC>
+__global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
+  __shared__ float red[64];
+  using C = Chunk<Tag>;
+  const int64_t r = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  if (trow < 0) return;
+  const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  for (int k = tid; k < p.K; k += NT) {
+    const int64_t id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
+    p.zk[trow * p.K + k] = (id >= 0 && id < p.V) ? load_as_float(row, Tag::id, id) * p.inv_T : 0.f;
+  }
+  const float a = p.inv_T * LOG2E;
+  float m = -INFINITY, sm = 0.f;
+  if (VEC) {
+    const int64_t nch = p.V / C::N;
+    for (int64_t c0 = 0; c0 < nch; c0 += 4 * NT) {          // four 16-byte loads in flight per thread
+      u32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t ch = c0 + (int64_t)u * NT + tid;
+        v[u] = ch < nch ? load16_stream(row + ch * 16) : C::neg_inf();
+      }
+      float cm = -INFINITY;
+      float f[4][C::N];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        C::unpack(v[u], f[u]);
+#pragma unroll
+        for (int e = 0; e < C::N; ++e) cm = fmaxf(cm, f[u][e]);
+      }
+      if (cm > m) { sm *= fast_exp2((m - cm) * a); m = cm; }
+      const float mb = m * a;
+      if (m > -INFINITY) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[u][e], a, -mb));
+      }
+    }
+  } else {
+    for (int64_t j = tid; j < p.V; j += NT) {
+      const float f = load_as_float(row, Tag::id, j);
+      if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
+      sm += fast_exp2(fmaf(f, a, -m * a));
+    }
+  }
+  const float mx = block_max<NT>(m, red);
+  sm = (m == -INFINITY) ? 0.f : sm * fast_exp2((m - mx) * a);
+  sm = block_sum<NT>(sm, red);
+  if (tid == 0) p.lse[trow] = (mx * a + fast_log2(sm)) * LN2;
+}
+
+// ---- phase 2 -------------------------------------------------------------------------------
+// One workgroup per (row, column part of NT*NCH chunks).
+template <class Tag, int NT, int NCH, bool VEC>
+__global__ __launch_bounds__(NT) void rowcoef_grad_kernel(const StatsParams p, int parts) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  using C = Chunk<Tag>;
+  const int Kp = (p.K + 15) & ~15;
+  int* s_idx = reinterpret_cast<int*>(smem);
+  float* s_c = reinterpret_cast<float*>(s_idx + Kp);
+  const int64_t r = blockIdx.x / parts;
+  const int h = (int)(blockIdx.x % parts);
+  const int tid = threadIdx.x;
+  const int64_t per_part = (int64_t)NT * NCH * C::N;                 // columns per part
+  const int64_t lo = h * per_part, hi = min(p.V, lo + per_part);
+  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  char* grow = reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes;
+  const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  if (trow < 0) {
+    if (VEC) zero_row<Tag, NT>(grow + lo * Tag::bytes, (hi - lo) / C::N);
+    else for (int64_t j = lo + tid; j < hi; j += NT) store_from_float(grow, Tag::id, j, 0.f);
+    return;
+  }
+  for (int k = tid; k < Kp; k += NT) {
+    int64_t id = -1;
+    float cv = 0.f;
+    if (k < p.K) {
+      id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
+      cv = p.coef_zk[trow * p.K + k];
+    }
+    s_idx[k] = (id >= lo && id < hi) ? (int)id : -1;
+    s_c[k] = cv;
+  }
+  const float a = p.inv_T * LOG2E;
+  const float b = p.lse[trow] * LOG2E;
+  const float w = p.coef_lse[trow] * p.inv_T;
+  if (VEC) {
+    const int64_t c_lo = lo / C::N, c_hi = hi / C::N;
+    u32x4 v[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int64_t ch = c_lo + (int64_t)i * NT + tid;
+      v[i] = ch < c_hi ? load16_stream(row + ch * 16) : C::neg_inf();
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int64_t ch = c_lo + (int64_t)i * NT + tid;
+      if (ch < c_hi) {
+        float f[C::N];
+        C::unpack(v[i], f);
+#pragma unroll
+        for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * w;
+        store16_stream(grow + ch * 16, C::pack(f));
+      }
+    }
+  } else {
+    for (int64_t j = lo + tid; j < hi; j += NT)
+      store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * w);
+  }
+  __syncthreads();          // LDS entries staged; dense stores ordered before the sparse additions
+  for (int k = tid; k < Kp; k += NT) {
+    const int id = s_idx[k];
+    if (id < 0) continue;
+    float cs = 0.f;           // every entry with this id contributes; all of them write the same total
+    for (int j = 0; j < Kp; ++j) cs += (s_idx[j] == id) ? s_c[j] : 0.f;
+    const float dense = fast_exp2(fmaf(load_as_float(row, Tag::id, id), a, -b)) * w;
+    store_from_float(grow, Tag::id, id, dense + cs * p.inv_T);
+  }
+}
+
+static bool aligned16(const void* ptr, int64_t stride, int eb) {
+  return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (stride * eb) % 16 == 0;
+}
+
+template <class Tag>
+static hipError_t launch_stats(const StatsParams& p, bool vec, hipStream_t st) {
+  if (vec) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, true>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((rowstats_kernel<Tag, 256, false>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
+  return hipGetLastError();
+}
+
+template <class Tag>
+static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
+  constexpr int NT = 256, NCH = 8;
+  const int64_t per_part = (int64_t)NT * NCH * Tag::epc;
+  const int parts = (int)((p.V + per_part - 1) / per_part);
+  const size_t lds = (size_t)((p.K + 15) & ~15) * 8;
+  const dim3 grid((unsigned)(p.n_rows * parts));
+  if (vec) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, true>), grid, dim3(NT), lds, st, p, parts);
+  else hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, false>), grid, dim3(NT), lds, st, p, parts);
+  return hipGetLastError();
+}
+
+static int check_common(const void* logits, int dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                        const void* t_idx, int itype, int K, int64_t n_trows) {
+  if (!logits || !t_idx) return DL_ERR_NULL;
+  if (dtype < DL_F32 || dtype > DL_F16 || (itype != DL_I32 && itype != DL_I64)) return DL_ERR_DTYPE;
+  if (n_rows < 0 || V <= 0 || K <= 0 || n_trows < 0 || row_stride < V) return DL_ERR_SHAPE;
+  if (K > DL_MAX_TOPK || V > 0x7fffffffLL || n_rows > 0x7fffffffLL) return DL_ERR_LIMIT;
+  return DL_OK;
+}
+
+}  // namespace dl
+
+extern "C" int dl_rowstats_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                                const int32_t* row_map, const void* t_idx, int t_idx_itype, int K,
+                                int64_t n_teacher_rows, float inv_T, float* lse, float* zk, void* stream) {
+  using namespace dl;
+  const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_teacher_rows);
+  if (rc != DL_OK) return rc;
+  if (!lse || !zk) return DL_ERR_NULL;
+  if (n_rows == 0) return DL_OK;
+  const int eb = logits_dtype == DL_F32 ? 4 : 2;
+  const bool vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb);
+  StatsParams p{logits, row_stride, n_rows, V, row_map, t_idx, t_idx_itype, K, n_teacher_rows, inv_T, lse, zk,
+                nullptr, nullptr, nullptr, 0};
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const hipError_t e = logits_dtype == DL_F32 ? launch_stats<TagF32>(p, vec, st)
+                       : logits_dtype == DL_BF16 ? launch_stats<TagBF16>(p, vec, st)
+                                                 : launch_stats<TagF16>(p, vec, st);
+  return e == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}
+
+extern "C" int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
+                                    int64_t V, const int32_t* row_map, const void* t_idx, int t_idx_itype, int K,
+                                    int64_t n_teacher_rows, float inv_T, const float* lse, const float* coef_lse,
+                                    const float* coef_zk, void* grad, int64_t grad_stride, void* stream) {
+  using namespace dl;
+  const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_teacher_rows);
+  if (rc != DL_OK) return rc;
+  if (!lse || !coef_lse || !coef_zk || !grad) return DL_ERR_NULL;
+  if (grad_stride < V) return DL_ERR_SHAPE;
+  if (n_rows == 0) return DL_OK;
+  const int eb = logits_dtype == DL_F32 ? 4 : 2;
+  const bool vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb) && aligned16(grad, grad_stride, eb);
+  StatsParams p{logits, row_stride, n_rows, V, row_map, t_idx, t_idx_itype, K, n_teacher_rows, inv_T,
+                const_cast<float*>(lse), nullptr, coef_lse, coef_zk, grad, grad_stride};
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const hipError_t e = logits_dtype == DL_F32 ? launch_coef<TagF32>(p, vec, st)
+                       : logits_dtype == DL_BF16 ? launch_coef<TagBF16>(p, vec, st)
+                                                 : launch_coef<TagF16>(p, vec, st);
+  return e == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}

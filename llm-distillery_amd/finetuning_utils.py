@@ -1,0 +1,107 @@
+"""Drop-in for the loss entry point of the reference, `utils/finetuning_utils.py`.
+
+`calculate_divergence` keeps the reference's name, positional arguments and its
+nine result keys (utils/finetuning_utils.py:47,112-122).  The two full-vocabulary
+steps of the reference -- `F.log_softmax` over V and `torch.gather` at the teacher
+ids (:88,:92), and their autograd replay -- run in the HIP kernels behind the
+`distillery_amd::rowstats_topk` custom op; what is left is K-wide arithmetic on
+[N, K] tensors, written with the same torch routines the reference uses so that
+its quirks carry over unchanged (crop rule and valid-mean fill of the top-K cross
+entropy, pad-by-one and non-detached max of the alpha weighting).
+
+`distill_loss` is the extended entry point: it takes the model's logits in their
+native dtype, un-gathered, with the row selection and the temperature folded
+into the kernels (classes/student/model.py:408,420-421).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+
+from . import ops
+
+LOSS_KEYS = ("train_loss", "custom loss", "CE loss", "kl_div", "reverse kl_div",
+             "weighted kl_div", "weighted rev. kl_div", "teacher CE loss", "CE diff")
+
+
+def _kl_per_token(inp_logp: Tensor, tgt_logp: Tensor) -> Tensor:
+    return F.kl_div(inp_logp, tgt_logp, reduction="none", log_target=True).sum(dim=-1)
+
+
+def _topk_cross_entropy(logprobs: Tensor, labels: Tensor, indices: Tensor, ignore_rows: Tensor) -> Tensor:
+    """utils/finetuning_utils.py:68-84 on K-wide tensors."""
+    stop = -1 if labels.size(-1) < logprobs.size(0) else 0
+    hit = labels.unsqueeze(-1) == indices[:stop]
+    hit[ignore_rows] = False
+    valid = hit.any(dim=-1)
+    picked = torch.zeros_like(valid, dtype=torch.float32)
+    picked[valid] = logprobs[:stop][hit].squeeze(-1)
+    picked[~valid] = picked[valid].mean()
+    return -picked
+
+
+def _alpha_weighted(per_token: Tensor, alpha, ce_per_token: Tensor) -> Tensor:
+    """utils/finetuning_utils.py:58-66."""
+    if ce_per_token.numel() < per_token.numel():
+        ce_per_token = torch.cat((ce_per_token, torch.zeros(1, device=ce_per_token.device)))
+    w = (per_token / per_token.max() + 1).pow(alpha) + ce_per_token
+    return (per_token * w).mean()
+
+
+def _assemble(s_sup: Tensor, t: Tensor, indices: Tensor, labels: Tensor, alpha, avoid: Tensor) -> dict[str, Tensor]:
+    ce_s = _topk_cross_entropy(s_sup, labels, indices, avoid)
+    ce_t = _topk_cross_entropy(t, labels, indices, avoid)
+    ce_diff = ce_s - ce_t
+    ce_pos = torch.where(ce_diff < 0, torch.zeros_like(ce_diff), ce_diff)
+    kl = _kl_per_token(s_sup, t)
+    rkl = _kl_per_token(t, F.log_softmax(s_sup, dim=-1))
+    wkl = _alpha_weighted(kl, alpha, ce_pos)
+    wrkl = _alpha_weighted(rkl, alpha, ce_pos)
+    total = (wkl + wrkl) / 2
+    return dict(zip(LOSS_KEYS, (total, total, ce_s.mean(), kl.mean(), rkl.mean(), wkl, wrkl, ce_t.mean(),
+                                ce_diff.mean())))
+
+
+def calculate_divergence(student_logits: Tensor, teacher_logits: Tensor, indices: Tensor | None,
+                         convo_CE_tokens: Tensor, alpha, avoid_indices: Tensor) -> dict[str, Tensor]:
+    """Same contract as the reference's `calculate_divergence`: `student_logits` [N, V] (already
+    divided by the temperature, any floating dtype), `teacher_logits` [N, K] stored log-probs divided
+    by the temperature, `indices` [N, K], the cross-entropy labels and the rows to ignore.  Returns
+    the nine-key dict; `train_loss` carries autograd history back to `student_logits`.
+
+    `indices=None` (dense teacher) raises, as the reference's own training path does.
+    """
+    if indices is None:
+        raise TypeError("calculate_divergence needs top-K indices: the dense-teacher form of the reference "
+                        "composite is not executable (use dense_divergence for dense teachers)")
+    n = min(student_logits.size(0), teacher_logits.size(0), indices.size(0))
+    logits = student_logits[:n]
+    idx = indices[:n]
+    lse, zk = ops.rowstats_topk(logits, idx, None, 1.0)
+    s_sup = zk - lse.unsqueeze(-1)                       # log_softmax over V, gathered at the ids
+    t = F.log_softmax(teacher_logits[:n].float(), dim=-1)
+    return _assemble(s_sup, t, idx, convo_CE_tokens[:n], alpha, avoid_indices)
+
+
+def distill_loss(model_logits: Tensor, content_rows: Tensor, teacher_logprobs: Tensor, indices: Tensor,
+                 convo_CE_tokens: Tensor, alpha, avoid_indices: Tensor, temperature: float = 1.0,
+                 crop_to_size: int | None = None, teacher_temperature: float | None = None) -> dict[str, Tensor]:
+    """The composite loss of one conversation straight from the model output.
+
+    model_logits [S, V_model] in the model's dtype; `content_rows` int [N] positions of the content
+    tokens (classes/student/model.py:87-91); `teacher_logprobs` [N, K] as stored (not yet divided by
+    the temperature).  Slice, cast, temperature and row selection happen inside the kernels.
+    `teacher_temperature=1` reproduces the validation loop, which scales only the student
+    (classes/student/model.py:501-502).
+    """
+    x = model_logits if crop_to_size is None else model_logits[:, :crop_to_size]
+    S = x.shape[0]
+    n = min(content_rows.numel(), teacher_logprobs.size(0), indices.size(0))
+    row_map = torch.full((S,), -1, dtype=torch.int32, device=x.device)
+    row_map[content_rows[:n].long()] = torch.arange(n, dtype=torch.int32, device=x.device)
+    lse, zk = ops.rowstats_topk(x, indices[:n], row_map, 1.0 / temperature)
+    s_sup = zk - lse.unsqueeze(-1)
+    tT = temperature if teacher_temperature is None else teacher_temperature
+    t = F.log_softmax(teacher_logprobs[:n].float() / tT, dim=-1)
+    return _assemble(s_sup, t, indices[:n], convo_CE_tokens[:n], alpha, avoid_indices)

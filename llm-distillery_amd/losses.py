@@ -1,0 +1,92 @@
+"""Accumulator for the loss dicts of a batch, mirroring `classes/losses.py` of the reference
+(same method names and behaviour: sum over conversations, `backward(divisor)`, logging by key)."""
+from __future__ import annotations
+
+import torch
+
+
+class Losses:
+    """Sums loss dicts across the conversations of a batch (classes/losses.py:16-47), runs the
+    backward pass on the summed `train_loss` (:70-79) and logs the other keys (:56-68).
+
+    `logger` is anything with `.log(dict, step=int)` (the reference passes a wandb run); None
+    disables logging.
+    """
+
+    def __init__(self, logger=None, validation: bool = False):
+        self.loss_dict: dict[str, torch.Tensor] = {}
+        self.validation = validation
+        self.device = None
+        self.logger = logger
+        self.num_steps_accumulated = 0
+
+    def add_losses(self, new_losses: dict[str, torch.Tensor]) -> None:
+        """Every key except `train_loss` is detached and cloned; the first dict is adopted, later
+        ones are added key by key.  Raises ValueError on an empty dict."""
+        if not new_losses:
+            raise ValueError("No losses to add to the loss dictionary.")
+        self.num_steps_accumulated += 1
+        for key in list(new_losses):
+            if key != "train_loss":
+                new_losses[key] = new_losses[key].clone().detach()
+        if not self.loss_dict:
+            self.loss_dict = new_losses
+            return
+        for key, value in new_losses.items():
+            if key in self.loss_dict:
+                self.loss_dict[key] = self.loss_dict[key] + value
+            else:
+                self.loss_dict[key] = value
+
+    def empty(self) -> None:
+        self.loss_dict = {}
+        self.num_steps_accumulated = 0
+
+    def log(self, step: int, average: bool = True) -> None:
+        if self.logger is None:
+            return
+        prefix = "Val Loss" if self.validation else "Loss"
+        for key, value in self.loss_dict.items():
+            if key == "train_loss":
+                continue
+            shown = value / self.num_steps_accumulated if average else value
+            self.logger.log({f"{prefix}/{key}": shown}, step=step)
+
+    def backward(self, divisor: int = 1) -> None:
+        """`train_loss / divisor` backward, then the key is dropped: the sum over the batch's
+        conversations divided by the gradient-accumulation count, not a batch mean."""
+        loss = self.loss_dict["train_loss"] / divisor
+        loss.backward()
+        del self.loss_dict["train_loss"]
+
+    def _scaled(self, fn) -> "Losses":
+        out = Losses(self.logger, self.validation)
+        out.loss_dict = {k: fn(v) for k, v in self.loss_dict.items()}
+        out.num_steps_accumulated = self.num_steps_accumulated
+        return out
+
+    def __truediv__(self, other):
+        if isinstance(other, (int, float, torch.Tensor)):
+            return self._scaled(lambda v: v / other)
+        return NotImplemented
+
+    def __itruediv__(self, other):
+        if isinstance(other, (int, float, torch.Tensor)):
+            self.loss_dict = {k: v / other for k, v in self.loss_dict.items()}
+            return self
+        return NotImplemented
+
+    def __mul__(self, other):
+        if isinstance(other, (int, float, torch.Tensor)):
+            return self._scaled(lambda v: v * other)
+        return NotImplemented
+
+    def __imul__(self, other):
+        if isinstance(other, (int, float, torch.Tensor)):
+            self.loss_dict = {k: v * other for k, v in self.loss_dict.items()}
+            return self
+        return NotImplemented
+
+    def __str__(self) -> str:
+        head = " Validation Losses:\n" if self.validation else " Training Losses:\n"
+        return head + "".join(f"{k}: {v.item():.4f}\n" for k, v in self.loss_dict.items())

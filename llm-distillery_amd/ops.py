@@ -3,6 +3,8 @@ stream; all arithmetic happens in the HIP kernels.  No fallbacks: a CPU tensor o
 a missing library raises."""
 from __future__ import annotations
 
+from typing import Optional, Tuple
+
 import torch
 
 from . import _lib
@@ -101,6 +103,95 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
     if grad is not None and logits.dim() != 2 and grad_out is None:
         grad = grad.view(logits.shape)
     return row_loss, grad
+
+
+def _rowstats_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float):
+    """Phase 1 launch: (lse [N], zk [N, K]) for the valid rows of x [R, V]."""
+    _dev(x, "logits"), _dev(t_idx, "t_idx")
+    if x.dim() != 2 or x.stride(1) != 1 or x.dtype not in _DT:
+        raise RuntimeError("logits must be [rows, V] bf16/fp16/fp32, dense along V")
+    if t_idx.dim() != 2 or t_idx.dtype not in _IT:
+        raise RuntimeError("t_idx must be [N, K] int32/int64")
+    t_idx = t_idx.contiguous()
+    R, V = x.shape
+    N, K = t_idx.shape
+    if row_map is None and N < R:
+        raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
+    _, rm_ptr = _opt_i32(row_map, R, "row_map", x.device)
+    lse = torch.zeros(N, dtype=torch.float32, device=x.device)
+    zk = torch.zeros((N, K), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().dl_rowstats_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(),
+                                          _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), zk.data_ptr(),
+                                          _stream_ptr(x.device))
+    _lib.check(st, "dl_rowstats_topk")
+    return lse, zk
+
+
+def _rowcoef_grad_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float, lse: torch.Tensor,
+                      g_lse: torch.Tensor, g_zk: torch.Tensor) -> torch.Tensor:
+    """Phase 2 launch: d L / d x from dL/d lse and dL/d zk."""
+    t_idx = t_idx.contiguous()
+    R, V = x.shape
+    N, K = t_idx.shape
+    _, rm_ptr = _opt_i32(row_map, R, "row_map", x.device)
+    g_lse = g_lse.to(torch.float32).contiguous()
+    g_zk = g_zk.to(torch.float32).contiguous()
+    grad = torch.empty((R, V), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().dl_rowcoef_grad_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(),
+                                              _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), g_lse.data_ptr(),
+                                              g_zk.data_ptr(), grad.data_ptr(), grad.stride(0),
+                                              _stream_ptr(x.device))
+    _lib.check(st, "dl_rowcoef_grad_topk")
+    return grad
+
+
+@torch.library.custom_op("distillery_amd::rowstats_topk", mutates_args=())
+def rowstats_topk(logits: torch.Tensor, t_idx: torch.Tensor, row_map: Optional[torch.Tensor],
+                  inv_T: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(lse [N] fp32, zk [N, K] fp32): full-vocabulary log-sum-exp of logits * inv_T and the scaled
+    logits at the teacher ids, for the rows selected by row_map.  Differentiable w.r.t. logits."""
+    return _rowstats_raw(logits, t_idx, row_map, inv_T)
+
+
+@rowstats_topk.register_fake
+def _(logits, t_idx, row_map, inv_T):
+    N, K = t_idx.shape
+    return (logits.new_empty((N,), dtype=torch.float32), logits.new_empty((N, K), dtype=torch.float32))
+
+
+@torch.library.custom_op("distillery_amd::rowcoef_grad_topk", mutates_args=())
+def rowcoef_grad_topk(logits: torch.Tensor, t_idx: torch.Tensor, row_map: Optional[torch.Tensor], inv_T: float,
+                      lse: torch.Tensor, g_lse: torch.Tensor, g_zk: torch.Tensor) -> torch.Tensor:
+    return _rowcoef_grad_raw(logits, t_idx, row_map, inv_T, lse, g_lse, g_zk)
+
+
+@rowcoef_grad_topk.register_fake
+def _(logits, t_idx, row_map, inv_T, lse, g_lse, g_zk):
+    return torch.empty_like(logits)
+
+
+def _rowstats_setup(ctx, inputs, output):
+    logits, t_idx, row_map, inv_T = inputs
+    lse, _ = output
+    ctx.save_for_backward(logits, t_idx, lse, *([row_map] if row_map is not None else []))
+    ctx.has_map = row_map is not None
+    ctx.inv_T = inv_T
+
+
+def _rowstats_backward(ctx, g_lse, g_zk):
+    saved = ctx.saved_tensors
+    logits, t_idx, lse = saved[:3]
+    row_map = saved[3] if ctx.has_map else None
+    if g_lse is None:
+        g_lse = torch.zeros_like(lse)
+    if g_zk is None:
+        g_zk = torch.zeros((t_idx.shape[0], t_idx.shape[1]), dtype=torch.float32, device=lse.device)
+    return rowcoef_grad_topk(logits, t_idx, row_map, ctx.inv_T, lse, g_lse, g_zk), None, None, None
+
+
+rowstats_topk.register_autograd(_rowstats_backward, setup_context=_rowstats_setup)
 
 
 def reduce_sum(values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:

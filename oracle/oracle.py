@@ -251,7 +251,8 @@ def topk_cross_entropy(logprobs: torch.Tensor, labels: torch.Tensor, idx: torch.
     hit = labels.unsqueeze(-1) == idx[:stop]
     hit[ignore_rows] = False
     valid = hit.any(dim=-1)
-    picked = torch.zeros_like(valid, dtype=torch.float32)
+    # the reference allocates float32 here; the float64 "truth" variant keeps its precision
+    picked = torch.zeros_like(valid, dtype=torch.float64 if logprobs.dtype == torch.float64 else torch.float32)
     picked[valid] = logprobs[:stop][hit].squeeze(-1)
     picked[~valid] = picked[valid].mean()
     return -picked
@@ -264,7 +265,7 @@ def alpha_weighted(per_token: torch.Tensor, alpha, ce_per_token: torch.Tensor) -
     maximum is part of the autograd graph (not detached).
     """
     if ce_per_token.numel() < per_token.numel():
-        ce_per_token = torch.cat((ce_per_token, torch.zeros(1, device=ce_per_token.device)))
+        ce_per_token = torch.cat((ce_per_token, torch.zeros(1, device=ce_per_token.device, dtype=ce_per_token.dtype)))
     w = (per_token / per_token.max() + 1).pow(alpha) + ce_per_token
     return (per_token * w).mean()
 
