@@ -93,6 +93,26 @@ int dl_div_topk(int kind,
 int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V);
 
 /*
+ * Forward KL (DL_FKL), reverse KL (DL_RKL) or Jensen-Shannon divergence (DL_JSD) against a dense
+ * teacher, loss and gradient in one launch.  Replaces, with K = V:
+ *   classes/student/model.py:408,420-421, utils/finetuning_utils.py:88,94 (both log_softmax),
+ *   utils/finetuning_utils.py:49-56,104-105 (kl_div + sum), classes/losses.py:77-78 (autograd replay).
+ * The reference's training side cannot run a dense teacher (it raises on indices=None) and has no
+ * JSD, so the conventions are this library's: teacher entries of -inf logit carry zero mass and
+ * contribute 0 to FKL/JSD; RKL renormalises the student over the teacher's support
+ * {j : t_logits[j] > -inf}, as the reference renormalises it over the top-K ids; JSD is
+ * 0.5 KL(P||M) + 0.5 KL(Q||M), natural log.
+ * t_logits [n_teacher_rows, V] (stride t_stride): teacher logits or log-probs (any per-row constant
+ * is irrelevant), scaled by inv_T_teacher.  Other arguments as for dl_div_topk.
+ */
+int dl_div_dense(int kind,
+                 const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                 const int32_t* row_map,
+                 const void* t_logits, int t_dtype, int64_t t_stride, int64_t n_teacher_rows,
+                 float inv_T_student, float inv_T_teacher, float grad_scale,
+                 float* row_loss, void* grad, int64_t grad_stride, void* stream);
+
+/*
  * Phase 1 of the general (two-phase) path: per valid row r with teacher row t = row_map[r],
  *   lse[t]   = logsumexp_j(logits[r, j] * inv_T)                       (fp32, natural log)
  *   zk[t, k] = logits[r, t_idx[t, k]] * inv_T                          (fp32; 0 for ids outside [0, V))

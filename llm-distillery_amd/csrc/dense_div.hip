@@ -1,0 +1,170 @@
+// Kernels and C entry point for divergences against a dense teacher stored in memory.
+#include "dense_div.hpp"
+
+namespace dl {
+
+struct DenseParams {
+  int kind;
+  const void* logits; int s_dtype; int64_t row_stride; int64_t n_rows; int64_t V;
+  const int32_t* row_map;
+  const void* t_logits; int t_dtype; int64_t t_stride; int64_t n_trows;
+  float inv_T_s, inv_T_t, grad_scale;
+  float* row_loss; void* grad; int64_t grad_stride;
+};
+
+// Both rows in registers: NU units of 8 columns per thread.
+template <class TagS, class TagT, int NT, int NU>
+struct RegRows {
+  Unit<TagS> s[NU];
+  Unit<TagT> t[NU];
+  int64_t nunits;
+  __device__ __forceinline__ void load(const char* srow, const char* trow, int64_t nu) {
+    nunits = nu;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * NT + threadIdx.x;
+      if (u < nunits) { s[i].load(srow, u); t[i].load(trow, u); }
+      else { s[i].fill_neg_inf(); t[i].fill_neg_inf(); }
+    }
+  }
+  template <class F>
+  __device__ __forceinline__ void sweep(F f) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * NT + threadIdx.x;
+      if (u < nunits) {
+        float a[8], b[8];
+        s[i].unpack(a);
+        t[i].unpack(b);
+        f(u, a, b);
+      }
+    }
+  }
+};
+
+template <class TagS, class TagT, int NT, int NU>
+__global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
+  __shared__ float red[64];
+  const int64_t r = blockIdx.x;
+  const int tid = threadIdx.x;
+  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
+  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  if (trow < 0) {
+    if (grow) zero_row<TagS, NT>(grow, p.V / TagS::epc);
+    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    return;
+  }
+  RegRows<TagS, TagT, NT, NU> rows;
+  rows.load(reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes,
+            reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * TagT::bytes, p.V / 8);
+  const DenseStats st = dense_stats<NT>(p.kind, rows, p.inv_T_s, p.inv_T_t, red);
+  if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
+  if (grow) dense_grad_sweep<TagS>(p.kind, rows, st, p.inv_T_s * p.grad_scale, grow);
+}
+
+// Any size, any alignment, any dtype pair: four scalar passes over global memory.
+template <int NT>
+__global__ __launch_bounds__(NT) void dense_stream_kernel(const DenseParams p) {
+  __shared__ float red[64];
+  const int64_t r = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t V = p.V;
+  const int sb = p.s_dtype == F32 ? 4 : 2, tb = p.t_dtype == F32 ? 4 : 2;
+  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * sb : nullptr;
+  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  if (trow < 0) {
+    if (grow) for (int64_t j = tid; j < V; j += NT) store_from_float(grow, p.s_dtype, j, 0.f);
+    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    return;
+  }
+  const char* srow = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * sb;
+  const char* trw = reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * tb;
+  const int kind = p.kind;
+  const float a_s = p.inv_T_s * LOG2E, a_t = p.inv_T_t * LOG2E;
+  float ms = -INFINITY, mt = -INFINITY;
+  for (int64_t j = tid; j < V; j += NT) {
+    const float s = load_as_float(srow, p.s_dtype, j), t = load_as_float(trw, p.t_dtype, j);
+    mt = fmaxf(mt, t);
+    ms = fmaxf(ms, (kind == DL_RKL && t == -INFINITY) ? -INFINITY : s);
+  }
+  block_max2<NT>(ms, mt, red);
+  const float bs = ms * a_s, bt = mt * a_t;
+  float ss = 0.f, stt = 0.f;
+  for (int64_t j = tid; j < V; j += NT) {
+    const float s = load_as_float(srow, p.s_dtype, j), t = load_as_float(trw, p.t_dtype, j);
+    ss += (kind == DL_RKL && t == -INFINITY) ? 0.f : fast_exp2(fmaf(s, a_s, -bs));
+    stt += fast_exp2(fmaf(t, a_t, -bt));
+  }
+  block_sum2<NT>(ss, stt, red);
+  const float ls = bs + fast_log2(ss), lt = bt + fast_log2(stt);
+  float x = 0.f, y = 0.f;
+  for (int64_t j = tid; j < V; j += NT) {
+    const float lp = fmaf(load_as_float(srow, p.s_dtype, j), a_s, -ls);
+    const float lq = fmaf(load_as_float(trw, p.t_dtype, j), a_t, -lt);
+    if (kind == DL_FKL) fkl_term(lp, lq, x);
+    else if (kind == DL_RKL) rkl_term(lp, lq, x);
+    else jsd_term(lp, lq, x, y);
+  }
+  block_sum2<NT>(x, y, red);
+  const float loss = kind == DL_JSD ? 0.5f * LN2 * (x + y) : x * LN2;
+  const float aux = x * LN2;
+  if (tid == 0 && p.row_loss) p.row_loss[r] = loss;
+  if (grow) {
+    const float c = p.inv_T_s * p.grad_scale;
+    for (int64_t j = tid; j < V; j += NT) {
+      const float lp = fmaf(load_as_float(srow, p.s_dtype, j), a_s, -ls);
+      const float lq = fmaf(load_as_float(trw, p.t_dtype, j), a_t, -lt);
+      store_from_float(grow, p.s_dtype, j, dense_grad(kind, lp, lq, aux) * c);
+    }
+  }
+}
+
+template <class TagS, class TagT, int NU>
+static bool launch_dense_reg(const DenseParams& p, hipStream_t st) {
+  const int64_t units = p.V / 8;
+  const dim3 grid((unsigned)p.n_rows);
+  if (units <= 256 * NU) hipLaunchKernelGGL((dense_reg_kernel<TagS, TagT, 256, NU>), grid, dim3(256), 0, st, p);
+  else if (units <= 512 * NU) hipLaunchKernelGGL((dense_reg_kernel<TagS, TagT, 512, NU>), grid, dim3(512), 0, st, p);
+  else if (units <= 1024 * NU) hipLaunchKernelGGL((dense_reg_kernel<TagS, TagT, 1024, NU>), grid, dim3(1024), 0, st, p);
+  else return false;
+  return true;
+}
+
+// Register path for the dtype pairs that occur: teacher stored like the student, or in fp32.
+static bool launch_dense_pair(const DenseParams& p, hipStream_t st) {
+  if (p.s_dtype == F32 && p.t_dtype == F32) return launch_dense_reg<TagF32, TagF32, 4>(p, st);
+  if (p.s_dtype == BF16 && p.t_dtype == BF16) return launch_dense_reg<TagBF16, TagBF16, 8>(p, st);
+  if (p.s_dtype == F16 && p.t_dtype == F16) return launch_dense_reg<TagF16, TagF16, 8>(p, st);
+  if (p.s_dtype == BF16 && p.t_dtype == F32) return launch_dense_reg<TagBF16, TagF32, 4>(p, st);
+  if (p.s_dtype == F16 && p.t_dtype == F32) return launch_dense_reg<TagF16, TagF32, 4>(p, st);
+  return false;
+}
+
+}  // namespace dl
+
+extern "C" int dl_div_dense(int kind, const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
+                            int64_t V, const int32_t* row_map, const void* t_logits, int t_dtype, int64_t t_stride,
+                            int64_t n_teacher_rows, float inv_T_student, float inv_T_teacher, float grad_scale,
+                            float* row_loss, void* grad, int64_t grad_stride, void* stream) {
+  using namespace dl;
+  if (!logits || !t_logits) return DL_ERR_NULL;
+  if (kind < DL_FKL || kind > DL_JSD || logits_dtype < DL_F32 || logits_dtype > DL_F16 || t_dtype < DL_F32 ||
+      t_dtype > DL_F16)
+    return DL_ERR_DTYPE;
+  if (n_rows < 0 || V <= 0 || n_teacher_rows < 0 || row_stride < V || t_stride < V || (grad && grad_stride < V))
+    return DL_ERR_SHAPE;
+  if (n_rows > 0x7fffffffLL || V > 0x7fffffffLL) return DL_ERR_LIMIT;
+  if (n_rows == 0) return DL_OK;
+  const int sb = logits_dtype == DL_F32 ? 4 : 2, tb = t_dtype == DL_F32 ? 4 : 2;
+  auto ok16 = [](const void* ptr, int64_t stride, int eb) {
+    return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (stride * eb) % 16 == 0;
+  };
+  const bool vec = V % 8 == 0 && ok16(logits, row_stride, sb) && ok16(t_logits, t_stride, tb) &&
+                   (!grad || ok16(grad, grad_stride, sb));
+  DenseParams p{kind, logits, logits_dtype, row_stride, n_rows, V, row_map, t_logits, t_dtype, t_stride,
+                n_teacher_rows, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride};
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (!(vec && launch_dense_pair(p, st)))
+    hipLaunchKernelGGL((dense_stream_kernel<1024>), dim3((unsigned)n_rows), dim3(1024), 0, st, p);
+  return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}

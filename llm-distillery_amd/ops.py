@@ -105,6 +105,44 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
     return row_loss, grad
 
 
+def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_map: torch.Tensor | None = None,
+              T: float = 1.0, teacher_T: float | None = None, grad_scale: float = 1.0, want_grad: bool = True,
+              grad_out: torch.Tensor | None = None):
+    """Per-token "fkl", "rkl" or "jsd" against a dense teacher [N, V] and, in the same launch,
+    d(sum of row losses)/d(logits) * grad_scale.  Returns (row_loss fp32 [rows], grad or None)."""
+    if kind not in KINDS:
+        raise ValueError("kind must be 'fkl', 'rkl' or 'jsd'")
+    _dev(logits, "logits"), _dev(t_logits, "t_logits")
+    x = _rows_2d(logits)
+    t = _rows_2d(t_logits)
+    R, V = x.shape
+    dev = x.device
+    if x.dtype not in _DT or t.dtype not in _DT:
+        raise RuntimeError("unsupported dtype")
+    if t.shape[1] != V:
+        raise RuntimeError(f"teacher has {t.shape[1]} columns, logits {V}")
+    N = t.shape[0]
+    if row_map is None and N < R:
+        raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
+    _, rm_ptr = _opt_i32(row_map, R, "row_map", dev)
+    row_loss = torch.empty(R, dtype=torch.float32, device=dev)
+    grad, g_ptr, g_stride = None, 0, V
+    if want_grad:
+        grad = grad_out if grad_out is not None else torch.empty((R, V), dtype=x.dtype, device=dev)
+        if grad.shape != (R, V) or grad.dtype != x.dtype or grad.stride(1) != 1 or grad.device != dev:
+            raise RuntimeError("grad_out must match logits as a [rows, V] tensor")
+        g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_div_dense(KINDS[kind], x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr,
+                                      t.data_ptr(), _DT[t.dtype], t.stride(0), N, 1.0 / T,
+                                      1.0 / (T if teacher_T is None else teacher_T), grad_scale,
+                                      row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
+    _lib.check(st, "dl_div_dense")
+    if grad is not None and logits.dim() != 2 and grad_out is None:
+        grad = grad.view(logits.shape)
+    return row_loss, grad
+
+
 def _rowstats_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float):
     """Phase 1 launch: (lse [N], zk [N, K]) for the valid rows of x [R, V]."""
     _dev(x, "logits"), _dev(t_idx, "t_idx")

@@ -57,3 +57,37 @@ def config3(device, rows: int = 8 * 4096, V: int = 128256, K: int = 200, seed: i
         logits[a:b] = chunk
         t_val[a:b], t_idx[a:b] = topk_teacher_for(chunk, K, min(20, K), g)
     return {"logits": logits, "t_val": t_val, "t_idx": t_idx, "T": 1.0, "kind": "fkl"}
+
+
+def row_map_from_valid(valid: torch.Tensor) -> torch.Tensor:
+    """int32 map for the kernels: position of each valid row among the valid rows, -1 elsewhere."""
+    rm = torch.full((valid.numel(),), -1, dtype=torch.int32, device=valid.device)
+    rm[valid] = torch.arange(int(valid.sum()), dtype=torch.int32, device=valid.device)
+    return rm
+
+
+def config1(device, B: int = 1, S: int = 512, V: int = 32000, seed: int = 1):
+    """Plumbing config: forward KL over the full vocabulary, fp32.  Student ~ N(0, 2^2), teacher =
+    student + N(0, 1), T = 1; the last ceil(10 %) positions of the sequence are padding (for
+    S = 512: 461 valid, 51 masked).  The dense teacher holds only the valid rows."""
+    g = _gen(device, seed)
+    logits = torch.randn((B * S, V), generator=g, device=device) * 2.0
+    teacher = logits + torch.randn((B * S, V), generator=g, device=device)
+    n_pad = -(-S // 10)
+    valid = (torch.arange(S, device=device) < S - n_pad).repeat(B)
+    return {"logits": logits, "t_logits": teacher[valid].contiguous(), "valid": valid,
+            "row_map": row_map_from_valid(valid), "T": 1.0, "kind": "fkl"}
+
+
+def config2(device, B: int = 4, S: int = 2048, V: int = 32000, seed: int = 2, dtype=torch.bfloat16):
+    """JSD over the full vocabulary, dense bf16 teacher, T = 2: student ~ N(0, 2^2), teacher =
+    0.8 * student + N(0, 1.5^2); per-sequence valid length uniform in [S/2, S], the rest masked."""
+    g = _gen(device, seed)
+    s32 = torch.randn((B * S, V), generator=g, device=device) * 2.0
+    teacher = (0.8 * s32 + torch.randn((B * S, V), generator=g, device=device) * 1.5).to(dtype)
+    logits = s32.to(dtype)
+    del s32
+    lengths = torch.randint(S // 2, S + 1, (B,), generator=g, device=device)
+    valid = (torch.arange(S, device=device).unsqueeze(0) < lengths.unsqueeze(1)).reshape(-1)
+    return {"logits": logits, "t_logits": teacher[valid].contiguous(), "valid": valid,
+            "row_map": row_map_from_valid(valid), "T": 2.0, "kind": "jsd", "lengths": lengths}

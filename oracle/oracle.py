@@ -149,8 +149,10 @@ def fwd_kl_dense_rows(z: torch.Tensor, t_logits: torch.Tensor) -> torch.Tensor:
     """
     s = F.log_softmax(z, dim=-1)
     t = F.log_softmax(t_logits, dim=-1)
-    term = torch.exp(t) * (t - s)
-    return torch.where(torch.isneginf(t), torch.zeros_like(term), term).sum(dim=-1)
+    zero = torch.isneginf(t)
+    t_safe = torch.where(zero, torch.zeros_like(t), t)
+    term = torch.exp(t_safe) * (t_safe - s)
+    return torch.where(zero, torch.zeros_like(term), term).sum(dim=-1)
 
 
 def rev_kl_dense_rows(z: torch.Tensor, t_logits: torch.Tensor) -> torch.Tensor:
@@ -165,7 +167,11 @@ def rev_kl_dense_rows(z: torch.Tensor, t_logits: torch.Tensor) -> torch.Tensor:
     t = F.log_softmax(t_logits, dim=-1)
     sup = ~torch.isneginf(t)
     s_sup = F.log_softmax(z.masked_fill(~sup, NEG_INF), dim=-1)
-    term = torch.exp(s_sup) * (s_sup - t)
+    # off the support both operands are replaced by finite stand-ins before the product, so that
+    # autograd does not turn 0 * inf into NaN gradients
+    s_safe = torch.where(sup, s_sup, torch.zeros_like(s_sup))
+    t_safe = torch.where(sup, t, torch.zeros_like(t))
+    term = torch.exp(s_safe) * (s_safe - t_safe)
     return torch.where(sup, term, torch.zeros_like(term)).sum(dim=-1)
 
 

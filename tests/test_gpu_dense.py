@@ -1,0 +1,124 @@
+"""GPU parity of the dense-teacher kernels (forward KL, reverse KL, JSD) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL = {torch.float32: 1e-4, torch.bfloat16: 2e-3, torch.float16: 2e-3}
+
+
+@pytest.fixture(scope="module")
+def D():
+    import llm_distillery_amd as d
+    d._lib.load()
+    return d
+
+
+def _check(D, kind, logits, t_logits, T, valid=None, teacher_T=None):
+    R, V = logits.shape
+    n_valid = R if valid is None else int(valid.sum())
+    loss64, rows64, grad64 = O.mean_loss_and_grad(kind, logits, T, t_logits=t_logits, valid=valid, t_T=teacher_T,
+                                                  dtype=torch.float64)
+    row_map = None
+    if valid is not None:
+        rm = torch.full((R,), -1, dtype=torch.int32)
+        rm[valid] = torch.arange(n_valid, dtype=torch.int32)
+        row_map = rm.to(DEV)
+    rl, grad = D.div_dense(kind, logits.to(DEV), t_logits.to(DEV), row_map=row_map, T=T, teacher_T=teacher_T,
+                           grad_scale=1.0 / n_valid)
+    loss = D.reduce_sum(rl, 1.0 / n_valid).item()
+    rows = rl.cpu()
+    g = grad.cpu()
+    if valid is not None:
+        assert torch.count_nonzero(rows[~valid]) == 0 and torch.count_nonzero(g[~valid]) == 0
+        rows = rows[valid]
+    np.testing.assert_allclose(loss, loss64.item(), rtol=1e-5)
+    np.testing.assert_allclose(rows.double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    err = (g.double() - grad64).abs()
+    bound = O.storage_tolerance(grad64, logits.dtype, RTOL[logits.dtype])
+    # A gradient entry is a difference of terms of size (p + q) * (1 + |log p/q| + loss) / (T n): where
+    # they cancel, fp32 evaluation (here and in the reference) keeps ~1e-6 of the TERMS, not of the result.
+    sel = torch.arange(R) if valid is None else torch.nonzero(valid).squeeze(-1)
+    lp = torch.log_softmax(logits[sel].double() / T, -1)
+    lq = torch.log_softmax(t_logits.double() / (T if teacher_T is None else teacher_T), -1)
+    ratio = torch.nan_to_num((lp - lq).abs(), nan=0.0, posinf=0.0)
+    terms = (lp.exp() + lq.exp()) * (1 + ratio + rows64.unsqueeze(-1)) / (T * n_valid)
+    bound[sel] += 4e-6 * terms
+    assert (err <= bound).all(), f"{int((err > bound).sum())} entries off, worst ratio {(err / bound).max():.2f}"
+
+
+def _pair(R, V, dtype, seed, t_dtype=None, noise=1.0, std=2.0):
+    g = torch.Generator().manual_seed(seed)
+    s = (torch.randn(R, V, generator=g) * std).to(dtype)
+    t = (s.float() * 0.8 + torch.randn(R, V, generator=g) * noise).to(t_dtype or dtype)
+    return s, t
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+@pytest.mark.parametrize("dtype,t_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                           (torch.float16, torch.float16), (torch.bfloat16, torch.float32)])
+def test_dense_small(D, kind, dtype, t_dtype):
+    s, t = _pair(21, 2048, dtype, 1, t_dtype)
+    _check(D, kind, s, t, T=1.0)
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+def test_dense_vocab_32000_bf16_temperature_ragged_mask(D, kind):
+    s, t = _pair(48, 32000, torch.bfloat16, 2, noise=1.5)
+    valid = torch.ones(48, dtype=torch.bool)
+    valid[30:41] = False
+    _check(D, kind, s, t[valid], T=2.0, valid=valid)
+
+
+def test_dense_fp32_vocab_32000_config1_shape(D):
+    s, t = _pair(32, 32000, torch.float32, 3)
+    valid = torch.arange(32) < 29
+    _check(D, "fkl", s, t[valid], T=1.0, valid=valid)
+    _check(D, "jsd", s, t[valid], T=1.5, valid=valid, teacher_T=1.0)
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+def test_teacher_with_zero_mass_entries(D, kind):
+    # -inf teacher logits: zero mass; RKL renormalises the student over the remaining support
+    s, t = _pair(10, 4096, torch.float32, 4)
+    g = torch.Generator().manual_seed(4)
+    drop = torch.rand(10, 4096, generator=g) < 0.6
+    t = t.masked_fill(drop, float("-inf"))
+    _check(D, kind, s, t, T=1.0)
+
+
+@pytest.mark.parametrize("V,dtype", [(1001, torch.float32), (70000, torch.bfloat16), (50264, torch.float32)])
+def test_dense_streaming_fallback(D, V, dtype):
+    # odd vocabulary / rows beyond the register budget take the scalar multi-pass kernel
+    s, t = _pair(5, V, dtype, 5)
+    for kind in ("fkl", "rkl", "jsd"):
+        _check(D, kind, s, t, T=1.3)
+
+
+def test_dense_identical_distributions_give_zero(D):
+    s, _ = _pair(8, 8192, torch.float32, 6)
+    for kind in ("fkl", "rkl", "jsd"):
+        rl, grad = D.div_dense(kind, s.to(DEV), s.to(DEV))
+        assert rl.abs().max().item() < 1e-5 and grad.abs().max().item() < 2e-6
+
+
+def test_jsd_bounded_by_ln2_on_disjoint_supports(D):
+    a = torch.full((2, 1024), float("-inf"))
+    b = a.clone()
+    a[:, :500] = torch.randn(2, 500)
+    b[:, 500:] = torch.randn(2, 524)
+    rl, _ = D.div_dense("jsd", a.to(DEV), b.to(DEV))
+    np.testing.assert_allclose(rl.cpu().numpy(), np.log(2.0), rtol=1e-5)
+
+
+def test_synthetic_configs_1_and_2_at_reduced_rows(D):
+    from llm_distillery_amd import synthetic as S
+    c = S.config1(DEV, B=1, S=64)
+    assert int(c["valid"].sum()) == 57                    # ceil(10 %) of 64 = 7 padded
+    _check(D, "fkl", c["logits"].cpu(), c["t_logits"].cpu(), 1.0, valid=c["valid"].cpu())
+    c = S.config2(DEV, B=2, S=48)
+    assert c["t_logits"].shape[0] == int(c["lengths"].sum())
+    _check(D, "jsd", c["logits"].cpu(), c["t_logits"].cpu(), 2.0, valid=c["valid"].cpu())
