@@ -139,6 +139,36 @@ int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_strid
                          const float* coef_zk, void* grad, int64_t grad_stride, void* stream);
 
 /*
+ * Weighted merge of n_teachers sparse teachers with an optional vocabulary id map
+ * (no reference counterpart; generalises classes/data_manager.py:231-240, which is unweighted,
+ * pairwise and has no map).  Per row: mass = weights[j] * exp(t_vals[j][row, k]); the id goes
+ * through id_map (int32 [Vt], teacher id -> student id, -1 = dropped; NULL = identity); entries
+ * outside [0, Vs) are dropped; entries on the same id are summed in entry order (teacher 0 first).
+ * Output, E = n_teachers * K columns per row: out_idx ascending ids (int32, -1 padding),
+ * out_logmass = log(summed mass) (fp32, -inf padding), out_cnt = survivors per row.  Feed these to
+ * dl_div_topk as (t_val = out_logmass, t_idx = out_idx, K = E, t_cnt = out_cnt): it renormalises.
+ * t_vals / t_idxs / weights are HOST arrays of n_teachers device pointers / floats.
+ * n_teachers <= DL_MAX_TEACHERS, n_teachers * K <= 4096.
+ */
+int dl_merge_remap_topk(int n_teachers, const void* const* t_vals, const void* const* t_idxs,
+                        int val_dtype, int idx_itype, int K, const float* weights, int64_t n_rows,
+                        const int32_t* id_map, int64_t Vt, int64_t Vs,
+                        int32_t* out_idx, float* out_logmass, int32_t* out_cnt, void* stream);
+
+/*
+ * The dataset manager's pairwise merge, classes/data_manager.py:198-261 (merge_topk): exp both
+ * inputs, per row sum the masses of equal ids, keep the K largest in descending order, log.
+ * Rows that only the longer input holds pass through in their stored order (:214-224,242-244).
+ * Ties between equal masses go to the smaller id (the reference leaves them to torch.topk).
+ * Outputs cover max(disk_rows, new_rows) rows: out_logmass fp32 [rows, K], out_idx int64 [rows, K].
+ * 2 * K <= 4096.
+ */
+int dl_merge_topk_pair(const void* disk_val, const void* disk_idx, int64_t disk_rows,
+                       const void* new_val, const void* new_idx, int64_t new_rows,
+                       int val_dtype, int idx_itype, int K, int64_t V,
+                       float* out_logmass, int64_t* out_idx, void* stream);
+
+/*
  * Deterministic sum of n fp32 values times `scale` into out[0] (fixed reduction tree,
  * double accumulation).  Replaces the `.mean()` of utils/finetuning_utils.py:54 /
  * the `+=` accumulation of classes/losses.py:43-47.

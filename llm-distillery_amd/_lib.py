@@ -32,6 +32,9 @@ _SIGNATURES = {
                                  _P, _P, _P]),
     "dl_rowcoef_grad_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int, c_int64, c_float,
                                      _P, _P, _P, _P, c_int64, _P]),
+    "dl_merge_remap_topk": (c_int, [c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, c_int64, c_int64,
+                                    _P, _P, _P, _P]),
+    "dl_merge_topk_pair": (c_int, [_P, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int64, _P, _P, _P]),
     "dl_set_option": (c_int, [c_char_p, c_int]),
     "dl_reduce_sum": (c_int, [_P, c_int64, c_float, _P, _P]),
     "dl_copy16": (c_int, [_P, _P, c_int64, _P]),

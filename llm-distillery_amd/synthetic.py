@@ -91,3 +91,31 @@ def config2(device, B: int = 4, S: int = 2048, V: int = 32000, seed: int = 2, dt
     valid = (torch.arange(S, device=device).unsqueeze(0) < lengths.unsqueeze(1)).reshape(-1)
     return {"logits": logits, "t_logits": teacher[valid].contiguous(), "valid": valid,
             "row_map": row_map_from_valid(valid), "T": 2.0, "kind": "jsd", "lengths": lengths}
+
+
+def vocab_id_map(device, Vt: int = 152064, Vs: int = 128256, drop: float = 0.05, seed: int = 40) -> torch.Tensor:
+    """Seeded int32 teacher->student id map: ~`drop` of the teacher ids map to -1 (dropped), the rest
+    to uniform student ids, so many teacher ids collide on one student id."""
+    g = _gen(device, seed)
+    m = torch.randint(0, Vs, (Vt,), generator=g, device=device, dtype=torch.int32)
+    m[torch.rand((Vt,), generator=g, device=device) < drop] = -1
+    return m
+
+
+def config4(device, rows: int = 4 * 8192, V: int = 128256, Vt: int = 152064, K: int = 200, n_teachers: int = 3,
+            seed: int = 4, dtype=torch.bfloat16):
+    """Multi-teacher merge + vocabulary remap, forward KL: three top-K=200 teachers over a
+    152064-id teacher vocabulary, weights (0.5, 0.3, 0.2), seeded id map into the 128256-id student
+    vocabulary (~5 % dropped, collisions sum), bf16 student logits ~ N(0, 3^2), T = 1."""
+    g = _gen(device, seed)
+    logits = torch.empty((rows, V), dtype=dtype, device=device)
+    vals = [torch.empty((rows, K), dtype=torch.float16, device=device) for _ in range(n_teachers)]
+    idxs = [torch.empty((rows, K), dtype=torch.int32, device=device) for _ in range(n_teachers)]
+    for a in range(0, rows, CHUNK_ROWS):
+        b = min(rows, a + CHUNK_ROWS)
+        chunk = (torch.randn((b - a, V), generator=g, device=device) * 3.0).to(dtype)
+        logits[a:b] = chunk
+        for j in range(n_teachers):
+            vals[j][a:b], idxs[j][a:b] = topk_teacher_for(chunk, K, 20, g, teacher_vocab=Vt)
+    return {"logits": logits, "t_vals": vals, "t_idxs": idxs, "weights": (0.5, 0.3, 0.2)[:n_teachers],
+            "id_map": vocab_id_map(device, Vt, V, seed=seed + 36), "T": 1.0, "kind": "fkl"}
