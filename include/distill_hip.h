@@ -169,6 +169,54 @@ int dl_merge_topk_pair(const void* disk_val, const void* disk_idx, int64_t disk_
                        float* out_logmass, int64_t* out_idx, void* stream);
 
 /*
+ * Byte-trie longest-prefix map between two tokenizers (no reference counterpart; the reference
+ * rejects cross-vocabulary distillation, collect_and_finetune.py:83-101).  HOST function, HOST
+ * pointers.  Vocabularies are given as concatenated byte strings plus int64 offsets [n + 1].
+ * out_t2s[t] = id of the student token whose bytes are the longest prefix of teacher token t
+ * (duplicate student strings: the smallest id), else byte_fallback[first byte] if that table
+ * (256 int32, may be NULL) holds an id >= 0, else -1; empty teacher tokens map to -1.
+ */
+int dl_trie_longest_prefix_map(const uint8_t* student_bytes, const int64_t* student_offsets, int64_t n_student,
+                               const uint8_t* teacher_bytes, const int64_t* teacher_offsets, int64_t n_teacher,
+                               const int32_t* byte_fallback, int32_t* out_t2s);
+
+/*
+ * CSR form of a teacher->student map (HOST function, HOST pointers): offsets int32 [n_student + 1],
+ * indices int32 [n_teacher] (the first *n_mapped entries are used) listing, per student id, the
+ * teacher ids mapped to it in ascending order; ids mapped to -1 are left out.
+ */
+int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int32_t* offsets,
+                    int32_t* indices, int64_t* n_mapped);
+
+/*
+ * marg[r, s] = sum of probs[r, t] over the teacher ids t with t2s[t] == s (probs [n_rows, Vt] in
+ * p_dtype, marg fp32 [n_rows, Vs]; out_log != 0 stores log(marg) instead).  Accumulates with LDS
+ * floating-point atomics: sums agree with the CSR form to fp32 rounding, not bit for bit.
+ */
+int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
+                       const int32_t* t2s, int64_t Vs, float* marg, int64_t marg_stride, int out_log,
+                       void* stream);
+
+/* The same marginal from the CSR form, each segment added in ascending teacher-id order (bit-reproducible). */
+int dl_marginalise_csr(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
+                       const int32_t* offsets, const int32_t* indices, int64_t Vs, float* marg,
+                       int64_t marg_stride, int out_log, void* stream);
+
+/*
+ * Fused: marginalise the dense teacher row t_probs[row_map[r]] (over Vt teacher ids) into the Vs
+ * student ids inside LDS, then reverse KL of the student logits[r] against
+ * softmax(log(marginal) * inv_T_teacher), loss and gradient, with the conventions of dl_div_dense
+ * (DL_RKL: student renormalised over the marginal's support).  The marginal never reaches memory.
+ * Vs <= 36864 (the fp32 marginal of one row must fit the CU's LDS), Vs % 8 == 0, logits / grad
+ * rows 16-byte aligned (else DL_ERR_LIMIT / DL_ERR_ALIGN: use dl_marginalise_map + dl_div_dense).
+ */
+int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs,
+                        const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
+                        int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s,
+                        float inv_T_student, float inv_T_teacher, float grad_scale,
+                        float* row_loss, void* grad, int64_t grad_stride, void* stream);
+
+/*
  * Deterministic sum of n fp32 values times `scale` into out[0] (fixed reduction tree,
  * double accumulation).  Replaces the `.mean()` of utils/finetuning_utils.py:54 /
  * the `+=` accumulation of classes/losses.py:43-47.

@@ -42,6 +42,7 @@ struct DenseStats {
   float ls, lt;          // log2-sum-exp2 of the scaled student (over the support for RKL) / teacher row
   float loss;            // natural-log divergence of the row
   float aux;             // FKL: unused; RKL: rkl; JSD: KL(P || M)
+  float tmax;            // largest teacher logit of the row (-inf: the teacher row carries no mass)
 };
 
 // Divergence terms of one column.  lp / lq: log2-probabilities of student / teacher.
@@ -91,6 +92,7 @@ __device__ __forceinline__ DenseStats dense_stats(int kind, Rows& rows, float in
     }
   });
   block_max2<NT>(ms, mt, red);
+  st.tmax = mt;
   const float bs = ms * st.a_s, bt = mt * st.a_t;
   float ss = 0.f, stt = 0.f;
   rows.sweep([&](int64_t, const float* s, const float* t) {

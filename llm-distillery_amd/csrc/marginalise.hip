@@ -1,0 +1,253 @@
+// Cross-tokenizer marginalisation: a dense teacher distribution over the TEACHER vocabulary is
+// summed into the student vocabulary along a many-to-one id map,
+//     marg[r, s] = sum over { t : t2s[t] == s } of p[r, t],
+// and, fused, the reverse KL of the student against that marginal with its gradient.
+//
+//   * map form (fast): one workgroup per row streams the teacher row once (16-byte loads of the
+//     probabilities and of the id map, which stays L2-resident) and accumulates into an LDS copy
+//     of the student vocabulary with ds_add_f32.  The order of the additions is not fixed, so the
+//     sums agree to fp32 rounding, not bit for bit.
+//   * CSR form (deterministic): one thread per student id adds its segment in ascending
+//     teacher-id order.
+//   * fused reverse KL: the marginal never leaves LDS; its logarithm is the teacher row of the
+//     dense-divergence sweeps, the student row sits in registers.
+#include "dense_div.hpp"
+
+namespace dl {
+
+constexpr int MARG_NT = 1024;
+constexpr int MARG_MAX_VS = 36864;          // fp32 marginal of one row in LDS: 144 KiB of the CU's 160
+
+struct MargParams {
+  const void* probs; int p_dtype; int64_t p_stride; int64_t n_rows; int64_t Vt;
+  const int32_t* t2s; int64_t Vs;
+  float* marg; int64_t marg_stride; int out_log;
+  // fused reverse KL
+  const void* logits; int s_dtype; int64_t row_stride; int64_t n_srows; const int32_t* row_map;
+  float inv_T_s, inv_T_t, grad_scale; float* row_loss; void* grad; int64_t grad_stride;
+};
+
+// Accumulate the slice [s_lo, s_lo + s_n) of one row's marginal into `acc` (LDS, zeroed here).
+template <bool VEC>
+__device__ __forceinline__ void accumulate_marginal(const MargParams& p, const char* prow, float* acc, int s_lo,
+                                                    int s_n) {
+  const int tid = threadIdx.x;
+  for (int j = tid; j < s_n; j += MARG_NT) acc[j] = 0.f;
+  __syncthreads();
+  if (VEC) {       // fp32 probabilities, 16-byte aligned: four columns per load
+    const int64_t n4 = p.Vt / 4;
+    for (int64_t c0 = 0; c0 < n4; c0 += 2 * MARG_NT) {
+      u32x4 pv[2], iv[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int64_t c = c0 + (int64_t)u * MARG_NT + tid;
+        if (c < n4) {
+          pv[u] = load16_stream(prow + c * 16);
+          iv[u] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.t2s) + c * 16);
+        } else {
+          pv[u] = u32x4{0u, 0u, 0u, 0u};
+          iv[u] = u32x4{~0u, ~0u, ~0u, ~0u};
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int s = (int)iv[u][e] - s_lo;
+          if (s >= 0 && s < s_n)
+            __hip_atomic_fetch_add(&acc[s], __uint_as_float(pv[u][e]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+  } else {
+    for (int64_t t = tid; t < p.Vt; t += MARG_NT) {
+      const int s = p.t2s[t] - s_lo;
+      if (s >= 0 && s < s_n)
+        __hip_atomic_fetch_add(&acc[s], load_as_float(prow, p.p_dtype, t), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  }
+  __syncthreads();
+}
+
+// marg (or log marg) to memory; student vocabularies wider than the LDS slice take several passes.
+template <bool VEC>
+__global__ __launch_bounds__(MARG_NT) void marginalise_map_kernel(const MargParams p) {
+  extern __shared__ __align__(16) float acc[];
+  const int64_t r = blockIdx.x;
+  const int pb = p.p_dtype == F32 ? 4 : 2;
+  const char* prow = reinterpret_cast<const char*>(p.probs) + r * p.p_stride * pb;
+  float* out = p.marg + r * p.marg_stride;
+  for (int64_t s_lo = 0; s_lo < p.Vs; s_lo += MARG_MAX_VS) {
+    const int s_n = (int)min((int64_t)MARG_MAX_VS, p.Vs - s_lo);
+    accumulate_marginal<VEC>(p, prow, acc, (int)s_lo, s_n);
+    for (int j = threadIdx.x; j < s_n; j += MARG_NT) out[s_lo + j] = p.out_log ? logf(acc[j]) : acc[j];
+    __syncthreads();
+  }
+}
+
+// Deterministic form: thread per student id, segment summed in ascending teacher-id order.
+__global__ __launch_bounds__(256) void marginalise_csr_kernel(const void* probs, int p_dtype, int64_t p_stride,
+                                                             int64_t Vt, const int32_t* offsets,
+                                                             const int32_t* indices, int64_t Vs, float* marg,
+                                                             int64_t marg_stride, int out_log) {
+  const int64_t r = blockIdx.y;
+  const int64_t s = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (s >= Vs) return;
+  const char* prow = reinterpret_cast<const char*>(probs) + r * p_stride * (p_dtype == F32 ? 4 : 2);
+  float m = 0.f;
+  for (int e = offsets[s]; e < offsets[s + 1]; ++e) {
+    const int t = indices[e];
+    if (t >= 0 && t < Vt) m += load_as_float(prow, p_dtype, t);
+  }
+  marg[r * marg_stride + s] = out_log ? logf(m) : m;
+}
+
+// ---- fused: marginal in LDS -> reverse KL against the student row in registers -----------------
+template <class TagS, int NU>
+struct LdsTeacherRows {
+  Unit<TagS> s[NU];
+  const float* lt;      // log marginal, LDS
+  int64_t nunits;
+  __device__ __forceinline__ void load(const char* srow, int64_t nu) {
+    nunits = nu;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + threadIdx.x;
+      if (u < nunits) s[i].load(srow, u); else s[i].fill_neg_inf();
+    }
+  }
+  template <class F>
+  __device__ __forceinline__ void sweep(F f) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + threadIdx.x;
+      if (u < nunits) {
+        float a[8], b[8];
+        s[i].unpack(a);
+        const float4 b0 = *reinterpret_cast<const float4*>(lt + u * 8);
+        const float4 b1 = *reinterpret_cast<const float4*>(lt + u * 8 + 4);
+        b[0] = b0.x; b[1] = b0.y; b[2] = b0.z; b[3] = b0.w; b[4] = b1.x; b[5] = b1.y; b[6] = b1.z; b[7] = b1.w;
+        f(u, a, b);
+      }
+    }
+  }
+};
+
+template <class TagS, int NU, bool VEC>
+__global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargParams p) {
+  extern __shared__ __align__(16) float acc[];
+  __shared__ float red[64];
+  const int64_t r = blockIdx.x;
+  const int tid = threadIdx.x;
+  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
+  const int64_t trow = teacher_row(p.row_map, r, p.n_rows);
+  if (trow < 0) {
+    if (grow) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
+    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    return;
+  }
+  LdsTeacherRows<TagS, NU> rows;
+  rows.load(reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes, p.Vs / 8);   // in flight during the scatter
+  const int pb = p.p_dtype == F32 ? 4 : 2;
+  accumulate_marginal<VEC>(p, reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb, acc, 0, (int)p.Vs);
+  for (int j = tid; j < p.Vs; j += MARG_NT) acc[j] = fast_log2(acc[j]) * LN2;      // log 0 = -inf: off the support
+  __syncthreads();
+  rows.lt = acc;
+  const DenseStats st = dense_stats<MARG_NT>(DL_RKL, rows, p.inv_T_s, p.inv_T_t, red);
+  const bool empty = st.tmax == -INFINITY;        // the teacher row carried no mass at all
+  if (tid == 0 && p.row_loss) p.row_loss[r] = empty ? 0.f : st.loss;
+  if (grow) {
+    if (empty) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
+    else dense_grad_sweep<TagS>(DL_RKL, rows, st, p.inv_T_s * p.grad_scale, grow);
+  }
+}
+
+static bool ok16(const void* ptr, int64_t stride, int eb) {
+  return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (stride * eb) % 16 == 0;
+}
+
+}  // namespace dl
+
+extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
+                                  const int32_t* t2s, int64_t Vs, float* marg, int64_t marg_stride, int out_log,
+                                  void* stream) {
+  using namespace dl;
+  if (!probs || !t2s || !marg) return DL_ERR_NULL;
+  if (p_dtype < DL_F32 || p_dtype > DL_F16) return DL_ERR_DTYPE;
+  if (n_rows < 0 || Vt <= 0 || Vs <= 0 || p_stride < Vt || marg_stride < Vs) return DL_ERR_SHAPE;
+  if (n_rows > 0x7fffffffLL || Vt > 0x7fffffffLL || Vs > 0x7fffffffLL) return DL_ERR_LIMIT;
+  if (n_rows == 0) return DL_OK;
+  MargParams p{};
+  p.probs = probs; p.p_dtype = p_dtype; p.p_stride = p_stride; p.n_rows = n_rows; p.Vt = Vt; p.t2s = t2s; p.Vs = Vs;
+  p.marg = marg; p.marg_stride = marg_stride; p.out_log = out_log;
+  const size_t lds = (size_t)(Vs < MARG_MAX_VS ? Vs : MARG_MAX_VS) * 4;
+  const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(probs, p_stride, 4) && ok16(t2s, 0, 4);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  // more than 64 KiB of dynamic LDS has to be requested per kernel
+  hipFuncSetAttribute(reinterpret_cast<const void*>(&marginalise_map_kernel<true>),
+                      hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);
+  hipFuncSetAttribute(reinterpret_cast<const void*>(&marginalise_map_kernel<false>),
+                      hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);
+  if (vec) hipLaunchKernelGGL((marginalise_map_kernel<true>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
+  else hipLaunchKernelGGL((marginalise_map_kernel<false>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
+  return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}
+
+extern "C" int dl_marginalise_csr(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
+                                  const int32_t* offsets, const int32_t* indices, int64_t Vs, float* marg,
+                                  int64_t marg_stride, int out_log, void* stream) {
+  using namespace dl;
+  if (!probs || !offsets || !indices || !marg) return DL_ERR_NULL;
+  if (p_dtype < DL_F32 || p_dtype > DL_F16) return DL_ERR_DTYPE;
+  if (n_rows < 0 || Vt <= 0 || Vs <= 0 || p_stride < Vt || marg_stride < Vs) return DL_ERR_SHAPE;
+  if (n_rows > 65535 * 1024LL || Vs > 0x7fffffffLL) return DL_ERR_LIMIT;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  for (int64_t r0 = 0; r0 < n_rows; r0 += 65535) {        // grid.y limit
+    const int64_t nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    const int pb = p_dtype == DL_F32 ? 4 : 2;
+    hipLaunchKernelGGL(marginalise_csr_kernel, dim3((unsigned)((Vs + 255) / 256), (unsigned)nr), dim3(256), 0, st,
+                       reinterpret_cast<const char*>(probs) + r0 * p_stride * pb, p_dtype, p_stride, Vt, offsets,
+                       indices, Vs, marg + r0 * marg_stride, marg_stride, out_log);
+  }
+  return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}
+
+extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs,
+                                   const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
+                                   int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s, float inv_T_student,
+                                   float inv_T_teacher, float grad_scale, float* row_loss, void* grad,
+                                   int64_t grad_stride, void* stream) {
+  using namespace dl;
+  if (!logits || !t_probs || !t2s) return DL_ERR_NULL;
+  if (logits_dtype < DL_F32 || logits_dtype > DL_F16 || p_dtype < DL_F32 || p_dtype > DL_F16) return DL_ERR_DTYPE;
+  if (n_rows < 0 || Vs <= 0 || Vt <= 0 || n_teacher_rows < 0 || row_stride < Vs || p_stride < Vt ||
+      (grad && grad_stride < Vs))
+    return DL_ERR_SHAPE;
+  if (Vs > MARG_MAX_VS || n_rows > 0x7fffffffLL || Vt > 0x7fffffffLL) return DL_ERR_LIMIT;
+  const int sb = logits_dtype == DL_F32 ? 4 : 2;
+  if (Vs % 8 != 0 || !ok16(logits, row_stride, sb) || (grad && !ok16(grad, grad_stride, sb))) return DL_ERR_ALIGN;
+  if (n_rows == 0) return DL_OK;
+  MargParams p{};
+  p.probs = t_probs; p.p_dtype = p_dtype; p.p_stride = p_stride; p.n_rows = n_teacher_rows; p.Vt = Vt; p.t2s = t2s;
+  p.Vs = Vs; p.logits = logits; p.s_dtype = logits_dtype; p.row_stride = row_stride; p.n_srows = n_rows;
+  p.row_map = row_map; p.inv_T_s = inv_T_student; p.inv_T_t = inv_T_teacher; p.grad_scale = grad_scale;
+  p.row_loss = row_loss; p.grad = grad; p.grad_stride = grad_stride;
+  const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(t_probs, p_stride, 4) && ok16(t2s, 0, 4);
+  const size_t lds = (size_t)Vs * 4;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)n_rows), block(MARG_NT);
+#define DL_LAUNCH_RKLM(TAG)                                                                                  \
+  do {                                                                                                       \
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&rkl_marginalised_kernel<TAG, 8, true>),               \
+                        hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);                        \
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&rkl_marginalised_kernel<TAG, 8, false>),              \
+                        hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);                        \
+    if (vec) hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, 8, true>), grid, block, lds, st, p);           \
+    else hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, 8, false>), grid, block, lds, st, p);              \
+  } while (0)
+  if (logits_dtype == DL_F32) DL_LAUNCH_RKLM(TagF32);
+  else if (logits_dtype == DL_BF16) DL_LAUNCH_RKLM(TagBF16);
+  else DL_LAUNCH_RKLM(TagF16);
+#undef DL_LAUNCH_RKLM
+  return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}

@@ -119,3 +119,38 @@ def config4(device, rows: int = 4 * 8192, V: int = 128256, Vt: int = 152064, K: 
             vals[j][a:b], idxs[j][a:b] = topk_teacher_for(chunk, K, 20, g, teacher_vocab=Vt)
     return {"logits": logits, "t_vals": vals, "t_idxs": idxs, "weights": (0.5, 0.3, 0.2)[:n_teachers],
             "id_map": vocab_id_map(device, Vt, V, seed=seed + 36), "T": 1.0, "kind": "fkl"}
+
+
+def random_byte_vocab(n: int, seed: int, min_len: int = 1, max_len: int = 16, alphabet: int = 256,
+                      all_single_bytes: bool = False) -> list[bytes]:
+    """n random byte strings with lengths uniform in [min_len, max_len]; with `all_single_bytes`
+    the first 256 entries are the 256 one-byte strings (the byte-fallback tokens)."""
+    rng = np.random.default_rng(seed)
+    out: list[bytes] = [bytes([b]) for b in range(256)] if all_single_bytes else []
+    lens = rng.integers(min_len, max_len + 1, n - len(out))
+    blob = rng.integers(0, alphabet, int(lens.sum()), dtype=np.uint8).tobytes()
+    at = 0
+    for L in lens:
+        out.append(blob[at:at + int(L)])
+        at += int(L)
+    return out
+
+
+def config5(device, rows: int = 2 * 4096, Vs: int = 32000, Vt: int = 152064, seed: int = 5, dtype=torch.bfloat16,
+            alphabet: int = 256):
+    """Cross-tokenizer byte-trie marginalisation, then reverse KL: student vocabulary of `Vs` random
+    byte strings (lengths 1-16, all 256 single bytes included), teacher vocabulary of `Vt` random byte
+    strings; dense fp32 teacher softmax [rows, Vt]; bf16 student logits ~ N(0, 2^2); T = 1.5.
+    The id map / CSR come from the host trie."""
+    from . import vocab_utils
+    student_vocab = random_byte_vocab(Vs, seed * 100 + 1, all_single_bytes=True, alphabet=alphabet)
+    teacher_vocab = random_byte_vocab(Vt, seed * 100 + 2, alphabet=alphabet)
+    t2s = vocab_utils.longest_prefix_map(student_vocab, teacher_vocab)
+    g = _gen(device, seed)
+    logits = (torch.randn((rows, Vs), generator=g, device=device) * 2.0).to(dtype)
+    probs = torch.empty((rows, Vt), dtype=torch.float32, device=device)
+    for a in range(0, rows, CHUNK_ROWS):
+        b = min(rows, a + CHUNK_ROWS)
+        probs[a:b] = torch.softmax(torch.randn((b - a, Vt), generator=g, device=device) * 2.0, dim=-1)
+    return {"logits": logits, "t_probs": probs, "t2s": torch.as_tensor(t2s, device=device), "t2s_host": t2s,
+            "student_vocab": student_vocab, "teacher_vocab": teacher_vocab, "T": 1.5, "kind": "rkl"}

@@ -1,0 +1,125 @@
+"""Cross-tokenizer vocabulary tables and marginalisation.
+
+The reference's `utils/vocab_utils.py` only names tokenizer families and rejects distillation
+across vocabularies (collect_and_finetune.py:83-101); this module supplies what that case needs:
+a byte-trie longest-prefix map from teacher tokens to student tokens, its CSR form, the
+marginalisation of a dense teacher distribution into the student vocabulary, and the reverse KL
+against it.  The table builders are host C++ (libdistill_hip.so, no GPU needed); the
+marginalisation and the loss are HIP kernels.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+from .ops import _DT, _dev, _opt_i32, _rows_2d, _stream_ptr
+
+
+def _pack(vocab: Sequence[bytes]):
+    lens = np.fromiter((len(b) for b in vocab), dtype=np.int64, count=len(vocab))
+    offsets = np.zeros(len(vocab) + 1, dtype=np.int64)
+    np.cumsum(lens, out=offsets[1:])
+    blob = np.frombuffer(b"".join(bytes(b) for b in vocab), dtype=np.uint8) if offsets[-1] else np.zeros(1, np.uint8)
+    return np.ascontiguousarray(blob), offsets
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def longest_prefix_map(student_vocab: Sequence[bytes], teacher_vocab: Sequence[bytes],
+                       byte_fallback: Sequence[int] | None = None) -> np.ndarray:
+    """int32 [len(teacher_vocab)]: for every teacher token the id of the student token whose bytes
+    are the longest prefix of the teacher token's bytes; `byte_fallback[first byte]` (256 ids, -1 =
+    none) when no student token is a prefix; -1 otherwise."""
+    sb, so = _pack(student_vocab)
+    tb, to = _pack(teacher_vocab)
+    fb = None
+    if byte_fallback is not None:
+        fb = np.ascontiguousarray(np.asarray(byte_fallback, dtype=np.int32))
+        if fb.shape != (256,):
+            raise ValueError("byte_fallback must hold 256 ids")
+    out = np.empty(len(teacher_vocab), dtype=np.int32)
+    st = _lib.load().dl_trie_longest_prefix_map(_p(sb), _p(so), len(student_vocab), _p(tb), _p(to), len(teacher_vocab),
+                                                _p(fb) if fb is not None else None, _p(out))
+    _lib.check(st, "dl_trie_longest_prefix_map")
+    return out
+
+
+def csr_from_map(t2s: np.ndarray, n_student: int) -> tuple[np.ndarray, np.ndarray]:
+    """(offsets int32 [n_student + 1], indices int32 [#mapped]): teacher ids grouped by student id,
+    ascending inside a group; ids mapped to -1 are left out."""
+    t2s = np.ascontiguousarray(np.asarray(t2s, dtype=np.int32))
+    offsets = np.empty(n_student + 1, dtype=np.int32)
+    indices = np.empty(max(t2s.size, 1), dtype=np.int32)
+    n = ctypes.c_int64(0)
+    st = _lib.load().dl_csr_from_map(_p(t2s), t2s.size, n_student, _p(offsets), _p(indices), ctypes.byref(n))
+    _lib.check(st, "dl_csr_from_map")
+    return offsets, indices[:n.value].copy()
+
+
+def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=None, n_student: int,
+                log: bool = False) -> torch.Tensor:
+    """marg[r, s] = sum of probs[r, t] over the teacher ids mapped to s (fp32 [rows, n_student]).
+    `t2s` (int32 [Vt], on the GPU) selects the fast LDS-atomic form; `csr=(offsets, indices)` the
+    deterministic one.  `log=True` returns log(marg)."""
+    _dev(probs, "probs")
+    x = _rows_2d(probs)
+    if x.dtype not in _DT:
+        raise RuntimeError("unsupported dtype")
+    R, Vt = x.shape
+    out = torch.empty((R, n_student), dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        if csr is not None:
+            off, ind = csr
+            _dev(off, "offsets"), _dev(ind, "indices")
+            if off.dtype != torch.int32 or ind.dtype != torch.int32 or off.numel() != n_student + 1:
+                raise RuntimeError("csr must be (int32 offsets [n_student + 1], int32 indices)")
+            if int(off[-1].item()) > ind.numel():
+                raise RuntimeError("csr offsets run past the indices array")
+            st = lib.dl_marginalise_csr(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vt, off.contiguous().data_ptr(),
+                                        ind.contiguous().data_ptr(), n_student, out.data_ptr(), out.stride(0), int(log),
+                                        _stream_ptr(x.device))
+            _lib.check(st, "dl_marginalise_csr")
+        else:
+            _, _ = _opt_i32(t2s, Vt, "t2s", x.device)
+            st = lib.dl_marginalise_map(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vt, t2s.data_ptr(), n_student,
+                                        out.data_ptr(), out.stride(0), int(log), _stream_ptr(x.device))
+            _lib.check(st, "dl_marginalise_map")
+    return out
+
+
+def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: torch.Tensor, *,
+                     row_map: torch.Tensor | None = None, T: float = 1.0, teacher_T: float | None = None,
+                     grad_scale: float = 1.0, want_grad: bool = True, grad_out: torch.Tensor | None = None):
+    """Reverse KL of the student (logits [rows, Vs]) against the teacher's distribution
+    (teacher_probs [N, Vt]) marginalised into the student vocabulary along `t2s`, loss and gradient
+    in one launch; the marginal stays in LDS.  Returns (row_loss fp32 [rows], grad or None)."""
+    _dev(logits, "logits"), _dev(teacher_probs, "teacher_probs")
+    x, tp = _rows_2d(logits), _rows_2d(teacher_probs)
+    R, Vs = x.shape
+    N, Vt = tp.shape
+    dev = x.device
+    if x.dtype not in _DT or tp.dtype not in _DT:
+        raise RuntimeError("unsupported dtype")
+    if row_map is None and N < R:
+        raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
+    _, rm_ptr = _opt_i32(row_map, R, "row_map", dev)
+    _opt_i32(t2s, Vt, "t2s", dev)
+    row_loss = torch.empty(R, dtype=torch.float32, device=dev)
+    grad, g_ptr, g_stride = None, 0, Vs
+    if want_grad:
+        grad = grad_out if grad_out is not None else torch.empty((R, Vs), dtype=x.dtype, device=dev)
+        g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_rkl_marginalised(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vs, rm_ptr, tp.data_ptr(),
+                                             _DT[tp.dtype], tp.stride(0), N, Vt, t2s.data_ptr(), 1.0 / T,
+                                             1.0 / (T if teacher_T is None else teacher_T), grad_scale,
+                                             row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
+    _lib.check(st, "dl_rkl_marginalised")
+    return row_loss, grad

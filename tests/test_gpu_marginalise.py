@@ -1,0 +1,97 @@
+"""GPU parity of the cross-tokenizer marginalisation and the fused reverse KL against it."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def D():
+    import llm_distillery_amd as d
+    d._lib.load()
+    return d
+
+
+def _case(R, Vs, Vt, seed, alphabet=4, drop=0.0):
+    from llm_distillery_amd import synthetic as S
+    import llm_distillery_amd as d
+    student = S.random_byte_vocab(Vs, seed, alphabet=alphabet, max_len=6, all_single_bytes=(alphabet == 256))
+    teacher = S.random_byte_vocab(Vt, seed + 1, alphabet=alphabet, max_len=8)
+    t2s = d.vocab_utils.longest_prefix_map(student, teacher)
+    if drop:
+        t2s = t2s.copy()
+        t2s[np.random.default_rng(seed).random(Vt) < drop] = -1
+    g = torch.Generator().manual_seed(seed)
+    probs = torch.softmax(torch.randn(R, Vt, generator=g) * 2, -1)
+    return t2s, probs
+
+
+@pytest.mark.parametrize("Vs,Vt,alphabet", [(1000, 5000, 4), (32000, 152064, 256), (40000, 50001, 16)])
+def test_marginal_map_and_csr_forms(D, Vs, Vt, alphabet):
+    t2s, probs = _case(6, Vs, Vt, 1, alphabet, drop=0.02)
+    ref = O.marginalise_map(probs.numpy(), t2s, Vs)
+    off, ind = D.vocab_utils.csr_from_map(t2s, Vs)
+    np.testing.assert_allclose(ref, O.marginalise_csr(probs.numpy(), off, ind), rtol=1e-12, atol=1e-15)
+    m_map = D.vocab_utils.marginalise(probs.to(DEV), t2s=torch.tensor(t2s, device=DEV), n_student=Vs).cpu().numpy()
+    m_csr = D.vocab_utils.marginalise(probs.to(DEV), csr=(torch.tensor(off, device=DEV), torch.tensor(ind, device=DEV)),
+                                      n_student=Vs).cpu().numpy()
+    # marginal sums within fp32 tolerance; exact zeros where no teacher token maps
+    np.testing.assert_allclose(m_map, ref, rtol=2e-6, atol=1e-9)
+    np.testing.assert_allclose(m_csr, ref, rtol=2e-6, atol=1e-9)
+    assert np.array_equal(m_map == 0, ref == 0) and np.array_equal(m_csr == 0, ref == 0)
+    np.testing.assert_allclose(m_map.astype(np.float64).sum(-1), probs.double().numpy()[:, t2s >= 0].sum(-1), rtol=1e-5)
+    # the CSR form is bit-reproducible
+    again = D.vocab_utils.marginalise(probs.to(DEV), csr=(torch.tensor(off, device=DEV), torch.tensor(ind, device=DEV)),
+                                      n_student=Vs).cpu().numpy()
+    assert np.array_equal(m_csr, again)
+    lg = D.vocab_utils.marginalise(probs.to(DEV), t2s=torch.tensor(t2s, device=DEV), n_student=Vs, log=True).cpu().numpy()
+    with np.errstate(divide="ignore"):
+        np.testing.assert_allclose(lg[ref > 0], np.log(ref[ref > 0]), rtol=1e-5, atol=1e-5)
+    assert np.isneginf(lg[ref == 0]).all()
+
+
+def test_marginal_of_16bit_probabilities(D):
+    t2s, probs = _case(4, 512, 2048, 2)
+    got = D.vocab_utils.marginalise(probs.to(torch.bfloat16).to(DEV), t2s=torch.tensor(t2s, device=DEV), n_student=512)
+    ref = O.marginalise_map(probs.to(torch.bfloat16).double().numpy(), t2s, 512)
+    np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=2e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("dtype,Vs,Vt,alphabet,T", [(torch.bfloat16, 32000, 152064, 256, 1.5), (torch.float32, 2048, 9000, 4, 1.0),
+                                                    (torch.float16, 8192, 30000, 8, 0.8)])
+def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T):
+    R = 12
+    t2s, probs = _case(R, Vs, Vt, 3, alphabet, drop=0.01)
+    g = torch.Generator().manual_seed(9)
+    logits = (torch.randn(R + 3, Vs, generator=g) * 2).to(dtype)
+    valid = torch.ones(R + 3, dtype=torch.bool)
+    valid[[2, 5, 14]] = False
+    rm = torch.full((R + 3,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(R, dtype=torch.int32)
+    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), torch.tensor(t2s, device=DEV),
+                                              row_map=rm.to(DEV), T=T, grad_scale=1.0 / R)
+    marg = torch.tensor(O.marginalise_map(probs.numpy(), t2s, Vs))
+    with np.errstate(divide="ignore"):
+        t_logits = O.marginal_to_teacher_logits(marg)
+    loss64, rows64, grad64 = O.mean_loss_and_grad("rkl", logits, T, t_logits=t_logits, valid=valid, dtype=torch.float64)
+    np.testing.assert_allclose(D.reduce_sum(rl, 1.0 / R).item(), loss64.item(), rtol=1e-5)
+    np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    assert torch.count_nonzero(grad.cpu()[~valid]) == 0 and torch.count_nonzero(rl.cpu()[~valid]) == 0
+    err = (grad.cpu().double() - grad64).abs()
+    rtol = 1e-4 if dtype == torch.float32 else 2e-3
+    bound = O.storage_tolerance(grad64, dtype, rtol)
+    sel = torch.nonzero(valid).squeeze(-1)
+    bound[sel] += 4e-6 * torch.softmax(logits[sel].double() / T, -1) * (1 + rows64.unsqueeze(-1)) * 20 / (T * R)
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+    # the gradient is confined to the marginal's support
+    assert torch.count_nonzero(grad.cpu()[valid][:, (marg.sum(0) == 0)]) == 0
+
+
+def test_fused_path_limits_are_reported(D):
+    with pytest.raises(RuntimeError, match="exceeds"):
+        D.vocab_utils.rkl_marginalised(torch.zeros(2, 40000, device=DEV), torch.zeros(2, 64, device=DEV),
+                                       torch.zeros(64, dtype=torch.int32, device=DEV))
