@@ -24,7 +24,7 @@ V, K = 128256, 200
 BYTES_PER_TOKEN = V * 2 + V * 2 + K * (2 + 4)     # logits read + grad write + teacher (fp16 + int32)
 
 
-def cpu_baseline(rows: int, reps: int = 3):
+def cpu_baseline(rows: int, reps: int = 7):
     """The reference's op sequence (cast -> /T -> log_softmax -> gather -> kl_div -> mean
     -> backward) in PyTorch eager on the host cores, on a bounded row sample of the same
     workload (rows are independent, so tokens/s carries over to the full row count)."""
@@ -61,7 +61,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--rows", type=int, default=8 * 4096)
-    ap.add_argument("--cpu-rows", type=int, default=1024, help="row sample for the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="row sample for the CPU baseline (0 = skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's plain copy kernel over the logits buffer (known traffic: "
                          "rows*V*2 bytes each way), the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
@@ -120,7 +120,7 @@ def main():
         "loss": loss.item(),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(),
-                     "kernel": "fkl_topk_reg_kernel<bf16,1024,16>", "kernel_ms": kern_ms,
+                     "kernel": "fkl_topk_reg_kernel<bf16,256,16,split> (4 column parts per row)", "kernel_ms": kern_ms,
                      "algorithmic_bytes": algo_bytes},
         "cpu_baseline": cpu_baseline(args.cpu_rows) if args.cpu_rows > 0 else None,
     }
