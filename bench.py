@@ -1,10 +1,11 @@
 """Benchmark of the distillation-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--rows R]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3]
 
-One step = one pass of the fused forward-KL loss + gradient over one batch of
-synthetic input (8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200
-fp16/int32 teacher, T=1) followed by the deterministic mean reduction.  Inputs are
+One step = one pass of the fused loss + gradient over one batch of synthetic input followed by the
+deterministic mean reduction.  The default workload is the one the headline metric is quoted on
+(C3: 8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200 fp16/int32 teacher, T=1);
+`--workload c1|c2|c4|c5` measures the other configurations with the same harness.  Inputs are
 resident in HBM before the timed region.  Prints ONE JSON line.
 """
 from __future__ import annotations
@@ -20,37 +21,147 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
-V, K = 128256, 200
-BYTES_PER_TOKEN = V * 2 + V * 2 + K * (2 + 4)     # logits read + grad write + teacher (fp16 + int32)
 
 
-def cpu_baseline(rows: int, reps: int = 7):
-    """The reference's op sequence (cast -> /T -> log_softmax -> gather -> kl_div -> mean
-    -> backward) in PyTorch eager on the host cores, on a bounded row sample of the same
-    workload (rows are independent, so tokens/s carries over to the full row count)."""
+# ---------------------------------------------------------------------------------------------
+# workloads: build(device, rows) -> (step_fn, main_launch_fn, algorithmic_bytes, tokens, description, kernel)
+# step_fn runs the whole step and returns the loss tensor; main_launch_fn launches only the dominant kernel.
+# ---------------------------------------------------------------------------------------------
+def _wl_c3(D, S, dev, rows):
+    import torch
+    rows = rows or 8 * 4096
+    V, K = 128256, 200
+    c = S.config3(dev, rows=rows, seed=3)
+    grad = torch.empty_like(c["logits"])
+    scale = 1.0 / rows
+
+    def main():
+        return D.div_topk("fkl", c["logits"], c["t_val"], c["t_idx"], T=1.0, grad_scale=scale, grad_out=grad)[0]
+
+    return (lambda: D.reduce_sum(main(), scale), main, rows * (V * 2 + V * 2 + K * 6), rows,
+            f"C3 forward-KL fwd+bwd, top-K={K} fp16/int32 teacher, {rows} tokens x {V} vocab bf16 logits, T=1, "
+            "bf16 gradient", "fkl_topk_reg_kernel<bf16,256,16,split> (4 column parts per row)", c, grad)
+
+
+def _wl_c4(D, S, dev, rows):
+    import torch
+    rows = rows or 4 * 8192
+    V, Vt, K = 128256, 152064, 200
+    c = S.config4(dev, rows=rows, V=V, Vt=Vt, K=K)
+    grad = torch.empty_like(c["logits"])
+    scale = 1.0 / rows
+    state = {}
+
+    def merge():
+        state["m"] = D.merge_remap_topk(c["t_vals"], c["t_idxs"], c["weights"], c["id_map"], student_vocab=V)
+
+    def main():
+        ids, lm, cnt = state["m"]
+        return D.div_topk("fkl", c["logits"], lm, ids, t_cnt=cnt, T=1.0, grad_scale=scale, grad_out=grad)[0]
+
+    def step():
+        merge()
+        return D.reduce_sum(main(), scale)
+
+    merge()
+    return (step, main, rows * (V * 2 + V * 2 + 3 * K * 6) + Vt * 4, rows,
+            f"C4 3-teacher weighted merge + vocab remap ({Vt}->{V}) + forward-KL fwd+bwd, {rows} tokens, bf16",
+            "fkl_topk_reg_kernel<bf16,256,16,split> fed by merge_kernel", c, grad)
+
+
+def _wl_dense(kind_name):
+    def build(D, S, dev, rows):
+        import torch
+        if kind_name == "c1":
+            c = S.config1(dev) if not rows else S.config1(dev, B=1, S=rows)
+            eb, desc = 4, "C1 dense forward-KL fwd+bwd, fp32, T=1, last 10% of positions masked"
+        else:
+            c = S.config2(dev) if not rows else S.config2(dev, B=1, S=rows)
+            eb, desc = 2, "C2 dense JSD fwd+bwd, bf16, T=2, ragged valid lengths"
+        R, V = c["logits"].shape
+        nv = int(c["valid"].sum())
+        grad = torch.empty_like(c["logits"])
+        scale = 1.0 / nv
+
+        def main():
+            return D.div_dense(c["kind"], c["logits"], c["t_logits"], row_map=c["row_map"], T=c["T"], grad_scale=scale,
+                               grad_out=grad)[0]
+
+        return (lambda: D.reduce_sum(main(), scale), main, nv * V * 2 * eb + R * V * eb, R,
+                f"{desc}; {R} tokens ({nv} valid) x {V} vocab", f"dense_reg_kernel ({c['kind']})", c, grad)
+    return build
+
+
+def _wl_c5(D, S, dev, rows):
+    import torch
+    rows = rows or 2 * 4096
+    Vs, Vt = 32000, 152064
+    c = S.config5(dev, rows=rows, Vs=Vs, Vt=Vt)
+    grad = torch.empty_like(c["logits"])
+    scale = 1.0 / rows
+
+    def main():
+        return D.vocab_utils.rkl_marginalised(c["logits"], c["t_probs"], c["t2s"], T=c["T"], grad_scale=scale,
+                                              grad_out=grad)[0]
+
+    return (lambda: D.reduce_sum(main(), scale), main, rows * (Vt * 4 + Vs * 2 + Vs * 2) + Vt * 4, rows,
+            f"C5 byte-trie marginalisation ({Vt}->{Vs}) + reverse-KL fwd+bwd, {rows} tokens, fp32 teacher softmax, "
+            "bf16 student, T=1.5", "rkl_marginalised_kernel<bf16>", c, grad)
+
+
+WORKLOADS = {"c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c5": _wl_c5}
+
+
+# ---------------------------------------------------------------------------------------------
+def cpu_baseline(workload: str, rows: int, reps: int):
+    """The reference's op sequence (cast -> /T -> log_softmax -> gather -> kl_div -> mean -> backward) in
+    PyTorch eager on the host cores, on a bounded row sample of the same workload (rows are independent, so
+    tokens/s carries over to the full row count)."""
+    import numpy as np
     import torch
     from llm_distillery_amd import synthetic as S
     from oracle import oracle as O
 
-    c = S.config3("cpu", rows=rows, seed=3)
-    O.mean_loss_and_grad("fkl", c["logits"][:64], 1.0, t_vals=c["t_val"][:64], t_idx=c["t_idx"][:64].long())
+    if workload == "c3":
+        c = S.config3("cpu", rows=rows, seed=3)
+        fn = lambda: O.mean_loss_and_grad("fkl", c["logits"], 1.0, t_vals=c["t_val"], t_idx=c["t_idx"].long())
+        what = f"{rows} of 32768 rows at V=128256, K=200"
+    elif workload == "c4":
+        c = S.config4("cpu", rows=rows)
+        def fn():
+            ids, lq, cnt = O.merge_remap_padded([v.numpy() for v in c["t_vals"]], [i.numpy() for i in c["t_idxs"]],
+                                                c["weights"], c["id_map"].numpy())
+            z = c["logits"].float().requires_grad_(True)
+            O.fwd_kl_sparse_rows(z, ids, lq, cnt).mean().backward()
+        what = f"{rows} of 32768 rows at V=128256, 3 teachers x K=200 (dict/loop merge)"
+    elif workload in ("c1", "c2"):
+        c = S.config1("cpu", B=1, S=rows) if workload == "c1" else S.config2("cpu", B=1, S=rows)
+        fn = lambda: O.mean_loss_and_grad(c["kind"], c["logits"], c["T"], t_logits=c["t_logits"], valid=c["valid"])
+        what = f"{rows} rows at V=32000, dense teacher"
+    else:
+        c = S.config5("cpu", rows=rows)
+        def fn():
+            marg = torch.tensor(O.marginalise_map(c["t_probs"].numpy(), c["t2s_host"], 32000, dtype=np.float32))
+            with np.errstate(divide="ignore"):
+                O.mean_loss_and_grad("rkl", c["logits"], c["T"], t_logits=torch.log(marg))
+        what = f"{rows} of 8192 rows, Vt=152064 -> Vs=32000 (numpy scatter + torch eager)"
+    fn()
     times = []
     for _ in range(reps):
         t0 = time.perf_counter()
-        O.mean_loss_and_grad("fkl", c["logits"], 1.0, t_vals=c["t_val"], t_idx=c["t_idx"].long())
+        fn()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
     return {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"{rows} of 32768 rows at V={V}, K={K}, fp32 eager oracle fwd+bwd, median of {reps} "
-                      f"({med:.2f} s each; os.cpu_count()={os.cpu_count()})"}
+            "sample": f"{what}, fp32 eager oracle fwd+bwd, median of {reps} ({med:.2f} s each; "
+                      f"os.cpu_count()={os.cpu_count()})"}
 
 
-def measured_traffic():
+def measured_traffic(workload: str):
     """HBM bytes per launch from the committed rocprofv3 counter summary, if present."""
-    path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
-        with open(path) as f:
-            return json.load(f).get("fkl_topk_c3_bytes_per_launch")
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(f"{workload}_bytes_per_launch")
     except (OSError, ValueError):
         return None
 
@@ -60,11 +171,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--rows", type=int, default=8 * 4096)
-    ap.add_argument("--cpu-rows", type=int, default=4096, help="row sample for the CPU baseline (0 = skip)")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
+    ap.add_argument("--rows", type=int, default=0, help="override the workload's token count")
+    ap.add_argument("--cpu-rows", type=int, default=-1, help="row sample for the CPU baseline (0 = skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also launch the library's plain copy kernel over the logits buffer (known traffic: "
-                         "rows*V*2 bytes each way), the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
+                    help="also launch the library's plain copy kernel over the logits buffer (known traffic: its "
+                         "byte size each way), the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is row-parallel and every configuration fits one "
@@ -76,53 +188,46 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    rows = args.rows
-    c = S.config3(dev, rows=rows, seed=3)
-    logits, t_val, t_idx = c["logits"], c["t_val"], c["t_idx"]
-    grad = torch.empty_like(logits)
-    scale = 1.0 / rows
-
-    def step():
-        row_loss, _ = D.div_topk("fkl", logits, t_val, t_idx, T=1.0, grad_scale=scale, grad_out=grad)
-        return D.reduce_sum(row_loss, scale)
+    step, main_launch, algo_bytes, tokens, desc, kernel, c, grad = WORKLOADS[args.workload](D, S, dev, args.rows)
 
     for _ in range(args.warmup):
         loss = step()
     torch.cuda.synchronize()
     if args.calibrate_copy:
         for _ in range(3):
-            D.copy16(logits, grad)
+            D.copy16(c["logits"], grad)
         torch.cuda.synchronize()
 
-    # per-launch duration of the dominant kernel: events on the stream the kernel runs on
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    # whole step, wall clock between synchronisations
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # dominant kernel alone: events on the stream it is launched on (torch's current stream)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     for a, b in ev:
         a.record()
-        row_loss, _ = D.div_topk("fkl", logits, t_val, t_idx, T=1.0, grad_scale=scale, grad_out=grad)
+        main_launch()
         b.record()
-        loss = D.reduce_sum(row_loss, scale)
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     kern_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
-    ms_per_step = wall * 1e3 / args.steps
-    algo_bytes = rows * BYTES_PER_TOKEN
     achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
 
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c1": 512, "c2": 4096, "c5": 512}[args.workload]
     out = {
         "metric": "tokens/sec fused KL fwd+bwd @ vocab 128256 bf16; % of HBM peak GB/s",
-        "value": rows / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"C3 forward-KL fwd+bwd, top-K={K} fp16/int32 teacher, {rows} tokens x {V} vocab "
-                               "bf16 logits, T=1, bf16 gradient", "rows": rows, "vocab": V, "topk": K},
+        "vs_baseline": None, "dtype": "fp32" if args.workload == "c1" else "bf16", "data": "synthetic",
+        "config": {"workload": desc, "rows": tokens},
         "loss": loss.item(),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(),
-                     "kernel": "fkl_topk_reg_kernel<bf16,256,16,split> (4 column parts per row)", "kernel_ms": kern_ms,
-                     "algorithmic_bytes": algo_bytes},
-        "cpu_baseline": cpu_baseline(args.cpu_rows) if args.cpu_rows > 0 else None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload),
+                     "kernel": kernel, "kernel_ms": kern_ms, "algorithmic_bytes": algo_bytes},
+        "cpu_baseline": cpu_baseline(args.workload, cpu_rows, 7 if args.workload == "c3" else 3) if cpu_rows > 0 else None,
     }
     print(json.dumps(out))
 

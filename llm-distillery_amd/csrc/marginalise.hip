@@ -35,28 +35,44 @@ __device__ __forceinline__ void accumulate_marginal(const MargParams& p, const c
   for (int j = tid; j < s_n; j += MARG_NT) acc[j] = 0.f;
   __syncthreads();
   if (VEC) {       // fp32 probabilities, 16-byte aligned: four columns per load
+    // Double-buffered batches of U 16-byte loads of the probabilities and of the id map per thread:
+    // the next batch is in flight while the current one is scattered into LDS.
+    constexpr int U = 4;
     const int64_t n4 = p.Vt / 4;
-    for (int64_t c0 = 0; c0 < n4; c0 += 2 * MARG_NT) {
-      u32x4 pv[2], iv[2];
+    const char* mrow = reinterpret_cast<const char*>(p.t2s);
+    u32x4 pa[U], ia[U], pb[U], ib[U];
+    auto fetch = [&](int64_t c0, u32x4* pv, u32x4* iv) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < U; ++u) {
         const int64_t c = c0 + (int64_t)u * MARG_NT + tid;
         if (c < n4) {
           pv[u] = load16_stream(prow + c * 16);
-          iv[u] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.t2s) + c * 16);
+          iv[u] = *reinterpret_cast<const u32x4*>(mrow + c * 16);
         } else {
           pv[u] = u32x4{0u, 0u, 0u, 0u};
           iv[u] = u32x4{~0u, ~0u, ~0u, ~0u};
         }
       }
+    };
+    auto scatter = [&](u32x4* pv, u32x4* iv) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < U; ++u) {
+        forget(pv[u]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int s = (int)iv[u][e] - s_lo;
           if (s >= 0 && s < s_n)
             __hip_atomic_fetch_add(&acc[s], __uint_as_float(pv[u][e]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
+      }
+    };
+    constexpr int64_t STEP = (int64_t)U * MARG_NT;
+    fetch(0, pa, ia);
+    for (int64_t c0 = 0; c0 < n4; c0 += 2 * STEP) {
+      fetch(c0 + STEP, pb, ib);            // beyond the row: nothing is loaded, sentinel ids
+      scatter(pa, ia);
+      fetch(c0 + 2 * STEP, pa, ia);
+      scatter(pb, ib);
     }
   } else {
     for (int64_t t = tid; t < p.Vt; t += MARG_NT) {
@@ -166,6 +182,29 @@ static bool ok16(const void* ptr, int64_t stride, int eb) {
   return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (stride * eb) % 16 == 0;
 }
 
+// More than 64 KiB of dynamic LDS has to be requested per kernel; once per process and device is
+// enough (the call is slow, so it must not sit on the launch path).
+template <class K>
+static void allow_large_lds_for(K kernel) {
+  hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                      MARG_MAX_VS * 4);
+}
+static void allow_large_lds() {
+  static thread_local int done_for = -1;
+  int dev = 0;
+  hipGetDevice(&dev);
+  if (done_for == dev) return;
+  allow_large_lds_for(&marginalise_map_kernel<true>);
+  allow_large_lds_for(&marginalise_map_kernel<false>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF32, 8, true>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF32, 8, false>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagBF16, 8, true>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagBF16, 8, false>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF16, 8, true>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF16, 8, false>);
+  done_for = dev;
+}
+
 }  // namespace dl
 
 extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
@@ -183,11 +222,7 @@ extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stri
   const size_t lds = (size_t)(Vs < MARG_MAX_VS ? Vs : MARG_MAX_VS) * 4;
   const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(probs, p_stride, 4) && ok16(t2s, 0, 4);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  // more than 64 KiB of dynamic LDS has to be requested per kernel
-  hipFuncSetAttribute(reinterpret_cast<const void*>(&marginalise_map_kernel<true>),
-                      hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);
-  hipFuncSetAttribute(reinterpret_cast<const void*>(&marginalise_map_kernel<false>),
-                      hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);
+  allow_large_lds();
   if (vec) hipLaunchKernelGGL((marginalise_map_kernel<true>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
   else hipLaunchKernelGGL((marginalise_map_kernel<false>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
@@ -236,12 +271,9 @@ extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t
   const size_t lds = (size_t)Vs * 4;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)n_rows), block(MARG_NT);
+  allow_large_lds();
 #define DL_LAUNCH_RKLM(TAG)                                                                                  \
   do {                                                                                                       \
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&rkl_marginalised_kernel<TAG, 8, true>),               \
-                        hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);                        \
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&rkl_marginalised_kernel<TAG, 8, false>),              \
-                        hipFuncAttributeMaxDynamicSharedMemorySize, MARG_MAX_VS * 4);                        \
     if (vec) hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, 8, true>), grid, block, lds, st, p);           \
     else hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, 8, false>), grid, block, lds, st, p);              \
   } while (0)
