@@ -57,7 +57,7 @@ def _wl_c4(D, S, dev, rows):
 
     def main():
         ids, lm, cnt = state["m"]
-        return D.div_topk("fkl", c["logits"], lm, ids, t_cnt=cnt, T=1.0, grad_scale=scale, grad_out=grad)[0]
+        return D.div_topk("fkl", c["logits"], lm, ids, t_cnt=cnt, T=1.0, grad_scale=scale, grad_out=grad, unique_ids=True)[0]
 
     def step():
         merge()

@@ -39,6 +39,7 @@ typedef enum {
 
 #define DL_MAX_TOPK 2048      /* entries per row a sparse teacher may hold        */
 #define DL_MAX_TEACHERS 8     /* teachers merged in one launch                    */
+#define DL_TOPK_UNIQUE_IDS 1   /* dl_div_topk flag: no id occurs twice in a row    */
 
 /* Library ABI revision; bumped when a signature changes. */
 int dl_abi_version(void);
@@ -78,6 +79,9 @@ int dl_set_option(const char* name, int value);
  *            of the register file are cut into column parts that meet through it; without a
  *            workspace (NULL or too small) such rows take a slower one-workgroup-per-row kernel.
  *            Two launches that may overlap in time must not share a workspace.
+ * flags      DL_TOPK_UNIQUE_IDS promises that no id occurs twice within a row (true for the output of
+ *            torch.topk and of dl_merge_remap_topk); the kernel then skips its duplicate scan.  With
+ *            the flag set and duplicates present, the gradient at a duplicated id is wrong.
  * K <= DL_MAX_TOPK.
  */
 int dl_div_topk(int kind,
@@ -87,7 +91,7 @@ int dl_div_topk(int kind,
                 int64_t n_teacher_rows, const int32_t* t_cnt,
                 float inv_T_student, float inv_T_teacher, float grad_scale,
                 float* row_loss, void* grad, int64_t grad_stride,
-                void* workspace, int64_t workspace_bytes, void* stream);
+                void* workspace, int64_t workspace_bytes, int flags, void* stream);
 
 /* Scratch size dl_div_topk can make use of for this problem (0 = none needed).  Host-only. */
 int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V);

@@ -18,13 +18,14 @@ DL_I32, DL_I64 = 0, 1
 DL_FKL, DL_RKL, DL_JSD = 0, 1, 2
 DL_MAX_TOPK = 2048
 DL_MAX_TEACHERS = 8
+DL_TOPK_UNIQUE_IDS = 1
 
 _P = c_void_p
 _SIGNATURES = {
     "dl_abi_version": (c_int, []),
     "dl_status_string": (c_char_p, [c_int]),
     "dl_div_topk": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, _P, c_int, c_int, c_int64, _P,
-                            c_float, c_float, c_float, _P, _P, c_int64, _P, c_int64, _P]),
+                            c_float, c_float, c_float, _P, _P, c_int64, _P, c_int64, c_int, _P]),
     "dl_div_topk_workspace_bytes": (c_int64, [c_int, c_int, c_int64, c_int64]),
     "dl_div_dense": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int64, c_int64,
                              c_float, c_float, c_float, _P, _P, c_int64, _P]),

@@ -48,26 +48,32 @@ __device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, int n
 }
 
 // Exclusive prefix sum over n_pow2 flags (each thread owns a contiguous run); returns the total.
+// Wave-level scans with lane shuffles, wave totals combined through LDS.
 __device__ __forceinline__ int block_scan_flags(const unsigned char* flag, int* pos, int n_pow2, int* scratch) {
-  const int per = n_pow2 / MERGE_NT > 0 ? n_pow2 / MERGE_NT : 1;
+  const int per = n_pow2 / MERGE_NT;              // n_pow2 >= MERGE_NT
   const int begin = threadIdx.x * per;
   int local = 0;
-  if (begin < n_pow2)
-    for (int i = 0; i < per; ++i) local += flag[begin + i];
-  scratch[threadIdx.x] = local;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int i = 0; i < MERGE_NT; ++i) { const int v = scratch[i]; scratch[i] = run; run += v; }
-    scratch[MERGE_NT] = run;
+  for (int i = 0; i < per; ++i) local += flag[begin + i];
+  int incl = local;
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const int up = __shfl_up(incl, o, WAVE);
+    if (lane >= o) incl += up;
   }
+  if (lane == WAVE - 1) scratch[w] = incl;
   __syncthreads();
-  if (begin < n_pow2) {
-    int run = scratch[threadIdx.x];
-    for (int i = 0; i < per; ++i) { pos[begin + i] = run; run += flag[begin + i]; }
+  int base = 0, total = 0;
+#pragma unroll
+  for (int i = 0; i < MERGE_NT / WAVE; ++i) {
+    const int v = scratch[i];
+    if (i < w) base += v;
+    total += v;
   }
+  int run = base + incl - local;
+  for (int i = 0; i < per; ++i) { pos[begin + i] = run; run += flag[begin + i]; }
   __syncthreads();
-  return scratch[MERGE_NT];
+  return total;
 }
 
 __global__ __launch_bounds__(MERGE_NT) void merge_kernel(const MergeParams p, int E, int Ep) {

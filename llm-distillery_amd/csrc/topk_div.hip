@@ -32,7 +32,7 @@ struct TopkParams {
   int64_t n_trows; const int32_t* t_cnt;
   float inv_T_s, inv_T_t, grad_scale;
   float* row_loss; void* grad; int64_t grad_stride;
-  void* workspace; int parts; int spin_limit;
+  void* workspace; int parts; int spin_limit; int flags;
 };
 
 constexpr int MAX_PARTS = 8;
@@ -89,6 +89,71 @@ struct TopkLds {
   }
   __host__ __device__ static size_t bytes(int K) { return 512 + (size_t)((K + 15) & ~15) * 16; }
 };
+
+// Teacher entries of one row held in registers between issue and use: J entries per thread,
+// entry k = tid + j * NT.  Issuing their (tiny) loads before the row's 16 big ones, and the
+// dependent gathers right behind those, keeps three global-memory latencies off the critical path.
+template <int J>
+struct TeacherEntries {
+  int id[J];
+  float tv[J];
+  float z[J];
+};
+
+template <int NT, int J>
+__device__ __forceinline__ void teacher_issue(const TopkParams& p, int64_t trow, TeacherEntries<J>& t) {
+  const int K = p.K;
+  const int cnt = p.t_cnt ? min(p.t_cnt[trow], K) : K;
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    const int k = threadIdx.x + j * NT;
+    int64_t id = -1;
+    float v = -INFINITY;
+    if (k < cnt) {
+      const int64_t at = trow * (int64_t)K + k;
+      id = load_index(p.t_idx, p.t_idx_itype, at);
+      v = load_as_float(p.t_val, p.t_val_dtype, at);       // independent of the id: both loads fly together
+    }
+    const bool ok = id >= 0 && id < p.V;
+    t.id[j] = ok ? (int)id : -1;
+    t.tv[j] = ok ? v * p.inv_T_t : -INFINITY;
+  }
+}
+
+template <class Tag, int J>
+__device__ __forceinline__ void teacher_gather(const char* row, int lo, int hi, TeacherEntries<J>& t) {
+#pragma unroll
+  for (int j = 0; j < J; ++j)
+    t.z[j] = (t.id[j] >= lo && t.id[j] < hi) ? load_as_float(row, Tag::id, t.id[j]) : 0.f;
+}
+
+// Registers -> LDS, then the teacher's log-sum-exp; same result layout as stage_teacher.
+template <int NT, int J>
+__device__ __forceinline__ float teacher_finish(const TopkLds& s, const TeacherEntries<J>& t) {
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    const int k = threadIdx.x + j * NT;
+    if (k < s.Kp) { s.idx[k] = t.id[j]; s.z[k] = t.z[j]; }
+    tmax = fmaxf(tmax, t.tv[j]);
+  }
+  tmax = block_max<NT>(tmax, s.red);     // barrier inside: LDS entries visible afterwards
+  if (tmax == -INFINITY) return tmax;
+  float part = 0.f;
+#pragma unroll
+  for (int j = 0; j < J; ++j) part += expf(t.tv[j] - tmax);
+  const float tlse = tmax + logf(block_sum<NT>(part, s.red));
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    const int k = threadIdx.x + j * NT;
+    if (k < s.Kp) {
+      const float lt = t.tv[j] - tlse;
+      s.t[k] = lt;
+      s.q[k] = expf(lt);
+    }
+  }
+  return tlse;
+}
 
 // Stage the teacher row: ids, scaled log-probs, and the student logits at the ids that fall into
 // the column range [lo, hi) this workgroup owns.  Returns the log-sum-exp of the scaled teacher
@@ -159,11 +224,11 @@ __device__ __forceinline__ float mass_on_id(const TopkLds& s, int k, int id) {
 // inside [lo, hi).  b is the row's log2-sum-exp2, a = inv_T * log2(e), c = inv_T * scale.
 template <class Tag, int NT>
 __device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int lo, int hi,
-                                               float a, float b, float c) {
+                                               float a, float b, float c, bool ids_unique) {
   for (int k = threadIdx.x; k < s.Kp; k += NT) {
     const int id = s.idx[k];
     if (id < lo || id >= hi) continue;
-    const float q = mass_on_id(s, k, id);
+    const float q = ids_unique ? s.q[k] : mass_on_id(s, k, id);
     store_from_float(grow, Tag::id, id, (fast_exp2(fmaf(s.z[k], a, -b)) - q) * c);
   }
 }
@@ -207,7 +272,9 @@ __device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, f
 // they land on the same XCD back to back (partners start together and meet through one L2).
 // Within a group of 8*P ids, id t serves row 8*group + t % 8, part t / 8.
 // ---------------------------------------------------------------------------------------
-template <class Tag, int NT, int NCH, bool SPLIT>
+// J > 0: the K <= J * NT teacher entries travel in registers (loads issued ahead of the row's);
+// J == 0: any K, staged by a plain loop.
+template <class Tag, int NT, int NCH, bool SPLIT, int J>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))     // <= 128 VGPRs: 16 waves per CU
 void fkl_topk_reg_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -233,6 +300,8 @@ void fkl_topk_reg_kernel(const TopkParams p) {
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
   const char* rpart = row + c0 * 16;
 
+  TeacherEntries<(J > 0 ? J : 1)> te;
+  if constexpr (J > 0) teacher_issue<NT, J>(p, trow, te);
   u32x4 reg[NCH];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
@@ -241,7 +310,13 @@ void fkl_topk_reg_kernel(const TopkParams p) {
   }
 
   // teacher side while the row is in flight
-  const float tlse = stage_teacher<Tag, NT>(p, s, trow, row, lo, hi);
+  float tlse;
+  if constexpr (J > 0) {
+    teacher_gather<Tag, J>(row, lo, hi, te);
+    tlse = teacher_finish<NT, J>(s, te);
+  } else {
+    tlse = stage_teacher<Tag, NT>(p, s, trow, row, lo, hi);
+  }
   if (tlse == -INFINITY) {            // no usable teacher entry: the row contributes nothing
     if (gpart) zero_row<Tag, NT>(gpart, nch);
     if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
@@ -322,7 +397,7 @@ void fkl_topk_reg_kernel(const TopkParams p) {
       }
     }
     __syncthreads();      // dense stores are ordered before the sparse corrections
-    fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c);
+    fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
   }
 }
 
@@ -374,7 +449,7 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
         store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * c);
     }
     __syncthreads();
-    fkl_sparse_fix<Tag, NT>(s, grow, 0, (int)V, a, b, c);
+    fkl_sparse_fix<Tag, NT>(s, grow, 0, (int)V, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
   }
 }
 
@@ -446,10 +521,18 @@ __global__ __launch_bounds__(256) void clear_workspace_kernel(u32x4* ws, int64_t
 // ---------------------------------------------------------------------------------------
 // host dispatch
 // ---------------------------------------------------------------------------------------
+template <class Tag, int NT, int NCH, bool SPLIT>
+static void launch_reg_j(const TopkParams& p, unsigned grid, hipStream_t st) {
+  const int Kp = (p.K + 15) & ~15;
+  const size_t lds = TopkLds::bytes(p.K);
+  if (Kp <= NT) hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 1>), dim3(grid), dim3(NT), lds, st, p);
+  else if (Kp <= 3 * NT) hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 3>), dim3(grid), dim3(NT), lds, st, p);
+  else hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 0>), dim3(grid), dim3(NT), lds, st, p);
+}
+
 template <class Tag, int NT, int NCH>
 static hipError_t launch_reg(const TopkParams& p, hipStream_t st) {
-  hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, false>), dim3((unsigned)p.n_rows), dim3(NT),
-                     TopkLds::bytes(p.K), st, p);
+  launch_reg_j<Tag, NT, NCH, false>(p, (unsigned)p.n_rows, st);
   return hipGetLastError();
 }
 
@@ -459,8 +542,7 @@ static hipError_t launch_split(TopkParams p, int parts, hipStream_t st) {
   const int64_t n16 = p.n_rows * parts;          // one 16-byte PartStats per (row, part)
   hipLaunchKernelGGL(clear_workspace_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
                      reinterpret_cast<u32x4*>(p.workspace), n16);
-  hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, true>), dim3((unsigned)((p.n_rows + 7) / 8 * 8 * parts)), dim3(NT),
-                     TopkLds::bytes(p.K), st, p);
+  launch_reg_j<Tag, NT, NCH, true>(p, (unsigned)((p.n_rows + 7) / 8 * 8 * parts), st);
   return hipGetLastError();
 }
 
@@ -542,7 +624,8 @@ extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64
                            int64_t V, const int32_t* row_map, const void* t_val, int t_val_dtype,
                            const void* t_idx, int t_idx_itype, int K, int64_t n_teacher_rows,
                            const int32_t* t_cnt, float inv_T_student, float inv_T_teacher, float grad_scale, float* row_loss,
-                           void* grad, int64_t grad_stride, void* workspace, int64_t workspace_bytes, void* stream) {
+                           void* grad, int64_t grad_stride, void* workspace, int64_t workspace_bytes, int flags,
+                           void* stream) {
   using namespace dl;
   if (!logits || !t_val || !t_idx) return DL_ERR_NULL;
   if (kind != DL_FKL && kind != DL_RKL) return DL_ERR_DTYPE;
@@ -559,7 +642,7 @@ extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64
                        (!grad || (reinterpret_cast<uintptr_t>(grad) % 16 == 0 && (grad_stride * eb) % 16 == 0));
   TopkParams p{logits, row_stride, n_rows, V, row_map, t_val, t_val_dtype, t_idx, t_idx_itype, K, n_teacher_rows,
                t_cnt, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride,
-               (reinterpret_cast<uintptr_t>(workspace) % 16 == 0) ? workspace : nullptr, 1, spin_limit()};
+               (reinterpret_cast<uintptr_t>(workspace) % 16 == 0) ? workspace : nullptr, 1, spin_limit(), flags};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   hipError_t e;
   if (kind == DL_FKL) {

@@ -105,3 +105,47 @@ def distill_loss(model_logits: Tensor, content_rows: Tensor, teacher_logprobs: T
     tT = temperature if teacher_temperature is None else teacher_temperature
     t = F.log_softmax(teacher_logprobs[:n].float() / tT, dim=-1)
     return _assemble(s_sup, t, indices[:n], convo_CE_tokens[:n], alpha, avoid_indices)
+
+
+def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float = 1.0,
+                       crop_to_size: int | None = None, teacher_temperature: float | None = None) -> list[dict[str, Tensor]]:
+    """The per-conversation composite losses of a whole batch with ONE pass over the logits.
+
+    Replaces the Python loop of classes/student/model.py:415-436 (one `calculate_divergence` call,
+    i.e. one full-vocabulary log-softmax + gather and its autograd replay, per conversation): the
+    V-wide work of all conversations runs as a single phase-1 launch over `model_logits`
+    [B, S, V_model] and, in backward, a single phase-2 launch; only the K-wide epilogue stays per
+    conversation, because its weights (max of the per-token KL, mean of the valid cross entropies)
+    are per-conversation quantities in the reference.
+
+    `convos[i]` = (content_rows int [N_i] positions inside sequence i, teacher_logprobs [N_i, K] as
+    stored, indices [N_i, K], convo_CE_tokens [N_i - 1], avoid_indices).  All conversations share K.
+    Returns one nine-key dict per conversation, in order; feed them to `Losses.add_losses` as the
+    reference does and call `Losses.backward` once.
+    """
+    if model_logits.dim() != 3:
+        raise RuntimeError("model_logits must be [batch, seq, vocab]")
+    B, S, _ = model_logits.shape
+    if len(convos) != B:
+        raise ValueError(f"{len(convos)} conversations for a batch of {B} sequences")
+    x = model_logits if crop_to_size is None else model_logits[:, :, :crop_to_size]
+    dev = x.device
+    counts = []
+    row_map = torch.full((B * S,), -1, dtype=torch.int32, device=dev)
+    idx_all, base = [], 0
+    for b, (rows, t_lp, idx, _, _) in enumerate(convos):
+        n = min(rows.numel(), t_lp.size(0), idx.size(0))
+        counts.append(n)
+        row_map[b * S + rows[:n].long()] = torch.arange(base, base + n, dtype=torch.int32, device=dev)
+        idx_all.append(idx[:n])
+        base += n
+    idx_cat = torch.cat(idx_all, dim=0)
+    lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature)
+    tT = temperature if teacher_temperature is None else teacher_temperature
+    out, base = [], 0
+    for (rows, t_lp, idx, labels, avoid), n in zip(convos, counts):
+        s_sup = zk[base:base + n] - lse[base:base + n].unsqueeze(-1)
+        t = F.log_softmax(t_lp[:n].float() / tT, dim=-1)
+        out.append(_assemble(s_sup, t, idx[:n], labels[:n], alpha, avoid))
+        base += n
+    return out

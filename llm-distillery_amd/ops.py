@@ -58,13 +58,14 @@ def _opt_i32(t, n, name, dev):
 def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor, *,
              row_map: torch.Tensor | None = None, t_cnt: torch.Tensor | None = None,
              T: float = 1.0, teacher_T: float | None = None, grad_scale: float = 1.0,
-             want_grad: bool = True, grad_out: torch.Tensor | None = None):
+             want_grad: bool = True, grad_out: torch.Tensor | None = None, unique_ids: bool = False):
     """Per-token forward ("fkl") or reverse ("rkl") KL against a top-K teacher and,
     in the same launch, d(sum of row losses)/d(logits) * grad_scale.
 
     logits [..., V] bf16/fp16/fp32 (native model dtype, rows evenly strided);
     t_val/t_idx [N, K] stored teacher log-probs and ids; row_map int32 [rows]
-    gives the teacher row of each logits row (negative = masked row).
+    gives the teacher row of each logits row (negative = masked row).  `unique_ids=True` promises
+    that no id repeats within a row (skips the duplicate scan).
     Returns (row_loss fp32 [rows], grad like logits or None).
     """
     if kind not in ("fkl", "rkl"):
@@ -98,7 +99,8 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
                              t_val.data_ptr(), _DT[t_val.dtype], t_idx.data_ptr(), _IT[t_idx.dtype], K, N,
                              cnt_ptr, 1.0 / T, 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
                              row_loss.data_ptr(), g_ptr, g_stride,
-                             ws.data_ptr() if ws is not None else 0, ws_bytes, _stream_ptr(dev))
+                             ws.data_ptr() if ws is not None else 0, ws_bytes,
+                             _lib.DL_TOPK_UNIQUE_IDS if unique_ids else 0, _stream_ptr(dev))
     _lib.check(st, "dl_div_topk")
     if grad is not None and logits.dim() != 2 and grad_out is None:
         grad = grad.view(logits.shape)

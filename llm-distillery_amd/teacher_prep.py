@@ -96,4 +96,4 @@ def fkl_multi_teacher(logits: torch.Tensor, vals: Sequence[torch.Tensor], idxs: 
     V = logits.shape[-1]
     ids, logmass, cnt = merge_remap_topk(vals, idxs, weights, id_map, student_vocab=V)
     return ops.div_topk("fkl", logits, logmass, ids, row_map=row_map, t_cnt=cnt, T=T, teacher_T=teacher_T,
-                        grad_scale=grad_scale, want_grad=want_grad, grad_out=grad_out)
+                        grad_scale=grad_scale, want_grad=want_grad, grad_out=grad_out, unique_ids=True)

@@ -150,3 +150,47 @@ def test_rowstats_raw_outputs_and_losses_accumulator_on_gpu(D):
     L.backward(divisor=2)
     assert all(s.grad is not None and torch.isfinite(s.grad).all() for s in leafs)
     assert total > 0 and L.num_steps_accumulated == 2
+
+
+def test_batched_caller_equals_the_per_conversation_loop(D):
+    """One pass over [B, S, V] for all conversations of a batch gives, conversation by conversation, the
+    dicts the reference's loop gives (restated on the CPU), and after Losses.backward the same gradient."""
+    g = torch.Generator().manual_seed(11)
+    B, S, Vm, crop, K, T, accum = 3, 60, 4160, 4096, 24, 1.3, 2
+    model_logits = (torch.randn(B, S, Vm, generator=g) * 2).to(torch.bfloat16)
+    specs = [[(4, 20), (30, 41)], [(0, 55)], [(10, 16), (20, 30), (44, 59)]]
+    lens = [41, 55, 59]
+    convos_cpu, convos_gpu = [], []
+    for b in range(B):
+        rows = torch.as_tensor(O.content_indices(specs[b]))
+        lab_pos, avoid = O.ce_indices(specs[b], 2048, lens[b])
+        N = rows.numel()
+        tfull = torch.log_softmax(model_logits[b, rows, :crop].float() + torch.randn(N, crop, generator=g), -1)
+        tv, ti = torch.topk(tfull, K)
+        tv = tv.to(torch.float16)
+        tokens = torch.randint(0, crop, (S + 1,), generator=g)
+        tokens[torch.as_tensor(lab_pos)] = ti[:len(lab_pos), 0]
+        labels = tokens[torch.as_tensor(lab_pos)]
+        convos_cpu.append((rows, tv, ti, labels, torch.as_tensor(avoid)))
+        convos_gpu.append((rows.to(DEV), tv.to(DEV), ti.to(torch.int32).to(DEV), labels.to(DEV), torch.as_tensor(avoid).to(DEV)))
+    # reference loop on the CPU in float64
+    z = O.scaled_student_logits(model_logits, crop, T, torch.float64).requires_grad_(True)
+    ref_dicts, total = [], 0
+    for b, (rows, tv, ti, labels, avoid) in enumerate(convos_cpu):
+        d = O.calculate_divergence(torch.index_select(z[b], 0, rows), tv.double() / T, ti, labels, 2.0, avoid)
+        ref_dicts.append(d)
+        total = total + d["train_loss"]
+    (total / accum).backward()
+    x = model_logits.to(DEV).requires_grad_(True)
+    L = D.Losses(None)
+    dicts = D.distill_loss_batch(x, convos_gpu, 2.0, temperature=T, crop_to_size=crop)
+    for d, r in zip(dicts, ref_dicts):
+        for k in D.LOSS_KEYS:
+            np.testing.assert_allclose(d[k].item(), r[k].item(), rtol=2e-5, atol=2e-6, err_msg=k)
+        L.add_losses(d)
+    L.backward(divisor=accum)
+    gref = torch.zeros(B, S, Vm, dtype=torch.float64)
+    gref[:, :, :crop] = z.grad / T
+    err = (x.grad.cpu().double() - gref).abs()
+    assert (err <= O.storage_tolerance(gref, torch.bfloat16, 2e-3)).all()
+    assert torch.count_nonzero(x.grad[0, 41:]) == 0            # rows outside every content range
