@@ -5,7 +5,8 @@
 One step = one pass of the fused loss + gradient over one batch of synthetic input followed by the
 deterministic mean reduction.  The default workload is the one the headline metric is quoted on
 (C3: 8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200 fp16/int32 teacher, T=1);
-`--workload c1|c2|c4|c5` measures the other configurations with the same harness.  Inputs are
+`--workload c1|c2|c4|c5|producer` measures the other configurations and the teacher producer with the
+same harness.  Inputs are
 resident in HBM before the timed region.  Prints ONE JSON line.
 """
 from __future__ import annotations
@@ -109,7 +110,26 @@ def _wl_c5(D, S, dev, rows):
             "bf16 student, T=1.5", "rkl_marginalised_kernel<bf16>", c, grad)
 
 
-WORKLOADS = {"c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c5": _wl_c5}
+def _wl_producer(D, S, dev, rows):
+    import torch
+    rows = rows or 8 * 4096
+    V, K = 128256, 200
+    c = S.config3(dev, rows=rows, seed=3)
+    out = {}
+
+    def main():
+        out["v"], out["i"] = D.teacher_topk(c["logits"], K)
+        return out["v"]
+
+    def step():
+        return main()[0, 0].float()
+
+    return (step, main, rows * (V * 2 + K * 6), rows,
+            f"teacher producer: log-softmax over {V} + top-{K}, {rows} rows bf16 -> fp16/int32", "topk_producer_kernel<bf16,1024,16>",
+            c, torch.empty_like(c["logits"]))
+
+
+WORKLOADS = {"producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c5": _wl_c5}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -138,6 +158,10 @@ def cpu_baseline(workload: str, rows: int, reps: int):
         c = S.config1("cpu", B=1, S=rows) if workload == "c1" else S.config2("cpu", B=1, S=rows)
         fn = lambda: O.mean_loss_and_grad(c["kind"], c["logits"], c["T"], t_logits=c["t_logits"], valid=c["valid"])
         what = f"{rows} rows at V=32000, dense teacher"
+    elif workload == "producer":
+        c = S.config3("cpu", rows=rows, seed=3)
+        fn = lambda: O.to_storage(*[t.reshape(-1, 200) for t in O.teacher_topk_producer(c["logits"], 128256, 200)])
+        what = f"{rows} of 32768 rows at V=128256, K=200 (log_softmax + torch.topk)"
     else:
         c = S.config5("cpu", rows=rows)
         def fn():
@@ -216,7 +240,7 @@ def main():
     kern_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
     achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
 
-    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c1": 512, "c2": 4096, "c5": 512}[args.workload]
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048}[args.workload]
     out = {
         "metric": "tokens/sec fused KL fwd+bwd @ vocab 128256 bf16; % of HBM peak GB/s",
         "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,

@@ -143,6 +143,21 @@ int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_strid
                          const float* coef_zk, void* grad, int64_t grad_stride, void* stream);
 
 /*
+ * Teacher producer: per selected row, log_softmax over the V (cropped) columns, then the K largest
+ * log-probs in descending order with their ids.  Replaces
+ *   classes/teacher/inference_worker.py:73-80  (F.log_softmax(logits[:, :, :crop].float()) -> torch.topk)
+ *   classes/teacher/result_processor_worker.py:27-35  (content-row selection, via row_list)
+ *   classes/data_manager.py:306,312  (cast to the storage dtypes: out_dtype DL_F16, out_itype DL_I32)
+ * No temperature is applied at collection time.  row_list (int32 [n_out], may be NULL = rows
+ * 0..n_out-1) names the logits row behind each output row.  Entries with equal log-prob are ordered
+ * by ascending id (the reference leaves tie order to torch.topk).
+ * K <= 1024, K <= V; V a multiple of 8 (4 for fp32), rows 16-byte aligned; V <= 131072 (65536 fp32).
+ */
+int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                    const int32_t* row_list, int64_t n_out, int K,
+                    void* out_val, int out_dtype, void* out_idx, int out_itype, void* stream);
+
+/*
  * Weighted merge of n_teachers sparse teachers with an optional vocabulary id map
  * (no reference counterpart; generalises classes/data_manager.py:231-240, which is unweighted,
  * pairwise and has no map).  Per row: mass = weights[j] * exp(t_vals[j][row, k]); the id goes

@@ -97,3 +97,29 @@ def fkl_multi_teacher(logits: torch.Tensor, vals: Sequence[torch.Tensor], idxs: 
     ids, logmass, cnt = merge_remap_topk(vals, idxs, weights, id_map, student_vocab=V)
     return ops.div_topk("fkl", logits, logmass, ids, row_map=row_map, t_cnt=cnt, T=T, teacher_T=teacher_T,
                         grad_scale=grad_scale, want_grad=want_grad, grad_out=grad_out, unique_ids=True)
+
+
+def teacher_topk(logits: torch.Tensor, K: int, *, crop_to_size: int | None = None, rows: torch.Tensor | None = None,
+                 val_dtype=torch.float16, idx_dtype=torch.int32):
+    """What the teacher's inference worker produces (classes/teacher/inference_worker.py:73-80) in
+    the dataset's storage layout: per row the K largest full-vocabulary log-probs, descending, and
+    their ids.  `rows` (int32 positions, e.g. the content rows) selects and orders the output rows.
+    Returns (log-probs [n, K] val_dtype, ids [n, K] idx_dtype)."""
+    _dev(logits, "logits")
+    x = ops._rows_2d(logits if crop_to_size is None else logits[..., :crop_to_size])
+    if x.dtype not in _DT or val_dtype not in (torch.float16, torch.float32) or idx_dtype not in _IT:
+        raise RuntimeError("unsupported dtype")
+    R, V = x.shape
+    dev = x.device
+    n_out, rl_ptr = R, 0
+    if rows is not None:
+        ops._opt_i32(rows, None, "rows", dev)
+        n_out, rl_ptr = rows.numel(), rows.data_ptr()
+    out_v = torch.empty((n_out, K), dtype=val_dtype, device=dev)
+    out_i = torch.empty((n_out, K), dtype=idx_dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_teacher_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rl_ptr, n_out, K,
+                                         out_v.data_ptr(), _DT[val_dtype], out_i.data_ptr(), _IT[idx_dtype],
+                                         _stream_ptr(dev))
+    _lib.check(st, "dl_teacher_topk")
+    return out_v, out_i

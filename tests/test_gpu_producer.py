@@ -1,0 +1,79 @@
+"""GPU parity of the teacher producer (log-softmax over V + top-K, storage layout) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def D():
+    import llm_distillery_amd as d
+    d._lib.load()
+    return d
+
+
+def _ref(logits, crop, K):
+    """torch.topk semantics with the tie rule made explicit: equal log-probs -> smaller id first
+    (a stable descending sort of the full-vocabulary log-softmax)."""
+    logp = torch.log_softmax(logits[..., :crop].double(), dim=-1)
+    order = torch.sort(logits[..., :crop].float(), dim=-1, descending=True, stable=True).indices[..., :K]
+    return torch.gather(logp, -1, order), order
+
+
+@pytest.mark.parametrize("dtype,V,K", [(torch.bfloat16, 32000, 200), (torch.bfloat16, 128256, 400), (torch.float16, 32000, 64),
+                                       (torch.float32, 32000, 200), (torch.float32, 50264, 1024), (torch.bfloat16, 2048, 17)])
+def test_topk_ids_bit_exact_values_close(D, dtype, V, K):
+    g = torch.Generator().manual_seed(V + K)
+    logits = (torch.randn(9, V, generator=g) * 3).to(dtype)
+    val, idx = D.teacher_topk(logits.to(DEV), K, val_dtype=torch.float32, idx_dtype=torch.int64)
+    rv, ri = _ref(logits, V, K)
+    assert torch.equal(idx.cpu(), ri), "ids (including tie order: smaller id first) must match exactly"
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), rtol=0, atol=2e-6 * max(1.0, float(rv.abs().max())))
+    assert (val[:, :-1] >= val[:, 1:]).all()
+    # the oracle's producer (torch.topk) returns the same value set
+    ov, _ = O.teacher_topk_producer(logits, V, K)
+    np.testing.assert_allclose(val.cpu().numpy(), ov.numpy(), rtol=0, atol=3e-6 * max(1.0, float(ov.abs().max())))
+
+
+def test_storage_layout_crop_and_content_rows(D):
+    g = torch.Generator().manual_seed(3)
+    B, S, Vm, crop, K = 2, 40, 32064, 32000, 100
+    logits = (torch.randn(B, S, Vm, generator=g) * 2).to(torch.bfloat16)
+    rows = torch.as_tensor(np.concatenate([O.content_indices([(3, 9), (20, 31)]), S + O.content_indices([(0, 40)])]), dtype=torch.int32)
+    val, idx = D.teacher_topk(logits.to(DEV), K, crop_to_size=crop, rows=rows.to(DEV))
+    assert val.dtype == torch.float16 and idx.dtype == torch.int32 and val.shape == (rows.numel(), K)
+    flat = logits.reshape(B * S, Vm)[rows.long()]
+    rv, ri = _ref(flat, crop, K)
+    assert torch.equal(idx.cpu().long(), ri) and int(idx.max()) < crop
+    assert torch.equal(val.cpu(), rv.to(torch.float32).to(torch.float16)) or \
+        (val.cpu().float() - rv.float()).abs().max() <= 2e-3 * rv.abs().max()
+    # round trip through the dataset's dtypes and into the loss: producer output is a valid sparse teacher
+    rl, _ = D.div_topk("fkl", logits.reshape(B * S, Vm)[:, :crop].to(DEV)[rows.long().to(DEV)].contiguous(), val, idx, unique_ids=True)
+    # a model distilled from itself: KL(q || p) = -log(student mass on the top-K support)
+    mass = torch.gather(torch.softmax(flat[:, :crop].double(), -1), 1, ri).sum(-1)
+    np.testing.assert_allclose(rl.cpu().double().numpy(), -torch.log(mass).numpy(), rtol=2e-3, atol=2e-3)
+
+
+def test_heavy_ties_and_constant_rows(D):
+    # quantised logits: thousands of entries share the threshold value; constant rows: all equal
+    g = torch.Generator().manual_seed(4)
+    V, K = 16384, 300
+    logits = torch.randint(-3, 4, (5, V), generator=g).to(torch.bfloat16)
+    logits[3] = 1.5
+    logits[4, ::2] = float("-inf")
+    val, idx = D.teacher_topk(logits.to(DEV), K, val_dtype=torch.float32, idx_dtype=torch.int32)
+    rv, ri = _ref(logits, V, K)
+    assert torch.equal(idx.cpu().long(), ri)
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), atol=1e-5)
+    assert idx[3].cpu().tolist() == list(range(K))
+
+
+def test_producer_limits(D):
+    with pytest.raises(RuntimeError):
+        D.teacher_topk(torch.zeros(2, 4096, device=DEV), 2000)
+    with pytest.raises(RuntimeError):
+        D.teacher_topk(torch.zeros(2, 1001, device=DEV), 10)
