@@ -100,14 +100,15 @@ def _wl_c5(D, S, dev, rows):
     c = S.config5(dev, rows=rows, Vs=Vs, Vt=Vt)
     grad = torch.empty_like(c["logits"])
     scale = 1.0 / rows
+    plan = D.vocab_utils.MarginalPlan(c["t2s_host"], Vs, dev)       # built once per tokenizer pair
 
     def main():
-        return D.vocab_utils.rkl_marginalised(c["logits"], c["t_probs"], c["t2s"], T=c["T"], grad_scale=scale,
+        return D.vocab_utils.rkl_marginalised(c["logits"], c["t_probs"], plan, T=c["T"], grad_scale=scale,
                                               grad_out=grad)[0]
 
     return (lambda: D.reduce_sum(main(), scale), main, rows * (Vt * 4 + Vs * 2 + Vs * 2) + Vt * 4, rows,
             f"C5 byte-trie marginalisation ({Vt}->{Vs}) + reverse-KL fwd+bwd, {rows} tokens, fp32 teacher softmax, "
-            "bf16 student, T=1.5", "rkl_marginalised_kernel<bf16>", c, grad)
+            "bf16 student, T=1.5", "rkl_marginalised_kernel<bf16> (planned marginal)", c, grad)
 
 
 def _wl_producer(D, S, dev, rows):

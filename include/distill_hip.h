@@ -208,13 +208,31 @@ int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_student, in
                     int32_t* indices, int64_t* n_mapped);
 
 /*
+ * Marginalisation plan (HOST function, HOST pointers; no reference counterpart): re-lays a
+ * teacher->student map for the planned kernels, which add every marginal in a fixed order without
+ * atomics.  Student id s is owned by thread s % 1024 of a 1024-thread workgroup; the teacher
+ * vocabulary is cut into tiles of *tile_out ids; for tile k and wave w, rows
+ * row_off[16k + w] .. row_off[16k + w + 1] of `ent` hold 64 entries each (one per lane,
+ * 0xffffffff = padding): (s << log2(tile) | t - k * tile), per thread sorted by (s, t).
+ * Call once with row_off = ent = NULL to learn *tile_out and *ent_rows_out, allocate
+ * row_off int32 [16 * ceil(n_teacher / tile) + 1] and ent uint32 [64 * ent_rows], call again.
+ * DL_ERR_LIMIT: the student vocabulary is too wide for a plan (fp32 marginal + 16 KiB tile must fit 159 KiB).
+ */
+int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int* tile_out,
+                           int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity, int64_t* ent_rows_out);
+
+/*
  * marg[r, s] = sum of probs[r, t] over the teacher ids t with t2s[t] == s (probs [n_rows, Vt] in
- * p_dtype, marg fp32 [n_rows, Vs]; out_log != 0 stores log(marg) instead).  Accumulates with LDS
- * floating-point atomics: sums agree with the CSR form to fp32 rounding, not bit for bit.
+ * p_dtype, marg fp32 [n_rows, Vs]; out_log != 0 stores log(marg) instead).  With a plan
+ * (plan_row_off / plan_ent device copies of dl_marginal_plan_build's arrays, plan_tile its tile;
+ * fp32 probabilities, 16-byte aligned rows) every sum is added in a fixed order: bit-reproducible.
+ * Without (NULL, NULL, 0) it accumulates with LDS floating-point atomics: sums then agree to fp32
+ * rounding, not bit for bit.
  */
 int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
-                       const int32_t* t2s, int64_t Vs, float* marg, int64_t marg_stride, int out_log,
-                       void* stream);
+                       const int32_t* t2s, int64_t Vs,
+                       const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                       float* marg, int64_t marg_stride, int out_log, void* stream);
 
 /* The same marginal from the CSR form, each segment added in ascending teacher-id order (bit-reproducible). */
 int dl_marginalise_csr(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
@@ -226,12 +244,14 @@ int dl_marginalise_csr(const void* probs, int p_dtype, int64_t p_stride, int64_t
  * student ids inside LDS, then reverse KL of the student logits[r] against
  * softmax(log(marginal) * inv_T_teacher), loss and gradient, with the conventions of dl_div_dense
  * (DL_RKL: student renormalised over the marginal's support).  The marginal never reaches memory.
+ * Optional plan as for dl_marginalise_map (faster and bit-reproducible).
  * Vs <= 36864 (the fp32 marginal of one row must fit the CU's LDS), Vs % 8 == 0, logits / grad
  * rows 16-byte aligned (else DL_ERR_LIMIT / DL_ERR_ALIGN: use dl_marginalise_map + dl_div_dense).
  */
 int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs,
                         const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
                         int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s,
+                        const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
                         float inv_T_student, float inv_T_teacher, float grad_scale,
                         float* row_loss, void* grad, int64_t grad_stride, void* stream);
 

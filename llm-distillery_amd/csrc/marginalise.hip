@@ -9,6 +9,13 @@
 //     sums agree to fp32 rounding, not bit for bit.
 //   * CSR form (deterministic): one thread per student id adds its segment in ascending
 //     teacher-id order.
+//   * planned form (fast and deterministic): the host lays the map out as a "plan": the teacher
+//     vocabulary is cut into tiles of `tile` ids; student id s belongs to thread s % 1024; for every
+//     (tile, wave) the entries (s, local teacher id) of the wave's 64 threads are stored row-wise
+//     (64 entries per row, padded), each thread's entries sorted by (s, t).  The kernel streams a
+//     teacher tile into LDS (coalesced), then every thread walks its entries, reads the tile at
+//     random (LDS), and adds runs of equal s into marg[s] -- a location only that thread ever
+//     touches, so no atomics, and the order of additions is fixed: bit-reproducible.
 //   * fused reverse KL: the marginal never leaves LDS; its logarithm is the teacher row of the
 //     dense-divergence sweeps, the student row sits in registers.
 #include "dense_div.hpp"
@@ -17,6 +24,7 @@ namespace dl {
 
 constexpr int MARG_NT = 1024;
 constexpr int MARG_MAX_VS = 36864;          // fp32 marginal of one row in LDS: 144 KiB of the CU's 160
+constexpr int MARG_MAX_DYN_LDS = 160 * 1024 - 1024;   // dynamic LDS a workgroup may request (planned form: marginal + tile)
 
 struct MargParams {
   const void* probs; int p_dtype; int64_t p_stride; int64_t n_rows; int64_t Vt;
@@ -25,7 +33,138 @@ struct MargParams {
   // fused reverse KL
   const void* logits; int s_dtype; int64_t row_stride; int64_t n_srows; const int32_t* row_map;
   float inv_T_s, inv_T_t, grad_scale; float* row_loss; void* grad; int64_t grad_stride;
+  // plan (all NULL/0: accumulate with LDS atomics along t2s instead)
+  const int32_t* plan_row_off; const uint32_t* plan_ent; int plan_tile; int plan_tile_bits;
 };
+
+constexpr unsigned PLAN_PAD = 0xffffffffu;
+
+// Marginal of one teacher row into marg[0, Vs) (LDS, zeroed here) along a plan; `tile` is LDS
+// scratch of plan_tile floats.  fp32 probabilities, 16-byte aligned rows.
+//
+// Latencies are kept off the critical path by batching: a thread holds a batch of PLAN_EB entries
+// in registers (the next tile's first batch is fetched while the current tile is consumed), reads
+// the tile for the whole batch at once, folds runs of equal student id in registers, and then
+// applies the run totals to marg with all reads issued before all writes (the ids inside one
+// thread's list are sorted, so the runs of a batch hit distinct addresses).
+constexpr int PLAN_EB = 8;           // entries per prefetched batch (measured: 16 is slower, more padding work)
+constexpr int PLAN_HB = 8;
+
+struct PlanRun {          // a run of equal student id still open at the end of a batch
+  int sid;
+  float sum;
+};
+
+__device__ __forceinline__ void plan_consume_half(const unsigned* e, const float* tile, float* marg,
+                                                  unsigned tmask, int bits, PlanRun& open) {
+  float val[PLAN_HB];
+#pragma unroll
+  for (int j = 0; j < PLAN_HB; ++j) val[j] = e[j] != PLAN_PAD ? tile[e[j] & tmask] : 0.f;
+  int fsid[PLAN_HB];       // student id whose run closes just before entry j (or -1)
+  float fsum[PLAN_HB];
+#pragma unroll
+  for (int j = 0; j < PLAN_HB; ++j) {
+    fsid[j] = -1;
+    fsum[j] = 0.f;
+    if (e[j] != PLAN_PAD) {
+      const int sid = (int)(e[j] >> bits);
+      if (sid != open.sid) {
+        fsid[j] = open.sid;
+        fsum[j] = open.sum;
+        open.sid = sid;
+        open.sum = 0.f;
+      }
+      open.sum += val[j];
+    }
+  }
+  float old[PLAN_HB];
+#pragma unroll
+  for (int j = 0; j < PLAN_HB; ++j) old[j] = fsid[j] >= 0 ? marg[fsid[j]] : 0.f;
+#pragma unroll
+  for (int j = 0; j < PLAN_HB; ++j)
+    if (fsid[j] >= 0) marg[fsid[j]] = old[j] + fsum[j];
+}
+
+__device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const float* tile, float* marg,
+                                             unsigned tmask, int bits, PlanRun& open) {
+#pragma unroll
+  for (int h = 0; h < PLAN_EB / PLAN_HB; ++h) plan_consume_half(e + h * PLAN_HB, tile, marg, tmask, bits, open);
+}
+
+// Teacher tiles are fetched PLAN_DEPTH tiles ahead (registers): with one 32 KiB tile in flight per
+// CU the chip holds 8 MB outstanding, which at HBM latency caps the stream near 1.5 TB/s.
+constexpr int PLAN_DEPTH = 4;
+
+__device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p, const char* prow, float* marg,
+                                                            float* tile) {
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1);
+  // the wave index as a scalar: plan offsets are then fetched with scalar loads, which have their own
+  // counter and do not queue behind the vector prefetches
+  const int w = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  constexpr int NW = MARG_NT / WAVE;
+  const int TS = p.plan_tile;
+  const int per = TS / 4 / MARG_NT;                 // 16-byte loads per thread per tile (1 or 2)
+  const int ntiles = (int)((p.Vt + TS - 1) / TS);
+  const int64_t n4 = p.Vt / 4;
+  const int bits = p.plan_tile_bits;
+  const unsigned tmask = (1u << bits) - 1u;
+  for (int j = tid; j < p.Vs; j += MARG_NT) marg[j] = 0.f;
+  u32x4 tbuf[PLAN_DEPTH][2];
+  auto fetch_tile = [&](int k, u32x4 (&buf)[2]) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      // Unconditional load from a clamped address, then a select: with branch-free loads the
+      // compiler knows how many are in flight and never has to drain the whole queue.
+      const int64_t c = (int64_t)k * (TS / 4) + (int64_t)u * MARG_NT + tid;
+      const bool live = u < per && c < n4;
+      const u32x4 v = load16_stream(prow + (live ? c : 0) * 16);
+      buf[u] = live ? v : u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto fetch_entries = [&](int r_first, int r_end, unsigned (&e)[PLAN_EB]) {
+#pragma unroll
+    for (int j = 0; j < PLAN_EB; ++j) {
+      const int r = r_first + j;
+      const unsigned v = p.plan_ent[(int64_t)(r < r_end ? r : 0) * WAVE + lane];
+      e[j] = r < r_end ? v : PLAN_PAD;
+    }
+  };
+  unsigned ea[PLAN_EB], eb[PLAN_EB];                // ping-pong entry batches (no register copies)
+#pragma unroll
+  for (int d = 0; d < PLAN_DEPTH; ++d) fetch_tile(d, tbuf[d]);
+  int r0 = p.plan_row_off[w], r1 = p.plan_row_off[w + 1];
+  fetch_entries(r0, r1, ea);
+  auto do_tile = [&](int k, u32x4 (&buf)[2], unsigned (&ecur)[PLAN_EB], unsigned (&enxt)[PLAN_EB]) {
+    __syncthreads();                                 // previous tile fully consumed (first pass: marg zeroed)
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      if (u < per) *reinterpret_cast<u32x4*>(tile + ((int64_t)u * MARG_NT + tid) * 4) = buf[u];
+    __syncthreads();
+    fetch_tile(k + PLAN_DEPTH, buf);                 // refill this buffer, PLAN_DEPTH tiles ahead
+    int n0 = 0, n1 = 0;
+    if (k + 1 < ntiles) {
+      n0 = p.plan_row_off[(k + 1) * NW + w];
+      n1 = p.plan_row_off[(k + 1) * NW + w + 1];
+    }
+    fetch_entries(n0, n1, enxt);                     // next tile's first entry batch
+    PlanRun open{-1, 0.f};
+    plan_consume(ecur, tile, marg, tmask, bits, open);
+    for (int r = r0 + PLAN_EB; r < r1; r += PLAN_EB) {      // long lists (hot student ids): further batches
+      fetch_entries(r, r1, ecur);
+      plan_consume(ecur, tile, marg, tmask, bits, open);
+    }
+    if (open.sid >= 0) marg[open.sid] += open.sum;
+    r0 = n0;
+    r1 = n1;
+  };
+  for (int k = 0; k < ntiles; k += PLAN_DEPTH) {     // unrolled by the depth: buffers are addressed statically
+    do_tile(k, tbuf[0], ea, eb);
+    if (k + 1 < ntiles) do_tile(k + 1, tbuf[1], eb, ea);
+    if (k + 2 < ntiles) do_tile(k + 2, tbuf[2], ea, eb);
+    if (k + 3 < ntiles) do_tile(k + 3, tbuf[3], eb, ea);
+  }
+  __syncthreads();
+}
 
 // Accumulate the slice [s_lo, s_lo + s_n) of one row's marginal into `acc` (LDS, zeroed here).
 template <bool VEC>
@@ -93,6 +232,11 @@ __global__ __launch_bounds__(MARG_NT) void marginalise_map_kernel(const MargPara
   const int pb = p.p_dtype == F32 ? 4 : 2;
   const char* prow = reinterpret_cast<const char*>(p.probs) + r * p.p_stride * pb;
   float* out = p.marg + r * p.marg_stride;
+  if (VEC && p.plan_ent) {
+    accumulate_marginal_planned(p, prow, acc, acc + ((p.Vs + 3) & ~(int64_t)3));
+    for (int j = threadIdx.x; j < p.Vs; j += MARG_NT) out[j] = p.out_log ? logf(acc[j]) : acc[j];
+    return;
+  }
   for (int64_t s_lo = 0; s_lo < p.Vs; s_lo += MARG_MAX_VS) {
     const int s_n = (int)min((int64_t)MARG_MAX_VS, p.Vs - s_lo);
     accumulate_marginal<VEC>(p, prow, acc, (int)s_lo, s_n);
@@ -163,9 +307,16 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
     return;
   }
   LdsTeacherRows<TagS, NU> rows;
-  rows.load(reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes, p.Vs / 8);   // in flight during the scatter
+  const char* srow = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes;
   const int pb = p.p_dtype == F32 ? 4 : 2;
-  accumulate_marginal<VEC>(p, reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb, acc, 0, (int)p.Vs);
+  const char* prow = reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb;
+  if (VEC && p.plan_ent) {
+    accumulate_marginal_planned(p, prow, acc, acc + ((p.Vs + 3) & ~(int64_t)3));   // needs the registers itself
+    rows.load(srow, p.Vs / 8);
+  } else {
+    rows.load(srow, p.Vs / 8);                   // in flight during the scatter
+    accumulate_marginal<VEC>(p, prow, acc, 0, (int)p.Vs);
+  }
   for (int j = tid; j < p.Vs; j += MARG_NT) acc[j] = fast_log2(acc[j]) * LN2;      // log 0 = -inf: off the support
   __syncthreads();
   rows.lt = acc;
@@ -186,13 +337,13 @@ static bool ok16(const void* ptr, int64_t stride, int eb) {
 // enough (the call is slow, so it must not sit on the launch path).
 template <class K>
 static void allow_large_lds_for(K kernel) {
-  hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                      MARG_MAX_VS * 4);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            MARG_MAX_DYN_LDS);
 }
 static void allow_large_lds() {
   static thread_local int done_for = -1;
   int dev = 0;
-  hipGetDevice(&dev);
+  (void)hipGetDevice(&dev);
   if (done_for == dev) return;
   allow_large_lds_for(&marginalise_map_kernel<true>);
   allow_large_lds_for(&marginalise_map_kernel<false>);
@@ -207,9 +358,22 @@ static void allow_large_lds() {
 
 }  // namespace dl
 
+// Fills the plan fields of `p` if a usable plan is given; returns the dynamic LDS bytes to request.
+static size_t attach_plan(dl::MargParams& p, const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile, bool vec,
+                          size_t lds_without_plan) {
+  if (!plan_row_off || !plan_ent || !vec) return lds_without_plan;
+  if (plan_tile != 4096 && plan_tile != 8192) return lds_without_plan;
+  const size_t need = (size_t)((p.Vs + 3) & ~(int64_t)3) * 4 + (size_t)plan_tile * 4;
+  if (need > (size_t)dl::MARG_MAX_DYN_LDS) return lds_without_plan;
+  p.plan_row_off = plan_row_off; p.plan_ent = plan_ent; p.plan_tile = plan_tile;
+  p.plan_tile_bits = plan_tile == 4096 ? 12 : 13;
+  return need;
+}
+
 extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
-                                  const int32_t* t2s, int64_t Vs, float* marg, int64_t marg_stride, int out_log,
-                                  void* stream) {
+                                  const int32_t* t2s, int64_t Vs, const int32_t* plan_row_off,
+                                  const uint32_t* plan_ent, int plan_tile, float* marg, int64_t marg_stride,
+                                  int out_log, void* stream) {
   using namespace dl;
   if (!probs || !t2s || !marg) return DL_ERR_NULL;
   if (p_dtype < DL_F32 || p_dtype > DL_F16) return DL_ERR_DTYPE;
@@ -219,8 +383,8 @@ extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stri
   MargParams p{};
   p.probs = probs; p.p_dtype = p_dtype; p.p_stride = p_stride; p.n_rows = n_rows; p.Vt = Vt; p.t2s = t2s; p.Vs = Vs;
   p.marg = marg; p.marg_stride = marg_stride; p.out_log = out_log;
-  const size_t lds = (size_t)(Vs < MARG_MAX_VS ? Vs : MARG_MAX_VS) * 4;
   const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(probs, p_stride, 4) && ok16(t2s, 0, 4);
+  const size_t lds = attach_plan(p, plan_row_off, plan_ent, plan_tile, vec, (size_t)(Vs < MARG_MAX_VS ? Vs : MARG_MAX_VS) * 4);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   allow_large_lds();
   if (vec) hipLaunchKernelGGL((marginalise_map_kernel<true>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
@@ -249,9 +413,10 @@ extern "C" int dl_marginalise_csr(const void* probs, int p_dtype, int64_t p_stri
 
 extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs,
                                    const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
-                                   int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s, float inv_T_student,
-                                   float inv_T_teacher, float grad_scale, float* row_loss, void* grad,
-                                   int64_t grad_stride, void* stream) {
+                                   int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s,
+                                   const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                                   float inv_T_student, float inv_T_teacher, float grad_scale, float* row_loss,
+                                   void* grad, int64_t grad_stride, void* stream) {
   using namespace dl;
   if (!logits || !t_probs || !t2s) return DL_ERR_NULL;
   if (logits_dtype < DL_F32 || logits_dtype > DL_F16 || p_dtype < DL_F32 || p_dtype > DL_F16) return DL_ERR_DTYPE;
@@ -268,7 +433,7 @@ extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t
   p.row_map = row_map; p.inv_T_s = inv_T_student; p.inv_T_t = inv_T_teacher; p.grad_scale = grad_scale;
   p.row_loss = row_loss; p.grad = grad; p.grad_stride = grad_stride;
   const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(t_probs, p_stride, 4) && ok16(t2s, 0, 4);
-  const size_t lds = (size_t)Vs * 4;
+  const size_t lds = attach_plan(p, plan_row_off, plan_ent, plan_tile, vec, (size_t)Vs * 4);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)n_rows), block(MARG_NT);
   allow_large_lds();

@@ -4,6 +4,7 @@
 #include "distill_hip.h"
 
 #include <cstdint>
+#include <algorithm>
 #include <cstring>
 #include <unordered_map>
 #include <vector>
@@ -100,5 +101,60 @@ extern "C" int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_
     if (s >= 0) indices[cursor[s]++] = (int32_t)t;
   }
   if (n_mapped) *n_mapped = offsets[n_student];
+  return DL_OK;
+}
+
+// ---- marginalisation plan --------------------------------------------------------------------
+// Layout consumed by the planned marginalisation kernels (1024 threads = 16 waves per workgroup):
+// the teacher vocabulary is cut into tiles of `tile` ids; student id s is owned by thread s % 1024;
+// for tile k and wave w, rows row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries
+// per row (one per lane, 0xffffffff = padding), the entries (s << log2(tile) | t - k*tile) of the
+// wave's threads, each thread's entries sorted by (s, t).
+extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int* tile_out,
+                                      int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity,
+                                      int64_t* ent_rows_out) {
+  constexpr int NT = 1024, WAVE = 64, NW = NT / WAVE;
+  constexpr int64_t LDS_BUDGET = 160 * 1024 - 1024;      // dynamic LDS one workgroup may use
+  if (!t2s || !tile_out || !ent_rows_out) return DL_ERR_NULL;
+  if (n_teacher <= 0 || n_student <= 0) return DL_ERR_SHAPE;
+  if (n_teacher > 0x7fffffffLL) return DL_ERR_LIMIT;
+  const int64_t marg_bytes = ((n_student + 3) & ~(int64_t)3) * 4;
+  int tile = 8192;
+  while (tile >= 4096 && marg_bytes + (int64_t)tile * 4 > LDS_BUDGET) tile >>= 1;
+  if (tile < 4096) return DL_ERR_LIMIT;                  // marginal + smallest tile do not fit the LDS
+  int tile_bits = 0;
+  while ((1 << tile_bits) < tile) ++tile_bits;
+  if (n_student >= (1LL << (32 - tile_bits)) - 1) return DL_ERR_LIMIT;
+  *tile_out = tile;
+  const int64_t ntiles = (n_teacher + tile - 1) / tile;
+  std::vector<std::vector<uint32_t>> bucket(NT);
+  int64_t rows = 0;
+  if (row_off) row_off[0] = 0;
+  for (int64_t k = 0; k < ntiles; ++k) {
+    for (auto& b : bucket) b.clear();
+    const int64_t t0 = k * tile, t1 = std::min<int64_t>(n_teacher, t0 + tile);
+    for (int64_t t = t0; t < t1; ++t) {
+      const int32_t sid = t2s[t];
+      if (sid >= n_student) return DL_ERR_SHAPE;
+      if (sid >= 0) bucket[sid % NT].push_back(((uint32_t)sid << tile_bits) | (uint32_t)(t - t0));
+    }
+    for (auto& b : bucket) std::sort(b.begin(), b.end());      // (s, t) ascending: s in the high bits
+    for (int w = 0; w < NW; ++w) {
+      size_t longest = 0;
+      for (int l = 0; l < WAVE; ++l) longest = std::max(longest, bucket[w * WAVE + l].size());
+      if (ent) {
+        if (rows + (int64_t)longest > ent_rows_capacity) return DL_ERR_SHAPE;
+        for (size_t j = 0; j < longest; ++j)
+          for (int l = 0; l < WAVE; ++l) {
+            const auto& b = bucket[w * WAVE + l];
+            ent[(rows + (int64_t)j) * WAVE + l] = j < b.size() ? b[j] : 0xffffffffu;
+          }
+      }
+      rows += (int64_t)longest;
+      if (rows > 0x7fffffffLL) return DL_ERR_LIMIT;
+      if (row_off) row_off[k * NW + w + 1] = (int32_t)rows;
+    }
+  }
+  *ent_rows_out = rows;
   return DL_OK;
 }

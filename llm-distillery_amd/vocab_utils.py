@@ -62,11 +62,46 @@ def csr_from_map(t2s: np.ndarray, n_student: int) -> tuple[np.ndarray, np.ndarra
     return offsets, indices[:n.value].copy()
 
 
-def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=None, n_student: int,
-                log: bool = False) -> torch.Tensor:
+class MarginalPlan:
+    """A teacher->student id map laid out for the planned marginalisation kernels (fixed summation
+    order, no atomics): build once per tokenizer pair, reuse for every batch.  Holds the device
+    copies of the map and of the plan arrays."""
+
+    def __init__(self, t2s: np.ndarray, n_student: int, device):
+        t2s = np.ascontiguousarray(np.asarray(t2s, dtype=np.int32))
+        self.n_student = int(n_student)
+        self.n_teacher = int(t2s.size)
+        self.t2s = torch.as_tensor(t2s, device=device)
+        self.row_off = self.ent = None
+        self.tile = 0
+        lib = _lib.load()
+        tile, rows = ctypes.c_int(0), ctypes.c_int64(0)
+        st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), None, None, 0, ctypes.byref(rows))
+        if st == -4:          # DL_ERR_LIMIT: student vocabulary too wide for a plan; the atomic path still works
+            return
+        _lib.check(st, "dl_marginal_plan_build")
+        ntiles = -(-t2s.size // tile.value)
+        row_off = np.zeros(16 * ntiles + 1, dtype=np.int32)
+        ent = np.empty((max(rows.value, 1), 64), dtype=np.uint32)
+        st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), _p(row_off), _p(ent), rows.value,
+                                        ctypes.byref(rows))
+        _lib.check(st, "dl_marginal_plan_build")
+        self.tile = tile.value
+        self.row_off = torch.as_tensor(row_off, device=device)
+        self.ent = torch.as_tensor(ent.view(np.int32), device=device)     # same bits; torch has no uint32 arithmetic need
+
+    def _args(self):
+        if self.ent is None:
+            return 0, 0, 0
+        return self.row_off.data_ptr(), self.ent.data_ptr(), self.tile
+
+
+def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=None, plan: MarginalPlan | None = None,
+                n_student: int, log: bool = False) -> torch.Tensor:
     """marg[r, s] = sum of probs[r, t] over the teacher ids mapped to s (fp32 [rows, n_student]).
-    `t2s` (int32 [Vt], on the GPU) selects the fast LDS-atomic form; `csr=(offsets, indices)` the
-    deterministic one.  `log=True` returns log(marg)."""
+    `plan` (a MarginalPlan) selects the planned form: fast and bit-reproducible; `t2s` (int32 [Vt],
+    on the GPU) the LDS-atomic form; `csr=(offsets, indices)` the thread-per-id deterministic one.
+    `log=True` returns log(marg)."""
     _dev(probs, "probs")
     x = _rows_2d(probs)
     if x.dtype not in _DT:
@@ -87,20 +122,29 @@ def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=Non
                                         _stream_ptr(x.device))
             _lib.check(st, "dl_marginalise_csr")
         else:
+            pro, pen, pti = (0, 0, 0)
+            if plan is not None:
+                t2s = plan.t2s
+                pro, pen, pti = plan._args()
             _, _ = _opt_i32(t2s, Vt, "t2s", x.device)
             st = lib.dl_marginalise_map(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vt, t2s.data_ptr(), n_student,
-                                        out.data_ptr(), out.stride(0), int(log), _stream_ptr(x.device))
+                                        pro, pen, pti, out.data_ptr(), out.stride(0), int(log), _stream_ptr(x.device))
             _lib.check(st, "dl_marginalise_map")
     return out
 
 
-def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: torch.Tensor, *,
+def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "torch.Tensor | MarginalPlan", *,
                      row_map: torch.Tensor | None = None, T: float = 1.0, teacher_T: float | None = None,
                      grad_scale: float = 1.0, want_grad: bool = True, grad_out: torch.Tensor | None = None):
     """Reverse KL of the student (logits [rows, Vs]) against the teacher's distribution
     (teacher_probs [N, Vt]) marginalised into the student vocabulary along `t2s`, loss and gradient
-    in one launch; the marginal stays in LDS.  Returns (row_loss fp32 [rows], grad or None)."""
+    in one launch; the marginal stays in LDS.  `t2s` is the int32 [Vt] map on the GPU or, better, a
+    MarginalPlan built from it.  Returns (row_loss fp32 [rows], grad or None)."""
     _dev(logits, "logits"), _dev(teacher_probs, "teacher_probs")
+    pro, pen, pti = (0, 0, 0)
+    if isinstance(t2s, MarginalPlan):
+        pro, pen, pti = t2s._args()
+        t2s = t2s.t2s
     x, tp = _rows_2d(logits), _rows_2d(teacher_probs)
     R, Vs = x.shape
     N, Vt = tp.shape
@@ -118,7 +162,7 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: tor
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
     with torch.cuda.device(dev):
         st = _lib.load().dl_rkl_marginalised(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vs, rm_ptr, tp.data_ptr(),
-                                             _DT[tp.dtype], tp.stride(0), N, Vt, t2s.data_ptr(), 1.0 / T,
+                                             _DT[tp.dtype], tp.stride(0), N, Vt, t2s.data_ptr(), pro, pen, pti, 1.0 / T,
                                              1.0 / (T if teacher_T is None else teacher_T), grad_scale,
                                              row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
     _lib.check(st, "dl_rkl_marginalised")

@@ -48,6 +48,12 @@ def test_marginal_map_and_csr_forms(D, Vs, Vt, alphabet):
     again = D.vocab_utils.marginalise(probs.to(DEV), csr=(torch.tensor(off, device=DEV), torch.tensor(ind, device=DEV)),
                                       n_student=Vs).cpu().numpy()
     assert np.array_equal(m_csr, again)
+    if Vs <= 36000:
+        plan = D.vocab_utils.MarginalPlan(t2s, Vs, DEV)
+        m_plan = D.vocab_utils.marginalise(probs.to(DEV), plan=plan, n_student=Vs).cpu().numpy()
+        np.testing.assert_allclose(m_plan, ref, rtol=2e-6, atol=1e-9)
+        assert np.array_equal(m_plan == 0, ref == 0)
+        assert np.array_equal(m_plan, D.vocab_utils.marginalise(probs.to(DEV), plan=plan, n_student=Vs).cpu().numpy())
     lg = D.vocab_utils.marginalise(probs.to(DEV), t2s=torch.tensor(t2s, device=DEV), n_student=Vs, log=True).cpu().numpy()
     with np.errstate(divide="ignore"):
         np.testing.assert_allclose(lg[ref > 0], np.log(ref[ref > 0]), rtol=1e-5, atol=1e-5)
@@ -61,9 +67,10 @@ def test_marginal_of_16bit_probabilities(D):
     np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=2e-6, atol=1e-9)
 
 
+@pytest.mark.parametrize("planned", [False, True])
 @pytest.mark.parametrize("dtype,Vs,Vt,alphabet,T", [(torch.bfloat16, 32000, 152064, 256, 1.5), (torch.float32, 2048, 9000, 4, 1.0),
                                                     (torch.float16, 8192, 30000, 8, 0.8)])
-def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T):
+def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T, planned):
     R = 12
     t2s, probs = _case(R, Vs, Vt, 3, alphabet, drop=0.01)
     g = torch.Generator().manual_seed(9)
@@ -72,8 +79,13 @@ def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T):
     valid[[2, 5, 14]] = False
     rm = torch.full((R + 3,), -1, dtype=torch.int32)
     rm[valid] = torch.arange(R, dtype=torch.int32)
-    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), torch.tensor(t2s, device=DEV),
-                                              row_map=rm.to(DEV), T=T, grad_scale=1.0 / R)
+    tmap = D.vocab_utils.MarginalPlan(t2s, Vs, DEV) if planned else torch.tensor(t2s, device=DEV)
+    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, row_map=rm.to(DEV), T=T,
+                                              grad_scale=1.0 / R)
+    if planned:       # fixed summation order: bit-reproducible
+        rl2, grad2 = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, row_map=rm.to(DEV), T=T,
+                                                    grad_scale=1.0 / R)
+        assert torch.equal(rl, rl2) and torch.equal(grad, grad2)
     marg = torch.tensor(O.marginalise_map(probs.numpy(), t2s, Vs))
     with np.errstate(divide="ignore"):
         t_logits = O.marginal_to_teacher_logits(marg)

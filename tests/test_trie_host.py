@@ -55,3 +55,35 @@ def test_config5_vocabularies_at_full_size():
     assert np.array_equal(t2s[sample], ref)
     off, ind = D.vocab_utils.csr_from_map(t2s, 32000)
     assert off[-1] == 152064 and np.array_equal(np.sort(ind), np.arange(152064))
+
+
+def test_marginal_plan_covers_every_mapped_id_once_in_owner_order():
+    rng = np.random.default_rng(7)
+    Vt, Vs = 20000, 3000
+    t2s = rng.integers(-1, Vs, Vt).astype(np.int32)
+    t2s[rng.random(Vt) < 0.5] = rng.integers(0, 8)            # a few very hot student ids
+    plan = D.vocab_utils.MarginalPlan(t2s, Vs, "cpu")
+    tile, bits = plan.tile, int(np.log2(plan.tile))
+    assert tile in (4096, 8192)
+    row_off = plan.row_off.numpy()
+    ent = plan.ent.numpy().view(np.uint32)
+    ntiles = -(-Vt // tile)
+    assert row_off.shape == (16 * ntiles + 1,) and row_off[0] == 0 and row_off[-1] == ent.shape[0]
+    seen = np.zeros(Vt, dtype=np.int32)
+    for k in range(ntiles):
+        for w in range(16):
+            rows = ent[row_off[16 * k + w]:row_off[16 * k + w + 1]]
+            for lane in range(64):
+                col = rows[:, lane]
+                live = col[col != 0xffffffff]
+                assert (col[len(live):] == 0xffffffff).all()            # padding only at the tail
+                assert (np.diff(live.astype(np.int64)) > 0).all()         # sorted by (s, t), no repeats
+                sid = (live >> bits).astype(np.int64)
+                t = (live & (tile - 1)).astype(np.int64) + k * tile
+                assert (sid % 1024 == w * 64 + lane).all()                # owned by this thread
+                assert (t2s[t] == sid).all()
+                seen[t] += 1
+    assert np.array_equal(seen, (t2s >= 0).astype(np.int32))
+    # too wide a student vocabulary: no plan, the atomic form remains
+    wide = D.vocab_utils.MarginalPlan(np.zeros(100, dtype=np.int32), 40000, "cpu")
+    assert wide.ent is None and wide.tile == 0
