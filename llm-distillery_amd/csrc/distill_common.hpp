@@ -35,6 +35,31 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // ---- 16-byte chunk <-> floats -------------------------------------------------
 template <class Tag> struct Chunk;
 
+// eight floats <-> eight fp16 in 16 bytes (round to nearest even)
+__device__ __forceinline__ void unpack_f16x8(const u32x4& c, float* f) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const unsigned u = c[i];   // copy first: bit_cast straight from a vector element reads element 0
+    f16x2 h = __builtin_bit_cast(f16x2, u);
+    f[2 * i] = (float)h[0];
+    f[2 * i + 1] = (float)h[1];
+  }
+}
+__device__ __forceinline__ u32x4 pack_f16x8(const float* f) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f16x2 h = __builtin_convertvector(f32x2{f[2 * i], f[2 * i + 1]}, f16x2);
+    r[i] = __builtin_bit_cast(unsigned, h);
+  }
+  return r;
+}
+
+// Chunk<Tag>: a 16-byte piece of a row.  unpack/pack convert to and from floats in the row's
+// dtype.  stash/unstash keep intermediate values in (0, 2^stash_bias] in the chunk's own 16 bytes
+// between two sweeps: exactly for fp32 rows, as fp16 (11-bit significand, values pre-scaled by
+// 2^15 so that 44 binades stay normal) for 16-bit rows.
+
 template <> struct Chunk<TagF32> {
   static constexpr int N = 4;
   __device__ static __forceinline__ u32x4 neg_inf() { return u32x4{0xff800000u, 0xff800000u, 0xff800000u, 0xff800000u}; }
@@ -45,6 +70,9 @@ template <> struct Chunk<TagF32> {
   __device__ static __forceinline__ u32x4 pack(const float* f) {
     return u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
   }
+  static constexpr float stash_bias = 0.f;
+  __device__ static __forceinline__ u32x4 stash(const float* f) { return pack(f); }
+  __device__ static __forceinline__ void unstash(const u32x4& c, float* f) { unpack(c, f); }
 };
 
 template <> struct Chunk<TagBF16> {
@@ -66,29 +94,19 @@ template <> struct Chunk<TagBF16> {
     }
     return r;
   }
+  static constexpr float stash_bias = 15.f;
+  __device__ static __forceinline__ u32x4 stash(const float* f) { return pack_f16x8(f); }
+  __device__ static __forceinline__ void unstash(const u32x4& c, float* f) { unpack_f16x8(c, f); }
 };
 
 template <> struct Chunk<TagF16> {
   static constexpr int N = 8;
   __device__ static __forceinline__ u32x4 neg_inf() { return u32x4{0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u}; }
-  __device__ static __forceinline__ void unpack(const u32x4& c, float* f) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const unsigned u = c[i];   // copy first: bit_cast straight from a vector element reads element 0
-      f16x2 h = __builtin_bit_cast(f16x2, u);
-      f[2 * i] = (float)h[0];
-      f[2 * i + 1] = (float)h[1];
-    }
-  }
-  __device__ static __forceinline__ u32x4 pack(const float* f) {
-    u32x4 r;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f16x2 h = __builtin_convertvector(f32x2{f[2 * i], f[2 * i + 1]}, f16x2);
-      r[i] = __builtin_bit_cast(unsigned, h);
-    }
-    return r;
-  }
+  __device__ static __forceinline__ void unpack(const u32x4& c, float* f) { unpack_f16x8(c, f); }
+  __device__ static __forceinline__ u32x4 pack(const float* f) { return pack_f16x8(f); }
+  static constexpr float stash_bias = 15.f;
+  __device__ static __forceinline__ u32x4 stash(const float* f) { return pack_f16x8(f); }
+  __device__ static __forceinline__ void unstash(const u32x4& c, float* f) { unpack_f16x8(c, f); }
 };
 
 // ---- scalar element access by runtime dtype (K-wide side arrays only) ----------

@@ -336,7 +336,10 @@ void fkl_topk_reg_kernel(const TopkParams p) {
     for (int e = 0; e < C::N; ++e) mx = fmaxf(mx, f[e]);
   }
   mx = block_max<NT>(mx, s.red);
+  // Second sweep: 2^(x a - max a + bias) takes the place of x in the registers; the gradient is
+  // that value times a row constant, so each element costs one exp2, not two.
   float mb = mx * a;
+  const float mb_own = mb - C::stash_bias;
   float sm = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
@@ -344,9 +347,14 @@ void fkl_topk_reg_kernel(const TopkParams p) {
     forget(reg[i]);
     C::unpack(reg[i], f);
 #pragma unroll
-    for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[e], a, -mb));
+    for (int e = 0; e < C::N; ++e) {
+      f[e] = fast_exp2(fmaf(f[e], a, -mb_own));
+      sm += f[e];
+    }
+    reg[i] = C::stash(f);
+    forget(reg[i]);         // pins the schedule chunk by chunk: no pile-up of unpacked values
   }
-  sm = block_sum<NT>(sm, s.red);
+  sm = block_sum<NT>(sm * __builtin_exp2f(-C::stash_bias), s.red);      // exact: a power of two
 
   if (SPLIT) {
     // publish this part's statistics, collect the others'
@@ -384,15 +392,16 @@ void fkl_topk_reg_kernel(const TopkParams p) {
 
   if (gpart) {
     const float c = p.inv_T_s * p.grad_scale;
+    const float kc = fast_exp2(mb_own - b) * c;       // stashed value -> gradient
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = (int64_t)i * NT + tid;
       if (ch < nch) {
         float f[C::N];
         forget(reg[i]);
-        C::unpack(reg[i], f);
+        C::unstash(reg[i], f);
 #pragma unroll
-        for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * c;
+        for (int e = 0; e < C::N; ++e) f[e] *= kc;
         store16_stream(gpart + ch * 16, C::pack(f));
       }
     }
