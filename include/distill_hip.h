@@ -34,7 +34,8 @@ typedef enum {
   DL_ERR_SHAPE = -3,    /* negative or inconsistent sizes                  */
   DL_ERR_LIMIT = -4,    /* a size exceeds what the kernels support         */
   DL_ERR_LAUNCH = -5,   /* the HIP runtime refused the launch              */
-  DL_ERR_ALIGN = -6     /* a pointer/stride breaks a stated alignment rule */
+  DL_ERR_ALIGN = -6,    /* a pointer/stride breaks a stated alignment rule */
+  DL_ERR_WORKSPACE = -7 /* a required workspace is too small               */
 } dl_status;
 
 #define DL_MAX_TOPK 2048      /* entries per row a sparse teacher may hold        */
@@ -151,11 +152,17 @@ int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_strid
  * No temperature is applied at collection time.  row_list (int32 [n_out], may be NULL = rows
  * 0..n_out-1) names the logits row behind each output row.  Entries with equal log-prob are ordered
  * by ascending id (the reference leaves tie order to torch.topk).
- * K <= 1024, K <= V; V a multiple of 8 (4 for fp32), rows 16-byte aligned; V <= 131072 (65536 fp32).
+ * K <= 1024, K <= V; V a multiple of 8 (4 for fp32), rows 16-byte aligned; V <= 262144 (131072 fp32).
+ * workspace: device memory, 16-byte aligned, at least dl_teacher_topk_workspace_bytes(...) bytes
+ * (per output row and 32768-column part: the part's best K candidates and its softmax statistics);
+ * contents need no initialisation and mean nothing afterwards.  Two launches that may overlap in
+ * time need different workspaces.
  */
 int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
                     const int32_t* row_list, int64_t n_out, int K,
-                    void* out_val, int out_dtype, void* out_idx, int out_itype, void* stream);
+                    void* out_val, int out_dtype, void* out_idx, int out_itype,
+                    void* workspace, int64_t workspace_bytes, void* stream);
+int64_t dl_teacher_topk_workspace_bytes(int logits_dtype, int64_t n_out, int64_t V, int K);
 
 /*
  * Weighted merge of n_teachers sparse teachers with an optional vocabulary id map

@@ -42,6 +42,7 @@ extern "C" const char* dl_status_string(int status) {
     case DL_ERR_LIMIT: return "a size exceeds what the kernels support";
     case DL_ERR_LAUNCH: return "the HIP runtime refused the launch";
     case DL_ERR_ALIGN: return "a pointer or stride breaks an alignment rule";
+    case DL_ERR_WORKSPACE: return "a required workspace is too small";
     default: return "unknown status";
   }
 }

@@ -117,9 +117,11 @@ def teacher_topk(logits: torch.Tensor, K: int, *, crop_to_size: int | None = Non
         n_out, rl_ptr = rows.numel(), rows.data_ptr()
     out_v = torch.empty((n_out, K), dtype=val_dtype, device=dev)
     out_i = torch.empty((n_out, K), dtype=idx_dtype, device=dev)
+    lib = _lib.load()
+    ws = torch.empty((max(16, lib.dl_teacher_topk_workspace_bytes(_DT[x.dtype], n_out, V, K)),), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        st = _lib.load().dl_teacher_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rl_ptr, n_out, K,
-                                         out_v.data_ptr(), _DT[val_dtype], out_i.data_ptr(), _IT[idx_dtype],
-                                         _stream_ptr(dev))
+        st = lib.dl_teacher_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rl_ptr, n_out, K,
+                                 out_v.data_ptr(), _DT[val_dtype], out_i.data_ptr(), _IT[idx_dtype],
+                                 ws.data_ptr(), ws.numel(), _stream_ptr(dev))
     _lib.check(st, "dl_teacher_topk")
     return out_v, out_i
