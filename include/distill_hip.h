@@ -152,7 +152,8 @@ int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_strid
  * No temperature is applied at collection time.  row_list (int32 [n_out], may be NULL = rows
  * 0..n_out-1) names the logits row behind each output row.  Entries with equal log-prob are ordered
  * by ascending id (the reference leaves tie order to torch.topk).
- * K <= 1024, K <= V; V a multiple of 8 (4 for fp32), rows 16-byte aligned; V <= 262144 (131072 fp32).
+ * K <= 1024, K <= V; V a multiple of 8 (4 for fp32), rows 16-byte aligned; V <= 262144 (131072 fp32);
+ * K * parts <= 4096 with parts = ceil(V / 32768) (fp32: ceil(V / 16384)).
  * workspace: device memory, 16-byte aligned, at least dl_teacher_topk_workspace_bytes(...) bytes
  * (per output row and 32768-column part: the part's best K candidates and its softmax statistics);
  * contents need no initialisation and mean nothing afterwards.  Two launches that may overlap in

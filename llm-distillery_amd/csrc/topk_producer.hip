@@ -19,15 +19,16 @@
 namespace dl {
 
 constexpr int PROD_MAX_K = 1024;
-constexpr int PROD_NT = 256, PROD_NCH = 16;
+constexpr int PROD_NT = 512, PROD_NCH = 8;
+constexpr int PROD_G_SMALL = 1024 / PROD_NT, PROD_G_LARGE = PROD_NCH;    // chunk groups per thread: 1024 or 4096 groups per part
 constexpr int PROD_CAP = 2048;              // candidates of a part held in LDS
-constexpr int PROD_RANK_SORT_MAX = 512;     // at most this many candidates are sorted by counting
 constexpr int PROD_MAX_PARTS = 8;
 
 typedef unsigned long long u64;
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
 
-struct PartHeader { float mx; float sm; int cnt; int pad; };     // 16 bytes, then cnt sorted u64 entries
+struct PartHeader { float mx; float sm; int cnt; int pad; };     // 16 bytes, then cnt u64 entries
 
 struct ProducerParams {
   const void* logits; int64_t row_stride; int64_t V;
@@ -37,7 +38,32 @@ struct ProducerParams {
   void* out_val; int out_dtype; void* out_idx; int out_itype;
 };
 
-__host__ __device__ inline int64_t producer_part_stride(int K) { return 16 + (((int64_t)K * 8 + 15) & ~15LL); }
+// Entries a part record can hold: a part with no more candidates than this hands all of them,
+// unsorted, to the merge (which runs at far higher occupancy than the part kernel); a part with more
+// sorts and keeps its best K.  parts * capacity <= 4096 (K <= 1024, parts <= 8 give at most 8192)
+// keeps the merge inside 64 KiB of LDS together with its list of selected words.
+__host__ __device__ inline int producer_record_cap(int K, int parts) {
+  int want = 2 * K > 256 ? 2 * K : 256;
+  if (want > PROD_CAP) want = PROD_CAP;
+  const int fit = (4096 / parts) & ~1;
+  if (want > fit) want = fit;
+  return want > K ? want : K;
+}
+// Selected words (K plus ties) the merge can sort apart from the rest.
+__host__ __device__ inline int producer_sel_cap(int K) {
+  int c = 512;
+  while (c < 2 * K && c < PROD_CAP) c <<= 1;
+  return c;
+}
+// Candidate slots of the merge: the records of all parts, rounded up to a power of two.
+__host__ __device__ inline int producer_merge_slots(int K, int parts) {
+  int n2 = 64;
+  while (n2 < parts * producer_record_cap(K, parts)) n2 <<= 1;
+  return n2;
+}
+__host__ __device__ inline int64_t producer_part_stride(int K, int parts) {
+  return 16 + (((int64_t)producer_record_cap(K, parts) * 8 + 15) & ~15LL);
+}
 
 // ---- order-preserving keys ---------------------------------------------------------------------
 // 16-bit storage types are handled as packed pairs of 16-bit keys, fp32 as 32-bit keys.
@@ -50,6 +76,7 @@ template <> struct Keys<TagF32> {
     return u ^ ((unsigned)((int)u >> 31) | 0x80000000u);
   }
   __device__ static __forceinline__ unsigned key(unsigned kd, int) { return kd; }
+  __device__ static __forceinline__ unsigned above(unsigned kd, unsigned lm1) { return kd > lm1 ? 1u : 0u; }
   __device__ static __forceinline__ unsigned dword_max(unsigned a, unsigned b) { return a > b ? a : b; }
   __device__ static __forceinline__ unsigned top_key(unsigned m) { return m; }
   __device__ static __forceinline__ float value(unsigned k) {
@@ -62,8 +89,13 @@ template <bool IS_BF16> struct Keys16 {
   static constexpr int BITS = 16;
   static constexpr int PER_DWORD = 2;
   __device__ static __forceinline__ unsigned encode(unsigned u) {
-    const unsigned neg = (u >> 15) & 0x00010001u;            // 1 per negative half
-    return u ^ (neg * 0x7fffu) ^ 0x80008000u;                // negative: flip all 16 bits; else flip the sign bit
+    const i16x2 neg = __builtin_bit_cast(i16x2, u) >> (short)15;              // 0xffff per negative half
+    return u ^ (__builtin_bit_cast(unsigned, neg) | 0x80008000u);             // negative: flip all 16 bits; else the sign bit
+  }
+  // nonzero iff a half of kd exceeds the matching half of lm1x2 (= (L - 1) in both halves, L >= 1)
+  __device__ static __forceinline__ unsigned above(unsigned kd, unsigned lm1x2) {
+    const u16x2 d = __builtin_elementwise_sub_sat(__builtin_bit_cast(u16x2, kd), __builtin_bit_cast(u16x2, lm1x2));
+    return __builtin_bit_cast(unsigned, d);
   }
   __device__ static __forceinline__ unsigned key(unsigned kd, int half) { return half ? (kd >> 16) : (kd & 0xffffu); }
   __device__ static __forceinline__ unsigned dword_max(unsigned a, unsigned b) {     // per 16-bit half
@@ -96,6 +128,25 @@ __device__ __forceinline__ int block_sum_int(int v, int* scratch) {
   return r;
 }
 
+// ---- candidate words -----------------------------------------------------------------------------
+// A candidate is one word that sorts ascending = key descending, column ascending.  Inside a part
+// the column needs 15 bits, so 16-bit keys give 31-bit words; fp32 keys need 64 bits.  The part
+// record and the merge use the 64-bit form (~key in the high word, row-wide column in the low).
+template <class Tag> struct Cand {
+  typedef unsigned W;
+  static constexpr W PAD = 0xffffffffu;
+  __device__ static __forceinline__ W make(unsigned k, int col) { return ((~k & 0xffffu) << 15) | (unsigned)col; }
+  __device__ static __forceinline__ u64 wide(W c, int lo) {
+    return ((u64)(0xffff0000u | (c >> 15)) << 32) | (unsigned)(lo + (int)(c & 0x7fffu));
+  }
+};
+template <> struct Cand<TagF32> {
+  typedef u64 W;
+  static constexpr W PAD = ~0ull;
+  __device__ static __forceinline__ W make(unsigned k, int col) { return ((u64)(~k) << 32) | (unsigned)col; }
+  __device__ static __forceinline__ u64 wide(W c, int lo) { return c + (unsigned)lo; }
+};
+
 // Number of entries of the part for which pred(key, column inside the part) holds.
 template <class Tag, int NT, int NCH, class Pred>
 __device__ __forceinline__ int count_entries(u32x4 (&reg)[NCH], int my_chunks, int* scratch, Pred pred) {
@@ -117,9 +168,10 @@ __device__ __forceinline__ int count_entries(u32x4 (&reg)[NCH], int my_chunks, i
   return block_sum_int<NT>(c, scratch);
 }
 
-// Appends the entries for which pred holds to cand (LDS); slots beyond PROD_CAP are counted, not written.
+// Appends the entries of chunk i for which pred holds to cand (LDS); slots beyond PROD_CAP are counted, not written.
 template <class Tag, int NT, int NCH, class Pred>
-__device__ __forceinline__ void collect_entries(const u32x4 (&reg)[NCH], int i, int lo, u64* cand, int* n_cand, Pred pred) {
+__device__ __forceinline__ void collect_entries(const u32x4 (&reg)[NCH], int i, typename Cand<Tag>::W* cand, int* n_cand,
+                                                Pred pred) {
   using KY = Keys<Tag>;
 #pragma unroll
   for (int d = 0; d < 4; ++d)
@@ -129,22 +181,87 @@ __device__ __forceinline__ void collect_entries(const u32x4 (&reg)[NCH], int i, 
       const int col = (i * NT + (int)threadIdx.x) * Chunk<Tag>::N + d * KY::PER_DWORD + h;
       if (pred(k, col)) {
         const int slot = atomicAdd(n_cand, 1);
-        if (slot < PROD_CAP) cand[slot] = ((u64)(~k) << 32) | (unsigned)(lo + col);     // ascending = key descending, id ascending
+        if (slot < PROD_CAP) cand[slot] = Cand<Tag>::make(k, col);
       }
     }
 }
 
-template <class Tag>
-__global__ __launch_bounds__(PROD_NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+__device__ __forceinline__ unsigned lane_xor(unsigned v, int m) { return (unsigned)__shfl_xor((int)v, m, WAVE); }
+__device__ __forceinline__ u64 lane_xor(u64 v, int m) {
+  const unsigned l = (unsigned)__shfl_xor((int)(unsigned)v, m, WAVE), h = (unsigned)__shfl_xor((int)(unsigned)(v >> 32), m, WAVE);
+  return ((u64)h << 32) | l;
+}
+
+// One wave sorts 64 * EPL words held in registers, element e = lane * EPL + j, ascending, with a
+// bitonic network: strides below EPL inside a lane, the others through lane exchanges.  No barriers.
+template <class W, int EPL>
+__device__ __forceinline__ void wave_sort(W (&c)[EPL]) {
+  const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+  for (int size = 2; size <= WAVE * EPL; size <<= 1) {
+#pragma unroll
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      if (stride < EPL) {
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) {
+          if ((j & stride) == 0) {
+            const bool up = ((lane * EPL + j) & size) == 0;
+            const W a = c[j], b = c[j + stride];
+            const W mn = a < b ? a : b, mx = a < b ? b : a;
+            c[j] = up ? mn : mx;
+            c[j + stride] = up ? mx : mn;
+          }
+        }
+      } else {
+        const int lm = stride / EPL;
+        const bool lower = (lane & lm) == 0;
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) {
+          const bool up = ((lane * EPL + j) & size) == 0;
+          const W o = lane_xor(c[j], lm);
+          const W mn = c[j] < o ? c[j] : o, mx = c[j] < o ? o : c[j];
+          c[j] = (lower == up) ? mn : mx;
+        }
+      }
+    }
+  }
+}
+
+// One wave sorts the n <= 64 * EPL candidate words of a part (LDS) and writes the best n_out to
+// the part record in the 64-bit form.
+template <class Tag, int EPL>
+__device__ __forceinline__ void wave_sort_emit(const typename Cand<Tag>::W* cand, int n, int n_out, int lo, u64* lst) {
+  typedef typename Cand<Tag>::W W;
+  const int lane = threadIdx.x & (WAVE - 1);
+  W c[EPL];
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const int e = lane * EPL + j;
+    c[j] = e < n ? cand[e] : Cand<Tag>::PAD;
+  }
+  wave_sort<W, EPL>(c);
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const int e = lane * EPL + j;
+    if (e < n_out) lst[e] = Cand<Tag>::wide(c[j], lo);
+  }
+}
+
+// G = chunk groups per thread whose maxima feed the threshold search: 256 * G groups per part must
+// be a few times K for the candidate set to stay close to K (4 for K <= 256, else 16).
+template <class Tag, int G>
+__global__ __launch_bounds__(PROD_NT) __attribute__((amdgpu_waves_per_eu(PROD_NT / 64, 8)))
 void topk_part_kernel(const ProducerParams p) {
-  constexpr int NT = PROD_NT, NCH = PROD_NCH, NW = NT / WAVE;
+  constexpr int NT = PROD_NT, NCH = PROD_NCH, NW = NT / WAVE, CPG = NCH / G;
   using C = Chunk<Tag>;
   using KY = Keys<Tag>;
+  typedef typename Cand<Tag>::W W;
   __shared__ float red[64];
   __shared__ int ired[NW];
   __shared__ int slots[2 * NW];
   __shared__ int s_n;
-  __shared__ __align__(16) u64 cand[PROD_CAP];
+  __shared__ unsigned s_L;
+  __shared__ __align__(16) W cand[PROD_CAP];      // before the collection: the group maxima (G == 4)
 
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), w = tid / WAVE;
@@ -159,6 +276,8 @@ void topk_part_kernel(const ProducerParams p) {
   const int Kp = min(p.K, n_elems);
   const char* rpart = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes + c0 * 16;
   char* rec = p.ws + ((int64_t)blockIdx.x) * p.part_stride;
+  // single-wave stages rotate over the waves (and so over the SIMDs) from workgroup to workgroup
+  const int select_wave = (int)(blockIdx.x & (NW - 1));
 
   u32x4 reg[NCH];
 #pragma unroll
@@ -191,43 +310,117 @@ void topk_part_kernel(const ProducerParams p) {
   }
   sm = block_sum<NT>(sm, red);
 
-  // raw bits -> ordered keys, in place; largest key of every chunk
+  // raw bits -> ordered keys, in place; largest key of every chunk group
   const int my_chunks = (nch - tid + NT - 1) / NT;                  // chunks i < my_chunks are inside the part
-  unsigned gm[NCH];
+  unsigned gm[G];
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    forget(reg[i]);
+  for (int g = 0; g < G; ++g) {
+    unsigned m = 0u;
 #pragma unroll
-    for (int d = 0; d < 4; ++d) reg[i][d] = KY::encode(reg[i][d]);
-    const unsigned m = KY::dword_max(KY::dword_max(reg[i][0], reg[i][1]), KY::dword_max(reg[i][2], reg[i][3]));
-    gm[i] = i < my_chunks ? KY::top_key(m) : 0u;
+    for (int j = 0; j < CPG; ++j) {
+      const int i = g * CPG + j;
+      forget(reg[i]);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) reg[i][d] = KY::encode(reg[i][d]);
+      const unsigned mc = KY::dword_max(KY::dword_max(reg[i][0], reg[i][1]), KY::dword_max(reg[i][2], reg[i][3]));
+      m = KY::dword_max(m, i < my_chunks ? mc : 0u);
+    }
+    gm[g] = KY::top_key(m);
   }
+  // groups that hold at least one chunk of the part: thread tid's group g starts at chunk (g * CPG) * NT + tid
+  int n_groups = 0;
+#pragma unroll
+  for (int g = 0; g < G; ++g) n_groups += max(0, min(NT, nch - g * CPG * NT));
 
-  // L = Kp-th largest chunk maximum, found bit by bit (0 when the part has fewer chunks than Kp)
+  // L = Kp-th largest group maximum, found bit by bit (0 when the part has fewer groups than Kp)
   unsigned L = 0;
-  if (nch >= Kp) {
-#pragma unroll 1
-    for (int b = KY::BITS - 1; b >= 0; --b) {
-      const unsigned t = L | (1u << b);
-      int c = 0;
+  if (n_groups >= Kp) {
+    if constexpr (G * NT == 1024) {
+      // one wave searches all 1024 maxima from its registers: no barrier per bit
+      unsigned* gms = reinterpret_cast<unsigned*>(cand);
 #pragma unroll
-      for (int i = 0; i < NCH; ++i) c += __popcll(__ballot(gm[i] >= t));
-      int* sl = slots + (b & 1) * NW;
-      if (lane == 0) sl[w] = c;
+      for (int g = 0; g < G; ++g) gms[g * NT + tid] = gm[g];
       __syncthreads();
-      int tot = 0;
+      if (w == select_wave) {
+        unsigned v[G * NW];
 #pragma unroll
-      for (int j = 0; j < NW; ++j) tot += sl[j];
-      if (tot >= Kp) L = t;
+        for (int j = 0; j < G * NW; ++j) v[j] = gms[j * WAVE + lane];
+        // the answer nearly always shares the top 6 bits of the largest key: try that prefix first
+        unsigned top = 0u;
+#pragma unroll
+        for (int j = 0; j < G * NW; ++j) top = max(top, v[j]);
+#pragma unroll
+        for (int o = WAVE / 2; o > 0; o >>= 1) top = max(top, (unsigned)__shfl_xor((int)top, o, WAVE));
+        const unsigned pre = top & ~((1u << (KY::BITS - 6)) - 1u);
+        int cpre = 0;
+#pragma unroll
+        for (int j = 0; j < G * NW; ++j) cpre += __popcll(__ballot(v[j] >= pre));
+        unsigned Lw = cpre >= Kp ? pre : 0u;
+        int b = cpre >= Kp ? KY::BITS - 7 : KY::BITS - 1;
+#pragma unroll 1
+        for (; b >= 0; --b) {
+          const unsigned t = Lw | (1u << b);
+          int c = 0;
+#pragma unroll
+          for (int j = 0; j < G * NW; ++j) c += __popcll(__ballot(v[j] >= t));
+          if (c >= Kp) Lw = t;
+        }
+        if (lane == 0) s_L = Lw;
+      }
+      __syncthreads();
+      L = s_L;
+    } else {
+#pragma unroll 1
+      for (int b = KY::BITS - 1; b >= 0; --b) {
+        const unsigned t = L | (1u << b);
+        int c = 0;
+#pragma unroll
+        for (int g = 0; g < G; ++g) c += __popcll(__ballot(gm[g] >= t));
+        int* sl = slots + (b & 1) * NW;
+        if (lane == 0) sl[w] = c;
+        __syncthreads();
+        int tot = 0;
+#pragma unroll
+        for (int j = 0; j < NW; ++j) tot += sl[j];
+        if (tot >= Kp) L = t;
+      }
+      __syncthreads();
     }
   }
-  __syncthreads();
 
-  // entries at or above L; the chunk maxima tell which chunks hold any
+  // entries at or above L; the group maxima tell which groups hold any, a packed test which dwords
+  if (L == 0) {
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    if (i < my_chunks && gm[i] >= L)
-      collect_entries<Tag, NT, NCH>(reg, i, lo, cand, &s_n, [L](unsigned k, int) { return k >= L; });
+    for (int i = 0; i < NCH; ++i) {
+      if (i < my_chunks) collect_entries<Tag, NT, NCH>(reg, i, cand, &s_n, [](unsigned, int) { return true; });
+    }
+  } else {
+    const unsigned lm1 = KY::PER_DWORD == 2 ? (L - 1) * 0x00010001u : L - 1;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      if (gm[g] >= L) {
+#pragma unroll
+        for (int j = 0; j < CPG; ++j) {
+          const int i = g * CPG + j;
+          if (i < my_chunks) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              if (KY::above(reg[i][d], lm1)) {
+#pragma unroll
+                for (int h = 0; h < KY::PER_DWORD; ++h) {
+                  const unsigned k = KY::key(reg[i][d], h);
+                  if (k >= L) {
+                    const int col = (i * NT + tid) * C::N + d * KY::PER_DWORD + h;
+                    const int slot = atomicAdd(&s_n, 1);
+                    if (slot < PROD_CAP) cand[slot] = Cand<Tag>::make(k, col);
+                  }
+                }
+              }
+            }
+          }
+        }
+      }
+    }
   }
   __syncthreads();
   int n = s_n;
@@ -254,102 +447,167 @@ void topk_part_kernel(const ProducerParams p) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       if (i < my_chunks)
-        collect_entries<Tag, NT, NCH>(reg, i, lo, cand, &s_n,
+        collect_entries<Tag, NT, NCH>(reg, i, cand, &s_n,
                                       [T, clo](unsigned k, int col) { return k > T || (k == T && col <= clo); });
     }
     __syncthreads();
     n = s_n;                                                        // == Kp
   }
 
-  // ---- sort the n >= Kp candidates, emit the best Kp -------------------------------------------
+  // ---- hand the candidates over; sort and cut to the best Kp only if the record cannot hold them all
+  const int capw = producer_record_cap(p.K, P);
+  const int n_keep = n <= capw ? n : Kp;
+  if (tid == 0) {
+    PartHeader hd{mx, sm, n_keep, 0};
+    *reinterpret_cast<PartHeader*>(rec) = hd;
+  }
   u64* lst = reinterpret_cast<u64*>(rec + 16);
-  if (n <= PROD_RANK_SORT_MAX) {
-    if (tid == 0 && (n & 1)) cand[n] = ~0ull;
-    __syncthreads();
-    const int pairs = (n + 1) / 2;
-    const ulonglong2* c2 = reinterpret_cast<const ulonglong2*>(cand);
-    for (int ai = tid; ai < n; ai += NT) {
-      const u64 a = cand[ai];
-      int rank = 0;
-#pragma unroll 4
-      for (int b = 0; b < pairs; ++b) {
-        const ulonglong2 v = c2[b];
-        rank += (v.x < a ? 1 : 0) + (v.y < a ? 1 : 0);
-      }
-      if (rank < Kp) lst[rank] = a;
-    }
+  if (n <= capw) {
+    for (int a = tid; a < n; a += NT) lst[a] = Cand<Tag>::wide(cand[a], lo);
+  } else if (n <= WAVE * 8) {
+    if (w == select_wave) wave_sort_emit<Tag, 8>(cand, n, Kp, lo, lst);
   } else {
     int n2 = 1024;
     while (n2 < n) n2 <<= 1;
-    for (int a = n + tid; a < n2; a += NT) cand[a] = ~0ull;
+    for (int a = n + tid; a < n2; a += NT) cand[a] = Cand<Tag>::PAD;
     __syncthreads();
     for (int size = 2; size <= n2; size <<= 1) {
       for (int stride = size >> 1; stride > 0; stride >>= 1) {
         for (int t = tid; t < n2 / 2; t += NT) {
           const int lo_i = 2 * t - (t & (stride - 1)), hi_i = lo_i + stride;
           const bool up = (lo_i & size) == 0;
-          const u64 a = cand[lo_i], b = cand[hi_i];
+          const W a = cand[lo_i], b = cand[hi_i];
           if ((a > b) == up) { cand[lo_i] = b; cand[hi_i] = a; }
         }
         __syncthreads();
       }
     }
-    for (int k = tid; k < Kp; k += NT) lst[k] = cand[k];
-  }
-  if (tid == 0) {
-    PartHeader hd{mx, sm, Kp, 0};
-    *reinterpret_cast<PartHeader*>(rec) = hd;
+    for (int k = tid; k < Kp; k += NT) lst[k] = Cand<Tag>::wide(cand[k], lo);
   }
 }
 
-// Merge of the parts of one row: log-sum-exp from the part statistics; every listed entry's final
-// position is its position in its own sorted list plus the number of smaller entries in the others
-// (no two entries are equal: the column is part of the sort word).
+// Emits sorted words [0, K) held as element e = lane * EPL + j of one wave.
+template <class Tag, int EPL>
+__device__ __forceinline__ void emit_sorted(const ProducerParams& p, int64_t ro, float lse, const u64 (&c)[EPL]) {
+  const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const int k = lane * EPL + j;
+    if (k < p.K) {
+      const float logp = Keys<Tag>::value(~(unsigned)(c[j] >> 32)) - lse;
+      const int col = (int)(unsigned)c[j];
+      store_from_float(p.out_val, p.out_dtype, ro * p.K + k, logp);
+      if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * p.K + k] = col;
+      else reinterpret_cast<int64_t*>(p.out_idx)[ro * p.K + k] = col;
+    }
+  }
+}
+
+// Merge of the parts of one row: log-sum-exp from the part statistics, and the K best of the parts'
+// candidates.  Words sort ascending = key descending, column ascending, and no two are equal (the
+// column is part of the word).  The K-th smallest high word (= K-th largest key) is found bit by
+// bit; the words at or below it (K plus ties) are compacted and sorted by one wave in registers.
+// More than 512 of them (a tie plateau): everything is sorted in LDS instead.
 template <class Tag>
 __global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  u64* lists = reinterpret_cast<u64*>(smem_raw);                    // parts x K
-  __shared__ int s_cnt[PROD_MAX_PARTS];
+  u64* all = reinterpret_cast<u64*>(smem_raw);                      // the parts' records; producer_merge_slots words
+  __shared__ int slots[2 * 4];
+  __shared__ int s_nsel;
   const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1), w = tid / WAVE;
   const int64_t ro = blockIdx.x;
   const int P = p.parts, K = p.K;
+  const int capw = producer_record_cap(K, P);
+  const int sel_cap = producer_sel_cap(K);
+  u64* sel = all + producer_merge_slots(K, P);                      // the selected words; sel_cap words
   const char* rec0 = p.ws + ro * P * p.part_stride;
 
   float M = -INFINITY;
   for (int q = 0; q < P; ++q) M = fmaxf(M, reinterpret_cast<const PartHeader*>(rec0 + q * p.part_stride)->mx);
   float S = 0.f;
+  int total = 0;
   for (int q = 0; q < P; ++q) {
     const PartHeader hd = *reinterpret_cast<const PartHeader*>(rec0 + q * p.part_stride);
     if (hd.mx != -INFINITY) S += hd.sm * fast_exp2((hd.mx - M) * LOG2E);
-    if (tid == 0) s_cnt[q] = hd.cnt;
+    const int cnt = min(max(hd.cnt, 0), capw);
     const u64* lst = reinterpret_cast<const u64*>(rec0 + q * p.part_stride + 16);
-    for (int j = tid; j < hd.cnt; j += 256) lists[q * K + j] = lst[j];
+    for (int j = tid; j < cnt; j += 256) all[total + j] = lst[j];
+    total += cnt;
   }
   const float lse = (M * LOG2E + fast_log2(S)) * LN2;
+  if (tid == 0) s_nsel = 0;
   __syncthreads();
 
-  for (int item = tid; item < P * K; item += 256) {
-    const int q = item / K, j = item - q * K;
-    if (j >= s_cnt[q]) continue;
-    const u64 a = lists[item];
-    int rank = j;
-    for (int o = 0; o < P; ++o) {
-      if (o == q) continue;
-      const u64* l = lists + o * K;
-      int lo = 0, hi = s_cnt[o];                                    // -> number of entries of list o below a
-      while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (l[mid] < a) lo = mid + 1; else hi = mid;
+  // U = smallest high word with at least K words at or below it; only the low Keys::BITS bits vary
+  constexpr int BITS = Keys<Tag>::BITS;
+  unsigned U = BITS == 32 ? 0u : 0xffff0000u;
+#pragma unroll 1
+  for (int b = BITS - 1; b >= 0; --b) {
+    const unsigned bound = U | ((1u << b) - 1u);                    // bit b left at zero
+    int c = 0;
+    for (int a = tid; a < total; a += 256) c += ((unsigned)(all[a] >> 32) <= bound) ? 1 : 0;
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) c += __shfl_xor(c, o, WAVE);
+    int* sl = slots + (b & 1) * 4;
+    if (lane == 0) sl[w] = c;
+    __syncthreads();
+    if (sl[0] + sl[1] + sl[2] + sl[3] < K) U |= 1u << b;
+  }
+  for (int a = tid; a < total; a += 256) {
+    const u64 v = all[a];
+    if ((unsigned)(v >> 32) <= U) {
+      const int slot = atomicAdd(&s_nsel, 1);
+      if (slot < sel_cap) sel[slot] = v;
+    }
+  }
+  __syncthreads();
+  const int n_sel = s_nsel;                                         // >= K when the parts delivered K or more
+  if (n_sel <= 256) {
+    if (w == 0) {
+      u64 c[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) c[j] = lane * 4 + j < n_sel ? sel[lane * 4 + j] : ~0ull;
+      wave_sort<u64, 4>(c);
+      emit_sorted<Tag, 4>(p, ro, lse, c);
+    }
+    return;
+  }
+  if (n_sel <= 512) {
+    if (w == 0) {
+      u64 c[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) c[j] = lane * 8 + j < n_sel ? sel[lane * 8 + j] : ~0ull;
+      wave_sort<u64, 8>(c);
+      emit_sorted<Tag, 8>(p, ro, lse, c);
+    }
+    return;
+  }
+  // LDS bitonic sort: of the selected words if they fit their list, else (a tie plateau) of everything
+  u64* arr = n_sel <= sel_cap ? sel : all;
+  const int n_arr = n_sel <= sel_cap ? n_sel : total;
+  int n2 = 64;
+  while (n2 < n_arr) n2 <<= 1;
+  for (int a = n_arr + tid; a < n2; a += 256) arr[a] = ~0ull;
+  __syncthreads();
+  for (int size = 2; size <= n2; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int t = tid; t < n2 / 2; t += 256) {
+        const int lo_i = 2 * t - (t & (stride - 1)), hi_i = lo_i + stride;
+        const bool up = (lo_i & size) == 0;
+        const u64 a = arr[lo_i], b = arr[hi_i];
+        if ((a > b) == up) { arr[lo_i] = b; arr[hi_i] = a; }
       }
-      rank += lo;
+      __syncthreads();
     }
-    if (rank < K) {
-      const float logp = Keys<Tag>::value(~(unsigned)(a >> 32)) - lse;
-      const int col = (int)(unsigned)a;
-      store_from_float(p.out_val, p.out_dtype, ro * K + rank, logp);
-      if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * K + rank] = col;
-      else reinterpret_cast<int64_t*>(p.out_idx)[ro * K + rank] = col;
-    }
+  }
+  for (int k = tid; k < K; k += 256) {
+    const u64 a = arr[k];
+    const float logp = Keys<Tag>::value(~(unsigned)(a >> 32)) - lse;
+    const int col = (int)(unsigned)a;
+    store_from_float(p.out_val, p.out_dtype, ro * K + k, logp);
+    if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * K + k] = col;
+    else reinterpret_cast<int64_t*>(p.out_idx)[ro * K + k] = col;
   }
 }
 
@@ -360,8 +618,11 @@ static int producer_parts(int64_t V, int logits_dtype) {
 
 template <class Tag>
 static int launch_producer(const ProducerParams& p, hipStream_t st) {
-  hipLaunchKernelGGL((topk_part_kernel<Tag>), dim3((unsigned)(p.n_out * p.parts)), dim3(PROD_NT), 0, st, p);
-  hipLaunchKernelGGL((topk_merge_kernel<Tag>), dim3((unsigned)p.n_out), dim3(256), (size_t)p.parts * p.K * 8, st, p);
+  const dim3 grid((unsigned)(p.n_out * p.parts));
+  if (p.K <= 256) hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_SMALL>), grid, dim3(PROD_NT), 0, st, p);
+  else hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_LARGE>), grid, dim3(PROD_NT), 0, st, p);
+  const size_t lds = (size_t)(producer_merge_slots(p.K, p.parts) + producer_sel_cap(p.K)) * 8;      // <= 48 KiB
+  hipLaunchKernelGGL((topk_merge_kernel<Tag>), dim3((unsigned)p.n_out), dim3(256), lds, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
@@ -369,7 +630,9 @@ static int launch_producer(const ProducerParams& p, hipStream_t st) {
 
 extern "C" int64_t dl_teacher_topk_workspace_bytes(int logits_dtype, int64_t n_out, int64_t V, int K) {
   if (n_out <= 0 || V <= 0 || K <= 0) return 0;
-  return n_out * dl::producer_parts(V, logits_dtype) * dl::producer_part_stride(K);
+  const int parts = dl::producer_parts(V, logits_dtype);
+  if (parts > dl::PROD_MAX_PARTS || K > dl::PROD_MAX_K || (int64_t)parts * K > 4096) return 0;
+  return n_out * parts * dl::producer_part_stride(K, parts);
 }
 
 extern "C" int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
@@ -383,7 +646,9 @@ extern "C" int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row
   if (n_rows < 0 || n_out < 0 || V <= 0 || K <= 0 || K > V || row_stride < V || (!row_list && n_out > n_rows))
     return DL_ERR_SHAPE;
   const int parts = producer_parts(V, logits_dtype);
-  if (K > PROD_MAX_K || parts > PROD_MAX_PARTS || V > 0x7fffffffLL || n_out * parts > 0x7fffffffLL) return DL_ERR_LIMIT;
+  if (K > PROD_MAX_K || parts > PROD_MAX_PARTS || (int64_t)parts * K > 4096 || V > 0x7fffffffLL ||
+      n_out * parts > 0x7fffffffLL)
+    return DL_ERR_LIMIT;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
   if (V % (16 / eb) != 0 || reinterpret_cast<uintptr_t>(logits) % 16 != 0 || (row_stride * eb) % 16 != 0)
     return DL_ERR_ALIGN;
@@ -392,7 +657,7 @@ extern "C" int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row
   if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return DL_ERR_ALIGN;
   if (workspace_bytes < dl_teacher_topk_workspace_bytes(logits_dtype, n_out, V, K)) return DL_ERR_WORKSPACE;
   ProducerParams p{logits, row_stride, V, row_list, n_out, K, parts, reinterpret_cast<char*>(workspace),
-                   producer_part_stride(K), out_val, out_dtype, out_idx, out_itype};
+                   producer_part_stride(K, parts), out_val, out_dtype, out_idx, out_itype};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   return logits_dtype == DL_F32 ? launch_producer<TagF32>(p, st)
          : logits_dtype == DL_BF16 ? launch_producer<TagBF16>(p, st)

@@ -72,6 +72,24 @@ def test_heavy_ties_and_constant_rows(D):
     assert idx[3].cpu().tolist() == list(range(K))
 
 
+@pytest.mark.parametrize("n_tied", [300, 1000, 3000])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_tie_plateaus_of_every_size(D, dtype, n_tied):
+    # a plateau of equal top values wider than K: the candidate set of a part outgrows its record
+    # (sorted and cut inside the part: in one wave, in LDS, or through the exact bisection select)
+    g = torch.Generator().manual_seed(n_tied)
+    V, K = 65536, 64
+    logits = (torch.randn(4, V, generator=g).clamp(max=3.0)).to(dtype)
+    for r in range(4):
+        pos = torch.randperm(V // 2, generator=g)[:n_tied] + (0 if r % 2 == 0 else V // 2)
+        logits[r, pos] = 5.0
+        logits[r, int(pos[0])] = 6.0
+    val, idx = D.teacher_topk(logits.to(DEV), K, val_dtype=torch.float32, idx_dtype=torch.int32)
+    rv, ri = _ref(logits, V, K)
+    assert torch.equal(idx.cpu().long(), ri)
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), atol=1e-5)
+
+
 def test_producer_limits(D):
     with pytest.raises(RuntimeError):
         D.teacher_topk(torch.zeros(2, 4096, device=DEV), 2000)
