@@ -126,7 +126,7 @@ def _wl_producer(D, S, dev, rows):
         return main()[0, 0].float()
 
     return (step, main, rows * (V * 2 + K * 6), rows,
-            f"teacher producer: log-softmax over {V} + top-{K}, {rows} rows bf16 -> fp16/int32", "topk_producer_kernel<bf16,1024,16>",
+            f"teacher producer: log-softmax over {V} + top-{K}, {rows} rows bf16 -> fp16/int32", "topk_part_kernel<bf16> (4 column parts per row) + topk_merge_kernel",
             c, torch.empty_like(c["logits"]))
 
 
