@@ -108,7 +108,8 @@ def distill_loss(model_logits: Tensor, content_rows: Tensor, teacher_logprobs: T
 
 
 def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float = 1.0,
-                       crop_to_size: int | None = None, teacher_temperature: float | None = None) -> list[dict[str, Tensor]]:
+                       crop_to_size: int | None = None, teacher_temperature: float | None = None,
+                       row_map: Tensor | None = None) -> list[dict[str, Tensor]]:
     """The per-conversation composite losses of a whole batch with ONE pass over the logits.
 
     Replaces the Python loop of classes/student/model.py:415-436 (one `calculate_divergence` call,
@@ -121,7 +122,9 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
     `convos[i]` = (content_rows int [N_i] positions inside sequence i, teacher_logprobs [N_i, K] as
     stored, indices [N_i, K], convo_CE_tokens [N_i - 1], avoid_indices).  All conversations share K.
     Returns one nine-key dict per conversation, in order; feed them to `Losses.add_losses` as the
-    reference does and call `Losses.backward` once.
+    reference does and call `Losses.backward` once.  `row_map` (int32 [B * S], from `BatchIndex`)
+    saves rebuilding the row map on the device; it is ignored if a teacher holds fewer rows than its
+    conversation has content rows.
     """
     if model_logits.dim() != 3:
         raise RuntimeError("model_logits must be [batch, seq, vocab]")
@@ -130,16 +133,14 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
         raise ValueError(f"{len(convos)} conversations for a batch of {B} sequences")
     x = model_logits if crop_to_size is None else model_logits[:, :, :crop_to_size]
     dev = x.device
-    counts = []
-    row_map = torch.full((B * S,), -1, dtype=torch.int32, device=dev)
-    idx_all, base = [], 0
-    for b, (rows, t_lp, idx, _, _) in enumerate(convos):
-        n = min(rows.numel(), t_lp.size(0), idx.size(0))
-        counts.append(n)
-        row_map[b * S + rows[:n].long()] = torch.arange(base, base + n, dtype=torch.int32, device=dev)
-        idx_all.append(idx[:n])
-        base += n
-    idx_cat = torch.cat(idx_all, dim=0)
+    counts = [min(rows.numel(), t_lp.size(0), idx.size(0)) for rows, t_lp, idx, _, _ in convos]
+    if row_map is None or row_map.numel() != B * S or any(n != rows.numel() for n, (rows, *_) in zip(counts, convos)):
+        row_map = torch.full((B * S,), -1, dtype=torch.int32, device=dev)
+        base = 0
+        for b, ((rows, *_), n) in enumerate(zip(convos, counts)):
+            row_map[b * S + rows[:n].long()] = torch.arange(base, base + n, dtype=torch.int32, device=dev)
+            base += n
+    idx_cat = torch.cat([idx[:n] for (_, _, idx, _, _), n in zip(convos, counts)], dim=0)
     lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature)
     tT = temperature if teacher_temperature is None else teacher_temperature
     out, base = [], 0
@@ -149,3 +150,17 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
         out.append(_assemble(s_sup, t, idx[:n], labels[:n], alpha, avoid))
         base += n
     return out
+
+
+def distill_loss_batch_indexed(model_logits: Tensor, index, tokens: Tensor, teachers, alpha,
+                               temperature: float = 1.0, crop_to_size: int | None = None,
+                               teacher_temperature: float | None = None) -> list[dict[str, Tensor]]:
+    """`distill_loss_batch` from a `BatchIndex` (all row / label / ignore indices of the batch built
+    and uploaded once), the batch's token ids [B, S] and `teachers[b]` = (stored log-probs [N_b, K],
+    ids [N_b, K]).  Covers classes/student/model.py:415-436 including the index construction of
+    `:87-116` and the label gather of `:423`."""
+    labels = index.labels(tokens)
+    convos = [(index.rows[b], t_lp, idx, labels[b], index.avoid[b]) for b, (t_lp, idx) in enumerate(teachers)]
+    return distill_loss_batch(model_logits, convos, alpha, temperature, crop_to_size, teacher_temperature,
+                              row_map=index.row_map)
+

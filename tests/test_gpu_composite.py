@@ -184,6 +184,7 @@ def test_batched_caller_equals_the_per_conversation_loop(D):
     x = model_logits.to(DEV).requires_grad_(True)
     L = D.Losses(None)
     dicts = D.distill_loss_batch(x, convos_gpu, 2.0, temperature=T, crop_to_size=crop)
+    values = [{k: d[k].item() for k in D.LOSS_KEYS} for d in dicts]
     for d, r in zip(dicts, ref_dicts):
         for k in D.LOSS_KEYS:
             np.testing.assert_allclose(d[k].item(), r[k].item(), rtol=2e-5, atol=2e-6, err_msg=k)
@@ -194,3 +195,19 @@ def test_batched_caller_equals_the_per_conversation_loop(D):
     err = (x.grad.cpu().double() - gref).abs()
     assert (err <= O.storage_tolerance(gref, torch.bfloat16, 2e-3)).all()
     assert torch.count_nonzero(x.grad[0, 41:]) == 0            # rows outside every content range
+    # the same batch from content ranges: every index array built on the host and uploaded once
+    x2 = model_logits.to(DEV).requires_grad_(True)
+    index = D.BatchIndex(specs, lens, S, 2048, DEV)
+    tokens_b = torch.zeros(B, S + 1, dtype=torch.long)
+    for b, (_, _, _, labels, _) in enumerate(convos_cpu):
+        tokens_b[b, torch.as_tensor(O.ce_indices(specs[b], 2048, lens[b])[0])] = labels
+    dicts2 = D.distill_loss_batch_indexed(x2, index, tokens_b.to(DEV), [(c[1], c[2]) for c in convos_gpu], 2.0,
+                                          temperature=T, crop_to_size=crop)
+    L2 = D.Losses(None)
+    for v, d2 in zip(values, dicts2):
+        for k in D.LOSS_KEYS:
+            assert v[k] == d2[k].item(), k
+        L2.add_losses(d2)
+    L2.backward(divisor=accum)
+    assert torch.equal(x.grad, x2.grad)
+
