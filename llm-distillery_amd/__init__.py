@@ -4,7 +4,7 @@ Hand-written gfx950 HIP kernels behind a C ABI (libdistill_hip.so), exposed
 through the reference's own Python boundary (`calculate_divergence`, `Losses`).
 """
 from . import _lib  # noqa: F401
-from .batch_index import BatchIndex, ce_rows, content_rows  # noqa: F401
+from .batch_index import BatchIndex, ce_rows, content_rows, teachers_from_outgoing_batch  # noqa: F401
 from .finetuning_utils import (LOSS_KEYS, calculate_divergence, distill_loss, distill_loss_batch,  # noqa: F401
                                distill_loss_batch_indexed)
 from .losses import Losses  # noqa: F401
@@ -15,4 +15,4 @@ from .ops import copy16, div_dense, div_topk, reduce_sum, rowcoef_grad_topk, row
 __all__ = ["BatchIndex", "LOSS_KEYS", "Losses", "calculate_divergence", "ce_rows", "content_rows", "copy16", "distill_loss",
            "distill_loss_batch", "distill_loss_batch_indexed", "div_dense", "div_topk", "fkl_multi_teacher",
            "merge_remap_topk", "merge_topk_pair", "reduce_sum", "rowcoef_grad_topk", "rowstats_topk", "set_option",
-           "teacher_topk", "vocab_utils"]
+           "teacher_topk", "teachers_from_outgoing_batch", "vocab_utils"]

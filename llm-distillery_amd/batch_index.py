@@ -101,3 +101,39 @@ class BatchIndex:
         """Cross-entropy labels per conversation from the batch's token ids [B, S]
         (classes/student/model.py:423: `batch_tokenized[i][CE_indices]`)."""
         return [tokens[b][pos] for b, pos in enumerate(self.label_pos)]
+
+
+def teachers_from_outgoing_batch(padded_batch: np.ndarray, batch_indices: Sequence[np.ndarray],
+                                 batch_padding: Sequence[int], device, storage: bool = True):
+    """Device-side teacher tensors from the tuple the dataset manager ships per batch
+    (`H5DataManager._make_outgoing_batch`, classes/data_manager.py:332-353): `padded_batch`
+    [B, max_len, K] log-probs zero-padded to the longest conversation, `batch_indices[b]` [N_b, K] ids,
+    `batch_padding[b]` = N_b.  Zero padding means log-prob 0, which is why the reference must slice
+    `[:batch_padding[i]]` before use (classes/student/model.py:421); here the padding never reaches
+    the device: the valid rows of all conversations are packed back to back and uploaded in two copies.
+
+    `storage=True` ships the dataset's own dtypes (fp16 log-probs — the cast back is exact because
+    that is what the file holds, classes/data_manager.py:306 — and int32 ids), a third of the
+    reference's fp32 + int64 bytes; the kernels read both layouts.
+    Returns `teachers` = [(log-probs [N_b, K], ids [N_b, K])] as views of the two packed tensors,
+    in the form `distill_loss_batch_indexed` takes."""
+    B = len(batch_padding)
+    if padded_batch.shape[0] != B or len(batch_indices) != B:
+        raise ValueError("one padding and one index array per conversation")
+    counts = [int(n) for n in batch_padding]
+    for b, n in enumerate(counts):
+        if n > padded_batch.shape[1] or batch_indices[b].shape[0] < n:
+            raise ValueError(f"conversation {b}: {n} rows announced, fewer shipped")
+    vals = np.concatenate([padded_batch[b, :n] for b, n in enumerate(counts)], axis=0)
+    ids = np.concatenate([np.asarray(batch_indices[b][:n]) for b, n in enumerate(counts)], axis=0)
+    if ids.size and (ids.min() < 0 or ids.max() > np.iinfo(np.int32).max):
+        raise ValueError("token ids outside int32")
+    vals = vals.astype(np.float16 if storage else np.float32, copy=False)
+    ids = ids.astype(np.int32 if storage else np.int64, copy=False)
+    dev = torch.device(device)
+    hv, hi = torch.from_numpy(np.ascontiguousarray(vals)), torch.from_numpy(np.ascontiguousarray(ids))
+    if dev.type == "cuda":
+        hv, hi = hv.pin_memory(), hi.pin_memory()
+    dv, di = hv.to(dev, non_blocking=True), hi.to(dev, non_blocking=True)
+    cuts = np.cumsum([0] + counts)
+    return [(dv[cuts[b]:cuts[b + 1]], di[cuts[b]:cuts[b + 1]]) for b in range(B)]

@@ -78,3 +78,21 @@ def test_batch_index_layout():
         assert lab.tolist() == (b * S + ix.label_pos[b]).tolist()
     with pytest.raises(ValueError):
         BI.BatchIndex([[(0, 70)]], [70], S, 2048, "cpu")
+
+
+def test_teachers_from_outgoing_batch_drops_the_zero_padding():
+    # the tuple classes/data_manager.py:332-353 ships: zero-padded fp32 [B, max_len, K], ids and lengths
+    rng = np.random.default_rng(0)
+    K, lens = 6, [5, 9, 1]
+    stored = [np.log(rng.random((n, K))).astype(np.float16) for n in lens]          # what the file holds
+    ids = [rng.integers(0, 50000, (n, K)).astype(np.int64) for n in lens]
+    padded = np.array([np.pad(d.astype(np.float32), ((0, max(lens) - len(d)), (0, 0))) for d in stored])
+    teachers = BI.teachers_from_outgoing_batch(padded, ids, lens, "cpu")
+    for (v, i), d, ix in zip(teachers, stored, ids):
+        assert v.dtype == torch.float16 and i.dtype == torch.int32
+        assert np.array_equal(v.numpy(), d) and np.array_equal(i.numpy(), ix)       # fp32 -> fp16 is exact here
+    wide = BI.teachers_from_outgoing_batch(padded, ids, lens, "cpu", storage=False)
+    assert wide[1][0].dtype == torch.float32 and wide[1][1].dtype == torch.int64
+    assert np.array_equal(wide[1][0].numpy(), padded[1, :9])
+    with pytest.raises(ValueError):
+        BI.teachers_from_outgoing_batch(padded, ids, [5, 10, 1], "cpu")
