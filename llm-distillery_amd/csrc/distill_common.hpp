@@ -239,6 +239,77 @@ __device__ __forceinline__ void forget(u32x4& c) {
   asm volatile("" : "+v"(c));
 }
 
+// ---- bitonic sort in registers ------------------------------------------------------------------
+__device__ __forceinline__ unsigned lane_xor(unsigned v, int m) { return (unsigned)__shfl_xor((int)v, m, WAVE); }
+__device__ __forceinline__ unsigned long long lane_xor(unsigned long long v, int m) {
+  const unsigned l = (unsigned)__shfl_xor((int)(unsigned)v, m, WAVE), h = (unsigned)__shfl_xor((int)(unsigned)(v >> 32), m, WAVE);
+  return ((unsigned long long)h << 32) | l;
+}
+
+template <class W, int EPL, int STRIDE>
+__device__ __forceinline__ void sort_stage_in_lane(W (&c)[EPL], int first, int size) {
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    if ((j & STRIDE) == 0 && j + STRIDE < EPL) {
+      const bool up = ((first + j) & size) == 0;
+      const W a = c[j], b = c[j + STRIDE];
+      const W mn = a < b ? a : b, mx = a < b ? b : a;
+      c[j] = up ? mn : mx;
+      c[j + STRIDE] = up ? mx : mn;
+    }
+  }
+}
+
+// The workgroup sorts NT * EPL words ascending; thread t holds elements t * EPL .. t * EPL + EPL - 1.
+// Strides below EPL are exchanged inside a thread, strides inside a wave through lane exchanges,
+// only the strides that cross waves through LDS (`xch`, NT * EPL words, free to reuse before and
+// after; two barriers per such stage).  Far less LDS traffic than sorting in LDS: a 1024-word sort
+// has 55 stages, of which 3 cross waves.
+template <class W, int NT, int EPL>
+__device__ __forceinline__ void block_sort(W (&c)[EPL], W* xch) {
+  static_assert(EPL == 1 || EPL == 2 || EPL == 4 || EPL == 8 || EPL == 16, "elements per thread");
+  const int tid = threadIdx.x;
+  const int first = tid * EPL;
+#pragma unroll 1
+  for (int size = 2; size <= NT * EPL; size <<= 1) {
+#pragma unroll 1
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      if (stride < EPL) {
+        switch (stride) {
+          case 1: sort_stage_in_lane<W, EPL, 1>(c, first, size); break;
+          case 2: sort_stage_in_lane<W, EPL, 2>(c, first, size); break;
+          case 4: sort_stage_in_lane<W, EPL, 4>(c, first, size); break;
+          default: sort_stage_in_lane<W, EPL, 8>(c, first, size); break;
+        }
+      } else {
+        const int tm = stride / EPL;                 // partner thread = tid ^ tm, same element slot
+        const bool lower = (tid & tm) == 0;
+        if (tm < WAVE) {
+#pragma unroll
+          for (int j = 0; j < EPL; ++j) {
+            const bool up = ((first + j) & size) == 0;
+            const W o = lane_xor(c[j], tm);
+            const W mn = c[j] < o ? c[j] : o, mx = c[j] < o ? o : c[j];
+            c[j] = (lower == up) ? mn : mx;
+          }
+        } else {
+          __syncthreads();
+#pragma unroll
+          for (int j = 0; j < EPL; ++j) xch[j * NT + tid] = c[j];
+          __syncthreads();
+#pragma unroll
+          for (int j = 0; j < EPL; ++j) {
+            const bool up = ((first + j) & size) == 0;
+            const W o = xch[j * NT + (tid ^ tm)];
+            const W mn = c[j] < o ? c[j] : o, mx = c[j] < o ? o : c[j];
+            c[j] = (lower == up) ? mn : mx;
+          }
+        }
+      }
+    }
+  }
+}
+
 // zero-fill one gradient row (masked / padded token positions)
 template <class Tag, int NT>
 __device__ __forceinline__ void zero_row(void* grad_row, int64_t nchunks) {

@@ -31,21 +31,36 @@ struct MergeParams {
   int32_t* out_idx32; int64_t* out_idx64; float* out_logm; int32_t* out_cnt; int64_t out_stride;
 };
 
-__device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, int n_pow2) {
-  for (int size = 2; size <= n_pow2; size <<= 1) {
-    for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      __syncthreads();
-      for (int t = threadIdx.x; t < n_pow2 / 2; t += MERGE_NT) {
-        const int lo = 2 * t - (t & (stride - 1));          // partner pairs (lo, lo + stride)
-        const int hi = lo + stride;
-        const bool up = (lo & size) == 0;
-        const unsigned long long a = keys[lo], b = keys[hi];
-        if ((a > b) == up) { keys[lo] = b; keys[hi] = a; }
-      }
-    }
-  }
+// Sorts keys[0, MERGE_NT * EPL) (LDS) ascending: through registers, see block_sort.
+template <class W, int EPL>
+__device__ __forceinline__ void sort_keys(W* keys) {
+  W c[EPL];
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) c[j] = keys[threadIdx.x * EPL + j];
+  block_sort<W, MERGE_NT, EPL>(c, keys);
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) keys[threadIdx.x * EPL + j] = c[j];
   __syncthreads();
 }
+
+// (id, entry) sort keys: 32-bit `id << log2(Ep) | entry` when the student vocabulary leaves room
+// (a third of the instructions of a 64-bit sort), else 64-bit `id << 32 | entry`.
+template <class W, int EPL> struct IdEntryKey;
+template <int EPL> struct IdEntryKey<unsigned, EPL> {
+  static constexpr int EBITS = __builtin_ctz(EPL * MERGE_NT);
+  static constexpr unsigned PAD = 0xffffffffu;
+  __device__ static __forceinline__ unsigned make(int64_t id, int e) { return ((unsigned)id << EBITS) | (unsigned)e; }
+  __device__ static __forceinline__ unsigned id(unsigned k) { return k >> EBITS; }
+  __device__ static __forceinline__ unsigned entry(unsigned k) { return k & ((1u << EBITS) - 1u); }
+};
+template <int EPL> struct IdEntryKey<unsigned long long, EPL> {
+  static constexpr unsigned long long PAD = ~0ull;
+  __device__ static __forceinline__ unsigned long long make(int64_t id, int e) { return ((unsigned long long)id << 32) | (unsigned)e; }
+  __device__ static __forceinline__ unsigned id(unsigned long long k) { return (unsigned)(k >> 32); }
+  __device__ static __forceinline__ unsigned entry(unsigned long long k) { return (unsigned)k; }
+};
 
 // Exclusive prefix sum over n_pow2 flags (each thread owns a contiguous run); returns the total.
 // Wave-level scans with lane shuffles, wave totals combined through LDS.
@@ -76,9 +91,13 @@ __device__ __forceinline__ int block_scan_flags(const unsigned char* flag, int* 
   return total;
 }
 
-__global__ __launch_bounds__(MERGE_NT) void merge_kernel(const MergeParams p, int E, int Ep) {
+template <int EPL, class W>
+__global__ __launch_bounds__(MERGE_NT) void merge_kernel(const MergeParams p, int E) {
+  constexpr int Ep = EPL * MERGE_NT;
+  using KY = IdEntryKey<W, EPL>;
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned long long* keys = reinterpret_cast<unsigned long long*>(smem);            // Ep
+  W* ikeys = reinterpret_cast<W*>(smem);                                              // the (id, entry) keys, same storage
   float* mass = reinterpret_cast<float*>(keys + Ep);                                  // Ep (by entry, later by slot)
   float* umass = mass + Ep;                                                           // Ep (by unique slot)
   int* uid = reinterpret_cast<int*>(umass + Ep);                                      // Ep
@@ -100,39 +119,51 @@ __global__ __launch_bounds__(MERGE_NT) void merge_kernel(const MergeParams p, in
     return;
   }
 
-  // stage: key = (id << 32 | entry), mass by entry
-  for (int e = tid; e < Ep; e += MERGE_NT) {
-    unsigned long long key = ~0ull;
-    float m = 0.f;
-    if (e < E) {
-      const int j = e / K, k = e - j * K;
-      if (r < p.rows[j]) {
-        const int64_t at = r * (int64_t)K + k;
-        int64_t id = load_index(p.idx[j], p.idx_itype, at);
-        if (p.id_map) id = (id >= 0 && id < p.Vt) ? (int64_t)p.id_map[id] : -1;
-        if (id >= 0 && id < p.Vs) {
-          m = p.weight[j] * expf(load_as_float(p.val[j], p.val_dtype, at));
-          key = ((unsigned long long)id << 32) | (unsigned)e;
-        }
-      }
-    }
-    keys[e] = key;
-    mass[e] = m;
+  // stage: key = (id << 32 | entry), mass by entry.  Three rounds of independent loads (ids and
+  // values, then the id map) instead of one dependent chain per entry.
+  int64_t id[EPL];
+  float lv[EPL], wt[EPL];
+#pragma unroll
+  for (int u = 0; u < EPL; ++u) {
+    const int e = u * MERGE_NT + tid;
+    const int j = e < E ? e / K : 0, k = e - j * K;
+    const bool live = e < E && r < p.rows[j];
+    const int64_t at = live ? r * (int64_t)K + k : 0;
+    const int64_t got = load_index(p.idx[j], p.idx_itype, at);
+    const float v = load_as_float(p.val[j], p.val_dtype, at);
+    id[u] = live ? got : -1;
+    lv[u] = v;
+    wt[u] = p.weight[j];
   }
-  bitonic_sort_u64(keys, Ep);
+  if (p.id_map) {
+#pragma unroll
+    for (int u = 0; u < EPL; ++u) {
+      const bool in = id[u] >= 0 && id[u] < p.Vt;
+      const int32_t mapped = p.id_map[in ? id[u] : 0];
+      id[u] = in ? (int64_t)mapped : -1;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < EPL; ++u) {
+    const int e = u * MERGE_NT + tid;
+    const bool keep = id[u] >= 0 && id[u] < p.Vs;
+    ikeys[e] = keep ? KY::make(id[u], e) : KY::PAD;
+    mass[e] = keep ? wt[u] * expf(lv[u]) : 0.f;
+  }
+  sort_keys<W, EPL>(ikeys);
 
   // segment heads in sorted order
   for (int i = tid; i < Ep; i += MERGE_NT) {
-    const unsigned long long k = keys[i];
-    flag[i] = (k != ~0ull && (i == 0 || (keys[i - 1] >> 32) != (k >> 32))) ? 1 : 0;
+    const W k = ikeys[i];
+    flag[i] = (k != KY::PAD && (i == 0 || KY::id(ikeys[i - 1]) != KY::id(k))) ? 1 : 0;
   }
   __syncthreads();
   const int n_unique = block_scan_flags(flag, pos, Ep, scratch);
   for (int i = tid; i < Ep; i += MERGE_NT) {
     if (flag[i]) {
-      const unsigned id = (unsigned)(keys[i] >> 32);
+      const unsigned id = KY::id(ikeys[i]);
       float m = 0.f;
-      for (int j = i; j < Ep && (unsigned)(keys[j] >> 32) == id; ++j) m += mass[(unsigned)keys[j]];   // entry order
+      for (int j = i; j < Ep && ikeys[j] != KY::PAD && KY::id(ikeys[j]) == id; ++j) m += mass[KY::entry(ikeys[j])];   // entry order
       uid[pos[i]] = (int)id;
       umass[pos[i]] = m;
     }
@@ -153,7 +184,7 @@ __global__ __launch_bounds__(MERGE_NT) void merge_kernel(const MergeParams p, in
   // top_k largest masses, descending; ties towards the smaller id
   for (int i = tid; i < Ep; i += MERGE_NT)
     keys[i] = i < n_unique ? ((unsigned long long)(~__float_as_uint(umass[i])) << 32) | (unsigned)uid[i] : ~0ull;
-  bitonic_sort_u64(keys, Ep);
+  sort_keys<unsigned long long, EPL>(keys);
   for (int u = tid; u < p.top_k; u += MERGE_NT) {
     const bool live = u < n_unique;
     const unsigned long long k = keys[u];
@@ -171,7 +202,21 @@ static int launch_merge(MergeParams& p, hipStream_t st) {
   int Ep = 256;
   while (Ep < E) Ep <<= 1;
   const size_t lds = (size_t)Ep * (8 + 4 + 4 + 4 + 4 + 1) + (MERGE_NT + 1) * 4 + 16;
-  hipLaunchKernelGGL(merge_kernel, dim3((unsigned)p.n_rows), dim3(MERGE_NT), lds, st, p, E, Ep);
+  const dim3 grid((unsigned)p.n_rows), block(MERGE_NT);
+  // 32-bit (id, entry) keys if every id plus the all-ones padding id fits beside log2(Ep) entry bits
+  const bool narrow = (uint64_t)p.Vs * (uint64_t)Ep < (1ull << 32) - (uint64_t)Ep;
+#define DL_MERGE_CASE(EPL)                                                                              \
+  if (narrow) hipLaunchKernelGGL((merge_kernel<EPL, unsigned>), grid, block, lds, st, p, E);             \
+  else hipLaunchKernelGGL((merge_kernel<EPL, unsigned long long>), grid, block, lds, st, p, E);          \
+  break;
+  switch (Ep / MERGE_NT) {
+    case 1: DL_MERGE_CASE(1)
+    case 2: DL_MERGE_CASE(2)
+    case 4: DL_MERGE_CASE(4)
+    case 8: DL_MERGE_CASE(8)
+    default: DL_MERGE_CASE(16)
+  }
+#undef DL_MERGE_CASE
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 

@@ -186,12 +186,6 @@ __device__ __forceinline__ void collect_entries(const u32x4 (&reg)[NCH], int i, 
     }
 }
 
-__device__ __forceinline__ unsigned lane_xor(unsigned v, int m) { return (unsigned)__shfl_xor((int)v, m, WAVE); }
-__device__ __forceinline__ u64 lane_xor(u64 v, int m) {
-  const unsigned l = (unsigned)__shfl_xor((int)(unsigned)v, m, WAVE), h = (unsigned)__shfl_xor((int)(unsigned)(v >> 32), m, WAVE);
-  return ((u64)h << 32) | l;
-}
-
 // One wave sorts 64 * EPL words held in registers, element e = lane * EPL + j, ascending, with a
 // bitonic network: strides below EPL inside a lane, the others through lane exchanges.  No barriers.
 template <class W, int EPL>
