@@ -35,10 +35,12 @@ def _topk_cross_entropy(logprobs: Tensor, labels: Tensor, indices: Tensor, ignor
     hit = labels.unsqueeze(-1) == indices[:stop]
     hit[ignore_rows] = False
     valid = hit.any(dim=-1)
-    picked = torch.zeros_like(valid, dtype=torch.float32)
-    picked[valid] = logprobs[:stop][hit].squeeze(-1)
-    picked[~valid] = picked[valid].mean()
-    return -picked
+    # masked sums instead of the reference's boolean-mask gathers (`picked[valid] = logprobs[hit]`,
+    # `picked[~valid] = picked[valid].mean()`): the same values, but nothing here makes the host wait
+    # for the device.  A row's ids are distinct, so at most one entry per row is hit.
+    own = torch.where(hit, logprobs[:stop], torch.zeros((), dtype=logprobs.dtype, device=logprobs.device)).sum(dim=-1)
+    mean_valid = own.sum() / valid.sum()              # no valid row: 0 / 0 = NaN, like the mean of nothing
+    return -torch.where(valid, own, mean_valid)
 
 
 def _alpha_weighted(per_token: Tensor, alpha, ce_per_token: Tensor) -> Tensor:
