@@ -5,7 +5,7 @@
 One step = one pass of the fused loss + gradient over one batch of synthetic input followed by the
 deterministic mean reduction.  The default workload is the one the headline metric is quoted on
 (C3: 8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200 fp16/int32 teacher, T=1);
-`--workload c1|c2|c4|c5|producer` measures the other configurations and the teacher producer with the
+`--workload c1|c2|c4|c5|producer|composite` measures the other configurations and the teacher producer with the
 same harness.  Inputs are
 resident in HBM before the timed region.  Prints ONE JSON line.
 """
@@ -130,7 +130,50 @@ def _wl_producer(D, S, dev, rows):
             c, torch.empty_like(c["logits"]))
 
 
-WORKLOADS = {"producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c5": _wl_c5}
+def _composite_batch(torch, S, dev, B, seq, V, K, seed=7):
+    """A batch as the reference's training loop sees it: [B, seq, V] bf16 logits, per conversation two
+    content ranges, stored fp16 / int32 teacher rows with distinct ids, labels mostly among the ids."""
+    c = S.config3(dev, rows=B * seq, seed=seed)
+    logits = c["logits"].view(B, seq, V)
+    convos = []
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    a, b = seq // 16, seq // 2
+    for i in range(B):
+        rows = torch.cat([torch.arange(a, b - a, device=dev), torch.arange(b, seq - 1, device=dev)])
+        ti = c["t_idx"].view(B, seq, K)[i][rows]
+        tv = c["t_val"].view(B, seq, K)[i][rows]
+        labels = ti[:-1, 1].long()
+        avoid = torch.tensor([b - 2 * a - 1], dtype=torch.long, device=dev)
+        convos.append((rows, tv, ti, labels, avoid))
+    return logits, convos
+
+
+def _wl_composite(D, S, dev, rows):
+    import torch
+    B, seq, V, K, T, alpha = 8, (rows // 8) if rows else 4096, 128256, 200, 1.0, 2.0
+    logits, convos = _composite_batch(torch, S, dev, B, seq, V, K)
+    x = logits.requires_grad_(True)
+    n_content = sum(c[0].numel() for c in convos)
+
+    def main():
+        x.grad = None
+        L = D.Losses(None)
+        for d in D.distill_loss_batch(x, convos, alpha, temperature=T):
+            L.add_losses(d)
+        total = L.loss_dict["train_loss"].detach()
+        L.backward(divisor=1)
+        return total
+
+    # phase 1 reads the content rows, phase 2 reads them again and writes every row of the gradient
+    algo = n_content * V * 2 * 2 + B * seq * V * 2 + n_content * K * (6 + 4 + 4 + 4)
+    return (main, main, algo, B * seq,
+            f"composite loss of the reference (calculate_divergence per conversation, Losses.backward) over a batch: "
+            f"{B} x {seq} tokens ({n_content} content) x {V} vocab bf16, K={K}, alpha={alpha}",
+            "rowstats_kernel + composite epilogue + rowcoef_grad_kernel (two-phase, whole fwd+bwd)", {"logits": logits}, x)
+
+
+WORKLOADS = {"composite": _wl_composite, "producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c5": _wl_c5}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -159,6 +202,18 @@ def cpu_baseline(workload: str, rows: int, reps: int):
         c = S.config1("cpu", B=1, S=rows) if workload == "c1" else S.config2("cpu", B=1, S=rows)
         fn = lambda: O.mean_loss_and_grad(c["kind"], c["logits"], c["T"], t_logits=c["t_logits"], valid=c["valid"])
         what = f"{rows} rows at V=32000, dense teacher"
+    elif workload == "composite":
+        seq = max(64, rows // 2)
+        logits, convos = _composite_batch(torch, S, "cpu", 2, seq, 128256, 200)
+        def fn():
+            z = O.scaled_student_logits(logits, 128256, 1.0).requires_grad_(True)
+            total = 0
+            for i, (r, tv, ti, labels, avoid) in enumerate(convos):
+                total = total + O.calculate_divergence(torch.index_select(z[i], 0, r), tv.float(), ti.long(), labels, 2.0,
+                                                       avoid)["train_loss"]
+            total.backward()
+        rows = 2 * seq
+        what = f"2 conversations x {seq} tokens at V=128256, K=200 (the reference's per-conversation loop)"
     elif workload == "producer":
         c = S.config3("cpu", rows=rows, seed=3)
         fn = lambda: O.to_storage(*[t.reshape(-1, 200) for t in O.teacher_topk_producer(c["logits"], 128256, 200)])
@@ -241,7 +296,7 @@ def main():
     kern_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
     achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
 
-    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048}[args.workload]
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048, "composite": 2048}[args.workload]
     out = {
         "metric": "tokens/sec fused KL fwd+bwd @ vocab 128256 bf16; % of HBM peak GB/s",
         "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,

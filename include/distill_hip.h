@@ -144,6 +144,41 @@ int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_strid
                          const float* coef_zk, void* grad, int64_t grad_stride, void* stream);
 
 /*
+ * The K-wide half of the composite loss for all conversations of a batch, from phase 1's outputs.
+ * Replaces utils/finetuning_utils.py:58-84 (abomination_loss, custom_ce_loss), :91 (teacher
+ * log_softmax over K), :96-110 (CE, CE diff, forward / reverse KL per token, the two weighted means
+ * and their average) and :112-122 (the nine values), and in backward the autograd replay of those
+ * lines.  Conversation c owns rows [row_off[c], row_off[c+1]) of lse / zk / t_val / t_idx, labels
+ * [label_off[c], label_off[c+1]) of `labels` (row i of the conversation carries label i; the caller
+ * guarantees #labels == #rows - 1, the only case the reference's code runs without raising) and
+ * entries [avoid_off[c], avoid_off[c+1]) of `avoid` (conversation-local rows excluded from the cross
+ * entropy; entries outside [0, #labels) are ignored).  The teacher rows are renormalised over their
+ * K entries after scaling by inv_T_teacher.
+ * out [n_convos, 9] in the reference's key order: train_loss, custom loss, CE loss, kl_div,
+ * reverse kl_div, weighted kl_div, weighted rev. kl_div, teacher CE loss, CE diff.
+ * row_records (32 bytes per row) and row_coef (16 bytes per row, may be NULL when no gradient is
+ * wanted) are caller-owned device buffers that carry the per-row state to dl_composite_backward.
+ * The gradient of max(kl) is shared evenly among tied rows, as torch.max's is.
+ */
+int dl_composite_forward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
+                         float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
+                         const int64_t* labels, const int32_t* avoid, const int32_t* row_off,
+                         const int32_t* label_off, const int32_t* avoid_off, int n_convos,
+                         int64_t n_rows, float alpha, void* row_records, void* row_coef, float* out,
+                         void* stream);
+
+/*
+ * Backward of dl_composite_forward for upstream gradients g_train [n_convos] on each conversation's
+ * train_loss: g_lse [n_rows] = dL/dlse and g_zk [n_rows, K] = dL/dzk, the inputs of
+ * dl_rowcoef_grad_topk.  Replaces the autograd replay started at classes/losses.py:77-78.
+ */
+int dl_composite_backward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
+                          float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
+                          const int32_t* row_off, int n_convos, int64_t n_rows, const void* row_records,
+                          const void* row_coef, const float* g_train, float* g_lse, float* g_zk,
+                          void* stream);
+
+/*
  * Teacher producer: per selected row, log_softmax over the V (cropped) columns, then the K largest
  * log-probs in descending order with their ids.  Replaces
  *   classes/teacher/inference_worker.py:73-80  (F.log_softmax(logits[:, :, :crop].float()) -> torch.topk)

@@ -43,6 +43,10 @@ _SIGNATURES = {
     "dl_marginalise_csr": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int64, _P, c_int64, c_int, _P]),
     "dl_rkl_marginalised": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int64, c_int64, c_int64, _P,
                                     _P, _P, c_int, c_float, c_float, c_float, _P, _P, c_int64, _P]),
+    "dl_composite_forward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, _P, _P, _P, _P, c_int, c_int64,
+                                     c_float, _P, _P, _P, _P]),
+    "dl_composite_backward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, c_int, c_int64, _P, _P, _P, _P, _P,
+                                      _P]),
     "dl_teacher_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, c_int, _P, c_int, _P, c_int, _P, c_int64, _P]),
     "dl_teacher_topk_workspace_bytes": (c_int64, [c_int, c_int64, c_int64, c_int]),
     "dl_set_option": (c_int, [c_char_p, c_int]),

@@ -65,6 +65,62 @@ def _assemble(s_sup: Tensor, t: Tensor, indices: Tensor, labels: Tensor, alpha, 
                                 ce_diff.mean())))
 
 
+def _packed_rows(tensors) -> Tensor:
+    """The row-wise concatenation of 2-D tensors; no copy when they already lie back to back in
+    memory (consecutive slices of one packed tensor, as `teachers_from_outgoing_batch` returns)."""
+    if len(tensors) == 1:
+        return tensors[0].contiguous()
+    first = tensors[0]
+    at = first.data_ptr()
+    for t in tensors:
+        if not t.is_contiguous() or t.dtype != first.dtype or t.data_ptr() != at or \
+                t.untyped_storage().data_ptr() != first.untyped_storage().data_ptr():
+            return torch.cat(tensors, dim=0)
+        at += t.numel() * t.element_size()
+    rows = sum(t.shape[0] for t in tensors)
+    return torch.as_strided(first, (rows, first.shape[1]), (first.shape[1], 1))
+
+
+def _fusable(counts, labels, alpha) -> bool:
+    """The fused epilogue covers what the reference's code can run: a Python-number alpha and, per
+    conversation, exactly one label fewer than rows (anything else raises inside the reference's
+    cross entropy or weighting, and the torch form below reproduces that)."""
+    return not isinstance(alpha, Tensor) and all(lab.dim() == 1 and lab.numel() == n - 1 for n, lab in zip(counts, labels))
+
+
+def _fused_dicts(lse: Tensor, zk: Tensor, counts, t_vals, t_idxs, labels, avoids, inv_T_teacher: float, alpha):
+    """Nine-key dicts of all conversations from one forward launch pair; `train_loss` / `custom loss`
+    carry the autograd history, the seven logged values do not (the reference's `Losses.add_losses`
+    detaches them before any use, classes/losses.py:35-37)."""
+    dev = zk.device
+    n_lab = [int(lab.numel()) for lab in labels]
+    n_avoid = [int(a.numel()) for a in avoids]
+    offs = torch.tensor([[0] + list(_cumsum(counts)), [0] + list(_cumsum(n_lab)), [0] + list(_cumsum(n_avoid))],
+                        dtype=torch.int32)
+    offs = (offs.pin_memory() if dev.type == "cuda" else offs).to(dev, non_blocking=True)
+    lab_cat = torch.cat([lab.to(torch.int64) for lab in labels]) if len(labels) > 1 else labels[0].to(torch.int64)
+    avoid_cat = torch.cat([a.to(torch.int32) for a in avoids]) if len(avoids) > 1 else avoids[0].to(torch.int32)
+    if lab_cat.numel() == 0:
+        lab_cat = torch.zeros(1, dtype=torch.int64, device=dev)
+    if avoid_cat.numel() == 0:
+        avoid_cat = torch.zeros(1, dtype=torch.int32, device=dev)
+    train, nine = ops.composite_epilogue(lse, zk, _packed_rows(t_vals), _packed_rows(t_idxs), lab_cat, avoid_cat, offs,
+                                         inv_T_teacher, alpha)
+    out = []
+    for c in range(len(counts)):
+        d = {k: nine[c, j] for j, k in enumerate(LOSS_KEYS)}
+        d["train_loss"] = d["custom loss"] = train[c]
+        out.append(d)
+    return out
+
+
+def _cumsum(values):
+    total = 0
+    for v in values:
+        total += int(v)
+        yield total
+
+
 def calculate_divergence(student_logits: Tensor, teacher_logits: Tensor, indices: Tensor | None,
                          convo_CE_tokens: Tensor, alpha, avoid_indices: Tensor) -> dict[str, Tensor]:
     """Same contract as the reference's `calculate_divergence`: `student_logits` [N, V] (already
@@ -81,9 +137,12 @@ def calculate_divergence(student_logits: Tensor, teacher_logits: Tensor, indices
     logits = student_logits[:n]
     idx = indices[:n]
     lse, zk = ops.rowstats_topk(logits, idx, None, 1.0)
+    labels = convo_CE_tokens[:n]
+    if _fusable([n], [labels], alpha) and teacher_logits.dtype in ops._DT:
+        return _fused_dicts(lse, zk, [n], [teacher_logits[:n]], [idx], [labels], [avoid_indices], 1.0, alpha)[0]
     s_sup = zk - lse.unsqueeze(-1)                       # log_softmax over V, gathered at the ids
     t = F.log_softmax(teacher_logits[:n].float(), dim=-1)
-    return _assemble(s_sup, t, idx, convo_CE_tokens[:n], alpha, avoid_indices)
+    return _assemble(s_sup, t, idx, labels, alpha, avoid_indices)
 
 
 def distill_loss(model_logits: Tensor, content_rows: Tensor, teacher_logprobs: Tensor, indices: Tensor,
@@ -103,10 +162,14 @@ def distill_loss(model_logits: Tensor, content_rows: Tensor, teacher_logprobs: T
     row_map = torch.full((S,), -1, dtype=torch.int32, device=x.device)
     row_map[content_rows[:n].long()] = torch.arange(n, dtype=torch.int32, device=x.device)
     lse, zk = ops.rowstats_topk(x, indices[:n], row_map, 1.0 / temperature)
-    s_sup = zk - lse.unsqueeze(-1)
     tT = temperature if teacher_temperature is None else teacher_temperature
+    labels = convo_CE_tokens[:n]
+    if _fusable([n], [labels], alpha) and teacher_logprobs.dtype in ops._DT:
+        return _fused_dicts(lse, zk, [n], [teacher_logprobs[:n]], [indices[:n]], [labels], [avoid_indices], 1.0 / tT,
+                            alpha)[0]
+    s_sup = zk - lse.unsqueeze(-1)
     t = F.log_softmax(teacher_logprobs[:n].float() / tT, dim=-1)
-    return _assemble(s_sup, t, indices[:n], convo_CE_tokens[:n], alpha, avoid_indices)
+    return _assemble(s_sup, t, indices[:n], labels, alpha, avoid_indices)
 
 
 def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float = 1.0,
@@ -142,9 +205,13 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
         for b, ((rows, *_), n) in enumerate(zip(convos, counts)):
             row_map[b * S + rows[:n].long()] = torch.arange(base, base + n, dtype=torch.int32, device=dev)
             base += n
-    idx_cat = torch.cat([idx[:n] for (_, _, idx, _, _), n in zip(convos, counts)], dim=0)
+    idx_cat = _packed_rows([idx[:n] for (_, _, idx, _, _), n in zip(convos, counts)])
     lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature)
     tT = temperature if teacher_temperature is None else teacher_temperature
+    labels_all = [labels[:n] for (_, _, _, labels, _), n in zip(convos, counts)]
+    if _fusable(counts, labels_all, alpha) and all(c[1].dtype in ops._DT for c in convos):
+        return _fused_dicts(lse, zk, counts, [t_lp[:n] for (_, t_lp, _, _, _), n in zip(convos, counts)],
+                            [idx_cat], labels_all, [c[4] for c in convos], 1.0 / tT, alpha)
     out, base = [], 0
     for (rows, t_lp, idx, labels, avoid), n in zip(convos, counts):
         s_sup = zk[base:base + n] - lse[base:base + n].unsqueeze(-1)

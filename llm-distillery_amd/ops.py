@@ -234,6 +234,69 @@ def _rowstats_backward(ctx, g_lse, g_zk):
 rowstats_topk.register_autograd(_rowstats_backward, setup_context=_rowstats_setup)
 
 
+class _CompositeEpilogue(torch.autograd.Function):
+    """K-wide composite loss of a batch of conversations (dl_composite_forward / _backward).
+    Returns (train_loss [C], the nine values [C, 9]); only train_loss is differentiable."""
+
+    @staticmethod
+    def forward(ctx, lse, zk, t_val, t_idx, labels, avoid, offsets, inv_T_teacher: float, alpha: float):
+        dev = zk.device
+        N, K = zk.shape
+        C = offsets.shape[1] - 1
+        need_grad = lse.requires_grad or zk.requires_grad
+        rec = torch.empty((N, 8), dtype=torch.float32, device=dev)
+        coef = torch.empty((N, 4), dtype=torch.float32, device=dev) if need_grad else None
+        out = torch.empty((C, 9), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            st = _lib.load().dl_composite_forward(
+                lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
+                _IT[t_idx.dtype], K, labels.data_ptr(), avoid.data_ptr(), offsets[0].data_ptr(), offsets[1].data_ptr(),
+                offsets[2].data_ptr(), C, N, float(alpha), rec.data_ptr(), coef.data_ptr() if need_grad else 0,
+                out.data_ptr(), _stream_ptr(dev))
+        _lib.check(st, "dl_composite_forward")
+        if need_grad:
+            ctx.save_for_backward(lse, zk, t_val, t_idx, offsets, rec, coef)
+        ctx.inv_T_teacher = inv_T_teacher
+        train = out[:, 0].contiguous()
+        ctx.mark_non_differentiable(out)
+        return train, out
+
+    @staticmethod
+    def backward(ctx, g_train, _g_logged):
+        lse, zk, t_val, t_idx, offsets, rec, coef = ctx.saved_tensors
+        dev = zk.device
+        N, K = zk.shape
+        g = g_train.to(torch.float32).contiguous()
+        g_lse = torch.empty_like(lse)
+        g_zk = torch.empty_like(zk)
+        with torch.cuda.device(dev):
+            st = _lib.load().dl_composite_backward(
+                lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], ctx.inv_T_teacher, t_idx.data_ptr(),
+                _IT[t_idx.dtype], K, offsets[0].data_ptr(), offsets.shape[1] - 1, N, rec.data_ptr(), coef.data_ptr(),
+                g.data_ptr(), g_lse.data_ptr(), g_zk.data_ptr(), _stream_ptr(dev))
+        _lib.check(st, "dl_composite_backward")
+        return g_lse, g_zk, None, None, None, None, None, None, None
+
+
+def composite_epilogue(lse: torch.Tensor, zk: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor,
+                       labels: torch.Tensor, avoid: torch.Tensor, offsets: torch.Tensor, inv_T_teacher: float,
+                       alpha: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(train_loss [C], nine values [C, 9]) of C conversations from phase 1's `lse` [N] / `zk` [N, K],
+    the stored teacher rows `t_val` / `t_idx` [N, K], the concatenated int64 `labels` and int32
+    `avoid` rows, and `offsets` int32 [3, C + 1] (first row, first label, first avoid entry of every
+    conversation).  See dl_composite_forward."""
+    _dev(zk, "zk")
+    if lse.dtype != torch.float32 or zk.dtype != torch.float32 or not (lse.is_contiguous() and zk.is_contiguous()):
+        raise RuntimeError("lse / zk must be contiguous fp32 (phase 1's outputs)")
+    if t_val.dtype not in _DT or t_idx.dtype not in _IT or labels.dtype != torch.int64 or avoid.dtype != torch.int32 \
+            or offsets.dtype != torch.int32:
+        raise RuntimeError("unsupported dtype")
+    if t_val.shape != zk.shape or t_idx.shape != zk.shape or offsets.dim() != 2 or offsets.shape[0] != 3:
+        raise RuntimeError("shape mismatch")
+    return _CompositeEpilogue.apply(lse, zk, t_val.contiguous(), t_idx.contiguous(), labels.contiguous(),
+                                    avoid.contiguous(), offsets.contiguous(), float(inv_T_teacher), float(alpha))
+
+
 def reduce_sum(values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
     """Deterministic sum(values) * scale as a 0-d fp32 tensor."""
     _dev(values, "values")

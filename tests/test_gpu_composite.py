@@ -211,3 +211,70 @@ def test_batched_caller_equals_the_per_conversation_loop(D):
     L2.backward(divisor=accum)
     assert torch.equal(x.grad, x2.grad)
 
+
+
+def _ranged_convo(g, S, V, K, ranges, convo_len, label_hits=0.8):
+    """One conversation's pieces (CPU): content rows, stored teacher rows, labels, ignore rows."""
+    rows = torch.as_tensor(O.content_indices(ranges))
+    lab_pos, avoid = O.ce_indices(ranges, 2048, convo_len)
+    N = rows.numel()
+    ti = torch.stack([torch.randperm(V, generator=g)[:K] for _ in range(N)])
+    tv = torch.log_softmax(torch.randn(N, K, generator=g) * 2, -1).to(torch.float16)
+    labels = torch.where(torch.rand(len(lab_pos), generator=g) < label_hits, ti[:len(lab_pos), 3],
+                         torch.full((len(lab_pos),), V + 7))          # a label outside the row's ids: invalid row
+    return rows, tv, ti, labels, torch.as_tensor(avoid)
+
+
+@pytest.mark.parametrize("alpha", [2.0, 0.7])
+def test_fused_epilogue_equals_the_torch_epilogue(D, alpha):
+    """The fused K-wide epilogue (three launches per batch) against the same arithmetic written with
+    the torch routines the reference uses (taken when alpha is a tensor): all nine values per
+    conversation and the gradient of the logits, including an all-invalid conversation (NaN cross
+    entropies, as in the reference) and tied maxima (duplicated rows: max's gradient is shared)."""
+    g = torch.Generator().manual_seed(21)
+    B, S, V, K, T = 4, 48, 2048, 16, 1.7
+    specs = [[(2, 20), (25, 40)], [(0, 33)], [(5, 9), (12, 30), (31, 44)], [(1, 30)]]
+    lens = [40, 33, 44, 30]
+    convos = [_ranged_convo(g, S, V, K, specs[b], lens[b], label_hits=0.0 if b == 3 else 0.8) for b in range(B)]
+    logits = torch.randn(B, S, V, generator=g) * 2                # fp32: the gradients compare unrounded
+    logits[1, 7] = logits[1, 3]                                   # two identical rows ...
+    r, tv, ti, lab, av = convos[1]
+    tv[7], ti[7] = tv[3], ti[3]                                   # ... with identical teachers: tied kl and rkl
+    dev_convos = [tuple(t.to(DEV) for t in c) for c in convos]
+
+    def run(a):
+        x = logits.to(DEV).requires_grad_(True)
+        dicts = D.distill_loss_batch(x, dev_convos, a, temperature=T)
+        vals = [{k: d[k].item() for k in D.LOSS_KEYS} for d in dicts]
+        total = sum(d["train_loss"] for d in dicts[:3])          # conversation 3 is NaN by construction
+        total.backward()
+        return vals, x.grad, dicts
+
+    fused, g_fused, dicts = run(alpha)
+    plain, g_plain, _ = run(torch.tensor(alpha, device=DEV))      # a tensor alpha takes the torch epilogue
+    assert dicts[0]["train_loss"].requires_grad and not dicts[0]["kl_div"].requires_grad
+    assert type(dicts[0]["train_loss"].grad_fn).__name__ == "SelectBackward0"
+    for b in range(B):
+        for k in D.LOSS_KEYS:
+            if b == 3 and k not in ("kl_div", "reverse kl_div"):
+                assert np.isnan(fused[b][k]) and np.isnan(plain[b][k]), k
+            else:
+                np.testing.assert_allclose(fused[b][k], plain[b][k], rtol=3e-6, atol=1e-7, err_msg=f"{b} {k}")
+    err = (g_fused.float() - g_plain.float()).abs()
+    bound = O.storage_tolerance(g_plain.double().cpu(), torch.float32, 1e-4).to(DEV)
+    assert (err <= bound).all(), float((err / bound).max())
+    assert torch.count_nonzero(g_fused[3]) == 0
+
+
+def test_fused_epilogue_under_no_grad_and_label_count_mismatch(D):
+    g = torch.Generator().manual_seed(5)
+    rows, tv, ti, labels, avoid = _ranged_convo(g, 40, 1024, 8, [(3, 19)], 19)
+    z = (torch.randn(rows.numel(), 1024, generator=g)).to(DEV)
+    with torch.no_grad():
+        d = D.calculate_divergence(z, tv.float().to(DEV), ti.to(DEV), labels.to(DEV), 2.0, avoid.to(DEV))
+    ref = O.calculate_divergence(z.cpu().double(), tv.double(), ti, labels, 2.0, avoid)
+    for k in D.LOSS_KEYS:
+        np.testing.assert_allclose(d[k].item(), ref[k].item(), rtol=2e-5, atol=2e-6, err_msg=k)
+    # as many labels as rows: the reference raises (empty crop); so does the drop-in, from the same torch ops
+    with pytest.raises(RuntimeError):
+        D.calculate_divergence(z, tv.float().to(DEV), ti.to(DEV), torch.cat([labels, labels[:1]]).to(DEV), 2.0, avoid.to(DEV))
