@@ -76,7 +76,8 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
 // ---- phase 2 -------------------------------------------------------------------------------
 // One workgroup per (row, column part of NT*NCH chunks).
 template <class Tag, int NT, int NCH, bool VEC>
-__global__ __launch_bounds__(NT) void rowcoef_grad_kernel(const StatsParams p, int parts) {
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+void rowcoef_grad_kernel(const StatsParams p, int parts) {
   extern __shared__ __align__(16) unsigned char smem[];
   using C = Chunk<Tag>;
   const int Kp = (p.K + 15) & ~15;
@@ -132,11 +133,21 @@ __global__ __launch_bounds__(NT) void rowcoef_grad_kernel(const StatsParams p, i
       store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * w);
   }
   __syncthreads();          // LDS entries staged; dense stores ordered before the sparse additions
+  const int4* ids4 = reinterpret_cast<const int4*>(s_idx);
   for (int k = tid; k < Kp; k += NT) {
     const int id = s_idx[k];
     if (id < 0) continue;
-    float cs = 0.f;           // every entry with this id contributes; all of them write the same total
-    for (int j = 0; j < Kp; ++j) cs += (s_idx[j] == id) ? s_c[j] : 0.f;
+    int same = 0;             // ids of a row may repeat: every entry with this id contributes, all write the same total
+#pragma unroll 4
+    for (int j = 0; j < Kp / 4; ++j) {
+      const int4 q = ids4[j];
+      same += (q.x == id) + (q.y == id) + (q.z == id) + (q.w == id);
+    }
+    float cs = s_c[k];
+    if (same != 1) {
+      cs = 0.f;
+      for (int j = 0; j < Kp; ++j) cs += (s_idx[j] == id) ? s_c[j] : 0.f;
+    }
     const float dense = fast_exp2(fmaf(load_as_float(row, Tag::id, id), a, -b)) * w;
     store_from_float(grow, Tag::id, id, dense + cs * p.inv_T);
   }
@@ -155,7 +166,7 @@ static hipError_t launch_stats(const StatsParams& p, bool vec, hipStream_t st) {
 
 template <class Tag>
 static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
-  constexpr int NT = 256, NCH = 8;
+  constexpr int NT = 256, NCH = 16;
   const int64_t per_part = (int64_t)NT * NCH * Tag::epc;
   const int parts = (int)((p.V + per_part - 1) / per_part);
   const size_t lds = (size_t)((p.K + 15) & ~15) * 8;
