@@ -84,6 +84,8 @@ int dl_set_option(const char* name, int value);
  *            torch.topk and of dl_merge_remap_topk); the kernel then skips its duplicate scan.  With
  *            the flag set and duplicates present, the gradient at a duplicated id is wrong.
  * K <= DL_MAX_TOPK.
+ * With n_teacher_rows == 0 the teacher pointers may be NULL: every row then counts as masked
+ * (the same holds for dl_div_dense, dl_rowstats_topk and dl_rowcoef_grad_topk).
  */
 int dl_div_topk(int kind,
                 const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,

@@ -147,7 +147,7 @@ extern "C" int dl_div_dense(int kind, const void* logits, int logits_dtype, int6
                             int64_t n_teacher_rows, float inv_T_student, float inv_T_teacher, float grad_scale,
                             float* row_loss, void* grad, int64_t grad_stride, void* stream) {
   using namespace dl;
-  if (!logits || !t_logits) return DL_ERR_NULL;
+  if (!logits || (!t_logits && n_teacher_rows > 0)) return DL_ERR_NULL;      // no teacher rows: every row is masked
   if (kind < DL_FKL || kind > DL_JSD || logits_dtype < DL_F32 || logits_dtype > DL_F16 || t_dtype < DL_F32 ||
       t_dtype > DL_F16)
     return DL_ERR_DTYPE;

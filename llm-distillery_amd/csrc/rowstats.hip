@@ -178,7 +178,7 @@ static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
 
 static int check_common(const void* logits, int dtype, int64_t row_stride, int64_t n_rows, int64_t V,
                         const void* t_idx, int itype, int K, int64_t n_trows) {
-  if (!logits || !t_idx) return DL_ERR_NULL;
+  if (!logits || (!t_idx && n_trows > 0)) return DL_ERR_NULL;      // no teacher rows: every row is masked
   if (dtype < DL_F32 || dtype > DL_F16 || (itype != DL_I32 && itype != DL_I64)) return DL_ERR_DTYPE;
   if (n_rows < 0 || V <= 0 || K <= 0 || n_trows < 0 || row_stride < V) return DL_ERR_SHAPE;
   if (K > DL_MAX_TOPK || V > 0x7fffffffLL || n_rows > 0x7fffffffLL) return DL_ERR_LIMIT;
@@ -193,7 +193,7 @@ extern "C" int dl_rowstats_topk(const void* logits, int logits_dtype, int64_t ro
   using namespace dl;
   const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_teacher_rows);
   if (rc != DL_OK) return rc;
-  if (!lse || !zk) return DL_ERR_NULL;
+  if ((!lse || !zk) && n_teacher_rows > 0) return DL_ERR_NULL;
   if (n_rows == 0) return DL_OK;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
   const bool vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb);
@@ -213,7 +213,7 @@ extern "C" int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_
   using namespace dl;
   const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_teacher_rows);
   if (rc != DL_OK) return rc;
-  if (!lse || !coef_lse || !coef_zk || !grad) return DL_ERR_NULL;
+  if (((!lse || !coef_lse || !coef_zk) && n_teacher_rows > 0) || !grad) return DL_ERR_NULL;
   if (grad_stride < V) return DL_ERR_SHAPE;
   if (n_rows == 0) return DL_OK;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;

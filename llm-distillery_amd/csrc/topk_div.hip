@@ -636,7 +636,7 @@ extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64
                            void* grad, int64_t grad_stride, void* workspace, int64_t workspace_bytes, int flags,
                            void* stream) {
   using namespace dl;
-  if (!logits || !t_val || !t_idx) return DL_ERR_NULL;
+  if (!logits || ((!t_val || !t_idx) && n_teacher_rows > 0)) return DL_ERR_NULL;      // no teacher rows: every row is masked
   if (kind != DL_FKL && kind != DL_RKL) return DL_ERR_DTYPE;
   if (logits_dtype < DL_F32 || logits_dtype > DL_F16 || t_val_dtype < DL_F32 || t_val_dtype > DL_F16 ||
       (t_idx_itype != DL_I32 && t_idx_itype != DL_I64))

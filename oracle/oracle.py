@@ -389,13 +389,15 @@ def merge_dense_pair(disk_logp: np.ndarray, new_logp: np.ndarray) -> np.ndarray:
 
 def merge_remap_rows(vals: Sequence[np.ndarray], idxs: Sequence[np.ndarray],
                      weights: Sequence[float], id_map: np.ndarray | None,
-                     T: float = 1.0):
+                     T: float = 1.0, n_student: int | None = None):
     """Weighted sum of several top-K teachers after mapping their ids.
 
     Parity unpinned (no reference counterpart; generalises
     classes/data_manager.py:231-240 with weights and an id map).  Per row:
     mass_e = w_teacher * exp(logp_e) in fp32; the id goes through `id_map`
-    (teacher id -> student id, -1 = dropped, its mass is removed); entries that
+    (teacher id -> student id, -1 = dropped, its mass is removed; ids outside
+    the map, and student ids outside [0, n_student) when that is given, are
+    dropped as well); entries that
     land on the same student id are summed in entry order (teacher 0's entries
     first); the surviving ids are listed in ascending order; the teacher
     distribution is log_softmax(log(mass) / T) over the survivors.
@@ -411,8 +413,11 @@ def merge_remap_rows(vals: Sequence[np.ndarray], idxs: Sequence[np.ndarray],
             m = (np.float32(w) * np.exp(np.asarray(v[r], dtype=np.float32))).astype(np.float32)
             for e in range(m.shape[0]):
                 tid = int(ix[r][e])
-                sid = tid if id_map is None else int(id_map[tid])
-                if sid < 0:
+                if id_map is None:
+                    sid = tid
+                else:
+                    sid = int(id_map[tid]) if 0 <= tid < len(id_map) else -1      # outside the teacher vocabulary: dropped
+                if sid < 0 or (n_student is not None and sid >= n_student):
                     continue
                 acc[sid] = np.float32(acc.get(sid, np.float32(0.0)) + m[e])
         ids = np.asarray(sorted(acc), dtype=np.int32)
@@ -426,10 +431,10 @@ def merge_remap_rows(vals: Sequence[np.ndarray], idxs: Sequence[np.ndarray],
     return out
 
 
-def merge_remap_padded(vals, idxs, weights, id_map, T: float = 1.0):
+def merge_remap_padded(vals, idxs, weights, id_map, T: float = 1.0, n_student: int | None = None):
     """`merge_remap_rows` packed into padded arrays: ids int32 [N,E] (pad -1),
     logq fp32 [N,E] (pad -inf), count int32 [N]; E = total entries per row."""
-    rows = merge_remap_rows(vals, idxs, weights, id_map, T)
+    rows = merge_remap_rows(vals, idxs, weights, id_map, T, n_student)
     E = sum(v.shape[1] for v in vals)
     N = len(rows)
     ids = np.full((N, E), -1, dtype=np.int32)
