@@ -255,21 +255,27 @@ int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_student, in
 /*
  * Marginalisation plan (HOST function, HOST pointers; no reference counterpart): re-lays a
  * teacher->student map for the planned kernels, which add every marginal in a fixed order without
- * atomics.  Student id s is owned by thread s % 1024 of a 1024-thread workgroup; the teacher
- * vocabulary is cut into tiles of *tile_out ids; for tile k and wave w, rows
+ * atomics: every accumulator word in LDS belongs to one thread of a 1024-thread workgroup.  Slot s
+ * (< n_student) accumulates student id s; ids with far more than an even share of the teacher ids
+ * get replica slots (n_student rounded up to 4, + j), *n_extra_out in all, folded into the id's
+ * slot after the last tile as listed in `fold` (int32 triples: id, first replica slot, replica
+ * count).  The teacher vocabulary is cut into tiles of *tile_out ids; for tile k and wave w, rows
  * row_off[16k + w] .. row_off[16k + w + 1] of `ent` hold 64 entries each (one per lane,
- * 0xffffffff = padding): (s << log2(tile) | t - k * tile), per thread sorted by (s, t).
- * Call once with row_off = ent = NULL to learn *tile_out and *ent_rows_out, allocate
- * row_off int32 [16 * ceil(n_teacher / tile) + 1] and ent uint32 [64 * ent_rows], call again.
+ * 0xffffffff = padding): (slot << log2(tile) | t - k * tile), per thread sorted by (slot, t).
+ * Call once with row_off = ent = fold = NULL to learn *tile_out, *ent_rows_out, *n_fold_out and
+ * *n_extra_out, allocate row_off int32 [16 * ceil(n_teacher / tile) + 1], ent uint32
+ * [64 * ent_rows] and fold int32 [3 * n_fold], call again.
  * DL_ERR_LIMIT: the student vocabulary is too wide for a plan (fp32 marginal + 16 KiB tile must fit 159 KiB).
  */
 int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int* tile_out,
-                           int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity, int64_t* ent_rows_out);
+                           int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity, int64_t* ent_rows_out,
+                           int32_t* fold, int64_t fold_capacity, int64_t* n_fold_out, int* n_extra_out);
 
 /*
  * marg[r, s] = sum of probs[r, t] over the teacher ids t with t2s[t] == s (probs [n_rows, Vt] in
  * p_dtype, marg fp32 [n_rows, Vs]; out_log != 0 stores log(marg) instead).  With a plan
- * (plan_row_off / plan_ent device copies of dl_marginal_plan_build's arrays, plan_tile its tile;
+ * (plan_row_off / plan_ent / plan_fold device copies of dl_marginal_plan_build's arrays, plan_tile,
+ * plan_n_fold and plan_n_extra its tile, fold count and replica count;
  * fp32 probabilities, 16-byte aligned rows) every sum is added in a fixed order: bit-reproducible.
  * Without (NULL, NULL, 0) it accumulates with LDS floating-point atomics: sums then agree to fp32
  * rounding, not bit for bit.
@@ -277,6 +283,7 @@ int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_stud
 int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
                        const int32_t* t2s, int64_t Vs,
                        const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                       const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
                        float* marg, int64_t marg_stride, int out_log, void* stream);
 
 /* The same marginal from the CSR form, each segment added in ascending teacher-id order (bit-reproducible). */
@@ -297,6 +304,7 @@ int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride
                         const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
                         int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s,
                         const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                        const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
                         float inv_T_student, float inv_T_teacher, float grad_scale,
                         float* row_loss, void* grad, int64_t grad_stride, void* stream);
 

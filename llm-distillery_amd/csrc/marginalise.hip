@@ -35,7 +35,13 @@ struct MargParams {
   float inv_T_s, inv_T_t, grad_scale; float* row_loss; void* grad; int64_t grad_stride;
   // plan (all NULL/0: accumulate with LDS atomics along t2s instead)
   const int32_t* plan_row_off; const uint32_t* plan_ent; int plan_tile; int plan_tile_bits;
+  const int32_t* plan_fold; int plan_n_fold; int plan_n_extra;       // replica slots behind the marginal and how they fold
 };
+
+// LDS words of the planned form before the tile: the marginal and the replica slots, both padded to 16 bytes
+__host__ __device__ inline int64_t plan_slot_words(int64_t Vs, int n_extra) {
+  return ((Vs + 3) & ~(int64_t)3) + (((int64_t)n_extra + 3) & ~(int64_t)3);
+}
 
 constexpr unsigned PLAN_PAD = 0xffffffffu;
 
@@ -108,7 +114,8 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
   const int64_t n4 = p.Vt / 4;
   const int bits = p.plan_tile_bits;
   const unsigned tmask = (1u << bits) - 1u;
-  for (int j = tid; j < p.Vs; j += MARG_NT) marg[j] = 0.f;
+  const int n_slots = (int)plan_slot_words(p.Vs, p.plan_n_extra);
+  for (int j = tid; j < n_slots; j += MARG_NT) marg[j] = 0.f;
   u32x4 tbuf[PLAN_DEPTH][2];
   auto fetch_tile = [&](int k, u32x4 (&buf)[2]) {
 #pragma unroll
@@ -162,6 +169,14 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
     if (k + 1 < ntiles) do_tile(k + 1, tbuf[1], eb, ea);
     if (k + 2 < ntiles) do_tile(k + 2, tbuf[2], ea, eb);
     if (k + 3 < ntiles) do_tile(k + 3, tbuf[3], eb, ea);
+  }
+  __syncthreads();
+  // replicas into their id's slot: own slot first, then the replicas in ascending order
+  for (int f = tid; f < p.plan_n_fold; f += MARG_NT) {
+    const int sid = p.plan_fold[3 * f], first = p.plan_fold[3 * f + 1], cnt = p.plan_fold[3 * f + 2];
+    float a = marg[sid];
+    for (int j = 0; j < cnt; ++j) a += marg[first + j];
+    marg[sid] = a;
   }
   __syncthreads();
 }
@@ -233,7 +248,7 @@ __global__ __launch_bounds__(MARG_NT) void marginalise_map_kernel(const MargPara
   const char* prow = reinterpret_cast<const char*>(p.probs) + r * p.p_stride * pb;
   float* out = p.marg + r * p.marg_stride;
   if (VEC && p.plan_ent) {
-    accumulate_marginal_planned(p, prow, acc, acc + ((p.Vs + 3) & ~(int64_t)3));
+    accumulate_marginal_planned(p, prow, acc, acc + plan_slot_words(p.Vs, p.plan_n_extra));
     for (int j = threadIdx.x; j < p.Vs; j += MARG_NT) out[j] = p.out_log ? logf(acc[j]) : acc[j];
     return;
   }
@@ -311,7 +326,7 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
   const int pb = p.p_dtype == F32 ? 4 : 2;
   const char* prow = reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb;
   if (VEC && p.plan_ent) {
-    accumulate_marginal_planned(p, prow, acc, acc + ((p.Vs + 3) & ~(int64_t)3));   // needs the registers itself
+    accumulate_marginal_planned(p, prow, acc, acc + plan_slot_words(p.Vs, p.plan_n_extra));   // needs the registers itself
     rows.load(srow, p.Vs / 8);
   } else {
     rows.load(srow, p.Vs / 8);                   // in flight during the scatter
@@ -359,20 +374,23 @@ static void allow_large_lds() {
 }  // namespace dl
 
 // Fills the plan fields of `p` if a usable plan is given; returns the dynamic LDS bytes to request.
-static size_t attach_plan(dl::MargParams& p, const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile, bool vec,
-                          size_t lds_without_plan) {
+static size_t attach_plan(dl::MargParams& p, const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                          const int32_t* plan_fold, int plan_n_fold, int plan_n_extra, bool vec, size_t lds_without_plan) {
   if (!plan_row_off || !plan_ent || !vec) return lds_without_plan;
   if (plan_tile != 4096 && plan_tile != 8192) return lds_without_plan;
-  const size_t need = (size_t)((p.Vs + 3) & ~(int64_t)3) * 4 + (size_t)plan_tile * 4;
+  if (plan_n_fold < 0 || plan_n_extra < 0 || (plan_n_fold > 0 && !plan_fold)) return lds_without_plan;
+  const size_t need = (size_t)dl::plan_slot_words(p.Vs, plan_n_extra) * 4 + (size_t)plan_tile * 4;
   if (need > (size_t)dl::MARG_MAX_DYN_LDS) return lds_without_plan;
   p.plan_row_off = plan_row_off; p.plan_ent = plan_ent; p.plan_tile = plan_tile;
   p.plan_tile_bits = plan_tile == 4096 ? 12 : 13;
+  p.plan_fold = plan_fold; p.plan_n_fold = plan_n_fold; p.plan_n_extra = plan_n_extra;
   return need;
 }
 
 extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
                                   const int32_t* t2s, int64_t Vs, const int32_t* plan_row_off,
-                                  const uint32_t* plan_ent, int plan_tile, float* marg, int64_t marg_stride,
+                                  const uint32_t* plan_ent, int plan_tile, const int32_t* plan_fold, int plan_n_fold,
+                                  int plan_n_extra, float* marg, int64_t marg_stride,
                                   int out_log, void* stream) {
   using namespace dl;
   if (!probs || !t2s || !marg) return DL_ERR_NULL;
@@ -384,7 +402,8 @@ extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stri
   p.probs = probs; p.p_dtype = p_dtype; p.p_stride = p_stride; p.n_rows = n_rows; p.Vt = Vt; p.t2s = t2s; p.Vs = Vs;
   p.marg = marg; p.marg_stride = marg_stride; p.out_log = out_log;
   const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(probs, p_stride, 4) && ok16(t2s, 0, 4);
-  const size_t lds = attach_plan(p, plan_row_off, plan_ent, plan_tile, vec, (size_t)(Vs < MARG_MAX_VS ? Vs : MARG_MAX_VS) * 4);
+  const size_t lds = attach_plan(p, plan_row_off, plan_ent, plan_tile, plan_fold, plan_n_fold, plan_n_extra, vec,
+                                 (size_t)(Vs < MARG_MAX_VS ? Vs : MARG_MAX_VS) * 4);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   allow_large_lds();
   if (vec) hipLaunchKernelGGL((marginalise_map_kernel<true>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
@@ -415,6 +434,7 @@ extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t
                                    const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
                                    int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s,
                                    const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                                   const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
                                    float inv_T_student, float inv_T_teacher, float grad_scale, float* row_loss,
                                    void* grad, int64_t grad_stride, void* stream) {
   using namespace dl;
@@ -433,7 +453,7 @@ extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t
   p.row_map = row_map; p.inv_T_s = inv_T_student; p.inv_T_t = inv_T_teacher; p.grad_scale = grad_scale;
   p.row_loss = row_loss; p.grad = grad; p.grad_stride = grad_stride;
   const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(t_probs, p_stride, 4) && ok16(t2s, 0, 4);
-  const size_t lds = attach_plan(p, plan_row_off, plan_ent, plan_tile, vec, (size_t)Vs * 4);
+  const size_t lds = attach_plan(p, plan_row_off, plan_ent, plan_tile, plan_fold, plan_n_fold, plan_n_extra, vec, (size_t)Vs * 4);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)n_rows), block(MARG_NT);
   allow_large_lds();

@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cstring>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 namespace {
@@ -105,28 +106,108 @@ extern "C" int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_
 }
 
 // ---- marginalisation plan --------------------------------------------------------------------
-// Layout consumed by the planned marginalisation kernels (1024 threads = 16 waves per workgroup):
-// the teacher vocabulary is cut into tiles of `tile` ids; student id s is owned by thread s % 1024;
-// for tile k and wave w, rows row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries
-// per row (one per lane, 0xffffffff = padding), the entries (s << log2(tile) | t - k*tile) of the
-// wave's threads, each thread's entries sorted by (s, t).
+// Layout consumed by the planned marginalisation kernels (1024 threads = 16 waves per workgroup).
+// Every accumulator word in LDS is touched by one thread only, so no atomics are needed and the
+// summation order is fixed.  Accumulator slots: slot s < n_student is student id s; a student id
+// that receives far more teacher ids than an even share (real vocabularies: the single-byte and
+// other short tokens) gets extra slots n_student_padded + j ("replicas") so that its load can be
+// split over several threads; after the last tile the replicas are folded into their id's slot in
+// a fixed order (fold table: triples id, first replica slot, replica count).  Slots are dealt to
+// threads by descending load onto the least-loaded thread; inside a tile an entry of a replicated
+// id goes to the replica whose owner holds the fewest entries of that tile so far.
+// The teacher vocabulary is cut into tiles of `tile` ids; for tile k and wave w, rows
+// row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries per row (one per lane,
+// 0xffffffff = padding), the entries (slot << log2(tile) | t - k*tile) of the wave's threads, each
+// thread's entries sorted by (slot, t).
 extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int* tile_out,
                                       int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity,
-                                      int64_t* ent_rows_out) {
+                                      int64_t* ent_rows_out, int32_t* fold, int64_t fold_capacity,
+                                      int64_t* n_fold_out, int* n_extra_out) {
   constexpr int NT = 1024, WAVE = 64, NW = NT / WAVE;
   constexpr int64_t LDS_BUDGET = 160 * 1024 - 1024;      // dynamic LDS one workgroup may use
-  if (!t2s || !tile_out || !ent_rows_out) return DL_ERR_NULL;
+  if (!t2s || !tile_out || !ent_rows_out || !n_fold_out || !n_extra_out) return DL_ERR_NULL;
   if (n_teacher <= 0 || n_student <= 0) return DL_ERR_SHAPE;
   if (n_teacher > 0x7fffffffLL) return DL_ERR_LIMIT;
-  const int64_t marg_bytes = ((n_student + 3) & ~(int64_t)3) * 4;
+  const int64_t n_pad = (n_student + 3) & ~(int64_t)3;
+  const int64_t marg_bytes = n_pad * 4;
   int tile = 8192;
   while (tile >= 4096 && marg_bytes + (int64_t)tile * 4 > LDS_BUDGET) tile >>= 1;
   if (tile < 4096) return DL_ERR_LIMIT;                  // marginal + smallest tile do not fit the LDS
   int tile_bits = 0;
   while ((1 << tile_bits) < tile) ++tile_bits;
-  if (n_student >= (1LL << (32 - tile_bits)) - 1) return DL_ERR_LIMIT;
   *tile_out = tile;
   const int64_t ntiles = (n_teacher + tile - 1) / tile;
+
+  // loads per student id
+  std::vector<int64_t> count(n_student, 0);
+  int64_t n_mapped = 0;
+  for (int64_t t = 0; t < n_teacher; ++t) {
+    const int32_t sid = t2s[t];
+    if (sid >= n_student) return DL_ERR_SHAPE;
+    if (sid >= 0) { ++count[sid]; ++n_mapped; }
+  }
+  // replicas: LDS words left beside the marginal and the tile, handed one at a time to the id with
+  // the largest load per slot, down to a quarter of a thread's even share
+  int64_t budget = ((LDS_BUDGET - marg_bytes - (int64_t)tile * 4) / 4) & ~(int64_t)3;
+  const int64_t slot_limit = (1LL << (32 - tile_bits)) - 1;                 // slot ids must fit beside the tile offset
+  if (n_pad >= slot_limit) return DL_ERR_LIMIT;
+  budget = std::min<int64_t>(budget, slot_limit - n_pad);
+  const double share = (double)n_mapped / NT;
+  std::vector<int32_t> reps(n_student, 1);
+  {
+    auto per_slot = [&](int32_t s) { return (double)count[s] / reps[s]; };
+    auto worse = [&](int32_t a, int32_t b) { const double la = per_slot(a), lb = per_slot(b); return la != lb ? la < lb : a > b; };
+    std::vector<int32_t> heap;
+    for (int64_t s = 0; s < n_student; ++s)
+      if ((double)count[s] > std::max(share / 4, 8.0)) heap.push_back((int32_t)s);
+    std::make_heap(heap.begin(), heap.end(), worse);
+    while (budget > 0 && !heap.empty()) {
+      std::pop_heap(heap.begin(), heap.end(), worse);
+      const int32_t s = heap.back();
+      if (per_slot(s) <= std::max(share / 4, 8.0)) break;                   // the heaviest is light enough: done
+      ++reps[s];
+      --budget;
+      std::push_heap(heap.begin(), heap.end(), worse);
+    }
+  }
+  // slots: own slot of every id that is hit, plus the replicas; fold table in ascending id order
+  struct Slot { int32_t slot; double load; };
+  std::vector<Slot> slots;
+  std::vector<int32_t> first_extra(n_student, -1);
+  int64_t n_extra = 0, n_fold = 0;
+  for (int64_t s = 0; s < n_student; ++s) {
+    if (count[s] == 0) continue;
+    const double load = (double)count[s] / reps[s];
+    slots.push_back({(int32_t)s, load});
+    if (reps[s] > 1) {
+      first_extra[s] = (int32_t)(n_pad + n_extra);
+      for (int j = 1; j < reps[s]; ++j) slots.push_back({(int32_t)(n_pad + n_extra + j - 1), load});
+      if (fold) {
+        if (n_fold >= fold_capacity) return DL_ERR_SHAPE;
+        fold[3 * n_fold] = (int32_t)s; fold[3 * n_fold + 1] = first_extra[s]; fold[3 * n_fold + 2] = reps[s] - 1;
+      }
+      n_extra += reps[s] - 1;
+      ++n_fold;
+    }
+  }
+  *n_fold_out = n_fold;
+  *n_extra_out = (int)n_extra;
+  // owners: heaviest slot first onto the least-loaded thread (ties: lower thread number)
+  std::stable_sort(slots.begin(), slots.end(), [](const Slot& a, const Slot& b) { return a.load > b.load; });
+  std::vector<int32_t> owner(n_pad + n_extra, -1);
+  {
+    std::vector<std::pair<double, int>> th(NT);
+    for (int i = 0; i < NT; ++i) th[i] = {0.0, i};
+    auto heavier = [](const std::pair<double, int>& a, const std::pair<double, int>& b) { return a > b; };
+    std::make_heap(th.begin(), th.end(), heavier);                          // min-heap on (load, thread)
+    for (const Slot& sl : slots) {
+      std::pop_heap(th.begin(), th.end(), heavier);
+      owner[sl.slot] = th.back().second;
+      th.back().first += sl.load;
+      std::push_heap(th.begin(), th.end(), heavier);
+    }
+  }
+
   std::vector<std::vector<uint32_t>> bucket(NT);
   int64_t rows = 0;
   if (row_off) row_off[0] = 0;
@@ -135,10 +216,17 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
     const int64_t t0 = k * tile, t1 = std::min<int64_t>(n_teacher, t0 + tile);
     for (int64_t t = t0; t < t1; ++t) {
       const int32_t sid = t2s[t];
-      if (sid >= n_student) return DL_ERR_SHAPE;
-      if (sid >= 0) bucket[sid % NT].push_back(((uint32_t)sid << tile_bits) | (uint32_t)(t - t0));
+      if (sid < 0) continue;
+      int32_t slot = sid;
+      size_t best = bucket[owner[sid]].size();
+      for (int j = 1; j < reps[sid]; ++j) {                                 // the replica whose owner is least busy in this tile
+        const int32_t cand = first_extra[sid] + j - 1;
+        const size_t sz = bucket[owner[cand]].size();
+        if (sz < best) { best = sz; slot = cand; }
+      }
+      bucket[owner[slot]].push_back(((uint32_t)slot << tile_bits) | (uint32_t)(t - t0));
     }
-    for (auto& b : bucket) std::sort(b.begin(), b.end());      // (s, t) ascending: s in the high bits
+    for (auto& b : bucket) std::sort(b.begin(), b.end());      // (slot, t) ascending: slot in the high bits
     for (int w = 0; w < NW; ++w) {
       size_t longest = 0;
       for (int l = 0; l < WAVE; ++l) longest = std::max(longest, bucket[w * WAVE + l].size());

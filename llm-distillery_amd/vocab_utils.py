@@ -72,28 +72,33 @@ class MarginalPlan:
         self.n_student = int(n_student)
         self.n_teacher = int(t2s.size)
         self.t2s = torch.as_tensor(t2s, device=device)
-        self.row_off = self.ent = None
-        self.tile = 0
+        self.row_off = self.ent = self.fold = None
+        self.tile = self.n_fold = self.n_extra = 0
         lib = _lib.load()
-        tile, rows = ctypes.c_int(0), ctypes.c_int64(0)
-        st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), None, None, 0, ctypes.byref(rows))
+        tile, rows, n_fold, n_extra = ctypes.c_int(0), ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int(0)
+        st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), None, None, 0, ctypes.byref(rows),
+                                        None, 0, ctypes.byref(n_fold), ctypes.byref(n_extra))
         if st == -4:          # DL_ERR_LIMIT: student vocabulary too wide for a plan; the atomic path still works
             return
         _lib.check(st, "dl_marginal_plan_build")
         ntiles = -(-t2s.size // tile.value)
         row_off = np.zeros(16 * ntiles + 1, dtype=np.int32)
         ent = np.empty((max(rows.value, 1), 64), dtype=np.uint32)
+        fold = np.zeros((max(n_fold.value, 1), 3), dtype=np.int32)
         st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), _p(row_off), _p(ent), rows.value,
-                                        ctypes.byref(rows))
+                                        ctypes.byref(rows), _p(fold), n_fold.value, ctypes.byref(n_fold),
+                                        ctypes.byref(n_extra))
         _lib.check(st, "dl_marginal_plan_build")
-        self.tile = tile.value
+        self.tile, self.n_fold, self.n_extra = tile.value, int(n_fold.value), int(n_extra.value)
         self.row_off = torch.as_tensor(row_off, device=device)
         self.ent = torch.as_tensor(ent.view(np.int32), device=device)     # same bits; torch has no uint32 arithmetic need
+        self.fold = torch.as_tensor(fold, device=device)
 
     def _args(self):
+        """(row_off, ent, tile, fold, n_fold, n_extra) as the C ABI takes them."""
         if self.ent is None:
-            return 0, 0, 0
-        return self.row_off.data_ptr(), self.ent.data_ptr(), self.tile
+            return 0, 0, 0, 0, 0, 0
+        return self.row_off.data_ptr(), self.ent.data_ptr(), self.tile, self.fold.data_ptr(), self.n_fold, self.n_extra
 
 
 def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=None, plan: MarginalPlan | None = None,
@@ -122,13 +127,13 @@ def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=Non
                                         _stream_ptr(x.device))
             _lib.check(st, "dl_marginalise_csr")
         else:
-            pro, pen, pti = (0, 0, 0)
+            plan_args = (0, 0, 0, 0, 0, 0)
             if plan is not None:
                 t2s = plan.t2s
-                pro, pen, pti = plan._args()
+                plan_args = plan._args()
             _, _ = _opt_i32(t2s, Vt, "t2s", x.device)
             st = lib.dl_marginalise_map(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vt, t2s.data_ptr(), n_student,
-                                        pro, pen, pti, out.data_ptr(), out.stride(0), int(log), _stream_ptr(x.device))
+                                        *plan_args, out.data_ptr(), out.stride(0), int(log), _stream_ptr(x.device))
             _lib.check(st, "dl_marginalise_map")
     return out
 
@@ -141,9 +146,9 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
     in one launch; the marginal stays in LDS.  `t2s` is the int32 [Vt] map on the GPU or, better, a
     MarginalPlan built from it.  Returns (row_loss fp32 [rows], grad or None)."""
     _dev(logits, "logits"), _dev(teacher_probs, "teacher_probs")
-    pro, pen, pti = (0, 0, 0)
+    plan_args = (0, 0, 0, 0, 0, 0)
     if isinstance(t2s, MarginalPlan):
-        pro, pen, pti = t2s._args()
+        plan_args = t2s._args()
         t2s = t2s.t2s
     x, tp = _rows_2d(logits), _rows_2d(teacher_probs)
     R, Vs = x.shape
@@ -162,7 +167,7 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
     with torch.cuda.device(dev):
         st = _lib.load().dl_rkl_marginalised(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vs, rm_ptr, tp.data_ptr(),
-                                             _DT[tp.dtype], tp.stride(0), N, Vt, t2s.data_ptr(), pro, pen, pti, 1.0 / T,
+                                             _DT[tp.dtype], tp.stride(0), N, Vt, t2s.data_ptr(), *plan_args, 1.0 / T,
                                              1.0 / (T if teacher_T is None else teacher_T), grad_scale,
                                              row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
     _lib.check(st, "dl_rkl_marginalised")

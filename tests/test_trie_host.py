@@ -57,7 +57,7 @@ def test_config5_vocabularies_at_full_size():
     assert off[-1] == 152064 and np.array_equal(np.sort(ind), np.arange(152064))
 
 
-def test_marginal_plan_covers_every_mapped_id_once_in_owner_order():
+def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     rng = np.random.default_rng(7)
     Vt, Vs = 20000, 3000
     t2s = rng.integers(-1, Vs, Vt).astype(np.int32)
@@ -67,23 +67,42 @@ def test_marginal_plan_covers_every_mapped_id_once_in_owner_order():
     assert tile in (4096, 8192)
     row_off = plan.row_off.numpy()
     ent = plan.ent.numpy().view(np.uint32)
+    fold = plan.fold.numpy()[:plan.n_fold]
     ntiles = -(-Vt // tile)
     assert row_off.shape == (16 * ntiles + 1,) and row_off[0] == 0 and row_off[-1] == ent.shape[0]
+    # replica slots sit behind the padded marginal, each belongs to exactly one hot id
+    n_pad = (Vs + 3) & ~3
+    slot_id = np.arange(n_pad + plan.n_extra)
+    slot_id[Vs:] = -1
+    assert plan.n_extra == fold[:, 2].sum() and (np.diff(fold[:, 0]) > 0).all()
+    cursor = n_pad
+    for sid, first, cnt in fold:
+        assert first == cursor and cnt >= 1 and 0 <= sid < Vs
+        slot_id[first:first + cnt] = sid
+        cursor += cnt
+    assert cursor == n_pad + plan.n_extra and plan.n_fold > 0       # the hot ids did get replicas
     seen = np.zeros(Vt, dtype=np.int32)
+    owner = {}
+    longest = []
     for k in range(ntiles):
         for w in range(16):
             rows = ent[row_off[16 * k + w]:row_off[16 * k + w + 1]]
+            longest.append(rows.shape[0])
             for lane in range(64):
                 col = rows[:, lane]
                 live = col[col != 0xffffffff]
                 assert (col[len(live):] == 0xffffffff).all()            # padding only at the tail
-                assert (np.diff(live.astype(np.int64)) > 0).all()         # sorted by (s, t), no repeats
-                sid = (live >> bits).astype(np.int64)
+                assert (np.diff(live.astype(np.int64)) > 0).all()         # sorted by (slot, t), no repeats
+                slot = (live >> bits).astype(np.int64)
                 t = (live & (tile - 1)).astype(np.int64) + k * tile
-                assert (sid % 1024 == w * 64 + lane).all()                # owned by this thread
-                assert (t2s[t] == sid).all()
+                assert (slot < n_pad + plan.n_extra).all()
+                assert (t2s[t] == slot_id[slot]).all()                    # the entry lands on a slot of its own id
+                for sl in np.unique(slot):
+                    assert owner.setdefault(int(sl), w * 64 + lane) == w * 64 + lane      # one thread per LDS word, in every tile
                 seen[t] += 1
     assert np.array_equal(seen, (t2s >= 0).astype(np.int32))
+    # half of the entries sit on 8 ids: without replicas one thread would hold > 1200 entries of a tile
+    assert max(longest) <= 4 * (tile // 1024)
     # too wide a student vocabulary: no plan, the atomic form remains
     wide = D.vocab_utils.MarginalPlan(np.zeros(100, dtype=np.int32), 40000, "cpu")
     assert wide.ent is None and wide.tile == 0
