@@ -42,7 +42,7 @@ struct RegRows {
   }
 };
 
-template <class TagS, class TagT, int NT, int NU>
+template <int KIND, class TagS, class TagT, int NT, int NU>
 __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
   __shared__ float red[64];
   const int64_t r = blockIdx.x;
@@ -57,9 +57,9 @@ __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
   RegRows<TagS, TagT, NT, NU> rows;
   rows.load(reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes,
             reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * TagT::bytes, p.V / 8);
-  const DenseStats st = dense_stats<NT>(p.kind, rows, p.inv_T_s, p.inv_T_t, red);
+  const DenseStats st = dense_stats<KIND, NT>(rows, p.inv_T_s, p.inv_T_t, red);
   if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
-  if (grow) dense_grad_sweep<TagS>(p.kind, rows, st, p.inv_T_s * p.grad_scale, grow);
+  if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
 }
 
 // Any size, any alignment, any dtype pair: four scalar passes over global memory.
@@ -119,15 +119,22 @@ __global__ __launch_bounds__(NT) void dense_stream_kernel(const DenseParams p) {
   }
 }
 
-template <class TagS, class TagT, int NU>
-static bool launch_dense_reg(const DenseParams& p, hipStream_t st) {
+template <int KIND, class TagS, class TagT, int NU>
+static bool launch_dense_kind(const DenseParams& p, hipStream_t st) {
   const int64_t units = p.V / 8;
   const dim3 grid((unsigned)p.n_rows);
-  if (units <= 256 * NU) hipLaunchKernelGGL((dense_reg_kernel<TagS, TagT, 256, NU>), grid, dim3(256), 0, st, p);
-  else if (units <= 512 * NU) hipLaunchKernelGGL((dense_reg_kernel<TagS, TagT, 512, NU>), grid, dim3(512), 0, st, p);
-  else if (units <= 1024 * NU) hipLaunchKernelGGL((dense_reg_kernel<TagS, TagT, 1024, NU>), grid, dim3(1024), 0, st, p);
+  if (units <= 256 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 256, NU>), grid, dim3(256), 0, st, p);
+  else if (units <= 512 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 512, NU>), grid, dim3(512), 0, st, p);
+  else if (units <= 1024 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 1024, NU>), grid, dim3(1024), 0, st, p);
   else return false;
   return true;
+}
+
+template <class TagS, class TagT, int NU>
+static bool launch_dense_reg(const DenseParams& p, hipStream_t st) {
+  if (p.kind == DL_FKL) return launch_dense_kind<DL_FKL, TagS, TagT, NU>(p, st);
+  if (p.kind == DL_RKL) return launch_dense_kind<DL_RKL, TagS, TagT, NU>(p, st);
+  return launch_dense_kind<DL_JSD, TagS, TagT, NU>(p, st);
 }
 
 // Register path for the dtype pairs that occur: teacher stored like the student, or in fp32.

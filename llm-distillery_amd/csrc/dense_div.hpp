@@ -74,64 +74,81 @@ __device__ __forceinline__ float dense_grad(int kind, float lp, float lq, float 
   return 0.5f * fast_exp2(lp) * ((lp - log2_mix(lp, lq)) * LN2 - aux);
 }
 
-// The four sweeps over a row pair.  `Rows` provides
+// The sweeps over a row pair held in registers.  `Rows` provides
 //   template <class F> void sweep(F f)       calls f(u, s[8], t[8]) for every unit this thread owns
 // (values already unpacked to fp32, -inf beyond the row), and `red` is LDS scratch of 64 floats.
-template <int NT, class Rows>
-__device__ __forceinline__ DenseStats dense_stats(int kind, Rows& rows, float inv_T_s, float inv_T_t, float* red) {
+// KIND is a compile-time constant: the per-column code carries no branch on it.
+//
+// Forward and reverse KL need three sweeps, not four: with es = 2^(s a_s - bs), et = 2^(t a_t - bt)
+// (bs, bt the scaled maxima) and S = sum es, T = sum et,
+//   FKL = sum q (lq - lp) = (1/T) sum et ((t a_t - bt) - (s a_s - bs)) - log2 T + log2 S      (q = et / T)
+//   RKL = sum r (lp - lq) = (1/S) sum es ((s a_s - bs) - (t a_t - bt)) - log2 S + log2 T      (r = es / S, support only)
+// so the divergence sum rides along with the sums of exponentials.  JSD needs the normalised
+// probabilities inside a logarithm and keeps its own sweep.
+template <int KIND, int NT, class Rows>
+__device__ __forceinline__ DenseStats dense_stats(Rows& rows, float inv_T_s, float inv_T_t, float* red) {
   DenseStats st;
   st.a_s = inv_T_s * LOG2E;
   st.a_t = inv_T_t * LOG2E;
+  const float a_s = st.a_s, a_t = st.a_t;
   // maxima (for RKL the student maximum is taken over the teacher's support)
   float ms = -INFINITY, mt = -INFINITY;
   rows.sweep([&](int64_t, const float* s, const float* t) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       mt = fmaxf(mt, t[e]);
-      ms = fmaxf(ms, (kind == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
+      ms = fmaxf(ms, (KIND == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
     }
   });
   block_max2<NT>(ms, mt, red);
   st.tmax = mt;
-  const float bs = ms * st.a_s, bt = mt * st.a_t;
-  float ss = 0.f, stt = 0.f;
+  const float bs = ms * a_s, bt = mt * a_t;
+  float ss = 0.f, stt = 0.f, w = 0.f;
   rows.sweep([&](int64_t, const float* s, const float* t) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float es = fast_exp2(fmaf(s[e], st.a_s, -bs));
-      ss += (kind == DL_RKL && t[e] == -INFINITY) ? 0.f : es;
-      stt += fast_exp2(fmaf(t[e], st.a_t, -bt));
+      const float xs = fmaf(s[e], a_s, -bs), xt = fmaf(t[e], a_t, -bt);
+      const float es = fast_exp2(xs), et = fast_exp2(xt);
+      stt += et;
+      if (KIND == DL_RKL) {
+        const bool on = t[e] != -INFINITY;
+        ss += on ? es : 0.f;
+        w += (on && es > 0.f) ? es * (xs - xt) : 0.f;
+      } else {
+        ss += es;
+        if (KIND == DL_FKL) w += et > 0.f ? et * (xt - xs) : 0.f;
+      }
     }
   });
   block_sum2<NT>(ss, stt, red);
-  st.ls = bs + fast_log2(ss);
-  st.lt = bt + fast_log2(stt);
-  // divergence sums
+  const float l2s = fast_log2(ss), l2t = fast_log2(stt);
+  st.ls = bs + l2s;
+  st.lt = bt + l2t;
+  if (KIND != DL_JSD) {
+    w = block_sum<NT>(w, red);
+    const float x = KIND == DL_FKL ? w / stt - l2t + l2s : w / ss - l2s + l2t;
+    st.loss = x * LN2;
+    st.aux = st.loss;
+    return st;
+  }
   float x = 0.f, y = 0.f;
   rows.sweep([&](int64_t, const float* s, const float* t) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float lp = fmaf(s[e], st.a_s, -st.ls), lq = fmaf(t[e], st.a_t, -st.lt);
-      if (kind == DL_FKL) fkl_term(lp, lq, x);
-      else if (kind == DL_RKL) rkl_term(lp, lq, x);
-      else jsd_term(lp, lq, x, y);
-    }
+    for (int e = 0; e < 8; ++e) jsd_term(fmaf(s[e], a_s, -st.ls), fmaf(t[e], a_t, -st.lt), x, y);
   });
   block_sum2<NT>(x, y, red);
-  if (kind == DL_JSD) { st.loss = 0.5f * LN2 * (x + y); st.aux = x * LN2; }
-  else { st.loss = x * LN2; st.aux = st.loss; }
+  st.loss = 0.5f * LN2 * (x + y);
+  st.aux = x * LN2;
   return st;
 }
 
-template <class TagS, class Rows>
-__device__ __forceinline__ void dense_grad_sweep(int kind, Rows& rows, const DenseStats& st, float c, char* grow) {
+template <int KIND, class TagS, class Rows>
+__device__ __forceinline__ void dense_grad_sweep(Rows& rows, const DenseStats& st, float c, char* grow) {
+  const float a_s = st.a_s, a_t = st.a_t, ls = st.ls, lt = st.lt, aux = st.aux;
   rows.sweep([&](int64_t u, const float* s, const float* t) {
     float g[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float lp = fmaf(s[e], st.a_s, -st.ls), lq = fmaf(t[e], st.a_t, -st.lt);
-      g[e] = dense_grad(kind, lp, lq, st.aux) * c;
-    }
+    for (int e = 0; e < 8; ++e) g[e] = dense_grad(KIND, fmaf(s[e], a_s, -ls), fmaf(t[e], a_t, -lt), aux) * c;
     Unit<TagS>::store(grow, u, g);
   });
 }

@@ -335,12 +335,12 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
   for (int j = tid; j < p.Vs; j += MARG_NT) acc[j] = fast_log2(acc[j]) * LN2;      // log 0 = -inf: off the support
   __syncthreads();
   rows.lt = acc;
-  const DenseStats st = dense_stats<MARG_NT>(DL_RKL, rows, p.inv_T_s, p.inv_T_t, red);
+  const DenseStats st = dense_stats<DL_RKL, MARG_NT>(rows, p.inv_T_s, p.inv_T_t, red);
   const bool empty = st.tmax == -INFINITY;        // the teacher row carried no mass at all
   if (tid == 0 && p.row_loss) p.row_loss[r] = empty ? 0.f : st.loss;
   if (grow) {
     if (empty) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
-    else dense_grad_sweep<TagS>(DL_RKL, rows, st, p.inv_T_s * p.grad_scale, grow);
+    else dense_grad_sweep<DL_RKL, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
   }
 }
 
