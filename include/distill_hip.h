@@ -84,6 +84,9 @@ int dl_set_option(const char* name, int value);
  *            torch.topk and of dl_merge_remap_topk); the kernel then skips its duplicate scan.  With
  *            the flag set and duplicates present, the gradient at a duplicated id is wrong.
  * K <= DL_MAX_TOPK.
+ * grad may be the logits buffer itself (same pointer and stride): every kernel holds, or has
+ * consumed, what it still needs of a row before it writes there.  The same holds for dl_div_dense
+ * and dl_rkl_marginalised, not for dl_rowcoef_grad_topk.
  * With n_teacher_rows == 0 the teacher pointers may be NULL: every row then counts as masked
  * (the same holds for dl_div_dense, dl_rowstats_topk and dl_rowcoef_grad_topk).
  */

@@ -20,6 +20,7 @@
 // reads the row twice.
 #include "distill_common.hpp"
 #include "distill_hip.h"
+#include <algorithm>
 #include <atomic>
 #include <cstring>
 
@@ -67,6 +68,21 @@ __device__ __forceinline__ bool part_collect(PartStats* w, int limit, float& m, 
   }
   return false;
 }
+
+// Workspace of a split launch: n_rows * parts records, then a counter and the list of (row, part)
+// numbers that gave up waiting for a partner and are finished by a second launch.
+struct RetryList {
+  unsigned* count;
+  unsigned* entries;
+  __host__ __device__ RetryList(void* workspace, int64_t n_rows, int parts) {
+    char* base = reinterpret_cast<char*>(workspace) + n_rows * parts * (int64_t)sizeof(PartStats);
+    count = reinterpret_cast<unsigned*>(base);
+    entries = reinterpret_cast<unsigned*>(base + 16);
+  }
+  __host__ __device__ static int64_t bytes(int64_t n_rows, int parts) {
+    return n_rows * parts * (int64_t)(sizeof(PartStats) + 4) + 16;
+  }
+};
 
 // LDS carve-up shared by the kernels of this file.  The id array is padded to a multiple of 16
 // with -1 so that it can be scanned four ids per read.
@@ -274,18 +290,13 @@ __device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, f
 // ---------------------------------------------------------------------------------------
 // J > 0: the K <= J * NT teacher entries travel in registers (loads issued ahead of the row's);
 // J == 0: any K, staged by a plain loop.
-template <class Tag, int NT, int NCH, bool SPLIT, int J>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))     // <= 128 VGPRs: 16 waves per CU
-void fkl_topk_reg_kernel(const TopkParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K);
+// RETRY: second launch over the parts that gave up waiting in the first (see split_retry_list):
+// every record of the row is published by then, so nothing is waited for.
+template <class Tag, int NT, int NCH, bool SPLIT, int J, bool RETRY>
+__device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds& s, int64_t r, int h) {
   using C = Chunk<Tag>;
   const int tid = threadIdx.x;
   const int P = SPLIT ? p.parts : 1;
-  const unsigned grp = SPLIT ? blockIdx.x / (8u * P) : 0u, t_in = SPLIT ? blockIdx.x % (8u * P) : 0u;
-  const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : blockIdx.x;
-  const int h = SPLIT ? (int)(t_in >> 3) : 0;
-  if (SPLIT && r >= p.n_rows) return;
   const int64_t c0 = (int64_t)h * NT * NCH;                       // first chunk of this part
   const int64_t nch = min((int64_t)NT * NCH, p.V / C::N - c0);    // chunks of this part
   const int lo = (int)(c0 * C::N), hi = lo + (int)(nch * C::N);   // its column range
@@ -359,33 +370,29 @@ void fkl_topk_reg_kernel(const TopkParams p) {
   if (SPLIT) {
     // publish this part's statistics, collect the others'
     PartStats* ws = reinterpret_cast<PartStats*>(p.workspace) + r * P;
-    if (tid == 0) part_publish(ws + h, mx, sm, B);
+    if (tid == 0 && !RETRY) part_publish(ws + h, mx, sm, B);
     if (tid < P) {
       float om = mx, os = sm, ob = B;
-      const int ok = (tid == h) || part_collect(ws + tid, p.spin_limit, om, os, ob);
+      const int ok = (tid == h) || part_collect(ws + tid, RETRY ? 0x7fffffff : p.spin_limit, om, os, ob);
       s.xm[tid] = om; s.xs[tid] = os; s.xb[tid] = ob; s.xok[tid] = ok;
     }
     __syncthreads();
     bool all_ok = true;
     for (int j = 0; j < P; ++j) all_ok = all_ok && (s.xok[j] != 0);
-    if (all_ok) {
-      float M = s.xm[0];
-      for (int j = 1; j < P; ++j) M = fmaxf(M, s.xm[j]);
-      float S = 0.f, Bt = 0.f;
-      for (int j = 0; j < P; ++j) { S += s.xs[j] * fast_exp2((s.xm[j] - M) * a); Bt += s.xb[j]; }
-      mb = M * a; sm = S; B = Bt;
-    } else {
-      // a partner did not answer: rebuild the row statistics and the loss sum alone
-      __syncthreads();
-      for (int k = tid; k < s.Kp; k += NT) {
-        const int id = s.idx[k];
-        if (id >= 0 && (id < lo || id >= hi)) s.z[k] = load_as_float(row, Tag::id, id);
+    if (!all_ok) {
+      // A partner did not answer in time.  Nothing has been written yet: this part puts itself on
+      // the retry list and leaves; its own record is published, so the partners can finish.
+      if (tid == 0) {
+        RetryList list(p.workspace, p.n_rows, P);
+        list.entries[atomicAdd(list.count, 1u)] = (unsigned)(r * P + h);
       }
-      __syncthreads();
-      fkl_partials<NT>(p, s, tlse, 0, (int)p.V, B, Q);
-      row_stats_streamed<Tag, NT, true>(row, p.V, a, s.red, mx, sm);
-      mb = mx * a;
+      return;
     }
+    float M = s.xm[0];
+    for (int j = 1; j < P; ++j) M = fmaxf(M, s.xm[j]);
+    float S = 0.f, Bt = 0.f;
+    for (int j = 0; j < P; ++j) { S += s.xs[j] * fast_exp2((s.xm[j] - M) * a); Bt += s.xb[j]; }
+    mb = M * a; sm = S; B = Bt;
   }
   const float b = mb + fast_log2(sm);      // log2-sum-exp2 of the scaled row
   if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = B + (b * LN2) * Q;
@@ -407,6 +414,41 @@ void fkl_topk_reg_kernel(const TopkParams p) {
     }
     __syncthreads();      // dense stores are ordered before the sparse corrections
     fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
+  }
+}
+
+template <class Tag, int NT, int NCH, bool SPLIT, int J>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))     // <= 128 VGPRs: 16 waves per CU
+void fkl_topk_reg_kernel(const TopkParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const TopkLds s(smem, p.K);
+  const int P = SPLIT ? p.parts : 1;
+  const unsigned grp = SPLIT ? blockIdx.x / (8u * P) : 0u, t_in = SPLIT ? blockIdx.x % (8u * P) : 0u;
+  const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : blockIdx.x;
+  const int h = SPLIT ? (int)(t_in >> 3) : 0;
+  if (SPLIT && r >= p.n_rows) return;
+  fkl_topk_part<Tag, NT, NCH, SPLIT, J, false>(p, s, r, h);
+}
+
+// One listed part, as a real call: the loop around it then costs the body no registers.
+template <class Tag, int NT, int NCH, int J>
+__device__ __attribute__((noinline)) void fkl_topk_part_again(const TopkParams& p, const TopkLds& s, unsigned at) {
+  fkl_topk_part<Tag, NT, NCH, true, J, true>(p, s, (int64_t)(at / (unsigned)p.parts), (int)(at % (unsigned)p.parts));
+}
+
+// The parts on the retry list, a fixed grid striding over it (normally the list is empty and
+// every workgroup leaves after one load).
+template <class Tag, int NT, int NCH, int J>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+void fkl_topk_retry_kernel(const TopkParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const TopkLds s(smem, p.K);
+  const RetryList list(p.workspace, p.n_rows, p.parts);
+  const unsigned n = *list.count;
+#pragma unroll 1
+  for (unsigned e = blockIdx.x; e < n; e += gridDim.x) {
+    fkl_topk_part_again<Tag, NT, NCH, J>(p, s, list.entries[e]);
+    __syncthreads();      // LDS is reused by the next entry
   }
 }
 
@@ -474,14 +516,16 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   const int tid = threadIdx.x;
   const int64_t V = p.V;
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
-  if (grow) {
-    if (VEC) zero_row<Tag, NT>(grow, V / C::N);
-    else for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
-  }
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
   float tlse = -INFINITY;
   if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
+  // The zero fill comes after the K logits have been gathered (stage_teacher ends in barriers), so
+  // the gradient may be written over the logits.
+  if (grow) {
+    if (VEC) zero_row<Tag, NT>(grow, V / C::N);
+    else for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
+  }
   if (tlse == -INFINITY) {
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
@@ -540,6 +584,15 @@ static void launch_reg_j(const TopkParams& p, unsigned grid, hipStream_t st) {
 }
 
 template <class Tag, int NT, int NCH>
+static void launch_retry_j(const TopkParams& p, unsigned grid, hipStream_t st) {
+  const int Kp = (p.K + 15) & ~15;
+  const size_t lds = TopkLds::bytes(p.K);
+  if (Kp <= NT) hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 1>), dim3(grid), dim3(NT), lds, st, p);
+  else if (Kp <= 3 * NT) hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 3>), dim3(grid), dim3(NT), lds, st, p);
+  else hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 0>), dim3(grid), dim3(NT), lds, st, p);
+}
+
+template <class Tag, int NT, int NCH>
 static hipError_t launch_reg(const TopkParams& p, hipStream_t st) {
   launch_reg_j<Tag, NT, NCH, false>(p, (unsigned)p.n_rows, st);
   return hipGetLastError();
@@ -548,10 +601,11 @@ static hipError_t launch_reg(const TopkParams& p, hipStream_t st) {
 template <class Tag, int NT, int NCH>
 static hipError_t launch_split(TopkParams p, int parts, hipStream_t st) {
   p.parts = parts;
-  const int64_t n16 = p.n_rows * parts;          // one 16-byte PartStats per (row, part)
+  const int64_t n16 = p.n_rows * parts + 1;      // one 16-byte PartStats per (row, part), then the retry counter
   hipLaunchKernelGGL(clear_workspace_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
                      reinterpret_cast<u32x4*>(p.workspace), n16);
   launch_reg_j<Tag, NT, NCH, true>(p, (unsigned)((p.n_rows + 7) / 8 * 8 * parts), st);
+  launch_retry_j<Tag, NT, NCH>(p, (unsigned)std::min<int64_t>(p.n_rows * parts, 256), st);
   return hipGetLastError();
 }
 
@@ -577,8 +631,7 @@ static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes
     if (nch <= 512 * 16) return launch_reg<Tag, 512, 16>(p, st);
     if (nch <= 1024 * 16) {
       const int parts = split_parts(nch);
-      const bool ws_ok = p.workspace && ws_bytes >= p.n_rows * parts * (int64_t)sizeof(PartStats) &&
-                         p.n_rows * parts <= 0x7fffffffLL;
+      const bool ws_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, parts) && p.n_rows * parts <= 0x7fffffffLL;
       if (parts == 2 && ws_ok) return launch_split<Tag, 512, 16>(p, 2, st);
       if (parts == 4 && ws_ok) return launch_split<Tag, 256, 16>(p, 4, st);
       return launch_reg<Tag, 1024, 16>(p, st);
@@ -626,7 +679,7 @@ extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64
   if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
   const int64_t nch = V / (logits_dtype == DL_F32 ? 4 : 8);
   if (nch <= 512 * 16 || nch > 1024 * 16) return 0;
-  return n_rows * dl::MAX_PARTS * (int64_t)sizeof(dl::PartStats);
+  return dl::RetryList::bytes(n_rows, 4);
 }
 
 extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,

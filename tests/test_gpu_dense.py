@@ -122,3 +122,16 @@ def test_synthetic_configs_1_and_2_at_reduced_rows(D):
     c = S.config2(DEV, B=2, S=48)
     assert c["t_logits"].shape[0] == int(c["lengths"].sum())
     _check(D, "jsd", c["logits"].cpu(), c["t_logits"].cpu(), 2.0, valid=c["valid"].cpu())
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+@pytest.mark.parametrize("V,dtype", [(32000, torch.bfloat16), (1001, torch.float32)])
+def test_dense_gradient_may_overwrite_the_logits(D, kind, V, dtype):
+    g = torch.Generator().manual_seed(17)
+    x = (torch.randn(12, V, generator=g) * 2).to(dtype).to(DEV)
+    t = (0.7 * x.float() + torch.randn(12, V, generator=g).to(DEV)).to(dtype)
+    rl, grad = D.div_dense(kind, x, t, T=1.3)
+    y = x.clone()
+    rl2, g2 = D.div_dense(kind, y, t, T=1.3, grad_out=y)
+    assert g2.data_ptr() == y.data_ptr() and torch.equal(rl, rl2) and torch.equal(grad, y)
+

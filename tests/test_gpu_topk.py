@@ -171,15 +171,18 @@ def test_errors_are_python_exceptions(D):
 def test_split_row_parts_agree_and_give_up_path(D, parts):
     """A 128256-wide row is cut into column parts that exchange statistics through the workspace.
     Every setting must give the oracle's numbers, also when no part waits for its partners
-    (spin_limit 0: each part then rebuilds the row statistics alone)."""
+    (spin_limit 0: every part that finds a record missing leaves and is finished by the retry
+    launch), and the same bits as with waiting."""
     logits, tv, ti = _case(40, 128256, 200, torch.bfloat16, 12, std=3.0)
     valid = torch.ones(40, dtype=torch.bool)
     valid[[0, 7, 33]] = False
     try:
         D.set_option("split_parts", parts)
         _check(D, "fkl", logits, tv[:37], ti[:37], T=1.0, valid=valid)
+        waited = _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid)
         D.set_option("spin_limit", 0)
-        _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid)
+        retried = _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid)
+        assert torch.equal(waited, retried)
     finally:
         D.set_option("split_parts", 0)
         D.set_option("spin_limit", 20000)
@@ -187,3 +190,23 @@ def test_split_row_parts_agree_and_give_up_path(D, parts):
         D.set_option("split_parts", 3)
     with pytest.raises(RuntimeError):
         D.set_option("no_such_option", 1)
+
+
+@pytest.mark.parametrize("kind,V,dtype", [("fkl", 128256, torch.bfloat16), ("fkl", 32000, torch.bfloat16), ("fkl", 152064, torch.float16),
+                                          ("fkl", 1001, torch.float32), ("rkl", 32000, torch.bfloat16)])
+def test_gradient_may_overwrite_the_logits(D, kind, V, dtype):
+    """grad == logits (same buffer): every kernel holds, or has consumed, what it still needs of a
+    row before it writes there, and a split part that gives up leaves its columns untouched for the
+    retry launch; results are the bits of the out-of-place call."""
+    logits, tv, ti = _case(24, V, 64, dtype, 31)
+    x = logits.to(DEV)
+    rl, g = D.div_topk(kind, x, tv.to(DEV), ti.to(DEV), T=1.5)
+    for spin in (20000, 0):
+        try:
+            D.set_option("spin_limit", spin)
+            y = x.clone()
+            rl2, g2 = D.div_topk(kind, y, tv.to(DEV), ti.to(DEV), T=1.5, grad_out=y)
+        finally:
+            D.set_option("spin_limit", 20000)
+        assert g2.data_ptr() == y.data_ptr() and torch.equal(rl, rl2) and torch.equal(g, y)
+
