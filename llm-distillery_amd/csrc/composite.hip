@@ -36,11 +36,6 @@ struct CompositeParams {
   const float* g_train; float* g_lse; float* g_zk;
 };
 
-__device__ __forceinline__ int wave_sum_int(int v) {
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
-}
 __device__ __forceinline__ int wave_min_int(int v) {
 #pragma unroll
   for (int o = WAVE / 2; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, WAVE));

@@ -144,22 +144,6 @@ __device__ __forceinline__ void store16_stream(void* p, const u32x4& v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
-// ---- row access through buffer instructions ------------------------------------------
-// A row is described by a buffer resource (scalar registers: base address + byte size); every
-// access is `resource + 32-bit lane offset (one VGPR) + scalar chunk offset`, so walking a row
-// costs no 64-bit address VGPRs.  Reads beyond the row's size return 0 and writes beyond it are
-// dropped by the hardware.
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
-}
-__device__ __forceinline__ u32x4 buf_load16_stream(rsrc_t r, unsigned lane_off, unsigned chunk_off) {
-  return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, chunk_off, 2);      // 2 = non-temporal
-}
-__device__ __forceinline__ void buf_store16_stream(rsrc_t r, unsigned lane_off, unsigned chunk_off, const u32x4& v) {
-  __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, chunk_off, 2);
-}
-
 // ---- reductions: fixed butterfly order => bit-reproducible ----------------------
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
