@@ -507,6 +507,7 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p)
   extern __shared__ __align__(16) unsigned char smem_raw[];
   u64* all = reinterpret_cast<u64*>(smem_raw);                      // the parts' records; producer_merge_slots words
   __shared__ int slots[2 * 4];
+  __shared__ unsigned s_best[4];
   __shared__ int s_nsel;
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), w = tid / WAVE;
@@ -533,20 +534,37 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p)
   if (tid == 0) s_nsel = 0;
   __syncthreads();
 
-  // U = smallest high word with at least K words at or below it; only the low Keys::BITS bits vary
+  // U = smallest high word with at least K words at or below it; only the low Keys::BITS bits vary.
+  // Counting is ballot + popcount per wave, one barrier per probe; the first probe tries the six
+  // leading bits of the best word, which the K-th almost always shares.
   constexpr int BITS = Keys<Tag>::BITS;
-  unsigned U = BITS == 32 ? 0u : 0xffff0000u;
-#pragma unroll 1
-  for (int b = BITS - 1; b >= 0; --b) {
-    const unsigned bound = U | ((1u << b) - 1u);                    // bit b left at zero
+  const int trips = (total + 255) / 256;
+  int probe = 0;
+  auto count_le = [&](unsigned bound) {
     int c = 0;
-    for (int a = tid; a < total; a += 256) c += ((unsigned)(all[a] >> 32) <= bound) ? 1 : 0;
-#pragma unroll
-    for (int o = WAVE / 2; o > 0; o >>= 1) c += __shfl_xor(c, o, WAVE);
-    int* sl = slots + (b & 1) * 4;
+    for (int it = 0; it < trips; ++it) {
+      const int a = it * 256 + tid;
+      c += __popcll(__ballot(a < total && (unsigned)(all[a < total ? a : 0] >> 32) <= bound));
+    }
+    int* sl = slots + (probe++ & 1) * 4;
     if (lane == 0) sl[w] = c;
     __syncthreads();
-    if (sl[0] + sl[1] + sl[2] + sl[3] < K) U |= 1u << b;
+    return sl[0] + sl[1] + sl[2] + sl[3];
+  };
+  unsigned best = 0xffffffffu;
+  for (int a = tid; a < total; a += 256) best = min(best, (unsigned)(all[a] >> 32));
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) best = min(best, (unsigned)__shfl_xor((int)best, o, WAVE));
+  if (lane == 0) s_best[w] = best;
+  __syncthreads();
+  best = min(min(s_best[0], s_best[1]), min(s_best[2], s_best[3]));
+  const unsigned low = (1u << (BITS - 6)) - 1u;
+  unsigned U = BITS == 32 ? 0u : 0xffff0000u;
+  int b = BITS - 1;
+  if (count_le(best | low) >= K) { U = best & ~low; b = BITS - 7; }
+#pragma unroll 1
+  for (; b >= 0; --b) {
+    if (count_le(U | ((1u << b) - 1u)) < K) U |= 1u << b;          // probe with bit b left at zero
   }
   for (int a = tid; a < total; a += 256) {
     const u64 v = all[a];
