@@ -54,14 +54,11 @@ __device__ __forceinline__ void rkl_term(float lp, float lq, float& acc) {
   const float r = fast_exp2(lp);
   acc += (lq > -INFINITY && r > 0.f) ? r * (lp - lq) : 0.f;
 }
-__device__ __forceinline__ float log2_mix(float lp, float lq) {      // log2((2^lp + 2^lq) / 2)
-  const float hi = fmaxf(lp, lq), lo = fminf(lp, lq);
-  return hi + fast_log2(0.5f + 0.5f * fast_exp2(lo - hi));
-}
+// Three transcendentals per column: the mixture's logarithm is taken of the probabilities themselves.
+// Columns where both probabilities underflow contribute nothing (they are skipped by the guards).
 __device__ __forceinline__ void jsd_term(float lp, float lq, float& kl_pm, float& kl_qm) {
-  if (lp == -INFINITY && lq == -INFINITY) return;
-  const float lm = log2_mix(lp, lq);
   const float pr = fast_exp2(lp), q = fast_exp2(lq);
+  const float lm = fast_log2(0.5f * pr + 0.5f * q);
   kl_pm += pr > 0.f ? pr * (lp - lm) : 0.f;
   kl_qm += q > 0.f ? q * (lq - lm) : 0.f;
 }
@@ -70,8 +67,9 @@ __device__ __forceinline__ void jsd_term(float lp, float lq, float& kl_pm, float
 __device__ __forceinline__ float dense_grad(int kind, float lp, float lq, float aux) {
   if (kind == DL_FKL) return fast_exp2(lp) - fast_exp2(lq);
   if (kind == DL_RKL) return lq > -INFINITY ? fast_exp2(lp) * ((lp - lq) * LN2 - aux) : 0.f;
-  if (lp == -INFINITY) return 0.f;
-  return 0.5f * fast_exp2(lp) * ((lp - log2_mix(lp, lq)) * LN2 - aux);
+  const float pr = fast_exp2(lp);
+  if (!(pr > 0.f)) return 0.f;
+  return 0.5f * pr * ((lp - fast_log2(0.5f * pr + 0.5f * fast_exp2(lq))) * LN2 - aux);
 }
 
 // The sweeps over a row pair held in registers.  `Rows` provides
