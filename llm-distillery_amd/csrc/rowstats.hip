@@ -83,8 +83,13 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
   const int Kp = (p.K + 15) & ~15;
   int* s_idx = reinterpret_cast<int*>(smem);
   float* s_c = reinterpret_cast<float*>(s_idx + Kp);
-  const int64_t r = blockIdx.x / parts;
-  const int h = (int)(blockIdx.x % parts);
+  float* s_z = s_c + Kp;
+  // Workgroup ids are dealt round-robin to the 8 XCDs: within a group of 8 * parts ids, id t serves
+  // row 8 * group + t % 8, part t / 8, so the parts of a row run on one XCD back to back.
+  const unsigned grp = blockIdx.x / (8u * parts), t_in = blockIdx.x % (8u * parts);
+  const int64_t r = (int64_t)grp * 8 + (t_in & 7u);
+  const int h = (int)(t_in >> 3);
+  if (r >= p.n_rows) return;
   const int tid = threadIdx.x;
   const int64_t per_part = (int64_t)NT * NCH * C::N;                 // columns per part
   const int64_t lo = h * per_part, hi = min(p.V, lo + per_part);
@@ -96,19 +101,25 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     else for (int64_t j = lo + tid; j < hi; j += NT) store_from_float(grow, Tag::id, j, 0.f);
     return;
   }
-  for (int k = tid; k < Kp; k += NT) {
-    int64_t id = -1;
-    float cv = 0.f;
-    if (k < p.K) {
-      id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
-      cv = p.coef_zk[trow * p.K + k];
-    }
-    s_idx[k] = (id >= lo && id < hi) ? (int)id : -1;
-    s_c[k] = cv;
-  }
   const float a = p.inv_T * LOG2E;
   const float b = p.lse[trow] * LOG2E;
   const float w = p.coef_lse[trow] * p.inv_T;
+  // Teacher ids, their coefficients and the logits at the ids of this part go to LDS; issued behind
+  // the row's own loads so that their latencies overlap instead of trailing the dense sweep.
+  auto stage = [&]() {
+    for (int k = tid; k < Kp; k += NT) {
+      int64_t id = -1;
+      float cv = 0.f;
+      if (k < p.K) {
+        id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
+        cv = p.coef_zk[trow * p.K + k];
+      }
+      const bool mine = id >= lo && id < hi;
+      s_idx[k] = mine ? (int)id : -1;
+      s_c[k] = cv;
+      s_z[k] = mine ? load_as_float(row, Tag::id, id) : 0.f;
+    }
+  };
   if (VEC) {
     const int64_t c_lo = lo / C::N, c_hi = hi / C::N;
     u32x4 v[NCH];
@@ -117,6 +128,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
       v[i] = ch < c_hi ? load16_stream(row + ch * 16) : C::neg_inf();
     }
+    stage();
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
@@ -129,6 +141,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
       }
     }
   } else {
+    stage();
     for (int64_t j = lo + tid; j < hi; j += NT)
       store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * w);
   }
@@ -148,7 +161,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
       cs = 0.f;
       for (int j = 0; j < Kp; ++j) cs += (s_idx[j] == id) ? s_c[j] : 0.f;
     }
-    const float dense = fast_exp2(fmaf(load_as_float(row, Tag::id, id), a, -b)) * w;
+    const float dense = fast_exp2(fmaf(s_z[k], a, -b)) * w;
     store_from_float(grow, Tag::id, id, dense + cs * p.inv_T);
   }
 }
@@ -169,8 +182,8 @@ static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
   constexpr int NT = 256, NCH = 16;
   const int64_t per_part = (int64_t)NT * NCH * Tag::epc;
   const int parts = (int)((p.V + per_part - 1) / per_part);
-  const size_t lds = (size_t)((p.K + 15) & ~15) * 8;
-  const dim3 grid((unsigned)(p.n_rows * parts));
+  const size_t lds = (size_t)((p.K + 15) & ~15) * 12;
+  const dim3 grid((unsigned)((p.n_rows + 7) / 8 * 8 * parts));
   if (vec) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, true>), grid, dim3(NT), lds, st, p, parts);
   else hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, false>), grid, dim3(NT), lds, st, p, parts);
   return hipGetLastError();
