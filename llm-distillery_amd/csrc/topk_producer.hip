@@ -260,8 +260,12 @@ void topk_part_kernel(const ProducerParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), w = tid / WAVE;
   const int P = p.parts;
-  const int64_t ro = blockIdx.x / (unsigned)P;
-  const int h_part = (int)(blockIdx.x % (unsigned)P);
+  // Workgroup ids are dealt round-robin to the 8 XCDs: within a group of 8 * P ids, id t serves
+  // row 8 * group + t % 8, part t / 8, so the parts of a row run on one XCD back to back.
+  const unsigned grp = blockIdx.x / (8u * P), t_in = blockIdx.x % (8u * P);
+  const int64_t ro = (int64_t)grp * 8 + (t_in & 7u);
+  const int h_part = (int)(t_in >> 3);
+  if (ro >= p.n_out) return;
   const int64_t r = p.row_list ? (int64_t)p.row_list[ro] : ro;
   const int64_t c0 = (int64_t)h_part * NT * NCH;
   const int nch = (int)min((int64_t)NT * NCH, p.V / C::N - c0);      // chunks of this part, >= 1
@@ -269,9 +273,9 @@ void topk_part_kernel(const ProducerParams p) {
   const int n_elems = nch * C::N;
   const int Kp = min(p.K, n_elems);
   const char* rpart = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes + c0 * 16;
-  char* rec = p.ws + ((int64_t)blockIdx.x) * p.part_stride;
+  char* rec = p.ws + (ro * P + h_part) * p.part_stride;
   // single-wave stages rotate over the waves (and so over the SIMDs) from workgroup to workgroup
-  const int select_wave = (int)(blockIdx.x & (NW - 1));
+  const int select_wave = (int)((blockIdx.x >> 3) & (NW - 1));
 
   u32x4 reg[NCH];
 #pragma unroll
@@ -630,7 +634,7 @@ static int producer_parts(int64_t V, int logits_dtype) {
 
 template <class Tag>
 static int launch_producer(const ProducerParams& p, hipStream_t st) {
-  const dim3 grid((unsigned)(p.n_out * p.parts));
+  const dim3 grid((unsigned)((p.n_out + 7) / 8 * 8 * p.parts));
   if (p.K <= 256) hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_SMALL>), grid, dim3(PROD_NT), 0, st, p);
   else hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_LARGE>), grid, dim3(PROD_NT), 0, st, p);
   const size_t lds = (size_t)(producer_merge_slots(p.K, p.parts) + producer_sel_cap(p.K)) * 8;      // <= 48 KiB
