@@ -45,7 +45,8 @@ struct RegRows {
 template <int KIND, class TagS, class TagT, int NT, int NU>
 __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
   __shared__ float red[64];
-  const int64_t r = blockIdx.x;
+  const int64_t r = xcd_banded_row(blockIdx.x);
+  if (r >= p.n_rows) return;
   const int tid = threadIdx.x;
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(NT) void dense_stream_kernel(const DenseParams p) {
 template <int KIND, class TagS, class TagT, int NU>
 static bool launch_dense_kind(const DenseParams& p, hipStream_t st) {
   const int64_t units = p.V / 8;
-  const dim3 grid((unsigned)p.n_rows);
+  const dim3 grid(xcd_banded_grid(p.n_rows));
   if (units <= 256 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 256, NU>), grid, dim3(256), 0, st, p);
   else if (units <= 512 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 512, NU>), grid, dim3(512), 0, st, p);
   else if (units <= 1024 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 1024, NU>), grid, dim3(1024), 0, st, p);

@@ -243,7 +243,8 @@ __device__ __forceinline__ void accumulate_marginal(const MargParams& p, const c
 template <bool VEC>
 __global__ __launch_bounds__(MARG_NT) void marginalise_map_kernel(const MargParams p) {
   extern __shared__ __align__(16) float acc[];
-  const int64_t r = blockIdx.x;
+  const int64_t r = xcd_banded_row(blockIdx.x);
+  if (r >= p.n_rows) return;
   const int pb = p.p_dtype == F32 ? 4 : 2;
   const char* prow = reinterpret_cast<const char*>(p.probs) + r * p.p_stride * pb;
   float* out = p.marg + r * p.marg_stride;
@@ -312,7 +313,8 @@ template <class TagS, int NU, bool VEC>
 __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargParams p) {
   extern __shared__ __align__(16) float acc[];
   __shared__ float red[64];
-  const int64_t r = blockIdx.x;
+  const int64_t r = xcd_banded_row(blockIdx.x);
+  if (r >= p.n_srows) return;
   const int tid = threadIdx.x;
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_rows);
@@ -406,8 +408,8 @@ extern "C" int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stri
                                  (size_t)(Vs < MARG_MAX_VS ? Vs : MARG_MAX_VS) * 4);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   allow_large_lds();
-  if (vec) hipLaunchKernelGGL((marginalise_map_kernel<true>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
-  else hipLaunchKernelGGL((marginalise_map_kernel<false>), dim3((unsigned)n_rows), dim3(MARG_NT), lds, st, p);
+  if (vec) hipLaunchKernelGGL((marginalise_map_kernel<true>), dim3(xcd_banded_grid(n_rows)), dim3(MARG_NT), lds, st, p);
+  else hipLaunchKernelGGL((marginalise_map_kernel<false>), dim3(xcd_banded_grid(n_rows)), dim3(MARG_NT), lds, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
@@ -455,7 +457,7 @@ extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t
   const bool vec = p_dtype == DL_F32 && Vt % 4 == 0 && ok16(t_probs, p_stride, 4) && ok16(t2s, 0, 4);
   const size_t lds = attach_plan(p, plan_row_off, plan_ent, plan_tile, plan_fold, plan_n_fold, plan_n_extra, vec, (size_t)Vs * 4);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  const dim3 grid((unsigned)n_rows), block(MARG_NT);
+  const dim3 grid(xcd_banded_grid(n_rows)), block(MARG_NT);
   allow_large_lds();
 #define DL_LAUNCH_RKLM(TAG)                                                                                  \
   do {                                                                                                       \

@@ -424,9 +424,9 @@ void fkl_topk_reg_kernel(const TopkParams p) {
   const TopkLds s(smem, p.K);
   const int P = SPLIT ? p.parts : 1;
   const unsigned grp = SPLIT ? blockIdx.x / (8u * P) : 0u, t_in = SPLIT ? blockIdx.x % (8u * P) : 0u;
-  const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : blockIdx.x;
+  const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : xcd_banded_row(blockIdx.x);
   const int h = SPLIT ? (int)(t_in >> 3) : 0;
-  if (SPLIT && r >= p.n_rows) return;
+  if (r >= p.n_rows) return;
   fkl_topk_part<Tag, NT, NCH, SPLIT, J, false>(p, s, r, h);
 }
 
@@ -460,7 +460,8 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
   extern __shared__ __align__(16) unsigned char smem[];
   const TopkLds s(smem, p.K);
   using C = Chunk<Tag>;
-  const int64_t r = blockIdx.x;
+  const int64_t r = xcd_banded_row(blockIdx.x);
+  if (r >= p.n_rows) return;
   const int tid = threadIdx.x;
   const int64_t V = p.V;
   const int64_t nch = V / C::N;
@@ -512,7 +513,8 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const TopkLds s(smem, p.K);
   using C = Chunk<Tag>;
-  const int64_t r = blockIdx.x;
+  const int64_t r = xcd_banded_row(blockIdx.x);
+  if (r >= p.n_rows) return;
   const int tid = threadIdx.x;
   const int64_t V = p.V;
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
@@ -594,7 +596,7 @@ static void launch_retry_j(const TopkParams& p, unsigned grid, hipStream_t st) {
 
 template <class Tag, int NT, int NCH>
 static hipError_t launch_reg(const TopkParams& p, hipStream_t st) {
-  launch_reg_j<Tag, NT, NCH, false>(p, (unsigned)p.n_rows, st);
+  launch_reg_j<Tag, NT, NCH, false>(p, xcd_banded_grid(p.n_rows), st);
   return hipGetLastError();
 }
 
@@ -636,10 +638,10 @@ static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes
       if (parts == 4 && ws_ok) return launch_split<Tag, 256, 16>(p, 4, st);
       return launch_reg<Tag, 1024, 16>(p, st);
     }
-    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, true>), dim3((unsigned)p.n_rows), dim3(1024),
+    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
                        TopkLds::bytes(p.K), st, p);
   } else {
-    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, false>), dim3((unsigned)p.n_rows), dim3(1024),
+    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, false>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
                        TopkLds::bytes(p.K), st, p);
   }
   return hipGetLastError();
@@ -648,10 +650,10 @@ static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes
 template <class Tag>
 static hipError_t launch_rkl(const TopkParams& p, bool aligned, hipStream_t st) {
   if (aligned)
-    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, true>), dim3((unsigned)p.n_rows), dim3(256),
+    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
                        TopkLds::bytes(p.K), st, p);
   else
-    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, false>), dim3((unsigned)p.n_rows), dim3(256),
+    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, false>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
                        TopkLds::bytes(p.K), st, p);
   return hipGetLastError();
 }
