@@ -1,0 +1,60 @@
+"""Collected teacher data through the dataset file and back into the loss: producer kernel ->
+`DistributionStore.save_data` -> reopen -> `teachers_for_batch` (pinned host memory, storage dtypes)
+-> the batched loss.  fp16 / uint32 storage is exact for what the producer emits, so every number
+must equal the one computed from the tensors that never left the GPU."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def test_dataset_file_round_trip_feeds_the_same_loss(tmp_path):
+    import llm_distillery_amd as D
+    from llm_distillery_amd.h5_dataset import DistributionStore
+    D._lib.load()
+    g = torch.Generator().manual_seed(21)
+    B, S, V, K, T = 3, 48, 8192, 32, 1.5
+    specs = [[(2, 20), (25, 40)], [(0, 44)], [(5, 17)]]
+    lens = [40, 44, 17]
+    student = (torch.randn(B, S, V, generator=g) * 2).to(torch.bfloat16)
+    teacher = (student.float() + torch.randn(B, S, V, generator=g)).to(torch.bfloat16).to(DEV)
+    tokens = torch.randint(0, V, (B, S + 1), generator=g)
+    direct = []
+    path = str(tmp_path / "distributions.hdf5")
+    with DistributionStore(path, "w") as store:
+        store.set_vocab_family("llama_3"); store.set_topk(K)
+        for b in range(B):
+            rows = torch.as_tensor(O.content_indices(specs[b]), dtype=torch.int32).to(DEV)
+            tv, ti = D.teacher_topk(teacher[b], K, rows=rows)               # fp16 log-probs, int32 ids: the storage dtypes
+            direct.append((tv, ti))
+            lab_pos = torch.as_tensor(O.ce_indices(specs[b], 2048, lens[b])[0])
+            hit = torch.arange(len(lab_pos)) % 3 != 0                         # two labels in three lie on the teacher's support
+            tokens[b, lab_pos[hit]] = ti[:len(lab_pos), 1].cpu().long()[hit]
+            store.save_data(tv.cpu().numpy(), 100 + b, ti.cpu().numpy().astype(np.uint32), content_sha=f"s{b}", sample="")
+    index = D.BatchIndex(specs, lens, S, 2048, DEV)
+    with DistributionStore(path, "r") as store:
+        assert store.get_topk() == K and sorted(store.get_available_ids()) == [100, 101, 102]
+        from_file = store.teachers_for_batch([100, 101, 102], DEV)
+        padded, idx, pad = store.make_outgoing_batch([100, 101, 102])          # the reference's tuple gives the same tensors
+    for (tv, ti), (fv, fi) in zip(direct, from_file):
+        assert fv.dtype == torch.float16 and fi.dtype == torch.int32
+        assert torch.equal(tv, fv) and torch.equal(ti, fi)
+    via_tuple = D.teachers_from_outgoing_batch(padded, idx, pad, DEV)
+    for (tv, ti), (fv, fi) in zip(direct, via_tuple):
+        assert torch.equal(tv, fv) and torch.equal(ti, fi)
+    outs = []
+    for teachers in (direct, from_file):
+        x = student.to(DEV).requires_grad_(True)
+        dicts = D.distill_loss_batch_indexed(x, index, tokens.to(DEV), teachers, 2.0, temperature=T)
+        L = D.Losses(None)
+        vals = [{k: d[k].item() for k in D.LOSS_KEYS} for d in dicts]
+        for d in dicts:
+            L.add_losses(d)
+        L.backward(divisor=1)
+        outs.append((vals, x.grad.clone()))
+    assert outs[0][0] == outs[1][0] and torch.equal(outs[0][1], outs[1][1])
+    assert all(np.isfinite(v["train_loss"]) for v in outs[0][0])
