@@ -7,7 +7,7 @@ from . import _lib  # noqa: F401
 from .batch_index import BatchIndex, ce_rows, content_rows, teachers_from_outgoing_batch  # noqa: F401
 from .finetuning_utils import (LOSS_KEYS, calculate_divergence, distill_loss, distill_loss_batch,  # noqa: F401
                                distill_loss_batch_indexed)
-from .h5_dataset import DistributionStore  # noqa: F401
+from .h5_dataset import BatchPrefetcher, DistributionStore  # noqa: F401
 from .losses import Losses  # noqa: F401
 from .teacher_prep import fkl_multi_teacher, merge_remap_topk, merge_topk_pair, teacher_topk  # noqa: F401
 from . import vocab_utils  # noqa: F401

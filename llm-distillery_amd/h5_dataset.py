@@ -426,3 +426,98 @@ class DistributionStore:
                 og = out._group(self._key(cid))
                 og.attrs = dict(g.attrs)
                 og.dirty = True
+
+
+class BatchPrefetcher:
+    """`enqueue_get_batches` / `read_next_batch` / `read_only_mode` (classes/data_manager.py:379-398)
+    without the child process: a worker thread inflates the coming batches into pinned memory and
+    uploads them on a copy stream of its own (default priority) while the current batch trains; at
+    most `depth` batches wait.  Iterating yields, per batch, the list `teachers_for_batch` returns;
+    the consumer's current stream is made to wait for the upload, so the tensors can be used at once.
+    `loop=True` goes round the batches until `close()` (the reference's read-only mode).  The store
+    must not be written to while a prefetcher reads it."""
+
+    _END = object()
+
+    def __init__(self, store: DistributionStore, batches: Sequence[Sequence[int]], device, depth: int = 2, loop: bool = False):
+        import queue
+        import threading
+        import torch
+        self._torch = torch
+        self.store, self.batches, self.loop = store, [list(b) for b in batches], loop
+        self.device = torch.device(device)
+        self._queue: "queue.Queue" = queue.Queue(max(1, depth))
+        self._closing = threading.Event()
+        self._stream = torch.cuda.Stream(self.device) if self.device.type == "cuda" else None
+        self._thread = threading.Thread(target=self._work, name="distribution-prefetch", daemon=True)
+        self._thread.start()
+
+    def _put(self, item) -> bool:
+        import queue
+        while not self._closing.is_set():
+            try:
+                self._queue.put(item, timeout=0.05)
+                return True
+            except queue.Full:
+                continue
+        return False
+
+    def _work(self):
+        torch = self._torch
+        try:
+            while True:
+                for ids in self.batches:
+                    if self._closing.is_set():
+                        return
+                    vals, idx, counts = self.store.packed_batch(ids)
+                    if self._stream is not None:
+                        with torch.cuda.stream(self._stream):
+                            dv, di = vals.to(self.device, non_blocking=True), idx.to(self.device, non_blocking=True)
+                            ready = self._stream.record_event()
+                    else:
+                        dv, di, ready = vals, idx, None
+                    # the pinned staging tensors travel along: they must outlive the copies
+                    if not self._put((dv, di, counts, ready, (vals, idx))):
+                        return
+                if not self.loop:
+                    break
+            self._put(self._END)
+        except BaseException as e:                          # handed to the consumer, which re-raises it
+            self._put(e)
+
+    def __iter__(self):
+        return self
+
+    def __next__(self):
+        item = self._queue.get()
+        if item is self._END:
+            self._queue.put(item)                           # further calls keep ending
+            raise StopIteration
+        if isinstance(item, BaseException):
+            self._queue.put(item)
+            raise item
+        dv, di, counts, ready, _staging = item
+        if ready is not None:
+            cur = self._torch.cuda.current_stream(self.device)
+            cur.wait_event(ready)
+            dv.record_stream(cur)
+            di.record_stream(cur)
+            # the pinned staging tensors may go now: torch's host allocator holds a pinned block back
+            # until the copies that read it have finished
+        cuts = np.cumsum([0] + list(counts))
+        return [(dv[cuts[b]:cuts[b + 1]], di[cuts[b]:cuts[b + 1]]) for b in range(len(counts))]
+
+    def close(self):
+        self._closing.set()
+        while self._thread.is_alive():
+            try:
+                self._queue.get_nowait()
+            except Exception:
+                pass
+            self._thread.join(0.05)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()

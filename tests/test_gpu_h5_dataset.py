@@ -43,6 +43,10 @@ def test_dataset_file_round_trip_feeds_the_same_loss(tmp_path):
     for (tv, ti), (fv, fi) in zip(direct, from_file):
         assert fv.dtype == torch.float16 and fi.dtype == torch.int32
         assert torch.equal(tv, fv) and torch.equal(ti, fi)
+    with DistributionStore(path, "r") as store, D.BatchPrefetcher(store, [[100, 101], [102], [101, 102, 100]], DEV) as pf:
+        for ids, teachers in zip([[100, 101], [102], [101, 102, 100]], pf):      # uploaded on the prefetcher's copy stream
+            for cid, (fv, fi) in zip(ids, teachers):
+                assert fv.is_cuda and torch.equal(fv, direct[cid - 100][0]) and torch.equal(fi, direct[cid - 100][1])
     via_tuple = D.teachers_from_outgoing_batch(padded, idx, pad, DEV)
     for (tv, ti), (fv, fi) in zip(direct, via_tuple):
         assert torch.equal(tv, fv) and torch.equal(ti, fi)

@@ -5,7 +5,6 @@ round-trip; and, where an interpreter with h5py is installed (the build containe
 library must read what is written here, append to it, and have its own files appended to."""
 import gzip
 import os
-import shutil
 import subprocess
 
 import numpy as np
@@ -118,6 +117,28 @@ def test_outgoing_batch_matches_reference_layout(fixture_file, expected):
             s.packed_batch([0, 3], pin=False)
         with pytest.raises(ValueError, match="dense-mode"):
             s.packed_batch([12], pin=False)
+
+
+def test_prefetcher_yields_the_batches_in_order_and_ends(fixture_file, expected):
+    from llm_distillery_amd import BatchPrefetcher
+    batches = [[0], [7, 1299], [1299, 0, 7]]
+    with DistributionStore(fixture_file, "r", workers=2) as s:
+        with BatchPrefetcher(s, batches, "cpu", depth=1) as pf:
+            got = list(pf)
+            with pytest.raises(StopIteration):
+                next(pf)
+        assert len(got) == 3
+        for ids, teachers in zip(batches, got):
+            assert len(teachers) == len(ids)
+            for cid, (v, i) in zip(ids, teachers):
+                assert np.array_equal(_bits(v.numpy()), _bits(expected[f"d{cid}"])) and np.array_equal(i.numpy(), expected[f"i{cid}"].astype(np.int32))
+        with BatchPrefetcher(s, batches[:2], "cpu", depth=2, loop=True) as pf:      # read-only mode: round and round
+            seen = [len(next(pf)) for _ in range(7)]
+        assert seen == [1, 2, 1, 2, 1, 2, 1]
+        with BatchPrefetcher(s, [[0], [424242]], "cpu") as pf:                      # worker errors surface at the consumer
+            next(pf)
+            with pytest.raises(ValueError, match="not found"):
+                next(pf)
 
 
 # ---------------------------------------------------------------------------------------------
