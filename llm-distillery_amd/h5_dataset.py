@@ -30,6 +30,10 @@ from .h5_format import H5FormatError
 DISTR_KEY, INDICES_KEY = "distributions", "indices"
 
 
+def _to_numpy(x) -> np.ndarray:
+    return x.detach().cpu().numpy() if hasattr(x, "detach") else np.asarray(x)
+
+
 class _Group:
     __slots__ = ("address", "attrs", "members", "loaded", "dirty")
 
@@ -306,6 +310,35 @@ class DistributionStore:
             self._append(blob)
             g.members[INDICES_KEY] = addr
         g.dirty = True
+
+    def put_distribution(self, data, convo_id: int, indices, content_sha: str | None = None,
+                         sample: str | None = None, *, vocab: int, device="cuda:0"):
+        """One item of `_process_distributions` (classes/data_manager.py:180-195): a conversation that
+        is new is saved as it comes; one that is already stored is merged with what the file holds
+        (`_merge_data`, :198-261 — probabilities of shared ids add, the K largest stay, rows beyond
+        the shorter input pass through) by the GPU merge kernel, and the result replaces the stored
+        datasets while the group's attributes stay.  `data` / `indices`: [rows, K] log-probs and ids
+        (numpy or torch); `vocab`: the teachers' vocabulary size (ids must lie below it).
+        Dense-mode conversations (no `indices`) cannot be merged: the reference's own dense merge
+        fails too (it returns an unbound name), so this raises instead of guessing."""
+        import torch
+        from . import teacher_prep
+        name = self._key(convo_id)
+        if name not in self._groups:
+            self.save_data(_to_numpy(data), convo_id, None if indices is None else _to_numpy(indices), content_sha, sample)
+            return
+        if indices is None or INDICES_KEY not in self._group(name).members:
+            raise ValueError(f"Convo ID {convo_id}: dense-mode data cannot be merged")
+        disk_v, disk_i = self.load_id(convo_id, storage=True)
+        if int(disk_i.max(initial=0)) >= vocab:
+            raise ValueError(f"Convo ID {convo_id}: stored ids reach beyond a vocabulary of {vocab}")
+        dev = torch.device(device)
+        dv = torch.from_numpy(disk_v).to(dev).float()
+        di = torch.from_numpy(disk_i.view(np.int32)).to(dev)
+        nv = torch.as_tensor(_to_numpy(data)).to(dev).float()
+        ni = torch.as_tensor(_to_numpy(indices).astype(np.int32)).to(dev)
+        logmass, ids = teacher_prep.merge_topk_pair(dv, di, nv, ni, vocab)
+        self.save_data(logmass.cpu().numpy(), convo_id, ids.cpu().numpy())
 
     def clear_ids(self, ids: Iterable[int]):
         """`_clear_dataset` (classes/data_manager.py:355-367): drops the groups (missing ones are

@@ -62,3 +62,36 @@ def test_dataset_file_round_trip_feeds_the_same_loss(tmp_path):
         outs.append((vals, x.grad.clone()))
     assert outs[0][0] == outs[1][0] and torch.equal(outs[0][1], outs[1][1])
     assert all(np.isfinite(v["train_loss"]) for v in outs[0][0])
+
+
+def test_second_teacher_is_merged_into_the_stored_one(tmp_path):
+    """`put_distribution` on a stored conversation = the reference's `_merge_data` followed by
+    `_save_data`: the file then holds fp16(log(merged mass)) and the ids, rows beyond the shorter
+    teacher passed through; attributes stay."""
+    import llm_distillery_amd as D
+    from llm_distillery_amd.h5_dataset import DistributionStore
+    D._lib.load()
+    g = torch.Generator().manual_seed(5)
+    V, K = 32000, 24
+    def teacher(rows):
+        lp = torch.log_softmax(torch.randn(rows, V, generator=g) * 3, -1)
+        v, i = torch.topk(lp, K)
+        return v.to(torch.float16), i
+    av, ai = teacher(40)
+    bv, bi = teacher(33)                                   # shorter: the last 7 stored rows pass through
+    path = str(tmp_path / "distributions.hdf5")
+    with DistributionStore(path, "w") as store:
+        store.put_distribution(av.numpy(), 4, ai.numpy(), "sha4", "smp", vocab=V, device=DEV)      # new: saved as it comes
+        store.put_distribution(bv, 4, bi, "ignored", "ignored", vocab=V, device=DEV)              # stored: merged
+        with pytest.raises(ValueError, match="dense-mode"):
+            store.put_distribution(bv, 4, None, vocab=V, device=DEV)
+    rv, ri = O.merge_topk_pair(av.float().numpy(), bv.float().numpy(), ai.numpy(), bi.numpy())
+    with DistributionStore(path, "r") as store:
+        d, i = store.load_id(4, storage=True)
+        assert store.group_attrs(4) == {"content_sha": "sha4", "sample": "smp"}
+    assert d.shape == (40, K) and np.array_equal(i.astype(np.int64), ri)
+    # the merge kernel sums in fp32 like the reference; the file rounds to fp16 once
+    ref16 = rv.astype(np.float16)
+    ulp_off = np.abs(d.view(np.int16).astype(np.int32) - ref16.view(np.int16).astype(np.int32))
+    assert ulp_off.max() <= 1 and (ulp_off > 0).mean() < 0.01
+    assert np.array_equal(d[33:], av[33:].numpy()) and np.array_equal(i[33:].astype(np.int64), ai[33:].numpy())
