@@ -134,9 +134,14 @@ def calculate_divergence(student_logits: Tensor, teacher_logits: Tensor, indices
         raise TypeError("calculate_divergence needs top-K indices: the dense-teacher form of the reference "
                         "composite is not executable (use dense_divergence for dense teachers)")
     n = min(student_logits.size(0), teacher_logits.size(0), indices.size(0))
-    logits = student_logits[:n]
     idx = indices[:n]
-    lse, zk = ops.rowstats_topk(logits, idx, None, 1.0)
+    # Rows beyond n are masked through the row map instead of sliced away: the backward of a slice
+    # would zero-fill a second [N, V] buffer and copy the gradient into it.
+    row_map = None
+    if n < student_logits.size(0):
+        row_map = torch.full((student_logits.size(0),), -1, dtype=torch.int32, device=student_logits.device)
+        row_map[:n] = torch.arange(n, dtype=torch.int32, device=student_logits.device)
+    lse, zk = ops.rowstats_topk(student_logits, idx, row_map, 1.0)
     labels = convo_CE_tokens[:n]
     if _fusable([n], [labels], alpha) and teacher_logits.dtype in ops._DT:
         return _fused_dicts(lse, zk, [n], [teacher_logits[:n]], [idx], [labels], [avoid_indices], 1.0, alpha)[0]

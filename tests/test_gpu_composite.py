@@ -68,6 +68,26 @@ def test_calculate_divergence_against_oracle_fp32(D, V, K, N):
     assert (err <= O.storage_tolerance(ref_in.grad, torch.float32, 1e-4)).all()
 
 
+def test_student_rows_beyond_the_teacher_are_dropped_with_zero_gradient(D):
+    """utils/finetuning_utils.py:87-88: only the first min(#student, #teacher, #indices) rows count.
+    The extra student rows are masked inside the kernels (no slice of the [N, V] logits, whose
+    backward would cost a zero fill and a copy of that size); their gradient rows are zero."""
+    student, tv, ti, labels = _convo(30, 4096, 16, 8)
+    n = 23
+    avoid = torch.tensor([4])
+    ref_in = student.double().requires_grad_(True)
+    ref = O.calculate_divergence(ref_in, tv[:n].double(), ti[:n], labels[:n - 1], 2.0, avoid)
+    ref["train_loss"].backward()
+    s = student.to(DEV).requires_grad_(True)
+    res = D.calculate_divergence(s, tv[:n].to(DEV), ti[:n].to(DEV), labels[:n - 1].to(DEV), 2.0, avoid.to(DEV))
+    for k in D.LOSS_KEYS:
+        np.testing.assert_allclose(res[k].item(), ref[k].item(), rtol=1e-5, atol=1e-6, err_msg=k)
+    res["train_loss"].backward()
+    assert s.grad.shape == student.shape and torch.count_nonzero(s.grad[n:]) == 0
+    err = (s.grad.cpu().double() - ref_in.grad).abs()
+    assert (err <= O.storage_tolerance(ref_in.grad, torch.float32, 1e-4)).all()
+
+
 def test_under_no_grad_and_reference_error_behaviour(D):
     student, tv, ti, labels = _convo(12, 512, 8, 6)
     with torch.no_grad():
