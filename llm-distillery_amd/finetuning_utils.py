@@ -161,12 +161,12 @@ def distill_loss(model_logits: Tensor, content_rows: Tensor, teacher_logprobs: T
     `teacher_temperature=1` reproduces the validation loop, which scales only the student
     (classes/student/model.py:501-502).
     """
-    x = model_logits if crop_to_size is None else model_logits[:, :crop_to_size]
+    x = model_logits
     S = x.shape[0]
     n = min(content_rows.numel(), teacher_logprobs.size(0), indices.size(0))
     row_map = torch.full((S,), -1, dtype=torch.int32, device=x.device)
     row_map[content_rows[:n].long()] = torch.arange(n, dtype=torch.int32, device=x.device)
-    lse, zk = ops.rowstats_topk(x, indices[:n], row_map, 1.0 / temperature)
+    lse, zk = ops.rowstats_topk(x, indices[:n], row_map, 1.0 / temperature, int(crop_to_size or 0))
     tT = temperature if teacher_temperature is None else teacher_temperature
     labels = convo_CE_tokens[:n]
     if _fusable([n], [labels], alpha) and teacher_logprobs.dtype in ops._DT:
@@ -201,7 +201,7 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
     B, S, _ = model_logits.shape
     if len(convos) != B:
         raise ValueError(f"{len(convos)} conversations for a batch of {B} sequences")
-    x = model_logits if crop_to_size is None else model_logits[:, :, :crop_to_size]
+    x = model_logits
     dev = x.device
     counts = [min(rows.numel(), t_lp.size(0), idx.size(0)) for rows, t_lp, idx, _, _ in convos]
     if row_map is None or row_map.numel() != B * S or any(n != rows.numel() for n, (rows, *_) in zip(counts, convos)):
@@ -211,7 +211,7 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
             row_map[b * S + rows[:n].long()] = torch.arange(base, base + n, dtype=torch.int32, device=dev)
             base += n
     idx_cat = _packed_rows([idx[:n] for (_, _, idx, _, _), n in zip(convos, counts)])
-    lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature)
+    lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature, int(crop_to_size or 0))
     tT = temperature if teacher_temperature is None else teacher_temperature
     labels_all = [labels[:n] for (_, _, _, labels, _), n in zip(convos, counts)]
     if _fusable(counts, labels_all, alpha) and all(c[1].dtype in ops._DT for c in convos):

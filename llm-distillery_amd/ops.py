@@ -169,15 +169,17 @@ def _rowstats_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float):
 
 
 def _rowcoef_grad_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float, lse: torch.Tensor,
-                      g_lse: torch.Tensor, g_zk: torch.Tensor) -> torch.Tensor:
-    """Phase 2 launch: d L / d x from dL/d lse and dL/d zk."""
+                      g_lse: torch.Tensor, g_zk: torch.Tensor, grad_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Phase 2 launch: d L / d x from dL/d lse and dL/d zk (into `grad_out` [R, V], dense along V, if given)."""
     t_idx = t_idx.contiguous()
     R, V = x.shape
     N, K = t_idx.shape
     _, rm_ptr = _opt_i32(row_map, R, "row_map", x.device)
     g_lse = g_lse.to(torch.float32).contiguous()
     g_zk = g_zk.to(torch.float32).contiguous()
-    grad = torch.empty((R, V), dtype=x.dtype, device=x.device)
+    grad = grad_out if grad_out is not None else torch.empty((R, V), dtype=x.dtype, device=x.device)
+    if grad.shape != (R, V) or grad.dtype != x.dtype or grad.stride(1) != 1:
+        raise RuntimeError("grad_out must match the logits in shape and dtype and be dense along V")
     with torch.cuda.device(x.device):
         st = _lib.load().dl_rowcoef_grad_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(),
                                               _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), g_lse.data_ptr(),
@@ -187,37 +189,51 @@ def _rowcoef_grad_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: floa
     return grad
 
 
+def _cropped(logits: torch.Tensor, crop: int) -> torch.Tensor:
+    return logits[:, :crop] if 0 < crop < logits.shape[1] else logits
+
+
 @torch.library.custom_op("distillery_amd::rowstats_topk", mutates_args=())
 def rowstats_topk(logits: torch.Tensor, t_idx: torch.Tensor, row_map: Optional[torch.Tensor],
-                  inv_T: float) -> Tuple[torch.Tensor, torch.Tensor]:
+                  inv_T: float, crop: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
     """(lse [N] fp32, zk [N, K] fp32): full-vocabulary log-sum-exp of logits * inv_T and the scaled
-    logits at the teacher ids, for the rows selected by row_map.  Differentiable w.r.t. logits."""
-    return _rowstats_raw(logits, t_idx, row_map, inv_T)
+    logits at the teacher ids, for the rows selected by row_map.  Differentiable w.r.t. logits.
+    `crop` > 0 uses only the first `crop` columns (the reference's `[:, :, :crop_to_size]`,
+    classes/student/model.py:408) without a slice in the autograd graph, whose backward would
+    zero-fill and copy a second full-width gradient buffer."""
+    return _rowstats_raw(_cropped(logits, crop), t_idx, row_map, inv_T)
 
 
 @rowstats_topk.register_fake
-def _(logits, t_idx, row_map, inv_T):
+def _(logits, t_idx, row_map, inv_T, crop=0):
     N, K = t_idx.shape
     return (logits.new_empty((N,), dtype=torch.float32), logits.new_empty((N, K), dtype=torch.float32))
 
 
 @torch.library.custom_op("distillery_amd::rowcoef_grad_topk", mutates_args=())
 def rowcoef_grad_topk(logits: torch.Tensor, t_idx: torch.Tensor, row_map: Optional[torch.Tensor], inv_T: float,
-                      lse: torch.Tensor, g_lse: torch.Tensor, g_zk: torch.Tensor) -> torch.Tensor:
-    return _rowcoef_grad_raw(logits, t_idx, row_map, inv_T, lse, g_lse, g_zk)
+                      lse: torch.Tensor, g_lse: torch.Tensor, g_zk: torch.Tensor, crop: int = 0) -> torch.Tensor:
+    x = _cropped(logits, crop)
+    if x is logits:
+        return _rowcoef_grad_raw(logits, t_idx, row_map, inv_T, lse, g_lse, g_zk)
+    grad = torch.empty_like(logits)                      # full width; the kernel fills [:, :crop]
+    grad[:, crop:].zero_()
+    _rowcoef_grad_raw(x, t_idx, row_map, inv_T, lse, g_lse, g_zk, grad_out=grad[:, :crop])
+    return grad
 
 
 @rowcoef_grad_topk.register_fake
-def _(logits, t_idx, row_map, inv_T, lse, g_lse, g_zk):
+def _(logits, t_idx, row_map, inv_T, lse, g_lse, g_zk, crop=0):
     return torch.empty_like(logits)
 
 
 def _rowstats_setup(ctx, inputs, output):
-    logits, t_idx, row_map, inv_T = inputs
+    logits, t_idx, row_map, inv_T, crop = inputs
     lse, _ = output
     ctx.save_for_backward(logits, t_idx, lse, *([row_map] if row_map is not None else []))
     ctx.has_map = row_map is not None
     ctx.inv_T = inv_T
+    ctx.crop = crop
 
 
 def _rowstats_backward(ctx, g_lse, g_zk):
@@ -228,7 +244,7 @@ def _rowstats_backward(ctx, g_lse, g_zk):
         g_lse = torch.zeros_like(lse)
     if g_zk is None:
         g_zk = torch.zeros((t_idx.shape[0], t_idx.shape[1]), dtype=torch.float32, device=lse.device)
-    return rowcoef_grad_topk(logits, t_idx, row_map, ctx.inv_T, lse, g_lse, g_zk), None, None, None
+    return rowcoef_grad_topk(logits, t_idx, row_map, ctx.inv_T, lse, g_lse, g_zk, ctx.crop), None, None, None, None
 
 
 rowstats_topk.register_autograd(_rowstats_backward, setup_context=_rowstats_setup)
