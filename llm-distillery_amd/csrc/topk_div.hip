@@ -93,8 +93,13 @@ struct TopkLds {
   float* t;          // Kp  scaled teacher logit -> teacher log-probability over the K entries
   float* q;          // Kp  teacher probability
   float* z;          // Kp  gathered student logit
+  // in-register corrections (kernels that keep the row in registers; owners == 0 elsewhere):
+  float* val;        // Kp  final gradient value at the entry's column
+  int* next;         // Kp  next entry owned by the same thread, or -1
+  int* head;         // one per thread: first entry inside the thread's chunks, or -1
+  unsigned* own;     // one per thread: bit i set = chunk i of the thread holds an entry
   int Kp;
-  __device__ TopkLds(unsigned char* base, int K) {
+  __device__ TopkLds(unsigned char* base, int K, int owners = 0) {
     Kp = (K + 15) & ~15;
     red = reinterpret_cast<float*>(base);
     xm = red + 64; xs = xm + MAX_PARTS; xb = xs + MAX_PARTS; xok = reinterpret_cast<int*>(xb + MAX_PARTS);
@@ -102,8 +107,15 @@ struct TopkLds {
     t = reinterpret_cast<float*>(idx + Kp);
     q = t + Kp;
     z = q + Kp;
+    val = z + Kp;
+    next = reinterpret_cast<int*>(val + Kp);
+    head = next + Kp;
+    own = reinterpret_cast<unsigned*>(head + owners);
   }
-  __host__ __device__ static size_t bytes(int K) { return 512 + (size_t)((K + 15) & ~15) * 16; }
+  __host__ __device__ static size_t bytes(int K, int owners = 0) {
+    const size_t Kp = (size_t)((K + 15) & ~15);
+    return 512 + Kp * 16 + (owners ? Kp * 8 + (size_t)owners * 8 : 0);
+  }
 };
 
 // Teacher entries of one row held in registers between issue and use: J entries per thread,
@@ -249,6 +261,43 @@ __device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int
   }
 }
 
+// The same corrections for a row (part) held in registers, applied before the dense store instead of
+// after it: a 2-byte store into a line whose 16-byte stores are still on their way costs the memory
+// system a read-modify-write of the line and the workgroup a wait for the dense stores to land.
+// Step 1 (entry threads): final value of every entry inside [lo, hi) into s.val, the entry linked
+// into the list of the thread that holds its chunk (chunk c of the part sits in register
+// c / NT of thread c % NT), that thread's chunk mask updated.  Entries that share an id all carry
+// the same value, so the order in which a list is walked does not matter.
+template <class Tag, int NT>
+__device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, int hi, float a, float b, float c,
+                                                     bool ids_unique) {
+  using C = Chunk<Tag>;
+  for (int k = threadIdx.x; k < s.Kp; k += NT) {
+    const int id = s.idx[k];
+    if (id < lo || id >= hi) continue;
+    const float q = ids_unique ? s.q[k] : mass_on_id(s, k, id);
+    s.val[k] = (fast_exp2(fmaf(s.z[k], a, -b)) - q) * c;
+    const int crel = (id - lo) / C::N;
+    const int owner = crel % NT;
+    s.next[k] = atomicExch(&s.head[owner], k);
+    atomicOr(&s.own[owner], 1u << (crel / NT));
+  }
+}
+
+// Step 2 (owner thread, chunk i, f = the chunk's gradient values about to be packed).
+template <class Tag, int NT>
+__device__ __forceinline__ void fkl_apply_corrections(const TopkLds& s, int lo, int i, float (&f)[Chunk<Tag>::N]) {
+  using C = Chunk<Tag>;
+  for (int k = s.head[threadIdx.x]; k >= 0; k = s.next[k]) {
+    const int off = s.idx[k] - lo;
+    if (off / (C::N * NT) != i) continue;
+    const int e = off % C::N;
+    const float v = s.val[k];
+#pragma unroll
+    for (int j = 0; j < C::N; ++j) f[j] = (j == e) ? v : f[j];
+  }
+}
+
 // Full-row statistics straight from global memory (two uses: the streaming kernel, and a split
 // part whose partner did not answer in time).  Returns the row maximum and sum 2^((x - max) a).
 template <class Tag, int NT, bool VEC>
@@ -311,6 +360,8 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
   const char* rpart = row + c0 * 16;
 
+  s.head[tid] = -1;                   // own list of corrections, filled after the row statistics
+  s.own[tid] = 0u;
   TeacherEntries<(J > 0 ? J : 1)> te;
   if constexpr (J > 0) teacher_issue<NT, J>(p, trow, te);
   u32x4 reg[NCH];
@@ -400,6 +451,9 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   if (gpart) {
     const float c = p.inv_T_s * p.grad_scale;
     const float kc = fast_exp2(mb_own - b) * c;       // stashed value -> gradient
+    fkl_link_corrections<Tag, NT>(s, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
+    __syncthreads();
+    const unsigned mine = s.own[tid];
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = (int64_t)i * NT + tid;
@@ -409,11 +463,10 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
         C::unstash(reg[i], f);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
+        if (mine & (1u << i)) fkl_apply_corrections<Tag, NT>(s, lo, i, f);
         store16_stream(gpart + ch * 16, C::pack(f));
       }
     }
-    __syncthreads();      // dense stores are ordered before the sparse corrections
-    fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
   }
 }
 
@@ -421,7 +474,7 @@ template <class Tag, int NT, int NCH, bool SPLIT, int J>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))     // <= 128 VGPRs: 16 waves per CU
 void fkl_topk_reg_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K);
+  const TopkLds s(smem, p.K, NT);
   const int P = SPLIT ? p.parts : 1;
   const unsigned grp = SPLIT ? blockIdx.x / (8u * P) : 0u, t_in = SPLIT ? blockIdx.x % (8u * P) : 0u;
   const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : xcd_banded_row(blockIdx.x);
@@ -442,7 +495,7 @@ template <class Tag, int NT, int NCH, int J>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void fkl_topk_retry_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K);
+  const TopkLds s(smem, p.K, NT);
   const RetryList list(p.workspace, p.n_rows, p.parts);
   const unsigned n = *list.count;
 #pragma unroll 1
@@ -579,7 +632,7 @@ __global__ __launch_bounds__(256) void clear_workspace_kernel(u32x4* ws, int64_t
 template <class Tag, int NT, int NCH, bool SPLIT>
 static void launch_reg_j(const TopkParams& p, unsigned grid, hipStream_t st) {
   const int Kp = (p.K + 15) & ~15;
-  const size_t lds = TopkLds::bytes(p.K);
+  const size_t lds = TopkLds::bytes(p.K, NT);
   if (Kp <= NT) hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 1>), dim3(grid), dim3(NT), lds, st, p);
   else if (Kp <= 3 * NT) hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 3>), dim3(grid), dim3(NT), lds, st, p);
   else hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 0>), dim3(grid), dim3(NT), lds, st, p);
@@ -588,7 +641,7 @@ static void launch_reg_j(const TopkParams& p, unsigned grid, hipStream_t st) {
 template <class Tag, int NT, int NCH>
 static void launch_retry_j(const TopkParams& p, unsigned grid, hipStream_t st) {
   const int Kp = (p.K + 15) & ~15;
-  const size_t lds = TopkLds::bytes(p.K);
+  const size_t lds = TopkLds::bytes(p.K, NT);
   if (Kp <= NT) hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 1>), dim3(grid), dim3(NT), lds, st, p);
   else if (Kp <= 3 * NT) hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 3>), dim3(grid), dim3(NT), lds, st, p);
   else hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 0>), dim3(grid), dim3(NT), lds, st, p);

@@ -21,14 +21,18 @@ class Losses:
         self.num_steps_accumulated = 0
 
     def add_losses(self, new_losses: dict[str, torch.Tensor]) -> None:
-        """Every key except `train_loss` is detached and cloned; the first dict is adopted, later
-        ones are added key by key.  Raises ValueError on an empty dict."""
+        """Every key except `train_loss` is cut from the autograd graph; the first dict is adopted,
+        later ones are added key by key (out of place).  Raises ValueError on an empty dict.
+        The reference clones as well as detaches (classes/losses.py:35-37); a value that carries no
+        graph is only aliased here, since nothing in this class writes into a stored value and a copy
+        kernel per key and conversation is most of the host-side cost of a small batch."""
         if not new_losses:
             raise ValueError("No losses to add to the loss dictionary.")
         self.num_steps_accumulated += 1
         for key in list(new_losses):
             if key != "train_loss":
-                new_losses[key] = new_losses[key].clone().detach()
+                v = new_losses[key]
+                new_losses[key] = v.detach().clone() if v.requires_grad else v.detach()
         if not self.loss_dict:
             self.loss_dict = new_losses
             return
