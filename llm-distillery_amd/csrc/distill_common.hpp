@@ -144,6 +144,41 @@ __device__ __forceinline__ void store16_stream(void* p, const u32x4& v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
+// ---- sparse corrections of a row (part) held in registers -------------------------------------------
+// A few columns of a row get a value other than the dense formula's.  Writing them with 2-byte stores
+// after the dense 16-byte stores costs the memory system a read-modify-write of every touched line
+// and the workgroup a wait for its dense stores to land; instead the thread that holds a column's
+// chunk in its registers replaces the value before it stores the chunk.  Chunk c of the part
+// (column offset / Chunk::N) sits in register c / NT of thread c % NT.
+//   correction_link:  called by whoever computed entry k's final value: links k into the list of the
+//                     owning thread (head[owner] -> k -> next[k] ...) and marks the chunk in own[owner].
+//   correction_apply: called by the owner for its chunk i when bit i % 32 of own[] is set: walks its
+//                     list and overwrites the element of every entry that falls into chunk i.
+// head[] = -1 and own[] = 0 must be set (each thread its own slot) and a barrier passed before the
+// first link; a barrier separates the links from the applies.  Entries that share a column must
+// carry the same value: list order is arbitrary.
+template <class Tag, int NT>
+__device__ __forceinline__ void correction_link(int* head, unsigned* own, int* next, int k, int offset) {
+  const int c = offset / Chunk<Tag>::N;
+  const int owner = c % NT;
+  next[k] = atomicExch(&head[owner], k);
+  atomicOr(&own[owner], 1u << ((c / NT) & 31));
+}
+
+template <class Tag, int NT>
+__device__ __forceinline__ void correction_apply(const int* head, const int* next, const int* col, const float* val,
+                                                 int lo, int i, float (&f)[Chunk<Tag>::N]) {
+  using C = Chunk<Tag>;
+  for (int k = head[threadIdx.x]; k >= 0; k = next[k]) {
+    const int off = col[k] - lo;
+    if (off / (C::N * NT) != i) continue;
+    const int e = off % C::N;
+    const float v = val[k];
+#pragma unroll
+    for (int j = 0; j < C::N; ++j) f[j] = (j == e) ? v : f[j];
+  }
+}
+
 // ---- workgroup id -> row ---------------------------------------------------------------------------
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  For kernels that give a whole row to
 // one workgroup this mapping makes every XCD work on 8 consecutive rows (one contiguous stretch of the

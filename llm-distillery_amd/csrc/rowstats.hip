@@ -75,6 +75,22 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
 
 // ---- phase 2 -------------------------------------------------------------------------------
 // One workgroup per (row, column part of NT*NCH chunks).
+// Coefficient on the id of entry k, summed over every entry of the row that carries the same id
+// (ids of a row may repeat: each such entry then yields the same total).
+__device__ __forceinline__ float coef_on_id(const int* s_idx, const float* s_c, int Kp, int k, int id) {
+  const int4* ids4 = reinterpret_cast<const int4*>(s_idx);
+  int same = 0;
+#pragma unroll 4
+  for (int j = 0; j < Kp / 4; ++j) {
+    const int4 q = ids4[j];
+    same += (q.x == id) + (q.y == id) + (q.z == id) + (q.w == id);
+  }
+  if (same == 1) return s_c[k];
+  float cs = 0.f;
+  for (int j = 0; j < Kp; ++j) cs += (s_idx[j] == id) ? s_c[j] : 0.f;
+  return cs;
+}
+
 template <class Tag, int NT, int NCH, bool VEC>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void rowcoef_grad_kernel(const StatsParams p, int parts) {
@@ -84,6 +100,10 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
   int* s_idx = reinterpret_cast<int*>(smem);
   float* s_c = reinterpret_cast<float*>(s_idx + Kp);
   float* s_z = s_c + Kp;
+  float* s_val = s_z + Kp;                         // VEC: final value at the entry's column, owner lists
+  int* s_next = reinterpret_cast<int*>(s_val + Kp);
+  int* s_head = s_next + Kp;
+  unsigned* s_own = reinterpret_cast<unsigned*>(s_head + NT);
   // Workgroup ids are dealt round-robin to the 8 XCDs: within a group of 8 * parts ids, id t serves
   // row 8 * group + t % 8, part t / 8, so the parts of a row run on one XCD back to back.
   const unsigned grp = blockIdx.x / (8u * parts), t_in = blockIdx.x % (8u * parts);
@@ -128,7 +148,19 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
       v[i] = ch < c_hi ? load16_stream(row + ch * 16) : C::neg_inf();
     }
+    s_head[tid] = -1;
+    s_own[tid] = 0u;
     stage();
+    __syncthreads();
+    // final values of the columns that carry a teacher entry, handed to the threads that hold them
+    for (int k = tid; k < Kp; k += NT) {
+      const int id = s_idx[k];
+      if (id < 0) continue;
+      s_val[k] = fast_exp2(fmaf(s_z[k], a, -b)) * w + coef_on_id(s_idx, s_c, Kp, k, id) * p.inv_T;
+      correction_link<Tag, NT>(s_head, s_own, s_next, k, id - (int)lo);
+    }
+    __syncthreads();
+    const unsigned mine = s_own[tid];
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
@@ -137,32 +169,22 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
         C::unpack(v[i], f);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * w;
+        if (mine & (1u << i)) correction_apply<Tag, NT>(s_head, s_next, s_idx, s_val, (int)lo, i, f);
         store16_stream(grow + ch * 16, C::pack(f));
       }
     }
+    return;
   } else {
     stage();
     for (int64_t j = lo + tid; j < hi; j += NT)
       store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * w);
   }
   __syncthreads();          // LDS entries staged; dense stores ordered before the sparse additions
-  const int4* ids4 = reinterpret_cast<const int4*>(s_idx);
   for (int k = tid; k < Kp; k += NT) {
     const int id = s_idx[k];
     if (id < 0) continue;
-    int same = 0;             // ids of a row may repeat: every entry with this id contributes, all write the same total
-#pragma unroll 4
-    for (int j = 0; j < Kp / 4; ++j) {
-      const int4 q = ids4[j];
-      same += (q.x == id) + (q.y == id) + (q.z == id) + (q.w == id);
-    }
-    float cs = s_c[k];
-    if (same != 1) {
-      cs = 0.f;
-      for (int j = 0; j < Kp; ++j) cs += (s_idx[j] == id) ? s_c[j] : 0.f;
-    }
     const float dense = fast_exp2(fmaf(s_z[k], a, -b)) * w;
-    store_from_float(grow, Tag::id, id, dense + cs * p.inv_T);
+    store_from_float(grow, Tag::id, id, dense + coef_on_id(s_idx, s_c, Kp, k, id) * p.inv_T);
   }
 }
 
@@ -182,7 +204,7 @@ static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
   constexpr int NT = 256, NCH = 16;
   const int64_t per_part = (int64_t)NT * NCH * Tag::epc;
   const int parts = (int)((p.V + per_part - 1) / per_part);
-  const size_t lds = (size_t)((p.K + 15) & ~15) * 12;
+  const size_t lds = (size_t)((p.K + 15) & ~15) * 20 + (size_t)NT * 8;      // ids, coefficients, logits, values, links; heads, masks
   const dim3 grid((unsigned)((p.n_rows + 7) / 8 * 8 * parts));
   if (vec) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, true>), grid, dim3(NT), lds, st, p, parts);
   else hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, false>), grid, dim3(NT), lds, st, p, parts);

@@ -261,40 +261,18 @@ __device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int
   }
 }
 
-// The same corrections for a row (part) held in registers, applied before the dense store instead of
-// after it: a 2-byte store into a line whose 16-byte stores are still on their way costs the memory
-// system a read-modify-write of the line and the workgroup a wait for the dense stores to land.
-// Step 1 (entry threads): final value of every entry inside [lo, hi) into s.val, the entry linked
-// into the list of the thread that holds its chunk (chunk c of the part sits in register
-// c / NT of thread c % NT), that thread's chunk mask updated.  Entries that share an id all carry
-// the same value, so the order in which a list is walked does not matter.
+// The same corrections for a row (part) held in registers, applied by the threads that hold the
+// columns before they store them (correction_link / correction_apply): final value of every entry
+// inside [lo, hi) into s.val, the entry linked into its owner's list.
 template <class Tag, int NT>
 __device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, int hi, float a, float b, float c,
                                                      bool ids_unique) {
-  using C = Chunk<Tag>;
   for (int k = threadIdx.x; k < s.Kp; k += NT) {
     const int id = s.idx[k];
     if (id < lo || id >= hi) continue;
     const float q = ids_unique ? s.q[k] : mass_on_id(s, k, id);
     s.val[k] = (fast_exp2(fmaf(s.z[k], a, -b)) - q) * c;
-    const int crel = (id - lo) / C::N;
-    const int owner = crel % NT;
-    s.next[k] = atomicExch(&s.head[owner], k);
-    atomicOr(&s.own[owner], 1u << (crel / NT));
-  }
-}
-
-// Step 2 (owner thread, chunk i, f = the chunk's gradient values about to be packed).
-template <class Tag, int NT>
-__device__ __forceinline__ void fkl_apply_corrections(const TopkLds& s, int lo, int i, float (&f)[Chunk<Tag>::N]) {
-  using C = Chunk<Tag>;
-  for (int k = s.head[threadIdx.x]; k >= 0; k = s.next[k]) {
-    const int off = s.idx[k] - lo;
-    if (off / (C::N * NT) != i) continue;
-    const int e = off % C::N;
-    const float v = s.val[k];
-#pragma unroll
-    for (int j = 0; j < C::N; ++j) f[j] = (j == e) ? v : f[j];
+    correction_link<Tag, NT>(s.head, s.own, s.next, k, id - lo);
   }
 }
 
@@ -463,7 +441,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
         C::unstash(reg[i], f);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
-        if (mine & (1u << i)) fkl_apply_corrections<Tag, NT>(s, lo, i, f);
+        if (mine & (1u << i)) correction_apply<Tag, NT>(s.head, s.next, s.idx, s.val, lo, i, f);
         store16_stream(gpart + ch * 16, C::pack(f));
       }
     }
@@ -564,7 +542,7 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
 template <class Tag, int NT, bool VEC>
 __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K);
+  const TopkLds s(smem, p.K, NT);
   using C = Chunk<Tag>;
   const int64_t r = xcd_banded_row(blockIdx.x);
   if (r >= p.n_rows) return;
@@ -573,11 +551,13 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  s.head[tid] = -1;
+  s.own[tid] = 0u;
   float tlse = -INFINITY;
   if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
-  // The zero fill comes after the K logits have been gathered (stage_teacher ends in barriers), so
+  // Every store comes after the K logits have been gathered (stage_teacher ends in barriers), so
   // the gradient may be written over the logits.
-  if (grow) {
+  if (grow && (!VEC || tlse == -INFINITY)) {
     if (VEC) zero_row<Tag, NT>(grow, V / C::N);
     else for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
   }
@@ -609,13 +589,31 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   if (tid == 0 && p.row_loss) p.row_loss[r] = rkl;
   if (grow) {
     const float c = p.inv_T_s * p.grad_scale;
-    __syncthreads();    // zero fill precedes the sparse values
+    __syncthreads();    // zero fill precedes the sparse values (scalar path); s.q / s.z complete
     for (int k = tid; k < s.Kp; k += NT) {
       const int id = s.idx[k];
       if (id < 0) continue;
       float g = 0.f;
       for (int j = 0; j < s.Kp; ++j) g += (s.idx[j] == id) ? s.q[j] * (s.z[j] - rkl) : 0.f;
-      store_from_float(grow, Tag::id, id, g * c);
+      if (VEC) {
+        s.val[k] = g * c;             // placed by the thread that writes the column's chunk
+        correction_link<Tag, NT>(s.head, s.own, s.next, k, id);
+      } else {
+        store_from_float(grow, Tag::id, id, g * c);
+      }
+    }
+    if (VEC) {
+      // the row of zeros, each chunk written once with the support's values already in place
+      __syncthreads();
+      const unsigned mine = s.own[tid];
+      const int64_t nch = V / C::N;
+      for (int64_t ch = tid, i = 0; ch < nch; ch += NT, ++i) {
+        float f[C::N];
+#pragma unroll
+        for (int e = 0; e < C::N; ++e) f[e] = 0.f;
+        if (mine & (1u << (i & 31))) correction_apply<Tag, NT>(s.head, s.next, s.idx, s.val, 0, (int)i, f);
+        store16_stream(grow + ch * 16, C::pack(f));
+      }
     }
   }
 }
@@ -704,10 +702,10 @@ template <class Tag>
 static hipError_t launch_rkl(const TopkParams& p, bool aligned, hipStream_t st) {
   if (aligned)
     hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
-                       TopkLds::bytes(p.K), st, p);
+                       TopkLds::bytes(p.K, 256), st, p);
   else
     hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, false>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
-                       TopkLds::bytes(p.K), st, p);
+                       TopkLds::bytes(p.K, 256), st, p);
   return hipGetLastError();
 }
 
