@@ -150,32 +150,69 @@ __device__ __forceinline__ void store16_stream(void* p, const u32x4& v) {
 // and the workgroup a wait for its dense stores to land; instead the thread that holds a column's
 // chunk in its registers replaces the value before it stores the chunk.  Chunk c of the part
 // (column offset / Chunk::N) sits in register c / NT of thread c % NT.
-//   correction_link:  called by whoever computed entry k's final value: links k into the list of the
-//                     owning thread (head[owner] -> k -> next[k] ...) and marks the chunk in own[owner].
-//   correction_apply: called by the owner for its chunk i when bit i % 32 of own[] is set: walks its
-//                     list and overwrites the element of every entry that falls into chunk i.
-// head[] = -1 and own[] = 0 must be set (each thread its own slot) and a barrier passed before the
-// first link; a barrier separates the links from the applies.  Entries that share a column must
-// carry the same value: list order is arbitrary.
-template <class Tag, int NT>
-__device__ __forceinline__ void correction_link(int* head, unsigned* own, int* next, int k, int offset) {
-  const int c = offset / Chunk<Tag>::N;
-  const int owner = c % NT;
-  next[k] = atomicExch(&head[owner], k);
-  atomicOr(&own[owner], 1u << ((c / NT) & 31));
+//   correction_link:  called by whoever staged entry k: links k into the list of its chunk
+//                     (head[slot] -> k -> next[k] ...) and marks the chunk in own[owner].  There are
+//                     CORRECTION_HEADS list heads per workgroup, CORRECTION_HEADS / NT per thread:
+//                     chunks i and i + CORRECTION_HEADS / NT of a thread share a list.
+//   correction_apply: called by the owner for its chunk i when bit i % 32 of own[] is set: walks the
+//                     chunk's list and overwrites the element of every entry that falls into chunk i
+//                     with value(k, shared, first); `shared` tells that another entry names the same
+//                     column (entries of one column all sit in the list that starts at `first`), in
+//                     which case value() must return what all of them together make of the column,
+//                     summed in an order that does not depend on the list's, which the atomics leave
+//                     open (correction_shared_sum).  `check_shared` false skips that test (the caller
+//                     knows that no column repeats).
+// correction_clear (all threads) and a barrier come before the first link; a barrier separates the
+// links from the applies.
+constexpr int CORRECTION_HEADS = 2048;
+
+template <int NT>
+__device__ __forceinline__ void correction_clear(int* head, unsigned* own) {
+#pragma unroll
+  for (int j = 0; j < CORRECTION_HEADS / NT; ++j) head[j * NT + threadIdx.x] = -1;
+  own[threadIdx.x] = 0u;
 }
 
 template <class Tag, int NT>
-__device__ __forceinline__ void correction_apply(const int* head, const int* next, const int* col, const float* val,
-                                                 int lo, int i, float (&f)[Chunk<Tag>::N]) {
+__device__ __forceinline__ void correction_link(int* head, unsigned* own, int* next, int k, int offset) {
+  const int c = offset / Chunk<Tag>::N;
+  const int owner = c % NT, i = c / NT;
+  next[k] = atomicExch(&head[(i % (CORRECTION_HEADS / NT)) * NT + owner], k);
+  atomicOr(&own[owner], 1u << (i & 31));
+}
+
+template <class Tag, int NT, class Value>
+__device__ __forceinline__ void correction_apply(const int* head, const int* next, const int* col, int lo, int i,
+                                                 bool check_shared, float (&f)[Chunk<Tag>::N], Value value) {
   using C = Chunk<Tag>;
-  for (int k = head[threadIdx.x]; k >= 0; k = next[k]) {
+  const int first = head[(i % (CORRECTION_HEADS / NT)) * NT + threadIdx.x];
+  for (int k = first; k >= 0; k = next[k]) {
     const int off = col[k] - lo;
     if (off / (C::N * NT) != i) continue;
+    bool shared = false;
+    if (check_shared)
+      for (int j = first; j >= 0; j = next[j]) shared = shared || (j != k && col[j] == col[k]);
     const int e = off % C::N;
-    const float v = val[k];
+    const float v = value(k, shared, first);
 #pragma unroll
     for (int j = 0; j < C::N; ++j) f[j] = (j == e) ? v : f[j];
+  }
+}
+
+// Sum of term(j) over the entries j of the list starting at `first` that name the column of entry
+// k, taken in ascending j: the same bits whatever order the list happens to have.  Lists are a
+// few entries long.
+template <class Term>
+__device__ __forceinline__ float correction_shared_sum(const int* next, const int* col, int first, int k, Term term) {
+  float sum = 0.f;
+  int last = -1;
+  while (true) {
+    int pick = 0x7fffffff;
+    for (int j = first; j >= 0; j = next[j])
+      if (j > last && j < pick && col[j] == col[k]) pick = j;
+    if (pick == 0x7fffffff) return sum;
+    sum += term(pick);
+    last = pick;
   }
 }
 

@@ -103,7 +103,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
   float* s_val = s_z + Kp;                         // VEC: final value at the entry's column, owner lists
   int* s_next = reinterpret_cast<int*>(s_val + Kp);
   int* s_head = s_next + Kp;
-  unsigned* s_own = reinterpret_cast<unsigned*>(s_head + NT);
+  unsigned* s_own = reinterpret_cast<unsigned*>(s_head + CORRECTION_HEADS);
   // Workgroup ids are dealt round-robin to the 8 XCDs: within a group of 8 * parts ids, id t serves
   // row 8 * group + t % 8, part t / 8, so the parts of a row run on one XCD back to back.
   const unsigned grp = blockIdx.x / (8u * parts), t_in = blockIdx.x % (8u * parts);
@@ -148,15 +148,14 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
       v[i] = ch < c_hi ? load16_stream(row + ch * 16) : C::neg_inf();
     }
-    s_head[tid] = -1;
-    s_own[tid] = 0u;
+    correction_clear<NT>(s_head, s_own);
     stage();
     __syncthreads();
-    // final values of the columns that carry a teacher entry, handed to the threads that hold them
+    // dense part of the columns that carry a teacher entry, handed to the threads that hold them
     for (int k = tid; k < Kp; k += NT) {
       const int id = s_idx[k];
       if (id < 0) continue;
-      s_val[k] = fast_exp2(fmaf(s_z[k], a, -b)) * w + coef_on_id(s_idx, s_c, Kp, k, id) * p.inv_T;
+      s_val[k] = fast_exp2(fmaf(s_z[k], a, -b)) * w;
       correction_link<Tag, NT>(s_head, s_own, s_next, k, id - (int)lo);
     }
     __syncthreads();
@@ -169,7 +168,12 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
         C::unpack(v[i], f);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * w;
-        if (mine & (1u << i)) correction_apply<Tag, NT>(s_head, s_next, s_idx, s_val, (int)lo, i, f);
+        if (mine & (1u << i))
+          correction_apply<Tag, NT>(s_head, s_next, s_idx, (int)lo, i, true, f, [&](int k, bool shared, int first) {
+            const float cs = shared ? correction_shared_sum(s_next, s_idx, first, k, [&](int j) { return s_c[j]; })
+                                    : s_c[k];
+            return s_val[k] + cs * p.inv_T;
+          });
         store16_stream(grow + ch * 16, C::pack(f));
       }
     }
@@ -204,7 +208,7 @@ static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
   constexpr int NT = 256, NCH = 16;
   const int64_t per_part = (int64_t)NT * NCH * Tag::epc;
   const int parts = (int)((p.V + per_part - 1) / per_part);
-  const size_t lds = (size_t)((p.K + 15) & ~15) * 20 + (size_t)NT * 8;      // ids, coefficients, logits, values, links; heads, masks
+  const size_t lds = (size_t)((p.K + 15) & ~15) * 20 + (size_t)CORRECTION_HEADS * 4 + (size_t)NT * 4;   // ids, coefficients, logits, values, links; list heads, chunk masks
   const dim3 grid((unsigned)((p.n_rows + 7) / 8 * 8 * parts));
   if (vec) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, true>), grid, dim3(NT), lds, st, p, parts);
   else hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, false>), grid, dim3(NT), lds, st, p, parts);

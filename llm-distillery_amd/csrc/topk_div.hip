@@ -96,7 +96,7 @@ struct TopkLds {
   // in-register corrections (kernels that keep the row in registers; owners == 0 elsewhere):
   float* val;        // Kp  final gradient value at the entry's column
   int* next;         // Kp  next entry owned by the same thread, or -1
-  int* head;         // one per thread: first entry inside the thread's chunks, or -1
+  int* head;         // CORRECTION_HEADS list heads: first entry of a chunk's list, or -1
   unsigned* own;     // one per thread: bit i set = chunk i of the thread holds an entry
   int Kp;
   __device__ TopkLds(unsigned char* base, int K, int owners = 0) {
@@ -110,11 +110,11 @@ struct TopkLds {
     val = z + Kp;
     next = reinterpret_cast<int*>(val + Kp);
     head = next + Kp;
-    own = reinterpret_cast<unsigned*>(head + owners);
+    own = reinterpret_cast<unsigned*>(head + (owners ? CORRECTION_HEADS : 0));
   }
   __host__ __device__ static size_t bytes(int K, int owners = 0) {
     const size_t Kp = (size_t)((K + 15) & ~15);
-    return 512 + Kp * 16 + (owners ? Kp * 8 + (size_t)owners * 8 : 0);
+    return 512 + Kp * 16 + (owners ? Kp * 8 + (size_t)CORRECTION_HEADS * 4 + (size_t)owners * 4 : 0);
   }
 };
 
@@ -262,16 +262,16 @@ __device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int
 }
 
 // The same corrections for a row (part) held in registers, applied by the threads that hold the
-// columns before they store them (correction_link / correction_apply): final value of every entry
-// inside [lo, hi) into s.val, the entry linked into its owner's list.
+// columns before they store them (correction_link / correction_apply).  Entry threads leave the
+// student probability at the entry's column in s.val and link the entry into its owner's list; the
+// owner subtracts the teacher mass -- of all entries of that column, should ids repeat, which it
+// sees from its own list: no scan over the row's ids.
 template <class Tag, int NT>
-__device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, int hi, float a, float b, float c,
-                                                     bool ids_unique) {
+__device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, int hi, float a, float b) {
   for (int k = threadIdx.x; k < s.Kp; k += NT) {
     const int id = s.idx[k];
     if (id < lo || id >= hi) continue;
-    const float q = ids_unique ? s.q[k] : mass_on_id(s, k, id);
-    s.val[k] = (fast_exp2(fmaf(s.z[k], a, -b)) - q) * c;
+    s.val[k] = fast_exp2(fmaf(s.z[k], a, -b));
     correction_link<Tag, NT>(s.head, s.own, s.next, k, id - lo);
   }
 }
@@ -338,8 +338,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
   const char* rpart = row + c0 * 16;
 
-  s.head[tid] = -1;                   // own list of corrections, filled after the row statistics
-  s.own[tid] = 0u;
+  correction_clear<NT>(s.head, s.own);      // lists of corrections, filled after the row statistics
   TeacherEntries<(J > 0 ? J : 1)> te;
   if constexpr (J > 0) teacher_issue<NT, J>(p, trow, te);
   u32x4 reg[NCH];
@@ -429,9 +428,14 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   if (gpart) {
     const float c = p.inv_T_s * p.grad_scale;
     const float kc = fast_exp2(mb_own - b) * c;       // stashed value -> gradient
-    fkl_link_corrections<Tag, NT>(s, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
-    __syncthreads();
-    const unsigned mine = s.own[tid];
+    // 16 chunks of 4-byte logits leave no registers for placing the corrections during the sweep
+    // (it spills): those shapes write them behind the dense stores instead.
+    constexpr bool IN_REGISTERS = !(Tag::bytes == 4 && NCH == 16);
+    if (IN_REGISTERS) {
+      fkl_link_corrections<Tag, NT>(s, lo, hi, a, b);
+      __syncthreads();
+    }
+    const unsigned mine = IN_REGISTERS ? s.own[tid] : 0u;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = (int64_t)i * NT + tid;
@@ -441,15 +445,26 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
         C::unstash(reg[i], f);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
-        if (mine & (1u << i)) correction_apply<Tag, NT>(s.head, s.next, s.idx, s.val, lo, i, f);
+        if (mine & (1u << i))
+          correction_apply<Tag, NT>(s.head, s.next, s.idx, lo, i, (p.flags & DL_TOPK_UNIQUE_IDS) == 0, f,
+                                    [&](int k, bool shared, int first) {
+                                      const float q = shared ? correction_shared_sum(s.next, s.idx, first, k,
+                                                                                     [&](int j) { return s.q[j]; })
+                                                             : s.q[k];
+                                      return (s.val[k] - q) * c;
+                                    });
         store16_stream(gpart + ch * 16, C::pack(f));
       }
+    }
+    if (!IN_REGISTERS) {
+      __syncthreads();      // dense stores are ordered before the sparse corrections
+      fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
     }
   }
 }
 
 template <class Tag, int NT, int NCH, bool SPLIT, int J>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))     // <= 128 VGPRs: 16 waves per CU
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void fkl_topk_reg_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const TopkLds s(smem, p.K, NT);
@@ -551,8 +566,7 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
-  s.head[tid] = -1;
-  s.own[tid] = 0u;
+  correction_clear<NT>(s.head, s.own);
   float tlse = -INFINITY;
   if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
   // Every store comes after the K logits have been gathered (stage_teacher ends in barriers), so
@@ -593,12 +607,11 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
     for (int k = tid; k < s.Kp; k += NT) {
       const int id = s.idx[k];
       if (id < 0) continue;
-      float g = 0.f;
-      for (int j = 0; j < s.Kp; ++j) g += (s.idx[j] == id) ? s.q[j] * (s.z[j] - rkl) : 0.f;
       if (VEC) {
-        s.val[k] = g * c;             // placed by the thread that writes the column's chunk
-        correction_link<Tag, NT>(s.head, s.own, s.next, k, id);
+        correction_link<Tag, NT>(s.head, s.own, s.next, k, id);     // placed by the thread that writes the column's chunk
       } else {
+        float g = 0.f;
+        for (int j = 0; j < s.Kp; ++j) g += (s.idx[j] == id) ? s.q[j] * (s.z[j] - rkl) : 0.f;
         store_from_float(grow, Tag::id, id, g * c);
       }
     }
@@ -611,7 +624,11 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
         float f[C::N];
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = 0.f;
-        if (mine & (1u << (i & 31))) correction_apply<Tag, NT>(s.head, s.next, s.idx, s.val, 0, (int)i, f);
+        if (mine & (1u << (i & 31)))
+          correction_apply<Tag, NT>(s.head, s.next, s.idx, 0, (int)i, true, f, [&](int k, bool shared, int first) {
+            const auto term = [&](int j) { return s.q[j] * (s.z[j] - rkl); };
+            return (shared ? correction_shared_sum(s.next, s.idx, first, k, term) : term(k)) * c;
+          });
         store16_stream(grow + ch * 16, C::pack(f));
       }
     }
@@ -669,6 +686,7 @@ static std::atomic<int> g_spin_limit{20000};    // polls a part waits for a part
 // Number of column parts a row of `nch` 16-byte chunks is cut into (1 = one workgroup per row).
 static int split_parts(int64_t nch) {
   if (nch <= 512 * 16) return 1;
+  if (nch > 1024 * 16) return (int)((nch + 256 * 16 - 1) / (256 * 16));      // 5 .. MAX_PARTS parts of 256 x 16 chunks
   const int forced = g_split_parts.load();
   if (forced == 1 || forced == 2 || forced == 4) return forced;
   return 4;
@@ -677,18 +695,19 @@ static int split_parts(int64_t nch) {
 template <class Tag>
 static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipStream_t st) {
   const int64_t nch = p.V / Tag::epc;
-  if (aligned) {
+  if (aligned && nch <= (int64_t)MAX_PARTS * 256 * 16) {
     if (nch <= 256 * 4) return launch_reg<Tag, 256, 4>(p, st);
     if (nch <= 256 * 8) return launch_reg<Tag, 256, 8>(p, st);
-    if (nch <= 256 * 16) return launch_reg<Tag, 256, 16>(p, st);
+    // 4-byte logits: 8 chunks per thread from twice the threads keep the corrections in registers
+    if (nch <= 256 * 16) return Tag::bytes == 4 ? launch_reg<Tag, 512, 8>(p, st) : launch_reg<Tag, 256, 16>(p, st);
     if (nch <= 512 * 16) return launch_reg<Tag, 512, 16>(p, st);
-    if (nch <= 1024 * 16) {
-      const int parts = split_parts(nch);
-      const bool ws_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, parts) && p.n_rows * parts <= 0x7fffffffLL;
-      if (parts == 2 && ws_ok) return launch_split<Tag, 512, 16>(p, 2, st);
-      if (parts == 4 && ws_ok) return launch_split<Tag, 256, 16>(p, 4, st);
-      return launch_reg<Tag, 1024, 16>(p, st);
-    }
+    const int parts = split_parts(nch);
+    const bool ws_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, parts) && p.n_rows * parts <= 0x7fffffffLL;
+    if (parts == 2 && ws_ok) return launch_split<Tag, 512, 16>(p, 2, st);
+    if (parts >= 4 && ws_ok) return launch_split<Tag, 256, 16>(p, parts, st);
+    if (nch <= 1024 * 16) return launch_reg<Tag, 1024, 16>(p, st);      // no workspace: one workgroup per row
+  }
+  if (aligned) {
     hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
                        TopkLds::bytes(p.K), st, p);
   } else {
@@ -731,8 +750,8 @@ extern "C" int dl_set_option(const char* name, int value) {
 extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V) {
   if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
   const int64_t nch = V / (logits_dtype == DL_F32 ? 4 : 8);
-  if (nch <= 512 * 16 || nch > 1024 * 16) return 0;
-  return dl::RetryList::bytes(n_rows, 4);
+  if (nch <= 512 * 16 || nch > (int64_t)dl::MAX_PARTS * 256 * 16) return 0;
+  return dl::RetryList::bytes(n_rows, nch <= 1024 * 16 ? 4 : dl::MAX_PARTS);
 }
 
 extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,

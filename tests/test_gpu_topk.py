@@ -210,3 +210,19 @@ def test_gradient_may_overwrite_the_logits(D, kind, V, dtype):
             D.set_option("spin_limit", 20000)
         assert g2.data_ptr() == y.data_ptr() and torch.equal(rl, rl2) and torch.equal(g, y)
 
+
+
+@pytest.mark.parametrize("V,dtype", [(152064, torch.bfloat16), (128256, torch.float32), (262144, torch.float16)])
+def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
+    """Vocabularies beyond 131072 two-byte (65536 four-byte) entries are cut into 5..8 parts of 4096
+    chunks; with and without waiting for the partners the oracle's numbers and the same bits."""
+    logits, tv, ti = _case(10, V, 48, dtype, 41, std=3.0)
+    valid = torch.ones(10, dtype=torch.bool)
+    valid[4] = False
+    waited = _check(D, "fkl", logits, tv[:9], ti[:9], T=1.3, valid=valid)
+    try:
+        D.set_option("spin_limit", 0)
+        retried = _check(D, "fkl", logits, tv[:9], ti[:9], T=1.3, valid=valid)
+    finally:
+        D.set_option("spin_limit", 20000)
+    assert torch.equal(waited, retried)
