@@ -63,6 +63,64 @@ __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
   if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
 }
 
+// Rows too wide for the registers, 16-byte aligned: the same sweeps, every one of them over global
+// memory with 16-byte loads, two units per thread in flight (3-4 reads of both rows; all but the first
+// come from L2 / the memory-side cache as far as the rows of the workgroups in flight fit there).
+template <class TagS, class TagT, int NT>
+struct StreamRows {
+  const char* srow;
+  const char* trow;
+  int64_t nunits;
+  template <class Tag>
+  static __device__ __forceinline__ void fetch(Unit<Tag>& x, const char* row, int64_t u) {
+#pragma unroll
+    for (int k = 0; k < Unit<Tag>::NC; ++k) x.c[k] = *reinterpret_cast<const u32x4*>(row + (u * Unit<Tag>::NC + k) * 16);
+  }
+  template <class F>
+  __device__ __forceinline__ void sweep(F f) {
+    constexpr int U = 2;
+    for (int64_t u0 = threadIdx.x; u0 < nunits; u0 += (int64_t)U * NT) {
+      Unit<TagS> s[U];
+      Unit<TagT> t[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const int64_t u = u0 + (int64_t)j * NT;
+        if (u < nunits) { fetch(s[j], srow, u); fetch(t[j], trow, u); }
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const int64_t u = u0 + (int64_t)j * NT;
+        if (u < nunits) {
+          float a[8], b[8];
+          s[j].unpack(a);
+          t[j].unpack(b);
+          f(u, a, b);
+        }
+      }
+    }
+  }
+};
+
+template <int KIND, class TagS, class TagT, int NT>
+__global__ __launch_bounds__(NT) void dense_stream_vec_kernel(const DenseParams p) {
+  __shared__ float red[64];
+  const int64_t r = xcd_banded_row(blockIdx.x);
+  if (r >= p.n_rows) return;
+  const int tid = threadIdx.x;
+  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
+  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  if (trow < 0) {
+    if (grow) zero_row<TagS, NT>(grow, p.V / TagS::epc);
+    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    return;
+  }
+  StreamRows<TagS, TagT, NT> rows{reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes,
+                                  reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * TagT::bytes, p.V / 8};
+  const DenseStats st = dense_stats<KIND, NT>(rows, p.inv_T_s, p.inv_T_t, red);
+  if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
+  if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
+}
+
 // Any size, any alignment, any dtype pair: four scalar passes over global memory.
 template <int NT>
 __global__ __launch_bounds__(NT) void dense_stream_kernel(const DenseParams p) {
@@ -127,7 +185,7 @@ static bool launch_dense_kind(const DenseParams& p, hipStream_t st) {
   if (units <= 256 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 256, NU>), grid, dim3(256), 0, st, p);
   else if (units <= 512 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 512, NU>), grid, dim3(512), 0, st, p);
   else if (units <= 1024 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 1024, NU>), grid, dim3(1024), 0, st, p);
-  else return false;
+  else hipLaunchKernelGGL((dense_stream_vec_kernel<KIND, TagS, TagT, 1024>), grid, dim3(1024), 0, st, p);
   return true;
 }
 

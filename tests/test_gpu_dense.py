@@ -90,9 +90,10 @@ def test_teacher_with_zero_mass_entries(D, kind):
     _check(D, kind, s, t, T=1.0)
 
 
-@pytest.mark.parametrize("V,dtype", [(1001, torch.float32), (70000, torch.bfloat16), (50264, torch.float32)])
+@pytest.mark.parametrize("V,dtype", [(1001, torch.float32), (70000, torch.bfloat16), (50264, torch.float32),
+                                     (128256, torch.bfloat16)])
 def test_dense_streaming_fallback(D, V, dtype):
-    # odd vocabulary / rows beyond the register budget take the scalar multi-pass kernel
+    # rows beyond the register budget take the multi-pass kernel with 16-byte loads, odd vocabularies the scalar one
     s, t = _pair(5, V, dtype, 5)
     for kind in ("fkl", "rkl", "jsd"):
         _check(D, kind, s, t, T=1.3)
