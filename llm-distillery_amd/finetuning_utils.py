@@ -206,10 +206,8 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
     counts = [min(rows.numel(), t_lp.size(0), idx.size(0)) for rows, t_lp, idx, _, _ in convos]
     if row_map is None or row_map.numel() != B * S or any(n != rows.numel() for n, (rows, *_) in zip(counts, convos)):
         row_map = torch.full((B * S,), -1, dtype=torch.int32, device=dev)
-        base = 0
-        for b, ((rows, *_), n) in enumerate(zip(convos, counts)):
-            row_map[b * S + rows[:n].long()] = torch.arange(base, base + n, dtype=torch.int32, device=dev)
-            base += n
+        where = torch.cat([rows[:n].long() + b * S for b, ((rows, *_), n) in enumerate(zip(convos, counts))])
+        row_map[where] = torch.arange(where.numel(), dtype=torch.int32, device=dev)      # one scatter for the batch
     idx_cat = _packed_rows([idx[:n] for (_, _, idx, _, _), n in zip(convos, counts)])
     lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature, int(crop_to_size or 0))
     tT = temperature if teacher_temperature is None else teacher_temperature
