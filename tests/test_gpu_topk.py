@@ -65,7 +65,8 @@ def test_topk_small(D, dtype, kind):
     _check(D, kind, logits, tv, ti, T=1.0)
 
 
-@pytest.mark.parametrize("V,K", [(32000, 200), (128256, 200), (50264, 64), (8192, 400)])
+@pytest.mark.parametrize("V,K", [(32000, 200), (128256, 200), (50264, 64), (8192, 400), (32000, 2048), (128256, 1024),
+                                 (65536, 2048)])
 def test_fkl_topk_register_path_sizes(D, V, K):
     logits, tv, ti = _case(24, V, K, torch.bfloat16, 2, std=3.0)
     _check(D, "fkl", logits, tv, ti, T=1.0)
