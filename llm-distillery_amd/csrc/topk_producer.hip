@@ -14,7 +14,9 @@
 // ~95 % of the kernel's time at ~16 instructions per element (softmax sweeps ~8, key encoding and
 // group maxima ~2, collection ~6).  Counting each thread's entries first and reserving their slots
 // with one atomic per thread (instead of one wave-wide vote per entry position) was measured: more
-// vector instructions, 9 % slower.
+// vector instructions, 9 % slower.  So was a region of candidates per wave with the count in a scalar
+// register and every branch taken by whole waves (votes instead of atomics): no LDS atomics left, but
+// 12 % more vector instructions (each vote costs a select and a compare) and 10 % more time.
 // Ties go to the smaller id, deterministically; torch.topk, which the reference calls, leaves tie
 // order open.  Rows with more than 2048 entries at or above L (constant or coarsely quantised rows)
 // take an exact but slow select by bisection over key bits and then over columns.
