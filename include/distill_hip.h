@@ -81,7 +81,8 @@ int dl_set_option(const char* name, int value);
  *            workspace (NULL or too small) such rows take a slower one-workgroup-per-row kernel.
  *            Two launches that may overlap in time must not share a workspace.
  * flags      DL_TOPK_UNIQUE_IDS promises that no id occurs twice within a row (true for the output of
- *            torch.topk and of dl_merge_remap_topk); the kernel then skips its duplicate scan.  With
+ *            torch.topk and of dl_merge_remap_topk); the kernel then skips its check for repeated ids
+ *            (a few instructions per entry in the register kernels, a scan in the streaming one).  With
  *            the flag set and duplicates present, the gradient at a duplicated id is wrong.
  * K <= DL_MAX_TOPK.
  * grad may be the logits buffer itself (same pointer and stride): every kernel holds, or has

@@ -65,7 +65,7 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
     logits [..., V] bf16/fp16/fp32 (native model dtype, rows evenly strided);
     t_val/t_idx [N, K] stored teacher log-probs and ids; row_map int32 [rows]
     gives the teacher row of each logits row (negative = masked row).  `unique_ids=True` promises
-    that no id repeats within a row (skips the duplicate scan).
+    that no id repeats within a row (skips the check for repeated ids).
     Returns (row_loss fp32 [rows], grad like logits or None).
     """
     if kind not in ("fkl", "rkl"):
