@@ -4,7 +4,6 @@ K larger than the number of distinct ids; the product's host index construction 
 position-by-position brute force on random content ranges; the C++ byte trie against the dict
 brute force on random byte vocabularies."""
 import numpy as np
-import pytest
 from hypothesis import given, settings, strategies as st
 
 import llm_distillery_amd.batch_index as BI
