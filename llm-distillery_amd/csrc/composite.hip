@@ -112,24 +112,41 @@ __global__ __launch_bounds__(CMP_NT) void composite_rows_fwd_kernel(const Compos
 }
 
 // ---- conversations -----------------------------------------------------------------------------------
-template <int NT>
-__device__ __forceinline__ double block_sum_f64(double v, double* scratch) {
+// N sums over the workgroup at once (wave butterflies, then the wave totals in wave order): one pair of barriers for all of them.
+template <int NT, int N>
+__device__ __forceinline__ void block_sums_f64(double (&v)[N], double* scratch) {
   constexpr int NW = NT / WAVE;
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
   const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
-  if (lane == 0) scratch[w] = v;
-  __syncthreads();
-  double r = 0.0;
 #pragma unroll
-  for (int i = 0; i < NW; ++i) r += scratch[i];
+  for (int k = 0; k < N; ++k) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v[k] += __shfl_xor(v[k], o, WAVE);
+    if (lane == 0) scratch[k * NW + w] = v[k];
+  }
   __syncthreads();
-  return r;
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    double r = 0.0;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) r += scratch[k * NW + i];
+    v[k] = r;
+  }
+  __syncthreads();
 }
 
-__global__ __launch_bounds__(CMP_NT) void composite_convo_kernel(const CompositeParams p) {
+// x^alpha and x^(alpha - 1) for the weights; alpha = 2 (the reference's configuration) and 1 need no powf
+__device__ __forceinline__ void weight_powers(float x, float alpha, float& pa, float& pa1) {
+  if (alpha == 2.f) { pa = x * x; pa1 = x; }
+  else if (alpha == 1.f) { pa = x; pa1 = 1.f; }
+  else { pa1 = powf(x, alpha - 1.f); pa = powf(x, alpha); }
+}
+
+constexpr int CONVO_NT = 256;
+
+__global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const CompositeParams p) {
+  constexpr int CMP_NT = CONVO_NT;  // (shadows the row kernels' size inside this kernel)
   __shared__ float red[64];
-  __shared__ double dred[CMP_NT / WAVE];
+  __shared__ double dred[10 * CMP_NT / WAVE];
   const int c = blockIdx.x, tid = threadIdx.x;
   const int r0 = p.row_off[c], n = p.row_off[c + 1] - r0;
   const int m = p.label_off[c + 1] - p.label_off[c];          // labels; the host guarantees m == n - 1
@@ -152,11 +169,11 @@ __global__ __launch_bounds__(CMP_NT) void composite_convo_kernel(const Composite
     tie_k += r.kl == mk ? 1.0 : 0.0;
     tie_r += r.rkl == mr ? 1.0 : 0.0;
   }
-  nv = block_sum_f64<CMP_NT>(nv, dred);
-  sum_s = block_sum_f64<CMP_NT>(sum_s, dred);
-  sum_t = block_sum_f64<CMP_NT>(sum_t, dred);
-  tie_k = block_sum_f64<CMP_NT>(tie_k, dred);
-  tie_r = block_sum_f64<CMP_NT>(tie_r, dred);
+  {
+    double v[5] = {nv, sum_s, sum_t, tie_k, tie_r};
+    block_sums_f64<CMP_NT>(v, dred);
+    nv = v[0]; sum_s = v[1]; sum_t = v[2]; tie_k = v[3]; tie_r = v[4];
+  }
   const float mean_s = (float)(sum_s / nv), mean_t = (float)(sum_t / nv);       // 0 / 0 = NaN: no valid row
 
   // weighted sums, logged means, and the two sums the gradient of the maxima needs
@@ -175,22 +192,21 @@ __global__ __launch_bounds__(CMP_NT) void composite_convo_kernel(const Composite
       if (!r.valid && !(d < 0.f)) a_ginv += (double)(0.5f * inv_n * (r.kl + r.rkl));
     }
     const float Ak = r.kl / mk + 1.f, Ar = r.rkl / mr + 1.f;
-    const float wk = powf(Ak, alpha) + cpos, wr = powf(Ar, alpha) + cpos;
+    float pk, pk1, pr, pr1;
+    weight_powers(Ak, alpha, pk, pk1);
+    weight_powers(Ar, alpha, pr, pr1);
+    const float wk = pk + cpos, wr = pr + cpos;
     a_wkl += (double)(r.kl * wk); a_wrkl += (double)(r.rkl * wr);
     a_kl += (double)r.kl; a_rkl += (double)r.rkl;
-    a_gmk += (double)(r.kl * alpha * powf(Ak, alpha - 1.f) * (-r.kl / (mk * mk)));
-    a_gmr += (double)(r.rkl * alpha * powf(Ar, alpha - 1.f) * (-r.rkl / (mr * mr)));
+    a_gmk += (double)(r.kl * alpha * pk1 * (-r.kl / (mk * mk)));
+    a_gmr += (double)(r.rkl * alpha * pr1 * (-r.rkl / (mr * mr)));
   }
-  a_wkl = block_sum_f64<CMP_NT>(a_wkl, dred);
-  a_wrkl = block_sum_f64<CMP_NT>(a_wrkl, dred);
-  a_kl = block_sum_f64<CMP_NT>(a_kl, dred);
-  a_rkl = block_sum_f64<CMP_NT>(a_rkl, dred);
-  a_ces = block_sum_f64<CMP_NT>(a_ces, dred);
-  a_cet = block_sum_f64<CMP_NT>(a_cet, dred);
-  a_d = block_sum_f64<CMP_NT>(a_d, dred);
-  a_gmk = block_sum_f64<CMP_NT>(a_gmk, dred);
-  a_gmr = block_sum_f64<CMP_NT>(a_gmr, dred);
-  a_ginv = block_sum_f64<CMP_NT>(a_ginv, dred);
+  {
+    double v[10] = {a_wkl, a_wrkl, a_kl, a_rkl, a_ces, a_cet, a_d, a_gmk, a_gmr, a_ginv};
+    block_sums_f64<CMP_NT>(v, dred);
+    a_wkl = v[0]; a_wrkl = v[1]; a_kl = v[2]; a_rkl = v[3]; a_ces = v[4]; a_cet = v[5]; a_d = v[6];
+    a_gmk = v[7]; a_gmr = v[8]; a_ginv = v[9];
+  }
   if (tid == 0) {
     const float wkl = (float)(a_wkl / n), wrkl = (float)(a_wrkl / n);
     const float total = (wkl + wrkl) * 0.5f;
@@ -221,9 +237,12 @@ __global__ __launch_bounds__(CMP_NT) void composite_convo_kernel(const Composite
       }
     }
     const float Ak = r.kl / mk + 1.f, Ar = r.rkl / mr + 1.f;
+    float pk, pk1, pr, pr1;
+    weight_powers(Ak, alpha, pk, pk1);
+    weight_powers(Ar, alpha, pr, pr1);
     RowCoef o;
-    o.g_kl = 0.5f * inv_n * (powf(Ak, alpha) + cpos + r.kl * alpha * powf(Ak, alpha - 1.f) / mk) + (r.kl == mk ? gmk : 0.f);
-    o.g_rkl = 0.5f * inv_n * (powf(Ar, alpha) + cpos + r.rkl * alpha * powf(Ar, alpha - 1.f) / mr) + (r.rkl == mr ? gmr : 0.f);
+    o.g_kl = 0.5f * inv_n * (pk + cpos + r.kl * alpha * pk1 / mk) + (r.kl == mk ? gmk : 0.f);
+    o.g_rkl = 0.5f * inv_n * (pr + cpos + r.rkl * alpha * pr1 / mr) + (r.rkl == mr ? gmr : 0.f);
     o.g_own = g_own;
     o.pad = 0.f;
     coef[i] = o;
@@ -291,7 +310,7 @@ extern "C" int dl_composite_forward(const float* lse, const float* zk, const voi
   if (n_rows > 0)
     hipLaunchKernelGGL(composite_rows_fwd_kernel, dim3((unsigned)((n_rows + CMP_ROWS_PER_WG - 1) / CMP_ROWS_PER_WG)),
                        dim3(CMP_NT), 0, st, p);
-  hipLaunchKernelGGL(composite_convo_kernel, dim3((unsigned)n_convos), dim3(CMP_NT), 0, st, p);
+  hipLaunchKernelGGL(composite_convo_kernel, dim3((unsigned)n_convos), dim3(CONVO_NT), 0, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
