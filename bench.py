@@ -163,8 +163,7 @@ def _wl_composite(D, S, dev, rows):
     def main():
         x.grad = None
         L = D.Losses(None)
-        for d in D.distill_loss_batch(x, convos, alpha, temperature=T):
-            L.add_losses(d)
+        L.add_batch(D.distill_loss_batch(x, convos, alpha, temperature=T))
         total = L.loss_dict["train_loss"].detach()
         L.backward(divisor=1)
         return total

@@ -42,6 +42,29 @@ class Losses:
             else:
                 self.loss_dict[key] = value
 
+    def add_batch(self, batch_losses) -> None:
+        """The dicts of all conversations of a batch at once (what `distill_loss_batch` returns): the
+        same totals and step count as calling `add_losses` on each in turn, from two launches per
+        key (a stack and a sum) instead of one addition per key and conversation.  The order of the
+        float additions differs from the sequential form, so the last bit of a logged value may."""
+        batch_losses = list(batch_losses)
+        if not batch_losses:
+            raise ValueError("No losses to add to the loss dictionary.")
+        if len(batch_losses) == 1:
+            self.add_losses(batch_losses[0])
+            return
+        keys = list(batch_losses[0])
+        if any(list(d) != keys for d in batch_losses):
+            for d in batch_losses:                           # differing key sets: the sequential form handles them
+                self.add_losses(d)
+            return
+        summed = {}
+        for key in keys:
+            vals = [d[key] if key == "train_loss" else d[key].detach() for d in batch_losses]
+            summed[key] = torch.stack(vals).sum(0)
+        self.num_steps_accumulated += len(batch_losses) - 1  # add_losses counts the last one
+        self.add_losses(summed)
+
     def empty(self) -> None:
         self.loss_dict = {}
         self.num_steps_accumulated = 0

@@ -46,6 +46,29 @@ def test_losses_accumulates_sums_and_backward_divides():
     assert L.loss_dict == {} and L.num_steps_accumulated == 0
 
 
+def test_losses_add_batch_equals_adding_one_by_one():
+    leaf_a, leaf_b = torch.tensor(2.0, requires_grad=True), torch.tensor(2.0, requires_grad=True)
+    one, many = D.Losses(None), D.Losses(None)
+    one.add_losses(_dict(0.5, leaf_a))                         # something accumulated before the batch
+    many.add_losses(_dict(0.5, leaf_b))
+    for v in (1.0, 3.0, 4.0):
+        one.add_losses(_dict(v, leaf_a))
+    many.add_batch([_dict(v, leaf_b) for v in (1.0, 3.0, 4.0)])
+    assert one.num_steps_accumulated == many.num_steps_accumulated == 4
+    assert set(one.loss_dict) == set(many.loss_dict)
+    for k in one.loss_dict:
+        assert one.loss_dict[k].item() == pytest.approx(many.loss_dict[k].item())
+        assert k == "train_loss" or not many.loss_dict[k].requires_grad
+    one.backward(divisor=2)
+    many.backward(divisor=2)
+    assert leaf_a.grad.item() == pytest.approx(leaf_b.grad.item()) == pytest.approx(8.5 / 2)
+    with pytest.raises(ValueError):
+        many.add_batch([])
+    single = D.Losses(None)
+    single.add_batch([_dict(1.0, leaf_b)])
+    assert single.num_steps_accumulated == 1
+
+
 def test_losses_validation_prefix_and_scaling_operators():
     L = D.Losses(_Log(), validation=True)
     L.add_losses({"train_loss": torch.tensor(1.0), "kl_div": torch.tensor(4.0)})
