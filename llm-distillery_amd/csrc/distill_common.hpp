@@ -154,14 +154,16 @@ __device__ __forceinline__ void store16_stream(void* p, const u32x4& v) {
 //                     (head[slot] -> k -> next[k] ...) and marks the chunk in own[owner].  There are
 //                     CORRECTION_HEADS list heads per workgroup, CORRECTION_HEADS / NT per thread:
 //                     chunks i and i + CORRECTION_HEADS / NT of a thread share a list.
-//   correction_apply: called by the owner for its chunk i when bit i % 32 of own[] is set: walks the
-//                     chunk's list and overwrites the element of every entry that falls into chunk i
-//                     with value(k, shared, first); `shared` tells that another entry names the same
-//                     column (entries of one column all sit in the list that starts at `first`), in
-//                     which case value() must return what all of them together make of the column,
-//                     summed in an order that does not depend on the list's, which the atomics leave
-//                     open (correction_shared_sum).  `check_shared` false skips that test (the caller
-//                     knows that no column repeats).
+//   correction_apply: called by the owner for its chunk i when bit i % 32 of own[] is set: one walk
+//                     over the chunk's list puts finish(k, term(k)) in place of the element of every
+//                     entry k that falls into chunk i; returns true if an element was named more
+//                     than once (ids repeat inside the row).
+//   correction_repeats: called by the owner after its sweep for the chunks where correction_apply
+//                     said so: every such element gets finish(k, sum of term over all its entries),
+//                     written by an element-sized store behind the owner's own chunk store (same
+//                     thread, same address: ordered).  The sum is taken in fixed point
+//                     (correction_exact_sum), so it is the same whatever order the atomics gave the
+//                     list.  Kept out of the sweep so that the sweep's registers do not pay for it.
 // correction_clear (all threads) and a barrier come before the first link; a barrier separates the
 // links from the applies.
 constexpr int CORRECTION_HEADS = 2048;
@@ -181,38 +183,75 @@ __device__ __forceinline__ void correction_link(int* head, unsigned* own, int* n
   atomicOr(&own[owner], 1u << (i & 31));
 }
 
-template <class Tag, int NT, class Value>
-__device__ __forceinline__ void correction_apply(const int* head, const int* next, const int* col, int lo, int i,
-                                                 bool check_shared, float (&f)[Chunk<Tag>::N], Value value) {
+// Sum of term(k) over the entries of a list that name column `want`: order-independent and exact to
+// 2^-40 of the largest term.  Every term is scaled by a power of two chosen from the largest
+// magnitude (an exact operation), cut to an integer and added as such; a single term comes back
+// bit for bit.
+template <class Term>
+__device__ __forceinline__ float correction_exact_sum(const int* next, const int* col, int first, int want, Term term) {
+  float big = 0.f;
+  bool odd = false;                                   // NaN or infinity among the terms
+  for (int k = first; k >= 0; k = next[k])
+    if (col[k] == want) {
+      const float t = term(k);
+      odd = odd || !(fabsf(t) <= 3.0e38f);
+      big = fmaxf(big, fabsf(t));
+    }
+  if (odd || big == 0.f) {                            // nothing to scale by: plain sum (its value is NaN, an infinity or 0)
+    float sum = 0.f;
+    for (int k = first; k >= 0; k = next[k]) sum += col[k] == want ? term(k) : 0.f;
+    return sum;
+  }
+  int e;
+  (void)frexpf(big, &e);                              // big = m * 2^e, 0.5 <= m < 1
+  long long acc = 0;
+  for (int k = first; k >= 0; k = next[k])
+    if (col[k] == want) acc += (long long)ldexp((double)term(k), 40 - e);      // |.| < 2^40; up to 2048 of them: < 2^52
+  return (float)ldexp((double)acc, e - 40);
+}
+
+template <class Tag, int NT, class Term, class Finish>
+__device__ __forceinline__ bool correction_apply(const int* head, const int* next, const int* col, int lo, int i,
+                                                 float (&f)[Chunk<Tag>::N], Term term, Finish finish) {
   using C = Chunk<Tag>;
-  const int first = head[(i % (CORRECTION_HEADS / NT)) * NT + threadIdx.x];
-  for (int k = first; k >= 0; k = next[k]) {
+  unsigned seen = 0u, again = 0u;
+  for (int k = head[(i % (CORRECTION_HEADS / NT)) * NT + threadIdx.x]; k >= 0; k = next[k]) {
     const int off = col[k] - lo;
     if (off / (C::N * NT) != i) continue;
-    bool shared = false;
-    if (check_shared)
-      for (int j = first; j >= 0; j = next[j]) shared = shared || (j != k && col[j] == col[k]);
     const int e = off % C::N;
-    const float v = value(k, shared, first);
+    again |= seen & (1u << e);
+    seen |= 1u << e;
+    const float v = finish(k, term(k));
 #pragma unroll
     for (int j = 0; j < C::N; ++j) f[j] = (j == e) ? v : f[j];
   }
+  return again != 0u;
 }
 
-// Sum of term(j) over the entries j of the list starting at `first` that name the column of entry
-// k, taken in ascending j: the same bits whatever order the list happens to have.  Lists are a
-// few entries long.
-template <class Term>
-__device__ __forceinline__ float correction_shared_sum(const int* next, const int* col, int first, int k, Term term) {
-  float sum = 0.f;
-  int last = -1;
-  while (true) {
-    int pick = 0x7fffffff;
-    for (int j = first; j >= 0; j = next[j])
-      if (j > last && j < pick && col[j] == col[k]) pick = j;
-    if (pick == 0x7fffffff) return sum;
-    sum += term(pick);
-    last = pick;
+// `chunks`: bit i % 32 set for the chunks i whose correction_apply returned true; n_chunks: chunks
+// per thread; store(column, value) writes one element of the row.
+template <class Tag, int NT, class Term, class Finish, class Store>
+__device__ __forceinline__ void correction_repeats(const int* head, const int* next, const int* col, int lo,
+                                                   unsigned chunks, int n_chunks, Term term, Finish finish, Store store) {
+  using C = Chunk<Tag>;
+  for (int i = 0; i < n_chunks; ++i) {
+    if (!(chunks & (1u << (i & 31)))) continue;
+    const int first = head[(i % (CORRECTION_HEADS / NT)) * NT + threadIdx.x];
+    unsigned seen = 0u, again = 0u;
+    for (int k = first; k >= 0; k = next[k]) {
+      const int off = col[k] - lo;
+      if (off / (C::N * NT) != i) continue;
+      again |= seen & (1u << (off % C::N));
+      seen |= 1u << (off % C::N);
+    }
+    while (again) {
+      const int e = __ffs(again) - 1;
+      again &= again - 1u;
+      const int want = lo + (i * NT + (int)threadIdx.x) * C::N + e;
+      int any = -1;
+      for (int k = first; k >= 0 && any < 0; k = next[k]) any = col[k] == want ? k : -1;
+      store(want, finish(any, correction_exact_sum(next, col, first, want, term)));
+    }
   }
 }
 

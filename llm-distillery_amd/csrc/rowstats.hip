@@ -160,6 +160,9 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     }
     __syncthreads();
     const unsigned mine = s_own[tid];
+    const auto coef = [&](int k) { return s_c[k]; };
+    const auto value = [&](int k, float cs) { return s_val[k] + cs * p.inv_T; };
+    unsigned repeats = 0u;            // chunks in which an id occurs more than once
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
@@ -169,14 +172,13 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * w;
         if (mine & (1u << i))
-          correction_apply<Tag, NT>(s_head, s_next, s_idx, (int)lo, i, true, f, [&](int k, bool shared, int first) {
-            const float cs = shared ? correction_shared_sum(s_next, s_idx, first, k, [&](int j) { return s_c[j]; })
-                                    : s_c[k];
-            return s_val[k] + cs * p.inv_T;
-          });
+          if (correction_apply<Tag, NT>(s_head, s_next, s_idx, (int)lo, i, f, coef, value)) repeats |= 1u << i;
         store16_stream(grow + ch * 16, C::pack(f));
       }
     }
+    if (repeats)
+      correction_repeats<Tag, NT>(s_head, s_next, s_idx, (int)lo, repeats, NCH, coef, value,
+                                  [&](int column, float g) { store_from_float(grow, Tag::id, column, g); });
     return;
   } else {
     stage();

@@ -265,7 +265,7 @@ __device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int
 // columns before they store them (correction_link / correction_apply).  Entry threads leave the
 // student probability at the entry's column in s.val and link the entry into its owner's list; the
 // owner subtracts the teacher mass -- of all entries of that column, should ids repeat, which it
-// sees from its own list: no scan over the row's ids.
+// sees from the chunk's list: no scan over the row's ids.
 template <class Tag, int NT>
 __device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, int hi, float a, float b) {
   for (int k = threadIdx.x; k < s.Kp; k += NT) {
@@ -436,6 +436,10 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
       __syncthreads();
     }
     const unsigned mine = IN_REGISTERS ? s.own[tid] : 0u;
+    const bool may_repeat = (p.flags & DL_TOPK_UNIQUE_IDS) == 0;
+    const auto mass = [&](int k) { return s.q[k]; };
+    const auto value = [&](int k, float q) { return (s.val[k] - q) * c; };
+    unsigned repeats = 0u;            // chunks in which an id occurs more than once
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = (int64_t)i * NT + tid;
@@ -446,16 +450,13 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
         if (mine & (1u << i))
-          correction_apply<Tag, NT>(s.head, s.next, s.idx, lo, i, (p.flags & DL_TOPK_UNIQUE_IDS) == 0, f,
-                                    [&](int k, bool shared, int first) {
-                                      const float q = shared ? correction_shared_sum(s.next, s.idx, first, k,
-                                                                                     [&](int j) { return s.q[j]; })
-                                                             : s.q[k];
-                                      return (s.val[k] - q) * c;
-                                    });
+          if (correction_apply<Tag, NT>(s.head, s.next, s.idx, lo, i, f, mass, value)) repeats |= 1u << i;
         store16_stream(gpart + ch * 16, C::pack(f));
       }
     }
+    if (may_repeat && repeats)
+      correction_repeats<Tag, NT>(s.head, s.next, s.idx, lo, repeats, NCH, mass, value,
+                                  [&](int column, float v) { store_from_float(grow, Tag::id, column, v); });
     if (!IN_REGISTERS) {
       __syncthreads();      // dense stores are ordered before the sparse corrections
       fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
@@ -620,17 +621,22 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
       __syncthreads();
       const unsigned mine = s.own[tid];
       const int64_t nch = V / C::N;
+      const auto term = [&](int k) { return s.q[k] * (s.z[k] - rkl); };
+      const auto value = [&](int, float g) { return g * c; };
+      unsigned repeats = 0u;
+      int n_own = 0;
       for (int64_t ch = tid, i = 0; ch < nch; ch += NT, ++i) {
         float f[C::N];
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = 0.f;
         if (mine & (1u << (i & 31)))
-          correction_apply<Tag, NT>(s.head, s.next, s.idx, 0, (int)i, true, f, [&](int k, bool shared, int first) {
-            const auto term = [&](int j) { return s.q[j] * (s.z[j] - rkl); };
-            return (shared ? correction_shared_sum(s.next, s.idx, first, k, term) : term(k)) * c;
-          });
+          if (correction_apply<Tag, NT>(s.head, s.next, s.idx, 0, (int)i, f, term, value)) repeats |= 1u << (i & 31);
         store16_stream(grow + ch * 16, C::pack(f));
+        n_own = (int)i + 1;
       }
+      if (repeats)
+        correction_repeats<Tag, NT>(s.head, s.next, s.idx, 0, repeats, n_own, term, value,
+                                    [&](int column, float v) { store_from_float(grow, Tag::id, column, v); });
     }
   }
 }

@@ -227,3 +227,29 @@ def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
     finally:
         D.set_option("spin_limit", 20000)
     assert torch.equal(waited, retried)
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl"])
+def test_rows_whose_ids_all_repeat(D, kind):
+    """Every entry of a row on one id, on two ids of one 16-byte chunk, on a handful of ids: the
+    masses add per id (the thread that holds the chunk sums them from its list), the result is the
+    oracle's and the same bits on every run."""
+    g = torch.Generator().manual_seed(77)
+    R, V, K = 6, 4096, 512
+    logits = (torch.randn(R, V, generator=g) * 2).to(torch.bfloat16)
+    ti = torch.empty(R, K, dtype=torch.int64)
+    ti[0] = 1234
+    ti[1] = torch.where(torch.arange(K) % 2 == 0, 801, 806)
+    ti[2] = torch.randint(0, 5, (K,), generator=g) * 1000 + 3
+    ti[3] = torch.randint(0, V, (K,), generator=g)
+    ti[4] = torch.arange(K) % 16 + 64
+    ti[5] = V - 1
+    if kind == "rkl":
+        # on a single id the reverse-KL gradient is an exact zero made of 512 cancelling terms: nothing
+        # for a relative tolerance to hold on to; two ids instead
+        ti[0] = torch.where(torch.arange(K) % 3 == 0, 1234, 77)
+        ti[5] = torch.where(torch.arange(K) % 5 == 0, V - 1, 0)
+    tv = torch.randn(R, K, generator=g)
+    a = _check(D, kind, logits, tv, ti.to(torch.int32), T=1.2)
+    b = _check(D, kind, logits, tv, ti.to(torch.int32), T=1.2)
+    assert torch.equal(a, b)
