@@ -229,6 +229,21 @@ def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
     assert torch.equal(waited, retried)
 
 
+def test_repeated_ids_on_wide_four_byte_rows(D):
+    # 16 chunks of fp32 per thread: the shapes that write their corrections behind the dense stores
+    g = torch.Generator().manual_seed(78)
+    R, V, K = 5, 32000, 96
+    logits = torch.randn(R, V, generator=g) * 2
+    ti = torch.randint(0, 40, (R, K), generator=g) * 797 + 5
+    tv = torch.randn(R, K, generator=g)
+    a = _check(D, "fkl", logits, tv, ti.to(torch.int32), T=0.9)
+    b = _check(D, "fkl", logits, tv, ti.to(torch.int32), T=0.9)
+    assert torch.equal(a, b)
+    wide = torch.randn(3, 60000, generator=g) * 2                  # cut into 4 parts
+    ti = torch.randint(0, 30, (3, K), generator=g) * 1999 + 11
+    _check(D, "fkl", wide, tv[:3], ti.to(torch.int32), T=1.0)
+
+
 @pytest.mark.parametrize("kind", ["fkl", "rkl"])
 def test_rows_whose_ids_all_repeat(D, kind):
     """Every entry of a row on one id, on two ids of one 16-byte chunk, on a handful of ids: the
