@@ -65,30 +65,19 @@ __device__ __forceinline__ void plan_consume_half(const unsigned* e, const float
                                                   unsigned tmask, int bits, PlanRun& open) {
   float val[PLAN_HB];
 #pragma unroll
-  for (int j = 0; j < PLAN_HB; ++j) val[j] = e[j] != PLAN_PAD ? tile[e[j] & tmask] : 0.f;
-  int fsid[PLAN_HB];       // student id whose run closes just before entry j (or -1)
-  float fsum[PLAN_HB];
+  for (int j = 0; j < PLAN_HB; ++j) val[j] = e[j] != PLAN_PAD ? tile[e[j] & tmask] : 0.f;      // all reads in flight together
 #pragma unroll
   for (int j = 0; j < PLAN_HB; ++j) {
-    fsid[j] = -1;
-    fsum[j] = 0.f;
     if (e[j] != PLAN_PAD) {
       const int sid = (int)(e[j] >> bits);
-      if (sid != open.sid) {
-        fsid[j] = open.sid;
-        fsum[j] = open.sum;
+      if (sid != open.sid) {                 // a run of equal student id closes: its total goes to the slot (this thread owns it)
+        if (open.sid >= 0) marg[open.sid] += open.sum;
         open.sid = sid;
         open.sum = 0.f;
       }
       open.sum += val[j];
     }
   }
-  float old[PLAN_HB];
-#pragma unroll
-  for (int j = 0; j < PLAN_HB; ++j) old[j] = fsid[j] >= 0 ? marg[fsid[j]] : 0.f;
-#pragma unroll
-  for (int j = 0; j < PLAN_HB; ++j)
-    if (fsid[j] >= 0) marg[fsid[j]] = old[j] + fsum[j];
 }
 
 __device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const float* tile, float* marg,
