@@ -264,8 +264,9 @@ int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_student, in
  * get replica slots (n_student rounded up to 4, + j), *n_extra_out in all, folded into the id's
  * slot after the last tile as listed in `fold` (int32 triples: id, first replica slot, replica
  * count).  The teacher vocabulary is cut into tiles of *tile_out ids; for tile k and wave w, rows
- * row_off[16k + w] .. row_off[16k + w + 1] of `ent` hold 64 entries each (one per lane,
- * 0xffffffff = padding): (slot << log2(tile) | t - k * tile), per thread sorted by (slot, t).
+ * row_off[16k + w] .. row_off[16k + w + 1] of `ent` hold 64 entries each (one per lane):
+ * (slot << log2(tile) | t - k * tile), per thread sorted by (slot, t), with bit 31 set on the first
+ * entry of a slot in the thread's list of the tile and bit 30 on the last one; 0x80000000 = padding.
  * Call once with row_off = ent = fold = NULL to learn *tile_out, *ent_rows_out, *n_fold_out and
  * *n_extra_out, allocate row_off int32 [16 * ceil(n_teacher / tile) + 1], ent uint32
  * [64 * ent_rows] and fold int32 [3 * n_fold], call again.

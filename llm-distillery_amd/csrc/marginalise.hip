@@ -43,47 +43,37 @@ __host__ __device__ inline int64_t plan_slot_words(int64_t Vs, int n_extra) {
   return ((Vs + 3) & ~(int64_t)3) + (((int64_t)n_extra + 3) & ~(int64_t)3);
 }
 
-constexpr unsigned PLAN_PAD = 0xffffffffu;
+// Plan entry: bit 31 = first entry of a run of one slot in its thread's list of the tile, bit 30 =
+// last entry of that run, below them (slot << log2(tile)) | offset inside the tile.  Padding is a
+// "first" entry that is never a "last" one: it restarts the running sum and stores nothing.
+constexpr unsigned PLAN_FIRST = 0x80000000u, PLAN_LAST = 0x40000000u, PLAN_PAD = PLAN_FIRST;
 
 // Marginal of one teacher row into marg[0, Vs) (LDS, zeroed here) along a plan; `tile` is LDS
 // scratch of plan_tile floats.  fp32 probabilities, 16-byte aligned rows.
 //
 // Latencies are kept off the critical path by batching: a thread holds a batch of PLAN_EB entries
-// in registers (the next tile's first batch is fetched while the current tile is consumed), reads
-// the tile for the whole batch at once, folds runs of equal student id in registers, and then
-// applies the run totals to marg with all reads issued before all writes (the ids inside one
-// thread's list are sorted, so the runs of a batch hit distinct addresses).
-constexpr int PLAN_EB = 8;           // entries per prefetched batch (measured: 16 is slower, more padding work)
-constexpr int PLAN_HB = 8;
-
-struct PlanRun {          // a run of equal student id still open at the end of a batch
-  int sid;
-  float sum;
-};
-
-__device__ __forceinline__ void plan_consume_half(const unsigned* e, const float* tile, float* marg,
-                                                  unsigned tmask, int bits, PlanRun& open) {
-  float val[PLAN_HB];
-#pragma unroll
-  for (int j = 0; j < PLAN_HB; ++j) val[j] = e[j] != PLAN_PAD ? tile[e[j] & tmask] : 0.f;      // all reads in flight together
-#pragma unroll
-  for (int j = 0; j < PLAN_HB; ++j) {
-    if (e[j] != PLAN_PAD) {
-      const int sid = (int)(e[j] >> bits);
-      if (sid != open.sid) {                 // a run of equal student id closes: its total goes to the slot (this thread owns it)
-        if (open.sid >= 0) marg[open.sid] += open.sum;
-        open.sid = sid;
-        open.sum = 0.f;
-      }
-      open.sum += val[j];
-    }
-  }
-}
+// in registers while the following batch (of this tile, or the first one of the next tile) is in
+// flight; it reads the tile for the whole batch at once, and for the entries that end a run the
+// slot's present value as well, so that no store waits for a load issued next to it.  A slot
+// belongs to one thread and has one run per thread and tile, so those early reads see no store of
+// the same batch.  The run totals are added as slot + (0 + v0 + v1 + ...), in list order.
+constexpr int PLAN_EB = 8;           // entries per batch
 
 __device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const float* tile, float* marg,
-                                             unsigned tmask, int bits, PlanRun& open) {
+                                             unsigned tmask, int bits, float& run) {
+  float val[PLAN_EB], base[PLAN_EB];
 #pragma unroll
-  for (int h = 0; h < PLAN_EB / PLAN_HB; ++h) plan_consume_half(e + h * PLAN_HB, tile, marg, tmask, bits, open);
+  for (int j = 0; j < PLAN_EB; ++j) val[j] = tile[e[j] & tmask];
+#pragma unroll
+  for (int j = 0; j < PLAN_EB; ++j) {
+    base[j] = 0.f;
+    if (e[j] & PLAN_LAST) base[j] = marg[(e[j] & ~(PLAN_FIRST | PLAN_LAST)) >> bits];
+  }
+#pragma unroll
+  for (int j = 0; j < PLAN_EB; ++j) {
+    run = ((e[j] & PLAN_FIRST) ? 0.f : run) + val[j];
+    if (e[j] & PLAN_LAST) marg[(e[j] & ~(PLAN_FIRST | PLAN_LAST)) >> bits] = base[j] + run;
+  }
 }
 
 // Teacher tiles are fetched PLAN_DEPTH tiles ahead (registers): with one 32 KiB tile in flight per
@@ -125,12 +115,17 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
       e[j] = r < r_end ? v : PLAN_PAD;
     }
   };
-  unsigned ea[PLAN_EB], eb[PLAN_EB];                // ping-pong entry batches (no register copies)
+  // the constant address space tells the compiler that nothing in this kernel writes the offsets:
+  // only then does it fetch them with scalar loads
+  typedef const __attribute__((address_space(4))) int32_t* ConstI32;
+  ConstI32 row_off = (ConstI32)p.plan_row_off;
+  unsigned ecur[PLAN_EB], enxt[PLAN_EB];            // the batch being consumed and the one in flight
 #pragma unroll
   for (int d = 0; d < PLAN_DEPTH; ++d) fetch_tile(d, tbuf[d]);
-  int r0 = p.plan_row_off[w], r1 = p.plan_row_off[w + 1];
-  fetch_entries(r0, r1, ea);
-  auto do_tile = [&](int k, u32x4 (&buf)[2], unsigned (&ecur)[PLAN_EB], unsigned (&enxt)[PLAN_EB]) {
+  int r0 = row_off[w], r1 = row_off[w + 1];
+  fetch_entries(r0, r1, enxt);
+  float run = 0.f;
+  auto do_tile = [&](int k, u32x4 (&buf)[2]) {
     __syncthreads();                                 // previous tile fully consumed (first pass: marg zeroed)
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -139,25 +134,26 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
     fetch_tile(k + PLAN_DEPTH, buf);                 // refill this buffer, PLAN_DEPTH tiles ahead
     int n0 = 0, n1 = 0;
     if (k + 1 < ntiles) {
-      n0 = p.plan_row_off[(k + 1) * NW + w];
-      n1 = p.plan_row_off[(k + 1) * NW + w + 1];
+      n0 = row_off[(k + 1) * NW + w];
+      n1 = row_off[(k + 1) * NW + w + 1];
     }
-    fetch_entries(n0, n1, enxt);                     // next tile's first entry batch
-    PlanRun open{-1, 0.f};
-    plan_consume(ecur, tile, marg, tmask, bits, open);
-    for (int r = r0 + PLAN_EB; r < r1; r += PLAN_EB) {      // long lists (hot student ids): further batches
-      fetch_entries(r, r1, ecur);
-      plan_consume(ecur, tile, marg, tmask, bits, open);
-    }
-    if (open.sid >= 0) marg[open.sid] += open.sum;
+    int r = r0;
+    do {                                             // an empty list still holds one batch of padding
+#pragma unroll
+      for (int j = 0; j < PLAN_EB; ++j) ecur[j] = enxt[j];
+      r += PLAN_EB;
+      const bool more = r < r1;                      // wave-uniform
+      fetch_entries(more ? r : n0, more ? r1 : n1, enxt);
+      plan_consume(ecur, tile, marg, tmask, bits, run);
+    } while (r < r1);
     r0 = n0;
     r1 = n1;
   };
   for (int k = 0; k < ntiles; k += PLAN_DEPTH) {     // unrolled by the depth: buffers are addressed statically
-    do_tile(k, tbuf[0], ea, eb);
-    if (k + 1 < ntiles) do_tile(k + 1, tbuf[1], eb, ea);
-    if (k + 2 < ntiles) do_tile(k + 2, tbuf[2], ea, eb);
-    if (k + 3 < ntiles) do_tile(k + 3, tbuf[3], eb, ea);
+    do_tile(k, tbuf[0]);
+    if (k + 1 < ntiles) do_tile(k + 1, tbuf[1]);
+    if (k + 2 < ntiles) do_tile(k + 2, tbuf[2]);
+    if (k + 3 < ntiles) do_tile(k + 3, tbuf[3]);
   }
   __syncthreads();
   // replicas into their id's slot: own slot first, then the replicas in ascending order

@@ -116,14 +116,16 @@ extern "C" int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_
 // threads by descending load onto the least-loaded thread; inside a tile an entry of a replicated
 // id goes to the replica whose owner holds the fewest entries of that tile so far.
 // The teacher vocabulary is cut into tiles of `tile` ids; for tile k and wave w, rows
-// row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries per row (one per lane,
-// 0xffffffff = padding), the entries (slot << log2(tile) | t - k*tile) of the wave's threads, each
-// thread's entries sorted by (slot, t).
+// row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries per row (one per lane), the
+// entries (slot << log2(tile) | t - k*tile) of the wave's threads, each thread's entries sorted by
+// (slot, t); bit 31 marks the first entry of a slot in the thread's list, bit 30 the last one, and
+// 0x80000000 (a first entry that never ends) is padding.
 extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int* tile_out,
                                       int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity,
                                       int64_t* ent_rows_out, int32_t* fold, int64_t fold_capacity,
                                       int64_t* n_fold_out, int* n_extra_out) {
   constexpr int NT = 1024, WAVE = 64, NW = NT / WAVE;
+  constexpr uint32_t FIRST = 0x80000000u, LAST = 0x40000000u, PAD = FIRST;
   constexpr int64_t LDS_BUDGET = 160 * 1024 - 1024;      // dynamic LDS one workgroup may use
   if (!t2s || !tile_out || !ent_rows_out || !n_fold_out || !n_extra_out) return DL_ERR_NULL;
   if (n_teacher <= 0 || n_student <= 0) return DL_ERR_SHAPE;
@@ -149,7 +151,7 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
   // replicas: LDS words left beside the marginal and the tile, handed one at a time to the id with
   // the largest load per slot, down to a quarter of a thread's even share
   int64_t budget = ((LDS_BUDGET - marg_bytes - (int64_t)tile * 4) / 4) & ~(int64_t)3;
-  const int64_t slot_limit = (1LL << (32 - tile_bits)) - 1;                 // slot ids must fit beside the tile offset
+  const int64_t slot_limit = (1LL << (30 - tile_bits)) - 1;                 // slot ids must fit between the flags and the tile offset
   if (n_pad >= slot_limit) return DL_ERR_LIMIT;
   budget = std::min<int64_t>(budget, slot_limit - n_pad);
   const double share = (double)n_mapped / NT;
@@ -235,7 +237,13 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
         for (size_t j = 0; j < longest; ++j)
           for (int l = 0; l < WAVE; ++l) {
             const auto& b = bucket[w * WAVE + l];
-            ent[(rows + (int64_t)j) * WAVE + l] = j < b.size() ? b[j] : 0xffffffffu;
+            uint32_t e = PAD;
+            if (j < b.size()) {
+              e = b[j];
+              if (j == 0 || (b[j - 1] >> tile_bits) != (b[j] >> tile_bits)) e |= FIRST;
+              if (j + 1 == b.size() || (b[j + 1] >> tile_bits) != (b[j] >> tile_bits)) e |= LAST;
+            }
+            ent[(rows + (int64_t)j) * WAVE + l] = e;
           }
       }
       rows += (int64_t)longest;

@@ -90,10 +90,15 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
             longest.append(rows.shape[0])
             for lane in range(64):
                 col = rows[:, lane]
-                live = col[col != 0xffffffff]
-                assert (col[len(live):] == 0xffffffff).all()            # padding only at the tail
+                live = col[col != 0x80000000]
+                assert (col[len(live):] == 0x80000000).all()            # padding only at the tail
+                first, last = (live >> 31).astype(bool), ((live >> 30) & 1).astype(bool)
+                live = live & 0x3fffffff
                 assert (np.diff(live.astype(np.int64)) > 0).all()         # sorted by (slot, t), no repeats
                 slot = (live >> bits).astype(np.int64)
+                change = np.diff(slot) != 0                               # run flags: first / last entry of a slot
+                assert np.array_equal(first, np.concatenate(([True], change))[:len(live)])
+                assert np.array_equal(last, np.concatenate((change, [True]))[-len(live):] if len(live) else last)
                 t = (live & (tile - 1)).astype(np.int64) + k * tile
                 assert (slot < n_pad + plan.n_extra).all()
                 assert (t2s[t] == slot_id[slot]).all()                    # the entry lands on a slot of its own id
