@@ -88,7 +88,7 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
   const int w = __builtin_amdgcn_readfirstlane(tid / WAVE);
   constexpr int NW = MARG_NT / WAVE;
   const int TS = p.plan_tile;
-  const int per = TS / 4 / MARG_NT;                 // 16-byte loads per thread per tile (1 or 2)
+  const int q_tile = TS / 4;                        // 16-byte loads per tile: 1024 .. 2048, up to two per thread
   const int ntiles = (int)((p.Vt + TS - 1) / TS);
   const int64_t n4 = p.Vt / 4;
   const int bits = p.plan_tile_bits;
@@ -101,8 +101,8 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
     for (int u = 0; u < 2; ++u) {
       // Unconditional load from a clamped address, then a select: with branch-free loads the
       // compiler knows how many are in flight and never has to drain the whole queue.
-      const int64_t c = (int64_t)k * (TS / 4) + (int64_t)u * MARG_NT + tid;
-      const bool live = u < per && c < n4;
+      const int64_t c = (int64_t)k * q_tile + (int64_t)u * MARG_NT + tid;
+      const bool live = u * MARG_NT + tid < q_tile && c < n4;
       const u32x4 v = load16_stream(prow + (live ? c : 0) * 16);
       buf[u] = live ? v : u32x4{0u, 0u, 0u, 0u};
     }
@@ -129,7 +129,7 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
     __syncthreads();                                 // previous tile fully consumed (first pass: marg zeroed)
 #pragma unroll
     for (int u = 0; u < 2; ++u)
-      if (u < per) *reinterpret_cast<u32x4*>(tile + ((int64_t)u * MARG_NT + tid) * 4) = buf[u];
+      if (u * MARG_NT + tid < q_tile) *reinterpret_cast<u32x4*>(tile + ((int64_t)u * MARG_NT + tid) * 4) = buf[u];
     __syncthreads();
     fetch_tile(k + PLAN_DEPTH, buf);                 // refill this buffer, PLAN_DEPTH tiles ahead
     int n0 = 0, n1 = 0;
@@ -364,7 +364,7 @@ static void allow_large_lds() {
 static size_t attach_plan(dl::MargParams& p, const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
                           const int32_t* plan_fold, int plan_n_fold, int plan_n_extra, bool vec, size_t lds_without_plan) {
   if (!plan_row_off || !plan_ent || !vec) return lds_without_plan;
-  if (plan_tile != 4096 && plan_tile != 8192) return lds_without_plan;
+  if (plan_tile < 4096 || plan_tile > 8192 || plan_tile % 1024) return lds_without_plan;
   if (plan_n_fold < 0 || plan_n_extra < 0 || (plan_n_fold > 0 && !plan_fold)) return lds_without_plan;
   const size_t need = (size_t)dl::plan_slot_words(p.Vs, plan_n_extra) * 4 + (size_t)plan_tile * 4;
   if (need > (size_t)dl::MARG_MAX_DYN_LDS) return lds_without_plan;

@@ -107,148 +107,202 @@ extern "C" int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_
 
 // ---- marginalisation plan --------------------------------------------------------------------
 // Layout consumed by the planned marginalisation kernels (1024 threads = 16 waves per workgroup).
-// Every accumulator word in LDS is touched by one thread only, so no atomics are needed and the
-// summation order is fixed.  Accumulator slots: slot s < n_student is student id s; a student id
-// that receives far more teacher ids than an even share (real vocabularies: the single-byte and
-// other short tokens) gets extra slots n_student_padded + j ("replicas") so that its load can be
-// split over several threads; after the last tile the replicas are folded into their id's slot in
-// a fixed order (fold table: triples id, first replica slot, replica count).  Slots are dealt to
-// threads by descending load onto the least-loaded thread; inside a tile an entry of a replicated
-// id goes to the replica whose owner holds the fewest entries of that tile so far.
-// The teacher vocabulary is cut into tiles of `tile` ids; for tile k and wave w, rows
-// row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries per row (one per lane), the
-// entries (slot << log2(tile) | t - k*tile) of the wave's threads, each thread's entries sorted by
-// (slot, t); bit 31 marks the first entry of a slot in the thread's list, bit 30 the last one, and
-// 0x80000000 (a first entry that never ends) is padding.
+// The teacher vocabulary is cut into tiles; the kernel stages one tile of probabilities in LDS at
+// a time, with workgroup barriers between tiles.  Inside a tile every accumulator word ("slot") in
+// LDS is touched by one thread only, so no atomics are needed and the summation order is fixed;
+// from tile to tile a slot may change hands.  Slot s < n_student is student id s.  The entries of
+// one id inside one tile are cut into pieces of at most PIECE entries (PIECE = the kernel's batch
+// of 8 where the LDS allows); piece 0 goes to the id's own slot, piece j > 0 to replica slot
+// first_extra[id] + j - 1 behind the padded marginal, so an id owns as many replicas as its
+// busiest tile needs.  After the last tile the replicas are folded into their id's slot in a
+// fixed order (fold table: triples id, first replica slot, replica count).  Inside a tile the
+// pieces are dealt, largest first, onto the thread that holds the fewest entries so far: lists
+// come out level, which matters because every wave of the workgroup waits for the longest one.
+// The tile size is chosen among the multiples of 1024 ids from 8192 down to 4096: a smaller tile
+// leaves more LDS for replicas (shorter lists when a few ids are very hot) but costs more barriers.
+// For tile k and wave w, rows row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries
+// per row (one per lane), the entries (slot << bits | t - k*tile), bits = 12 for a tile of 4096 and
+// 13 above, of the wave's threads, each thread's entries sorted by (slot, t); bit 31 marks the first
+// entry of a slot in the thread's list, bit 30 the last one, and 0x80000000 (a first entry that
+// never ends) is padding.
+namespace {
+
+constexpr int PLAN_NT = 1024, PLAN_WAVE = 64, PLAN_NW = PLAN_NT / PLAN_WAVE;
+constexpr int PLAN_BATCH = 8;                                 // entries per batch in the kernels
+constexpr int64_t PLAN_LDS_BUDGET = 160 * 1024 - 1024;        // dynamic LDS one workgroup may use
+
+struct PlanLayout {
+  int tile = 0, tile_bits = 0, piece = 0;
+  int64_t ntiles = 0, n_pad = 0, n_extra = 0, n_fold = 0;
+  std::vector<int32_t> first_extra;                           // per student id, -1: no replicas
+  std::vector<int32_t> reps;                                  // slots per student id (own one included)
+};
+
+// Entries of tile k as (student id, t - k*tile), sorted by (id, t).
+void tile_entries(const int32_t* t2s, int64_t n_teacher, const PlanLayout& L, int64_t k,
+                  std::vector<std::pair<int32_t, int32_t>>& out) {
+  out.clear();
+  const int64_t t0 = k * L.tile, t1 = std::min<int64_t>(n_teacher, t0 + L.tile);
+  for (int64_t t = t0; t < t1; ++t)
+    if (t2s[t] >= 0) out.emplace_back(t2s[t], (int32_t)(t - t0));
+  std::sort(out.begin(), out.end());
+}
+
+// Replica counts for a tile size: the smallest piece size >= PLAN_BATCH whose replicas fit the LDS
+// left beside the marginal and the tile.  False: the tile does not fit at all.
+bool plan_layout(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int tile, PlanLayout& L) {
+  L = PlanLayout();
+  L.tile = tile;
+  while ((1 << L.tile_bits) < tile) ++L.tile_bits;
+  L.ntiles = (n_teacher + tile - 1) / tile;
+  L.n_pad = (n_student + 3) & ~(int64_t)3;
+  const int64_t marg_bytes = L.n_pad * 4;
+  if (marg_bytes + (int64_t)tile * 4 > PLAN_LDS_BUDGET) return false;
+  int64_t budget = ((PLAN_LDS_BUDGET - marg_bytes - (int64_t)tile * 4) / 4) & ~(int64_t)3;
+  const int64_t slot_limit = (1LL << (30 - L.tile_bits)) - 1;   // slot ids must fit between the flags and the tile offset
+  if (L.n_pad >= slot_limit) return false;
+  budget = std::min<int64_t>(budget, slot_limit - L.n_pad);
+  // busiest tile of every id
+  std::vector<int32_t> busiest(n_student, 0), in_tile(n_student, 0);
+  for (int64_t k = 0; k < L.ntiles; ++k) {
+    const int64_t t0 = k * tile, t1 = std::min<int64_t>(n_teacher, t0 + tile);
+    for (int64_t t = t0; t < t1; ++t)
+      if (t2s[t] >= 0) ++in_tile[t2s[t]];
+    for (int64_t t = t0; t < t1; ++t)
+      if (t2s[t] >= 0) {
+        busiest[t2s[t]] = std::max(busiest[t2s[t]], in_tile[t2s[t]]);
+        in_tile[t2s[t]] = 0;
+      }
+  }
+  auto extra_for = [&](int piece) {
+    int64_t n = 0;
+    for (int64_t s = 0; s < n_student; ++s)
+      if (busiest[s] > piece) n += (busiest[s] + piece - 1) / piece - 1;
+    return n;
+  };
+  int piece = PLAN_BATCH;
+  while (extra_for(piece) > budget) piece += std::max(1, piece / 8);
+  L.piece = piece;
+  L.reps.assign(n_student, 1);
+  L.first_extra.assign(n_student, -1);
+  for (int64_t s = 0; s < n_student; ++s)
+    if (busiest[s] > piece) {
+      L.reps[s] = (busiest[s] + piece - 1) / piece;
+      L.first_extra[s] = (int32_t)(L.n_pad + L.n_extra);
+      L.n_extra += L.reps[s] - 1;
+      ++L.n_fold;
+    }
+  return true;
+}
+
+// The lists of the 1024 threads for one tile (entries without flags, sorted per thread).
+void plan_deal_tile(const PlanLayout& L, const std::vector<std::pair<int32_t, int32_t>>& entries,
+                    std::vector<std::vector<uint32_t>>& bucket) {
+  struct Piece { int32_t slot; int32_t first, count; };       // entries[first, first + count)
+  std::vector<Piece> pieces;
+  for (size_t i = 0; i < entries.size();) {
+    size_t j = i;
+    while (j < entries.size() && entries[j].first == entries[i].first) ++j;
+    const int32_t sid = entries[i].first, c = (int32_t)(j - i);
+    const int32_t n = (c + L.piece - 1) / L.piece, base = c / n, rem = c % n;
+    int32_t at = (int32_t)i;
+    for (int32_t q = 0; q < n; ++q) {
+      const int32_t len = base + (q < rem ? 1 : 0);
+      pieces.push_back({q == 0 ? sid : L.first_extra[sid] + q - 1, at, len});
+      at += len;
+    }
+    i = j;
+  }
+  std::stable_sort(pieces.begin(), pieces.end(), [](const Piece& a, const Piece& b) { return a.count > b.count; });
+  for (auto& b : bucket) b.clear();
+  std::vector<std::pair<int32_t, int32_t>> th(PLAN_NT);       // (entries held, thread): min-heap
+  for (int i = 0; i < PLAN_NT; ++i) th[i] = {0, i};
+  auto heavier = [](const std::pair<int32_t, int32_t>& a, const std::pair<int32_t, int32_t>& b) { return a > b; };
+  std::make_heap(th.begin(), th.end(), heavier);
+  for (const Piece& pc : pieces) {
+    std::pop_heap(th.begin(), th.end(), heavier);
+    auto& b = bucket[th.back().second];
+    for (int32_t q = 0; q < pc.count; ++q)
+      b.push_back(((uint32_t)pc.slot << L.tile_bits) | (uint32_t)entries[pc.first + q].second);
+    th.back().first += pc.count;
+    std::push_heap(th.begin(), th.end(), heavier);
+  }
+  for (auto& b : bucket) std::sort(b.begin(), b.end());       // (slot, t) ascending: slot in the high bits
+}
+
+}  // namespace
+
 extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int* tile_out,
                                       int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity,
                                       int64_t* ent_rows_out, int32_t* fold, int64_t fold_capacity,
                                       int64_t* n_fold_out, int* n_extra_out) {
-  constexpr int NT = 1024, WAVE = 64, NW = NT / WAVE;
   constexpr uint32_t FIRST = 0x80000000u, LAST = 0x40000000u, PAD = FIRST;
-  constexpr int64_t LDS_BUDGET = 160 * 1024 - 1024;      // dynamic LDS one workgroup may use
   if (!t2s || !tile_out || !ent_rows_out || !n_fold_out || !n_extra_out) return DL_ERR_NULL;
   if (n_teacher <= 0 || n_student <= 0) return DL_ERR_SHAPE;
   if (n_teacher > 0x7fffffffLL) return DL_ERR_LIMIT;
-  const int64_t n_pad = (n_student + 3) & ~(int64_t)3;
-  const int64_t marg_bytes = n_pad * 4;
-  int tile = 8192;
-  while (tile >= 4096 && marg_bytes + (int64_t)tile * 4 > LDS_BUDGET) tile >>= 1;
-  if (tile < 4096) return DL_ERR_LIMIT;                  // marginal + smallest tile do not fit the LDS
-  int tile_bits = 0;
-  while ((1 << tile_bits) < tile) ++tile_bits;
-  *tile_out = tile;
-  const int64_t ntiles = (n_teacher + tile - 1) / tile;
+  for (int64_t t = 0; t < n_teacher; ++t)
+    if (t2s[t] >= n_student) return DL_ERR_SHAPE;
 
-  // loads per student id
-  std::vector<int64_t> count(n_student, 0);
-  int64_t n_mapped = 0;
-  for (int64_t t = 0; t < n_teacher; ++t) {
-    const int32_t sid = t2s[t];
-    if (sid >= n_student) return DL_ERR_SHAPE;
-    if (sid >= 0) { ++count[sid]; ++n_mapped; }
+  // tile size: the cheapest of the candidates, counting per tile its batches (every wave waits for
+  // the longest list of the tile) and a fixed share for staging and barriers
+  std::vector<std::pair<int32_t, int32_t>> entries;
+  std::vector<std::vector<uint32_t>> bucket(PLAN_NT);
+  PlanLayout best;
+  int64_t best_cost = -1;
+  for (int tile = 8192; tile >= 4096; tile -= 1024) {
+    PlanLayout L;
+    if (!plan_layout(t2s, n_teacher, n_student, tile, L)) continue;
+    int64_t cost = 0;
+    for (int64_t k = 0; k < L.ntiles; ++k) {
+      tile_entries(t2s, n_teacher, L, k, entries);
+      plan_deal_tile(L, entries, bucket);
+      size_t longest = 0;
+      for (const auto& b : bucket) longest = std::max(longest, b.size());
+      const int64_t batches = std::max<int64_t>(1, ((int64_t)longest + PLAN_BATCH - 1) / PLAN_BATCH);
+      cost += batches * PLAN_BATCH + PLAN_BATCH / 2;
+    }
+    if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = L; }
   }
-  // replicas: LDS words left beside the marginal and the tile, handed one at a time to the id with
-  // the largest load per slot, down to a quarter of a thread's even share
-  int64_t budget = ((LDS_BUDGET - marg_bytes - (int64_t)tile * 4) / 4) & ~(int64_t)3;
-  const int64_t slot_limit = (1LL << (30 - tile_bits)) - 1;                 // slot ids must fit between the flags and the tile offset
-  if (n_pad >= slot_limit) return DL_ERR_LIMIT;
-  budget = std::min<int64_t>(budget, slot_limit - n_pad);
-  const double share = (double)n_mapped / NT;
-  std::vector<int32_t> reps(n_student, 1);
-  {
-    auto per_slot = [&](int32_t s) { return (double)count[s] / reps[s]; };
-    auto worse = [&](int32_t a, int32_t b) { const double la = per_slot(a), lb = per_slot(b); return la != lb ? la < lb : a > b; };
-    std::vector<int32_t> heap;
+  if (best_cost < 0) return DL_ERR_LIMIT;                    // marginal + smallest tile do not fit the LDS
+  const PlanLayout& L = best;
+  *tile_out = L.tile;
+  *n_fold_out = L.n_fold;
+  *n_extra_out = (int)L.n_extra;
+  if (fold) {
+    if (L.n_fold > fold_capacity) return DL_ERR_SHAPE;
+    int64_t f = 0;
     for (int64_t s = 0; s < n_student; ++s)
-      if ((double)count[s] > std::max(share / 4, 8.0)) heap.push_back((int32_t)s);
-    std::make_heap(heap.begin(), heap.end(), worse);
-    while (budget > 0 && !heap.empty()) {
-      std::pop_heap(heap.begin(), heap.end(), worse);
-      const int32_t s = heap.back();
-      if (per_slot(s) <= std::max(share / 4, 8.0)) break;                   // the heaviest is light enough: done
-      ++reps[s];
-      --budget;
-      std::push_heap(heap.begin(), heap.end(), worse);
-    }
-  }
-  // slots: own slot of every id that is hit, plus the replicas; fold table in ascending id order
-  struct Slot { int32_t slot; double load; };
-  std::vector<Slot> slots;
-  std::vector<int32_t> first_extra(n_student, -1);
-  int64_t n_extra = 0, n_fold = 0;
-  for (int64_t s = 0; s < n_student; ++s) {
-    if (count[s] == 0) continue;
-    const double load = (double)count[s] / reps[s];
-    slots.push_back({(int32_t)s, load});
-    if (reps[s] > 1) {
-      first_extra[s] = (int32_t)(n_pad + n_extra);
-      for (int j = 1; j < reps[s]; ++j) slots.push_back({(int32_t)(n_pad + n_extra + j - 1), load});
-      if (fold) {
-        if (n_fold >= fold_capacity) return DL_ERR_SHAPE;
-        fold[3 * n_fold] = (int32_t)s; fold[3 * n_fold + 1] = first_extra[s]; fold[3 * n_fold + 2] = reps[s] - 1;
+      if (L.reps[s] > 1) {
+        fold[3 * f] = (int32_t)s; fold[3 * f + 1] = L.first_extra[s]; fold[3 * f + 2] = L.reps[s] - 1;
+        ++f;
       }
-      n_extra += reps[s] - 1;
-      ++n_fold;
-    }
-  }
-  *n_fold_out = n_fold;
-  *n_extra_out = (int)n_extra;
-  // owners: heaviest slot first onto the least-loaded thread (ties: lower thread number)
-  std::stable_sort(slots.begin(), slots.end(), [](const Slot& a, const Slot& b) { return a.load > b.load; });
-  std::vector<int32_t> owner(n_pad + n_extra, -1);
-  {
-    std::vector<std::pair<double, int>> th(NT);
-    for (int i = 0; i < NT; ++i) th[i] = {0.0, i};
-    auto heavier = [](const std::pair<double, int>& a, const std::pair<double, int>& b) { return a > b; };
-    std::make_heap(th.begin(), th.end(), heavier);                          // min-heap on (load, thread)
-    for (const Slot& sl : slots) {
-      std::pop_heap(th.begin(), th.end(), heavier);
-      owner[sl.slot] = th.back().second;
-      th.back().first += sl.load;
-      std::push_heap(th.begin(), th.end(), heavier);
-    }
   }
 
-  std::vector<std::vector<uint32_t>> bucket(NT);
   int64_t rows = 0;
   if (row_off) row_off[0] = 0;
-  for (int64_t k = 0; k < ntiles; ++k) {
-    for (auto& b : bucket) b.clear();
-    const int64_t t0 = k * tile, t1 = std::min<int64_t>(n_teacher, t0 + tile);
-    for (int64_t t = t0; t < t1; ++t) {
-      const int32_t sid = t2s[t];
-      if (sid < 0) continue;
-      int32_t slot = sid;
-      size_t best = bucket[owner[sid]].size();
-      for (int j = 1; j < reps[sid]; ++j) {                                 // the replica whose owner is least busy in this tile
-        const int32_t cand = first_extra[sid] + j - 1;
-        const size_t sz = bucket[owner[cand]].size();
-        if (sz < best) { best = sz; slot = cand; }
-      }
-      bucket[owner[slot]].push_back(((uint32_t)slot << tile_bits) | (uint32_t)(t - t0));
-    }
-    for (auto& b : bucket) std::sort(b.begin(), b.end());      // (slot, t) ascending: slot in the high bits
-    for (int w = 0; w < NW; ++w) {
+  for (int64_t k = 0; k < L.ntiles; ++k) {
+    tile_entries(t2s, n_teacher, L, k, entries);
+    plan_deal_tile(L, entries, bucket);
+    for (int w = 0; w < PLAN_NW; ++w) {
       size_t longest = 0;
-      for (int l = 0; l < WAVE; ++l) longest = std::max(longest, bucket[w * WAVE + l].size());
+      for (int l = 0; l < PLAN_WAVE; ++l) longest = std::max(longest, bucket[w * PLAN_WAVE + l].size());
       if (ent) {
         if (rows + (int64_t)longest > ent_rows_capacity) return DL_ERR_SHAPE;
         for (size_t j = 0; j < longest; ++j)
-          for (int l = 0; l < WAVE; ++l) {
-            const auto& b = bucket[w * WAVE + l];
+          for (int l = 0; l < PLAN_WAVE; ++l) {
+            const auto& b = bucket[w * PLAN_WAVE + l];
             uint32_t e = PAD;
             if (j < b.size()) {
               e = b[j];
-              if (j == 0 || (b[j - 1] >> tile_bits) != (b[j] >> tile_bits)) e |= FIRST;
-              if (j + 1 == b.size() || (b[j + 1] >> tile_bits) != (b[j] >> tile_bits)) e |= LAST;
+              if (j == 0 || (b[j - 1] >> L.tile_bits) != (b[j] >> L.tile_bits)) e |= FIRST;
+              if (j + 1 == b.size() || (b[j + 1] >> L.tile_bits) != (b[j] >> L.tile_bits)) e |= LAST;
             }
-            ent[(rows + (int64_t)j) * WAVE + l] = e;
+            ent[(rows + (int64_t)j) * PLAN_WAVE + l] = e;
           }
       }
       rows += (int64_t)longest;
       if (rows > 0x7fffffffLL) return DL_ERR_LIMIT;
-      if (row_off) row_off[k * NW + w + 1] = (int32_t)rows;
+      if (row_off) row_off[k * PLAN_NW + w + 1] = (int32_t)rows;
     }
   }
   *ent_rows_out = rows;
