@@ -267,6 +267,7 @@ int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_student, in
  * row_off[16k + w] .. row_off[16k + w + 1] of `ent` hold 64 entries each (one per lane):
  * (slot << log2(tile) | t - k * tile), per thread sorted by (slot, t), with bit 31 set on the first
  * entry of a slot in the thread's list of the tile and bit 30 on the last one; 0x80000000 = padding.
+ * Every (tile, wave) list is padded to a multiple of 8 rows, at least 8.
  * Call once with row_off = ent = fold = NULL to learn *tile_out, *ent_rows_out, *n_fold_out and
  * *n_extra_out, allocate row_off int32 [16 * ceil(n_teacher / tile) + 1], ent uint32
  * [64 * ent_rows] and fold int32 [3 * n_fold], call again.

@@ -107,13 +107,11 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
       buf[u] = live ? v : u32x4{0u, 0u, 0u, 0u};
     }
   };
-  auto fetch_entries = [&](int r_first, int r_end, unsigned (&e)[PLAN_EB]) {
+  // every (tile, wave) list of the plan is a whole number of batches (padding entries included)
+  auto fetch_entries = [&](int r_first, unsigned (&e)[PLAN_EB]) {
+    const unsigned* at = p.plan_ent + (int64_t)r_first * WAVE + lane;
 #pragma unroll
-    for (int j = 0; j < PLAN_EB; ++j) {
-      const int r = r_first + j;
-      const unsigned v = p.plan_ent[(int64_t)(r < r_end ? r : 0) * WAVE + lane];
-      e[j] = r < r_end ? v : PLAN_PAD;
-    }
+    for (int j = 0; j < PLAN_EB; ++j) e[j] = at[j * WAVE];
   };
   // the constant address space tells the compiler that nothing in this kernel writes the offsets:
   // only then does it fetch them with scalar loads
@@ -123,7 +121,7 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
 #pragma unroll
   for (int d = 0; d < PLAN_DEPTH; ++d) fetch_tile(d, tbuf[d]);
   int r0 = row_off[w], r1 = row_off[w + 1];
-  fetch_entries(r0, r1, enxt);
+  fetch_entries(r0, enxt);
   float run = 0.f;
   auto do_tile = [&](int k, u32x4 (&buf)[2]) {
     __syncthreads();                                 // previous tile fully consumed (first pass: marg zeroed)
@@ -132,7 +130,7 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
       if (u * MARG_NT + tid < q_tile) *reinterpret_cast<u32x4*>(tile + ((int64_t)u * MARG_NT + tid) * 4) = buf[u];
     __syncthreads();
     fetch_tile(k + PLAN_DEPTH, buf);                 // refill this buffer, PLAN_DEPTH tiles ahead
-    int n0 = 0, n1 = 0;
+    int n0 = 0, n1 = 0;                              // behind the last tile: the plan's first batch, fetched and dropped
     if (k + 1 < ntiles) {
       n0 = row_off[(k + 1) * NW + w];
       n1 = row_off[(k + 1) * NW + w + 1];
@@ -142,8 +140,7 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
 #pragma unroll
       for (int j = 0; j < PLAN_EB; ++j) ecur[j] = enxt[j];
       r += PLAN_EB;
-      const bool more = r < r1;                      // wave-uniform
-      fetch_entries(more ? r : n0, more ? r1 : n1, enxt);
+      fetch_entries(r < r1 ? r : n0, enxt);          // wave-uniform choice
       plan_consume(ecur, tile, marg, tmask, bits, run);
     } while (r < r1);
     r0 = n0;

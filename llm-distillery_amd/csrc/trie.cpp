@@ -124,7 +124,8 @@ extern "C" int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_
 // per row (one per lane), the entries (slot << bits | t - k*tile), bits = 12 for a tile of 4096 and
 // 13 above, of the wave's threads, each thread's entries sorted by (slot, t); bit 31 marks the first
 // entry of a slot in the thread's list, bit 30 the last one, and 0x80000000 (a first entry that
-// never ends) is padding.
+// never ends) is padding.  Every (tile, wave) list is padded to whole batches of PLAN_BATCH rows, at
+// least one, so the kernels fetch batches without looking at the list's end.
 namespace {
 
 constexpr int PLAN_NT = 1024, PLAN_WAVE = 64, PLAN_NW = PLAN_NT / PLAN_WAVE;
@@ -286,6 +287,7 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
     for (int w = 0; w < PLAN_NW; ++w) {
       size_t longest = 0;
       for (int l = 0; l < PLAN_WAVE; ++l) longest = std::max(longest, bucket[w * PLAN_WAVE + l].size());
+      longest = std::max<size_t>(PLAN_BATCH, (longest + PLAN_BATCH - 1) / PLAN_BATCH * PLAN_BATCH);   // whole batches, at least one
       if (ent) {
         if (rows + (int64_t)longest > ent_rows_capacity) return DL_ERR_SHAPE;
         for (size_t j = 0; j < longest; ++j)

@@ -89,6 +89,7 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
         for w in range(16):
             rows = ent[row_off[16 * k + w]:row_off[16 * k + w + 1]]
             longest.append(rows.shape[0])
+            assert rows.shape[0] >= 8 and rows.shape[0] % 8 == 0            # whole batches of the kernels
             for lane in range(64):
                 col = rows[:, lane]
                 live = col[col != 0x80000000]
