@@ -99,12 +99,13 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
   auto fetch_tile = [&](int k, u32x4 (&buf)[2]) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      // Unconditional load from a clamped address, then a select: with branch-free loads the
-      // compiler knows how many are in flight and never has to drain the whole queue.
+      // Unconditional load from a clamped address: with branch-free loads the compiler knows how
+      // many are in flight and never has to drain the whole queue.  What a clamped load brings is
+      // never used: no entry points behind the end of the row, and a select on the value here
+      // would make the thread wait for the load right away instead of PLAN_DEPTH tiles later.
       const int64_t c = (int64_t)k * q_tile + (int64_t)u * MARG_NT + tid;
       const bool live = u * MARG_NT + tid < q_tile && c < n4;
-      const u32x4 v = load16_stream(prow + (live ? c : 0) * 16);
-      buf[u] = live ? v : u32x4{0u, 0u, 0u, 0u};
+      buf[u] = load16_stream(prow + (live ? c : 0) * 16);
     }
   };
   // every (tile, wave) list of the plan is a whole number of batches (padding entries included)
@@ -117,40 +118,49 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
   // only then does it fetch them with scalar loads
   typedef const __attribute__((address_space(4))) int32_t* ConstI32;
   ConstI32 row_off = (ConstI32)p.plan_row_off;
-  unsigned ecur[PLAN_EB], enxt[PLAN_EB];            // the batch being consumed and the one in flight
+  // Per buffer in flight: the tile's data and the first batch of its list, both fetched PLAN_DEPTH
+  // tiles ahead.  Loads complete in issue order, so a thread that waits for the batch of the next
+  // tile also waits for everything issued before it: fetching the batches as far ahead as the
+  // tiles is what lets the tile loads stay in flight for several tiles.
+  unsigned ebuf[PLAN_DEPTH][PLAN_EB];
+  int r_first[PLAN_DEPTH], r_end[PLAN_DEPTH];
+  auto list_of = [&](int k, int& first, int& end) {  // behind the last tile: the plan's first batch, fetched and dropped
+    first = end = 0;
+    if (k < ntiles) {
+      first = row_off[k * NW + w];
+      end = row_off[k * NW + w + 1];
+    }
+  };
 #pragma unroll
-  for (int d = 0; d < PLAN_DEPTH; ++d) fetch_tile(d, tbuf[d]);
-  int r0 = row_off[w], r1 = row_off[w + 1];
-  fetch_entries(r0, enxt);
+  for (int d = 0; d < PLAN_DEPTH; ++d) {
+    fetch_tile(d, tbuf[d]);
+    list_of(d, r_first[d], r_end[d]);
+    fetch_entries(r_first[d], ebuf[d]);
+  }
   float run = 0.f;
-  auto do_tile = [&](int k, u32x4 (&buf)[2]) {
+  auto do_tile = [&](int k, u32x4 (&buf)[2], unsigned (&e)[PLAN_EB], int& first, int& end) {
     __syncthreads();                                 // previous tile fully consumed (first pass: marg zeroed)
 #pragma unroll
     for (int u = 0; u < 2; ++u)
       if (u * MARG_NT + tid < q_tile) *reinterpret_cast<u32x4*>(tile + ((int64_t)u * MARG_NT + tid) * 4) = buf[u];
     __syncthreads();
     fetch_tile(k + PLAN_DEPTH, buf);                 // refill this buffer, PLAN_DEPTH tiles ahead
-    int n0 = 0, n1 = 0;                              // behind the last tile: the plan's first batch, fetched and dropped
-    if (k + 1 < ntiles) {
-      n0 = row_off[(k + 1) * NW + w];
-      n1 = row_off[(k + 1) * NW + w + 1];
+    int n_first, n_end;
+    list_of(k + PLAN_DEPTH, n_first, n_end);
+    plan_consume(e, tile, marg, tmask, bits, run);
+    for (int r = first + PLAN_EB; r < end; r += PLAN_EB) {     // a list longer than one batch (rare: not enough LDS
+      fetch_entries(r, e);                                     // for replicas): fetched on the spot
+      plan_consume(e, tile, marg, tmask, bits, run);
     }
-    int r = r0;
-    do {                                             // an empty list still holds one batch of padding
-#pragma unroll
-      for (int j = 0; j < PLAN_EB; ++j) ecur[j] = enxt[j];
-      r += PLAN_EB;
-      fetch_entries(r < r1 ? r : n0, enxt);          // wave-uniform choice
-      plan_consume(ecur, tile, marg, tmask, bits, run);
-    } while (r < r1);
-    r0 = n0;
-    r1 = n1;
+    fetch_entries(n_first, e);
+    first = n_first;
+    end = n_end;
   };
   for (int k = 0; k < ntiles; k += PLAN_DEPTH) {     // unrolled by the depth: buffers are addressed statically
-    do_tile(k, tbuf[0]);
-    if (k + 1 < ntiles) do_tile(k + 1, tbuf[1]);
-    if (k + 2 < ntiles) do_tile(k + 2, tbuf[2]);
-    if (k + 3 < ntiles) do_tile(k + 3, tbuf[3]);
+    do_tile(k, tbuf[0], ebuf[0], r_first[0], r_end[0]);
+    if (k + 1 < ntiles) do_tile(k + 1, tbuf[1], ebuf[1], r_first[1], r_end[1]);
+    if (k + 2 < ntiles) do_tile(k + 2, tbuf[2], ebuf[2], r_first[2], r_end[2]);
+    if (k + 3 < ntiles) do_tile(k + 3, tbuf[3], ebuf[3], r_first[3], r_end[3]);
   }
   __syncthreads();
   // replicas into their id's slot: own slot first, then the replicas in ascending order
