@@ -34,45 +34,46 @@ struct MargParams {
   const void* logits; int s_dtype; int64_t row_stride; int64_t n_srows; const int32_t* row_map;
   float inv_T_s, inv_T_t, grad_scale; float* row_loss; void* grad; int64_t grad_stride;
   // plan (all NULL/0: accumulate with LDS atomics along t2s instead)
-  const int32_t* plan_row_off; const uint32_t* plan_ent; int plan_tile; int plan_tile_bits;
+  const int32_t* plan_row_off; const uint32_t* plan_ent; int plan_tile;
   const int32_t* plan_fold; int plan_n_fold; int plan_n_extra;       // replica slots behind the marginal and how they fold
 };
 
-// LDS words of the planned form before the tile: the marginal and the replica slots, both padded to 16 bytes
+// LDS words of the planned form behind the tile: the marginal and the replica slots, both padded to
+// 16 bytes, and one slot per lane for the run totals that are not final yet
+constexpr int PLAN_SPARE_SLOTS = 64;
 __host__ __device__ inline int64_t plan_slot_words(int64_t Vs, int n_extra) {
-  return ((Vs + 3) & ~(int64_t)3) + (((int64_t)n_extra + 3) & ~(int64_t)3);
+  return ((Vs + 3) & ~(int64_t)3) + (((int64_t)n_extra + 3) & ~(int64_t)3) + PLAN_SPARE_SLOTS;
 }
 
-// Plan entry: bit 31 = first entry of a run of one slot in its thread's list of the tile, bit 30 =
-// last entry of that run, below them (slot << log2(tile)) | offset inside the tile.  Padding is a
-// "first" entry that is never a "last" one: it restarts the running sum and stores nothing.
-constexpr unsigned PLAN_FIRST = 0x80000000u, PLAN_LAST = 0x40000000u, PLAN_PAD = PLAN_FIRST;
+// Plan entry: bit 31 = first entry of a run of one slot in its thread's list of the tile; bits
+// 15-30 = the slot on the last entry of the run, the lane's spare slot on the others; bits 0-14 =
+// byte offset of the probability inside the tile.  Padding is a first entry on the spare slot.
+constexpr unsigned PLAN_FIRST = 0x80000000u;
+constexpr int PLAN_SLOT_SHIFT = 15;
+constexpr unsigned PLAN_OFFSET_MASK = 0x7ffcu, PLAN_SLOT_MASK = 0xffffu;
 
 // Marginal of one teacher row into marg[0, Vs) (LDS, zeroed here) along a plan; `tile` is LDS
 // scratch of plan_tile floats.  fp32 probabilities, 16-byte aligned rows.
 //
-// Latencies are kept off the critical path by batching: a thread holds a batch of PLAN_EB entries
-// in registers while the following batch (of this tile, or the first one of the next tile) is in
-// flight; it reads the tile for the whole batch at once, and for the entries that end a run the
-// slot's present value as well, so that no store waits for a load issued next to it.  A slot
-// belongs to one thread and has one run per thread and tile, so those early reads see no store of
-// the same batch.  The run totals are added as slot + (0 + v0 + v1 + ...), in list order.
+// The hot loop is straight-line code: per entry a read of the tile, a read of the entry's slot, the
+// running sum of the run (restarted where the entry says so) and a store of slot + running sum.
+// Only the store of a run's last entry lands in the run's slot; the others go to the lane's spare
+// slot, which nobody reads for its value.  A slot belongs to one thread inside a tile and has one
+// run per thread and tile, so reading all slots of a batch before its stores changes nothing.
+// The run totals are added as slot + (0 + v0 + v1 + ...), in list order.
 constexpr int PLAN_EB = 8;           // entries per batch
 
-__device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const float* tile, float* marg,
-                                             unsigned tmask, int bits, float& run) {
+__device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const float* tile, float* marg, float& run) {
   float val[PLAN_EB], base[PLAN_EB];
 #pragma unroll
-  for (int j = 0; j < PLAN_EB; ++j) val[j] = tile[e[j] & tmask];
+  for (int j = 0; j < PLAN_EB; ++j)
+    val[j] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(tile) + (e[j] & PLAN_OFFSET_MASK));
+#pragma unroll
+  for (int j = 0; j < PLAN_EB; ++j) base[j] = marg[(e[j] >> PLAN_SLOT_SHIFT) & PLAN_SLOT_MASK];
 #pragma unroll
   for (int j = 0; j < PLAN_EB; ++j) {
-    base[j] = 0.f;
-    if (e[j] & PLAN_LAST) base[j] = marg[(e[j] & ~(PLAN_FIRST | PLAN_LAST)) >> bits];
-  }
-#pragma unroll
-  for (int j = 0; j < PLAN_EB; ++j) {
-    run = ((e[j] & PLAN_FIRST) ? 0.f : run) + val[j];
-    if (e[j] & PLAN_LAST) marg[(e[j] & ~(PLAN_FIRST | PLAN_LAST)) >> bits] = base[j] + run;
+    run = ((int)e[j] < 0 ? 0.f : run) + val[j];
+    marg[(e[j] >> PLAN_SLOT_SHIFT) & PLAN_SLOT_MASK] = base[j] + run;
   }
 }
 
@@ -91,8 +92,6 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
   const int q_tile = TS / 4;                        // 16-byte loads per tile: 1024 .. 2048, up to two per thread
   const int ntiles = (int)((p.Vt + TS - 1) / TS);
   const int64_t n4 = p.Vt / 4;
-  const int bits = p.plan_tile_bits;
-  const unsigned tmask = (1u << bits) - 1u;
   const int n_slots = (int)plan_slot_words(p.Vs, p.plan_n_extra);
   for (int j = tid; j < n_slots; j += MARG_NT) marg[j] = 0.f;
   u32x4 tbuf[PLAN_DEPTH][2];
@@ -147,10 +146,10 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
     fetch_tile(k + PLAN_DEPTH, buf);                 // refill this buffer, PLAN_DEPTH tiles ahead
     int n_first, n_end;
     list_of(k + PLAN_DEPTH, n_first, n_end);
-    plan_consume(e, tile, marg, tmask, bits, run);
+    plan_consume(e, tile, marg, run);
     for (int r = first + PLAN_EB; r < end; r += PLAN_EB) {     // a list longer than one batch (rare: not enough LDS
       fetch_entries(r, e);                                     // for replicas): fetched on the spot
-      plan_consume(e, tile, marg, tmask, bits, run);
+      plan_consume(e, tile, marg, run);
     }
     fetch_entries(n_first, e);
     first = n_first;
@@ -241,8 +240,9 @@ __global__ __launch_bounds__(MARG_NT) void marginalise_map_kernel(const MargPara
   const char* prow = reinterpret_cast<const char*>(p.probs) + r * p.p_stride * pb;
   float* out = p.marg + r * p.marg_stride;
   if (VEC && p.plan_ent) {
-    accumulate_marginal_planned(p, prow, acc, acc + plan_slot_words(p.Vs, p.plan_n_extra));
-    for (int j = threadIdx.x; j < p.Vs; j += MARG_NT) out[j] = p.out_log ? logf(acc[j]) : acc[j];
+    float* marg = acc + p.plan_tile;                // the tile sits first: its addresses are then plain offsets
+    accumulate_marginal_planned(p, prow, marg, acc);
+    for (int j = threadIdx.x; j < p.Vs; j += MARG_NT) out[j] = p.out_log ? logf(marg[j]) : marg[j];
     return;
   }
   for (int64_t s_lo = 0; s_lo < p.Vs; s_lo += MARG_MAX_VS) {
@@ -319,16 +319,18 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
   const char* srow = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes;
   const int pb = p.p_dtype == F32 ? 4 : 2;
   const char* prow = reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb;
+  float* marg = acc;
   if (VEC && p.plan_ent) {
-    accumulate_marginal_planned(p, prow, acc, acc + plan_slot_words(p.Vs, p.plan_n_extra));   // needs the registers itself
+    marg = acc + p.plan_tile;                    // the tile sits first: its addresses are then plain offsets
+    accumulate_marginal_planned(p, prow, marg, acc);   // needs the registers itself
     rows.load(srow, p.Vs / 8);
   } else {
     rows.load(srow, p.Vs / 8);                   // in flight during the scatter
     accumulate_marginal<VEC>(p, prow, acc, 0, (int)p.Vs);
   }
-  for (int j = tid; j < p.Vs; j += MARG_NT) acc[j] = fast_log2(acc[j]) * LN2;      // log 0 = -inf: off the support
+  for (int j = tid; j < p.Vs; j += MARG_NT) marg[j] = fast_log2(marg[j]) * LN2;    // log 0 = -inf: off the support
   __syncthreads();
-  rows.lt = acc;
+  rows.lt = marg;
   const DenseStats st = dense_stats<DL_RKL, MARG_NT>(rows, p.inv_T_s, p.inv_T_t, red);
   const bool empty = st.tmax == -INFINITY;        // the teacher row carried no mass at all
   if (tid == 0 && p.row_loss) p.row_loss[r] = empty ? 0.f : st.loss;
@@ -376,7 +378,6 @@ static size_t attach_plan(dl::MargParams& p, const int32_t* plan_row_off, const 
   const size_t need = (size_t)dl::plan_slot_words(p.Vs, plan_n_extra) * 4 + (size_t)plan_tile * 4;
   if (need > (size_t)dl::MARG_MAX_DYN_LDS) return lds_without_plan;
   p.plan_row_off = plan_row_off; p.plan_ent = plan_ent; p.plan_tile = plan_tile;
-  p.plan_tile_bits = plan_tile == 4096 ? 12 : 13;
   p.plan_fold = plan_fold; p.plan_n_fold = plan_n_fold; p.plan_n_extra = plan_n_extra;
   return need;
 }

@@ -121,16 +121,20 @@ extern "C" int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_
 // The tile size is chosen among the multiples of 1024 ids from 8192 down to 4096: a smaller tile
 // leaves more LDS for replicas (shorter lists when a few ids are very hot) but costs more barriers.
 // For tile k and wave w, rows row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries
-// per row (one per lane), the entries (slot << bits | t - k*tile), bits = 12 for a tile of 4096 and
-// 13 above, of the wave's threads, each thread's entries sorted by (slot, t); bit 31 marks the first
-// entry of a slot in the thread's list, bit 30 the last one, and 0x80000000 (a first entry that
-// never ends) is padding.  Every (tile, wave) list is padded to whole batches of PLAN_BATCH rows, at
-// least one, so the kernels fetch batches without looking at the list's end.
+// per row (one per lane), the entries of the wave's threads, each thread's entries sorted by
+// (slot, t).  A thread adds up a run of entries of one slot and stores slot + running sum after
+// every entry, so only the run's last entry may name the slot: bits 15-30 hold the slot there and
+// the lane's spare slot (behind the replicas, one per lane) on the other entries; bit 31 marks the
+// first entry of a run (the running sum restarts); bits 0-14 hold 4 * (t - k*tile), the byte offset
+// inside the tile.  Padding is a first entry on the spare slot with offset 0.  Every (tile, wave)
+// list is padded to whole batches of PLAN_BATCH rows, at least one, so the kernels fetch batches
+// without looking at the list's end.
 namespace {
 
 constexpr int PLAN_NT = 1024, PLAN_WAVE = 64, PLAN_NW = PLAN_NT / PLAN_WAVE;
 constexpr int PLAN_BATCH = 8;                                 // entries per batch in the kernels
-constexpr int64_t PLAN_LDS_BUDGET = 160 * 1024 - 1024;        // dynamic LDS one workgroup may use
+constexpr int64_t PLAN_LDS_BUDGET = 160 * 1024 - 1024 - 64 * 4;   // dynamic LDS one workgroup may use, less the spare slots
+constexpr int PLAN_SLOT_SHIFT = 15;
 
 struct PlanLayout {
   int tile = 0, tile_bits = 0, piece = 0;
@@ -160,7 +164,7 @@ bool plan_layout(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int t
   const int64_t marg_bytes = L.n_pad * 4;
   if (marg_bytes + (int64_t)tile * 4 > PLAN_LDS_BUDGET) return false;
   int64_t budget = ((PLAN_LDS_BUDGET - marg_bytes - (int64_t)tile * 4) / 4) & ~(int64_t)3;
-  const int64_t slot_limit = (1LL << (30 - L.tile_bits)) - 1;   // slot ids must fit between the flags and the tile offset
+  const int64_t slot_limit = (1LL << 16) - PLAN_WAVE - 4;       // slot ids (the spare ones included) take 16 bits of an entry
   if (L.n_pad >= slot_limit) return false;
   budget = std::min<int64_t>(budget, slot_limit - L.n_pad);
   // busiest tile of every id
@@ -237,7 +241,7 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
                                       int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity,
                                       int64_t* ent_rows_out, int32_t* fold, int64_t fold_capacity,
                                       int64_t* n_fold_out, int* n_extra_out) {
-  constexpr uint32_t FIRST = 0x80000000u, LAST = 0x40000000u, PAD = FIRST;
+  constexpr uint32_t FIRST = 0x80000000u;
   if (!t2s || !tile_out || !ent_rows_out || !n_fold_out || !n_extra_out) return DL_ERR_NULL;
   if (n_teacher <= 0 || n_student <= 0) return DL_ERR_SHAPE;
   if (n_teacher > 0x7fffffffLL) return DL_ERR_LIMIT;
@@ -279,6 +283,7 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
       }
   }
 
+  const uint32_t spare = (uint32_t)(L.n_pad + ((L.n_extra + 3) & ~(int64_t)3));   // first of the 64 spare slots
   int64_t rows = 0;
   if (row_off) row_off[0] = 0;
   for (int64_t k = 0; k < L.ntiles; ++k) {
@@ -293,11 +298,12 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
         for (size_t j = 0; j < longest; ++j)
           for (int l = 0; l < PLAN_WAVE; ++l) {
             const auto& b = bucket[w * PLAN_WAVE + l];
-            uint32_t e = PAD;
+            uint32_t e = FIRST | (spare + (uint32_t)l) << PLAN_SLOT_SHIFT;
             if (j < b.size()) {
-              e = b[j];
-              if (j == 0 || (b[j - 1] >> L.tile_bits) != (b[j] >> L.tile_bits)) e |= FIRST;
-              if (j + 1 == b.size() || (b[j + 1] >> L.tile_bits) != (b[j] >> L.tile_bits)) e |= LAST;
+              const uint32_t slot = b[j] >> L.tile_bits, offset = b[j] & ((1u << L.tile_bits) - 1u);
+              const bool first = j == 0 || (b[j - 1] >> L.tile_bits) != slot;
+              const bool last = j + 1 == b.size() || (b[j + 1] >> L.tile_bits) != slot;
+              e = (first ? FIRST : 0u) | (last ? slot : spare + (uint32_t)l) << PLAN_SLOT_SHIFT | offset << 2;
             }
             ent[(rows + (int64_t)j) * PLAN_WAVE + l] = e;
           }

@@ -60,6 +60,24 @@ def test_marginal_map_and_csr_forms(D, Vs, Vt, alphabet):
     assert np.isneginf(lg[ref == 0]).all()
 
 
+def test_planned_marginal_with_lists_longer_than_one_batch(D):
+    """A student vocabulary that leaves the LDS almost no room for replicas, and a few very hot ids:
+    the per-thread lists of a tile then run over several batches of the kernel."""
+    Vs, Vt, R = 36500, 30000, 5
+    rng = np.random.default_rng(11)
+    t2s = rng.integers(-1, Vs, Vt).astype(np.int32)
+    hot = rng.random(Vt) < 0.9
+    t2s[hot] = rng.integers(0, 16, int(hot.sum())) * 977
+    probs = torch.softmax(torch.randn(R, Vt, generator=torch.Generator().manual_seed(11)) * 2, -1)
+    plan = D.vocab_utils.MarginalPlan(t2s, Vs, DEV)
+    assert plan.ent is not None and int(np.diff(plan.row_off.cpu().numpy()).max()) > 8
+    ref = O.marginalise_map(probs.numpy(), t2s, Vs)
+    m_plan = D.vocab_utils.marginalise(probs.to(DEV), plan=plan, n_student=Vs).cpu().numpy()
+    np.testing.assert_allclose(m_plan, ref, rtol=4e-6, atol=1e-9)
+    assert np.array_equal(m_plan == 0, ref == 0)
+    assert np.array_equal(m_plan, D.vocab_utils.marginalise(probs.to(DEV), plan=plan, n_student=Vs).cpu().numpy())
+
+
 def test_marginal_of_16bit_probabilities(D):
     t2s, probs = _case(4, 512, 2048, 2)
     got = D.vocab_utils.marginalise(probs.to(torch.bfloat16).to(DEV), t2s=torch.tensor(t2s, device=DEV), n_student=512)

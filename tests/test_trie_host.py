@@ -65,7 +65,6 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     plan = D.vocab_utils.MarginalPlan(t2s, Vs, "cpu")
     tile = plan.tile
     assert 4096 <= tile <= 8192 and tile % 1024 == 0
-    bits = 12 if tile == 4096 else 13
     row_off = plan.row_off.numpy()
     ent = plan.ent.numpy().view(np.uint32)
     fold = plan.fold.numpy()[:plan.n_fold]
@@ -91,22 +90,23 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
             longest.append(rows.shape[0])
             assert rows.shape[0] >= 8 and rows.shape[0] % 8 == 0            # whole batches of the kernels
             for lane in range(64):
-                col = rows[:, lane]
-                live = col[col != 0x80000000]
-                assert (col[len(live):] == 0x80000000).all()            # padding only at the tail
-                first, last = (live >> 31).astype(bool), ((live >> 30) & 1).astype(bool)
-                live = live & 0x3fffffff
-                assert (np.diff(live.astype(np.int64)) > 0).all()         # sorted by (slot, t), no repeats
-                slot = (live >> bits).astype(np.int64)
-                change = np.diff(slot) != 0                               # run flags: first / last entry of a slot
-                assert np.array_equal(first, np.concatenate(([True], change))[:len(live)])
-                assert np.array_equal(last, np.concatenate((change, [True]))[-len(live):] if len(live) else last)
-                t = (live & ((1 << bits) - 1)).astype(np.int64) + k * tile
-                assert (slot < n_pad + plan.n_extra).all()
-                assert (t2s[t] == slot_id[slot]).all()                    # the entry lands on a slot of its own id
-                for sl in np.unique(slot):
+                col = rows[:, lane].astype(np.int64)
+                first, slot, offset = (col >> 31).astype(bool), (col >> 15) & 0xffff, col & 0x7fff
+                assert (offset % 4 == 0).all()
+                spare = n_pad + ((plan.n_extra + 3) & ~3) + lane          # where unfinished run totals are parked
+                ends = np.nonzero(slot != spare)[0]                      # the last entry of every run names the run's slot
+                n_live = ends[-1] + 1 if len(ends) else 0
+                assert (col[n_live:] == (1 << 31 | spare << 15)).all()   # padding only at the tail: restarts, parks, offset 0
+                starts = np.concatenate(([0], ends[:-1] + 1)) if len(ends) else ends
+                assert np.array_equal(np.nonzero(first[:n_live])[0], starts)        # the running sum restarts exactly at run starts
+                run_slot = slot[ends]
+                assert (np.diff(run_slot) > 0).all() and (run_slot < n_pad + plan.n_extra).all()   # one run per slot, ascending
+                for a, z, sl in zip(starts, ends, run_slot):
+                    t = offset[a:z + 1] // 4 + k * tile
+                    assert (np.diff(t) > 0).all() and (t < Vt).all()
+                    assert (t2s[t] == slot_id[sl]).all()                  # the entries land on a slot of their own id
                     assert owner.setdefault(int(sl), w * 64 + lane) == w * 64 + lane      # one thread per LDS word inside a tile
-                seen[t] += 1
+                    seen[t] += 1
     assert np.array_equal(seen, (t2s >= 0).astype(np.int32))
     # half of the entries sit on 8 ids: without replicas one thread would hold > 1200 entries of a tile
     assert max(longest) <= 4 * (tile // 1024)
