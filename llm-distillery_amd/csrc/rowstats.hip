@@ -146,7 +146,9 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
-      v[i] = ch < c_hi ? load16_stream(row + ch * 16) : C::neg_inf();
+      // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
+      // finds its lines in L2 instead of fetching them a second time
+      v[i] = ch < c_hi ? *reinterpret_cast<const u32x4*>(row + ch * 16) : C::neg_inf();
     }
     correction_clear<NT>(s_head, s_own);
     stage();

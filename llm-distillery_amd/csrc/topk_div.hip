@@ -345,7 +345,9 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int64_t c = (int64_t)i * NT + tid;
-    reg[i] = c < nch ? load16_stream(rpart + c * 16) : C::neg_inf();
+    // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
+    // finds its lines in L2 instead of fetching them a second time (0.47 GB less per 32768 rows of K = 200)
+    reg[i] = c < nch ? *reinterpret_cast<const u32x4*>(rpart + c * 16) : C::neg_inf();
   }
 
   // teacher side while the row is in flight
