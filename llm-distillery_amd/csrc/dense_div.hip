@@ -121,6 +121,99 @@ __global__ __launch_bounds__(NT) void dense_stream_vec_kernel(const DenseParams 
   if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
 }
 
+// Rows too wide for both to sit in registers, but not for the student's alone: the student row is
+// read from HBM once and kept on the CU, half of it in registers (NUS / 2 units per thread) and half
+// in LDS (128 KiB; all of it in registers leaves too few for the sweeps: the compiler spills).  The
+// teacher row is streamed through a ring of D units per thread in every sweep (its later reads come
+// from L2 as far as the rows in flight fit there).  Against streaming both rows this saves two or
+// three reads of the student row.
+template <class TagS, class TagT, int NT, int NUS>
+struct StudentRegRows {
+  static constexpr int D = Unit<TagT>::NC == 1 ? 4 : 2;      // teacher units in flight per thread
+  static constexpr int NR = NUS / 2;                         // student units in registers; the rest in LDS
+  static constexpr int NC = Unit<TagS>::NC;
+  static constexpr size_t LDS_BYTES = (size_t)(NUS - NR) * NC * NT * 16;
+  Unit<TagS> s[NR];
+  u32x4* lds;
+  const char* trow;
+  int64_t nunits;
+  __device__ __forceinline__ void load(const char* srow, const char* trow_, int64_t nu, u32x4* lds_) {
+    trow = trow_;
+    nunits = nu;
+    lds = lds_;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int64_t u = (int64_t)i * NT + threadIdx.x;
+      if (u < nunits) s[i].load(srow, u);
+      else s[i].fill_neg_inf();
+    }
+#pragma unroll
+    for (int i = NR; i < NUS; ++i) {         // every thread reads back only what it wrote: no barrier needed
+      const int64_t u = (int64_t)i * NT + threadIdx.x;
+      Unit<TagS> x;
+      if (u < nunits) x.load(srow, u);
+      else x.fill_neg_inf();
+#pragma unroll
+      for (int k = 0; k < NC; ++k) lds[((i - NR) * NC + k) * NT + threadIdx.x] = x.c[k];
+    }
+  }
+  template <class F>
+  __device__ __forceinline__ void sweep(F f) {
+    Unit<TagT> t[D];
+#pragma unroll
+    for (int d = 0; d < D && d < NUS; ++d) {
+      const int64_t u = (int64_t)d * NT + threadIdx.x;
+      if (u < nunits) StreamRows<TagS, TagT, NT>::fetch(t[d], trow, u);
+    }
+#pragma unroll
+    for (int i = 0; i < NUS; ++i) {
+      const int64_t u = (int64_t)i * NT + threadIdx.x;
+      if (u < nunits) {
+        float a[8], b[8];
+        if (i < NR) {
+          s[i].unpack(a);
+        } else {
+          Unit<TagS> x;
+#pragma unroll
+          for (int k = 0; k < NC; ++k) x.c[k] = lds[((i - NR) * NC + k) * NT + threadIdx.x];
+          x.unpack(a);
+        }
+        t[i % D].unpack(b);
+        f(u, a, b);
+      }
+      if (i + D < NUS) {                     // refill the slot just used
+        const int64_t un = (int64_t)(i + D) * NT + threadIdx.x;
+        if (un < nunits) StreamRows<TagS, TagT, NT>::fetch(t[i % D], trow, un);
+      }
+      // no memory access moves across this point: without it the compiler issues the loads of all
+      // units up front and spills the registers that hold them
+      asm volatile("" ::: "memory");
+    }
+  }
+};
+
+template <int KIND, class TagS, class TagT, int NT, int NUS>
+__global__ __launch_bounds__(NT) void dense_student_reg_kernel(const DenseParams p) {
+  extern __shared__ __align__(16) u32x4 student_half[];
+  __shared__ float red[64];
+  const int64_t r = xcd_banded_row(blockIdx.x);
+  if (r >= p.n_rows) return;
+  const int tid = threadIdx.x;
+  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
+  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  if (trow < 0) {
+    if (grow) zero_row<TagS, NT>(grow, p.V / TagS::epc);
+    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    return;
+  }
+  StudentRegRows<TagS, TagT, NT, NUS> rows;
+  rows.load(reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes,
+            reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * TagT::bytes, p.V / 8, student_half);
+  const DenseStats st = dense_stats<KIND, NT>(rows, p.inv_T_s, p.inv_T_t, red);
+  if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
+  if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
+}
+
 // Any size, any alignment, any dtype pair: four scalar passes over global memory.
 template <int NT>
 __global__ __launch_bounds__(NT) void dense_stream_kernel(const DenseParams p) {
@@ -181,10 +274,25 @@ __global__ __launch_bounds__(NT) void dense_stream_kernel(const DenseParams p) {
 template <int KIND, class TagS, class TagT, int NU>
 static bool launch_dense_kind(const DenseParams& p, hipStream_t st) {
   const int64_t units = p.V / 8;
+  constexpr int NUS = 256 / (16 * Unit<TagS>::NC);      // the student row alone: 256 bytes of registers per thread
   const dim3 grid(xcd_banded_grid(p.n_rows));
   if (units <= 256 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 256, NU>), grid, dim3(256), 0, st, p);
   else if (units <= 512 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 512, NU>), grid, dim3(512), 0, st, p);
   else if (units <= 1024 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, TagS, TagT, 1024, NU>), grid, dim3(1024), 0, st, p);
+  else if (units <= 1024 * NUS) {
+    // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device (the call is slow)
+    constexpr size_t lds = StudentRegRows<TagS, TagT, 1024, NUS>::LDS_BYTES;
+    static thread_local int allowed_on = -1;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (allowed_on != dev) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_student_reg_kernel<KIND, TagS, TagT, 1024, NUS>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return false;
+      allowed_on = dev;
+    }
+    hipLaunchKernelGGL((dense_student_reg_kernel<KIND, TagS, TagT, 1024, NUS>), grid, dim3(1024), lds, st, p);
+  }
   else hipLaunchKernelGGL((dense_stream_vec_kernel<KIND, TagS, TagT, 1024>), grid, dim3(1024), 0, st, p);
   return true;
 }

@@ -91,12 +91,21 @@ def test_teacher_with_zero_mass_entries(D, kind):
 
 
 @pytest.mark.parametrize("V,dtype", [(1001, torch.float32), (70000, torch.bfloat16), (50264, torch.float32),
-                                     (128256, torch.bfloat16)])
-def test_dense_streaming_fallback(D, V, dtype):
-    # rows beyond the register budget take the multi-pass kernel with 16-byte loads, odd vocabularies the scalar one
+                                     (128256, torch.bfloat16), (151936, torch.bfloat16), (70000, torch.float32)])
+def test_dense_rows_beyond_the_register_budget(D, V, dtype):
+    # up to 131072 16-bit / 65536 fp32 columns the student row stays on the CU and the teacher row is
+    # streamed; beyond, both are streamed (multi-pass, 16-byte loads); odd vocabularies take the scalar kernel
     s, t = _pair(5, V, dtype, 5)
     for kind in ("fkl", "rkl", "jsd"):
         _check(D, kind, s, t, T=1.3)
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+def test_dense_wide_16bit_student_fp32_teacher_with_masked_rows(D, kind):
+    s, t = _pair(9, 100000, torch.bfloat16, 6, torch.float32)
+    valid = torch.ones(9, dtype=torch.bool)
+    valid[[2, 7]] = False
+    _check(D, kind, s, t[valid], T=1.7, valid=valid, teacher_T=1.0)
 
 
 def test_dense_identical_distributions_give_zero(D):
@@ -126,7 +135,7 @@ def test_synthetic_configs_1_and_2_at_reduced_rows(D):
 
 
 @pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
-@pytest.mark.parametrize("V,dtype", [(32000, torch.bfloat16), (1001, torch.float32)])
+@pytest.mark.parametrize("V,dtype", [(32000, torch.bfloat16), (1001, torch.float32), (128256, torch.bfloat16)])
 def test_dense_gradient_may_overwrite_the_logits(D, kind, V, dtype):
     g = torch.Generator().manual_seed(17)
     x = (torch.randn(12, V, generator=g) * 2).to(dtype).to(DEV)
