@@ -10,12 +10,14 @@
 //   * CSR form (deterministic): one thread per student id adds its segment in ascending
 //     teacher-id order.
 //   * planned form (fast and deterministic): the host lays the map out as a "plan": the teacher
-//     vocabulary is cut into tiles of `tile` ids; student id s belongs to thread s % 1024; for every
-//     (tile, wave) the entries (s, local teacher id) of the wave's 64 threads are stored row-wise
-//     (64 entries per row, padded), each thread's entries sorted by (s, t).  The kernel streams a
-//     teacher tile into LDS (coalesced), then every thread walks its entries, reads the tile at
-//     random (LDS), and adds runs of equal s into marg[s] -- a location only that thread ever
-//     touches, so no atomics, and the order of additions is fixed: bit-reproducible.
+//     vocabulary is cut into tiles; inside a tile every accumulator slot (a student id, or one of
+//     the replicas of a student id that many teacher ids map to) belongs to one thread, and for
+//     every (tile, wave) the entries of the wave's 64 threads are stored row-wise (64 entries per
+//     row, padded to batches of 8 rows), each thread's entries sorted by (slot, t).  The kernel
+//     streams a teacher tile into LDS (coalesced), then every thread walks its entries, reads the
+//     tile at random (LDS), and adds runs of equal slot into LDS words only it touches in that
+//     tile, so no atomics, and the order of additions is fixed: bit-reproducible.  Replicas are
+//     folded into their id's slot after the last tile.
 //   * fused reverse KL: the marginal never leaves LDS; its logarithm is the teacher row of the
 //     dense-divergence sweeps, the student row sits in registers.
 #include "dense_div.hpp"
