@@ -78,6 +78,31 @@ def test_planned_marginal_with_lists_longer_than_one_batch(D):
     assert np.array_equal(m_plan, D.vocab_utils.marginalise(probs.to(DEV), plan=plan, n_student=Vs).cpu().numpy())
 
 
+@pytest.mark.parametrize("case", ["one_hot_id", "all_dropped", "short", "tiny_student", "zipf"])
+def test_planned_marginal_on_degenerate_maps(D, case):
+    rng = np.random.default_rng(3)
+    Vs, Vt, R = 3000, 20000, 4
+    if case == "one_hot_id":
+        t2s = np.where(rng.random(Vt) < 0.95, 17, rng.integers(0, Vs, Vt))
+    elif case == "all_dropped":
+        t2s = np.full(Vt, -1)
+    elif case == "short":
+        Vt = 1000
+        t2s = rng.integers(0, Vs, Vt)
+    elif case == "tiny_student":
+        Vs = 4
+        t2s = rng.integers(0, Vs, Vt)
+    else:
+        t2s = np.minimum(rng.zipf(1.2, Vt) - 1, Vs - 1)
+    t2s = t2s.astype(np.int32)
+    probs = torch.softmax(torch.randn(R, Vt, generator=torch.Generator().manual_seed(5)) * 2, -1)
+    plan = D.vocab_utils.MarginalPlan(t2s, Vs, DEV)
+    ref = O.marginalise_map(probs.numpy(), t2s, Vs)
+    m_plan = D.vocab_utils.marginalise(probs.to(DEV), plan=plan, n_student=Vs).cpu().numpy()
+    np.testing.assert_allclose(m_plan, ref, rtol=2e-5, atol=1e-9)
+    assert np.array_equal(m_plan == 0, ref == 0)
+
+
 def test_marginal_of_16bit_probabilities(D):
     t2s, probs = _case(4, 512, 2048, 2)
     got = D.vocab_utils.marginalise(probs.to(torch.bfloat16).to(DEV), t2s=torch.tensor(t2s, device=DEV), n_student=512)

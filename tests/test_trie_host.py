@@ -113,3 +113,69 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     # too wide a student vocabulary: no plan, the atomic form remains
     wide = D.vocab_utils.MarginalPlan(np.zeros(100, dtype=np.int32), 40000, "cpu")
     assert wide.ent is None and wide.tile == 0
+
+
+def _apply_plan(plan, probs, Vs):
+    """What the planned kernels compute, entry by entry in numpy: per tile and thread the running sum
+    restarts on bit 31, every entry stores slot + running sum into the slot its bits 15-30 name (spare
+    slots on unfinished runs), replicas are folded into their id after the last tile."""
+    tile = plan.tile
+    row_off = plan.row_off.numpy()
+    ent = plan.ent.numpy().view(np.uint32).astype(np.int64)
+    n_pad = (Vs + 3) & ~3
+    slots = np.zeros(n_pad + ((plan.n_extra + 3) & ~3) + 64, dtype=np.float32)
+    ntiles = -(-probs.size // tile)
+    for k in range(ntiles):
+        seg = np.zeros(tile, dtype=np.float32)
+        part = probs[k * tile:(k + 1) * tile]
+        seg[:part.size] = part
+        touched = {}
+        for w in range(16):
+            rows = ent[row_off[16 * k + w]:row_off[16 * k + w + 1]]
+            assert rows.shape[0] % 8 == 0 and rows.shape[0] >= 8
+            for lane in range(64):
+                run = np.float32(0)
+                for e in rows[:, lane]:
+                    slot, offset = (e >> 15) & 0xffff, (e & 0x7fff) >> 2
+                    assert slot < slots.size and offset < tile
+                    run = np.float32((0 if e >> 31 else run) + seg[offset])
+                    if slot < n_pad + plan.n_extra:      # a real slot: only this thread may touch it in this tile
+                        assert touched.setdefault(int(slot), (w, lane)) == (w, lane)
+                        slots[slot] = slots[slot] + run   # one store per run: slot value read before the batch == before the run
+                    # spare slots: value never used
+    for sid, first, cnt in plan.fold.numpy()[:plan.n_fold]:
+        for j in range(cnt):
+            slots[sid] = slots[sid] + slots[first + j]
+    return slots[:Vs]
+
+
+@pytest.mark.parametrize("case", ["uniform", "one_hot_id", "all_dropped", "short", "tiny_student", "wide_student", "zipf"])
+def test_marginal_plan_applied_in_numpy_equals_the_marginal(case):
+    rng = np.random.default_rng(3)
+    Vs, Vt = 3000, 20000
+    if case == "uniform":
+        t2s = rng.integers(-1, Vs, Vt)
+    elif case == "one_hot_id":
+        t2s = np.where(rng.random(Vt) < 0.95, 17, rng.integers(0, Vs, Vt))
+    elif case == "all_dropped":
+        t2s = np.full(Vt, -1)
+    elif case == "short":
+        Vt = 1000
+        t2s = rng.integers(0, Vs, Vt)
+    elif case == "tiny_student":
+        Vs = 4
+        t2s = rng.integers(0, Vs, Vt)
+    elif case == "wide_student":
+        Vs, Vt = 36500, 9000
+        t2s = np.where(rng.random(Vt) < 0.8, rng.integers(0, 6, Vt) * 5000, rng.integers(0, Vs, Vt))
+    else:
+        t2s = np.minimum(rng.zipf(1.2, Vt) - 1, Vs - 1)
+    t2s = t2s.astype(np.int32)
+    plan = D.vocab_utils.MarginalPlan(t2s, Vs, "cpu")
+    assert plan.ent is not None
+    probs = rng.random(Vt).astype(np.float32)
+    got = _apply_plan(plan, probs, Vs)
+    want = np.zeros(Vs, dtype=np.float64)
+    np.add.at(want, t2s[t2s >= 0], probs[t2s >= 0].astype(np.float64))
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-6)
+    assert np.array_equal(got == 0, want == 0)
