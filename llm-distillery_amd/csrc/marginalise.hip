@@ -26,6 +26,8 @@ namespace dl {
 
 constexpr int MARG_NT = 1024;
 constexpr int MARG_MAX_VS = 36864;          // fp32 marginal of one row in LDS: 144 KiB of the CU's 160
+constexpr int MARG_NU = 5;                  // units of 8 student columns per thread in the fused kernel
+static_assert(MARG_MAX_VS / 8 <= MARG_NU * MARG_NT, "the student row must fit the registers of the fused kernel");
 constexpr int MARG_MAX_DYN_LDS = 160 * 1024 - 1024;   // dynamic LDS a workgroup may request (planned form: marginal + tile)
 
 struct MargParams {
@@ -324,11 +326,8 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
   float* marg = acc;
   if (VEC && p.plan_ent) {
     marg = acc + p.plan_tile;                    // the tile sits first: its addresses are then plain offsets
-    // a 16-bit student row is in flight during the accumulation; an fp32 one would take the registers
-    // the accumulation needs (it spills) and is loaded afterwards
-    if (TagS::bytes == 2) rows.load(srow, p.Vs / 8);
+    rows.load(srow, p.Vs / 8);                   // in flight during the accumulation
     accumulate_marginal_planned(p, prow, marg, acc);
-    if (TagS::bytes != 2) rows.load(srow, p.Vs / 8);
   } else {
     rows.load(srow, p.Vs / 8);                   // in flight during the scatter
     accumulate_marginal<VEC>(p, prow, acc, 0, (int)p.Vs);
@@ -363,12 +362,12 @@ static void allow_large_lds() {
   if (done_for == dev) return;
   allow_large_lds_for(&marginalise_map_kernel<true>);
   allow_large_lds_for(&marginalise_map_kernel<false>);
-  allow_large_lds_for(&rkl_marginalised_kernel<TagF32, 8, true>);
-  allow_large_lds_for(&rkl_marginalised_kernel<TagF32, 8, false>);
-  allow_large_lds_for(&rkl_marginalised_kernel<TagBF16, 8, true>);
-  allow_large_lds_for(&rkl_marginalised_kernel<TagBF16, 8, false>);
-  allow_large_lds_for(&rkl_marginalised_kernel<TagF16, 8, true>);
-  allow_large_lds_for(&rkl_marginalised_kernel<TagF16, 8, false>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF32, MARG_NU, true>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF32, MARG_NU, false>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagBF16, MARG_NU, true>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagBF16, MARG_NU, false>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF16, MARG_NU, true>);
+  allow_large_lds_for(&rkl_marginalised_kernel<TagF16, MARG_NU, false>);
   done_for = dev;
 }
 
@@ -459,8 +458,8 @@ extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t
   allow_large_lds();
 #define DL_LAUNCH_RKLM(TAG)                                                                                  \
   do {                                                                                                       \
-    if (vec) hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, 8, true>), grid, block, lds, st, p);           \
-    else hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, 8, false>), grid, block, lds, st, p);              \
+    if (vec) hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, MARG_NU, true>), grid, block, lds, st, p);           \
+    else hipLaunchKernelGGL((rkl_marginalised_kernel<TAG, MARG_NU, false>), grid, block, lds, st, p);              \
   } while (0)
   if (logits_dtype == DL_F32) DL_LAUNCH_RKLM(TagF32);
   else if (logits_dtype == DL_BF16) DL_LAUNCH_RKLM(TagBF16);
