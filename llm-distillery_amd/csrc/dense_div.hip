@@ -15,6 +15,7 @@ struct DenseParams {
 // Both rows in registers: NU units of 8 columns per thread.
 template <class TagS, class TagT, int NT, int NU>
 struct RegRows {
+  static constexpr bool ONLINE = false;      // sweeps cost no memory traffic: maxima first, then sums
   Unit<TagS> s[NU];
   Unit<TagT> t[NU];
   int64_t nunits;
@@ -64,10 +65,11 @@ __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
 }
 
 // Rows too wide for the registers, 16-byte aligned: the same sweeps, every one of them over global
-// memory with 16-byte loads, two units per thread in flight (3-4 reads of both rows; all but the first
+// memory with 16-byte loads, two units per thread in flight (2-3 reads of both rows; all but the first
 // come from L2 / the memory-side cache as far as the rows of the workgroups in flight fit there).
 template <class TagS, class TagT, int NT>
 struct StreamRows {
+  static constexpr bool ONLINE = true;       // every sweep reads both rows: maxima and sums share one
   const char* srow;
   const char* trow;
   int64_t nunits;
@@ -125,10 +127,11 @@ __global__ __launch_bounds__(NT) void dense_stream_vec_kernel(const DenseParams 
 // read from HBM once and kept on the CU, half of it in registers (NUS / 2 units per thread) and half
 // in LDS (128 KiB; all of it in registers leaves too few for the sweeps: the compiler spills).  The
 // teacher row is streamed through a ring of D units per thread in every sweep (its later reads come
-// from L2 as far as the rows in flight fit there).  Against streaming both rows this saves two or
-// three reads of the student row.
+// from L2 as far as the rows in flight fit there).  Against streaming both rows this saves one or
+// two reads of the student row.
 template <class TagS, class TagT, int NT, int NUS>
 struct StudentRegRows {
+  static constexpr bool ONLINE = true;       // every sweep reads the teacher row: maxima and sums share one
   static constexpr int D = Unit<TagT>::NC == 1 ? 4 : 2;      // teacher units in flight per thread
   static constexpr int NR = NUS / 2;                         // student units in registers; the rest in LDS
   static constexpr int NC = Unit<TagS>::NC;

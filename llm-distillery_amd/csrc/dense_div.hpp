@@ -2,8 +2,9 @@
 // loss and gradient in one launch.
 //
 // One workgroup per token row.  Student and teacher rows are pulled into registers with 16-byte
-// non-temporal loads (each read from HBM once) and swept four times from there: maxima, sums of
-// exponentials, divergence sums, gradient.  All arithmetic runs in the log2 domain
+// non-temporal loads (each read from HBM once) and swept from there: maxima, sums of exponentials
+// (with the divergence sum of forward / reverse KL riding along; JSD takes a sweep of its own),
+// gradient.  Rows too wide for the registers are swept from memory, maxima and sums in one sweep.  All arithmetic runs in the log2 domain
 // (lp = x * inv_T * log2(e) - log2-sum-exp2), natural logs appear only in the results.
 //
 // The same sweeps serve the byte-trie path, where the teacher row is not read from memory but is
@@ -89,35 +90,80 @@ __device__ __forceinline__ DenseStats dense_stats(Rows& rows, float inv_T_s, flo
   st.a_s = inv_T_s * LOG2E;
   st.a_t = inv_T_t * LOG2E;
   const float a_s = st.a_s, a_t = st.a_t;
-  // maxima (for RKL the student maximum is taken over the teacher's support)
-  float ms = -INFINITY, mt = -INFINITY;
-  rows.sweep([&](int64_t, const float* s, const float* t) {
+  float ms = -INFINITY, mt = -INFINITY;     // maxima (for RKL the student maximum is taken over the teacher's support)
+  float ss = 0.f, stt = 0.f, w = 0.f;
+  if constexpr (Rows::ONLINE) {
+    // Rows that are read from memory in every sweep: maxima and sums in ONE sweep.  Each thread keeps
+    // running maxima; when a unit raises one, what has been summed so far is carried over to the new
+    // bias: with shifts ds, dt >= 0 of the two biases (log2 domain), es scales by 2^-ds, et by 2^-dt,
+    // and the divergence terms et (xt - xs) / es (xs - xt) follow from xs -= ds, xt -= dt.  A maximum
+    // of -inf means that nothing has been summed on that side yet (bias 0 keeps 2^(-inf - bias) = 0).
+    const auto carry = [&](float nms, float nmt) {
+      const float ds = ms == -INFINITY ? 0.f : (nms - ms) * a_s, dt = mt == -INFINITY ? 0.f : (nmt - mt) * a_t;
+      const float fs = fast_exp2(-ds), ft = fast_exp2(-dt);
+      if (KIND == DL_FKL) w = ft * (w - (dt - ds) * stt);
+      if (KIND == DL_RKL) w = fs * (w - (ds - dt) * ss);
+      ss *= fs;
+      stt *= ft;
+      ms = nms;
+      mt = nmt;
+    };
+    rows.sweep([&](int64_t, const float* s, const float* t) {
+      float ums = -INFINITY, umt = -INFINITY;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      mt = fmaxf(mt, t[e]);
-      ms = fmaxf(ms, (KIND == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
-    }
-  });
-  block_max2<NT>(ms, mt, red);
+      for (int e = 0; e < 8; ++e) {
+        umt = fmaxf(umt, t[e]);
+        ums = fmaxf(ums, (KIND == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
+      }
+      if (ums > ms || umt > mt) carry(fmaxf(ms, ums), fmaxf(mt, umt));
+      const float bs = ms == -INFINITY ? 0.f : ms * a_s, bt = mt == -INFINITY ? 0.f : mt * a_t;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xs = fmaf(s[e], a_s, -bs), xt = fmaf(t[e], a_t, -bt);
+        const float es = fast_exp2(xs), et = fast_exp2(xt);
+        stt += et;
+        if (KIND == DL_RKL) {
+          const bool on = t[e] != -INFINITY;
+          ss += on ? es : 0.f;
+          w += (on && es > 0.f) ? es * (xs - xt) : 0.f;
+        } else {
+          ss += es;
+          if (KIND == DL_FKL) w += et > 0.f ? et * (xt - xs) : 0.f;
+        }
+      }
+    });
+    float gs = ms, gt = mt;
+    block_max2<NT>(gs, gt, red);
+    carry(gs, gt);                          // this thread's sums on the row's biases
+  } else {
+    rows.sweep([&](int64_t, const float* s, const float* t) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        mt = fmaxf(mt, t[e]);
+        ms = fmaxf(ms, (KIND == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
+      }
+    });
+    block_max2<NT>(ms, mt, red);
+    const float bs = ms * a_s, bt = mt * a_t;
+    rows.sweep([&](int64_t, const float* s, const float* t) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xs = fmaf(s[e], a_s, -bs), xt = fmaf(t[e], a_t, -bt);
+        const float es = fast_exp2(xs), et = fast_exp2(xt);
+        stt += et;
+        if (KIND == DL_RKL) {
+          const bool on = t[e] != -INFINITY;
+          ss += on ? es : 0.f;
+          w += (on && es > 0.f) ? es * (xs - xt) : 0.f;
+        } else {
+          ss += es;
+          if (KIND == DL_FKL) w += et > 0.f ? et * (xt - xs) : 0.f;
+        }
+      }
+    });
+  }
   st.tmax = mt;
   const float bs = ms * a_s, bt = mt * a_t;
-  float ss = 0.f, stt = 0.f, w = 0.f;
-  rows.sweep([&](int64_t, const float* s, const float* t) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float xs = fmaf(s[e], a_s, -bs), xt = fmaf(t[e], a_t, -bt);
-      const float es = fast_exp2(xs), et = fast_exp2(xt);
-      stt += et;
-      if (KIND == DL_RKL) {
-        const bool on = t[e] != -INFINITY;
-        ss += on ? es : 0.f;
-        w += (on && es > 0.f) ? es * (xs - xt) : 0.f;
-      } else {
-        ss += es;
-        if (KIND == DL_FKL) w += et > 0.f ? et * (xt - xs) : 0.f;
-      }
-    }
-  });
   block_sum2<NT>(ss, stt, red);
   const float l2s = fast_log2(ss), l2t = fast_log2(stt);
   st.ls = bs + l2s;

@@ -277,6 +277,7 @@ __global__ __launch_bounds__(256) void marginalise_csr_kernel(const void* probs,
 // ---- fused: marginal in LDS -> reverse KL against the student row in registers -----------------
 template <class TagS, int NU>
 struct LdsTeacherRows {
+  static constexpr bool ONLINE = false;
   Unit<TagS> s[NU];
   const float* lt;      // log marginal, LDS
   int64_t nunits;

@@ -101,6 +101,23 @@ def test_dense_rows_beyond_the_register_budget(D, V, dtype):
 
 
 @pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+@pytest.mark.parametrize("V", [70000, 151936])
+def test_wide_rows_with_zero_mass_teacher_entries(D, kind, V):
+    # rows swept from memory take maxima and sums in one sweep with running maxima: stretches without any
+    # teacher mass (the first 20000 columns, and 60 % of the rest) must neither poison nor bias the sums,
+    # and the largest entries sit late in the row so that the running maxima do move
+    s, t = _pair(6, V, torch.bfloat16, 8)
+    g = torch.Generator().manual_seed(8)
+    drop = torch.rand(6, V, generator=g) < 0.6
+    drop[:, :20000] = True
+    t = t.float().masked_fill(drop, float("-inf"))
+    t[:, V - 5000:] += 6.0
+    s = s.float()
+    s[:, V // 2:] += 4.0
+    _check(D, kind, s.to(torch.bfloat16), t.to(torch.bfloat16), T=1.0)
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
 def test_dense_wide_16bit_student_fp32_teacher_with_masked_rows(D, kind):
     s, t = _pair(9, 100000, torch.bfloat16, 6, torch.float32)
     valid = torch.ones(9, dtype=torch.bool)
