@@ -94,6 +94,15 @@ class MarginalPlan:
         self.ent = torch.as_tensor(ent.view(np.int32), device=device)     # same bits; torch has no uint32 arithmetic need
         self.fold = torch.as_tensor(fold, device=device)
 
+    def check(self, n_student: int, n_teacher: int, device) -> None:
+        """Raises unless the plan was built for these vocabulary sizes and lives on `device`: the
+        kernels index LDS by what the plan says and cannot check it themselves."""
+        if self.n_student != int(n_student) or self.n_teacher != int(n_teacher):
+            raise RuntimeError(f"the plan maps {self.n_teacher} teacher ids onto {self.n_student} student ids, "
+                               f"the call has {int(n_teacher)} and {int(n_student)}")
+        if self.t2s.device != torch.device(device):
+            raise RuntimeError(f"the plan lives on {self.t2s.device}, the call runs on {device}")
+
     def _args(self):
         """(row_off, ent, tile, fold, n_fold, n_extra) as the C ABI takes them."""
         if self.ent is None:
@@ -129,6 +138,7 @@ def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=Non
         else:
             plan_args = (0, 0, 0, 0, 0, 0)
             if plan is not None:
+                plan.check(n_student, Vt, x.device)
                 t2s = plan.t2s
                 plan_args = plan._args()
             _, _ = _opt_i32(t2s, Vt, "t2s", x.device)
@@ -146,14 +156,15 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
     in one launch; the marginal stays in LDS.  `t2s` is the int32 [Vt] map on the GPU or, better, a
     MarginalPlan built from it.  Returns (row_loss fp32 [rows], grad or None)."""
     _dev(logits, "logits"), _dev(teacher_probs, "teacher_probs")
-    plan_args = (0, 0, 0, 0, 0, 0)
-    if isinstance(t2s, MarginalPlan):
-        plan_args = t2s._args()
-        t2s = t2s.t2s
     x, tp = _rows_2d(logits), _rows_2d(teacher_probs)
     R, Vs = x.shape
     N, Vt = tp.shape
     dev = x.device
+    plan_args = (0, 0, 0, 0, 0, 0)
+    if isinstance(t2s, MarginalPlan):
+        t2s.check(Vs, Vt, dev)
+        plan_args = t2s._args()
+        t2s = t2s.t2s
     if x.dtype not in _DT or tp.dtype not in _DT:
         raise RuntimeError("unsupported dtype")
     if row_map is None and N < R:

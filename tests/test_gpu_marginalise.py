@@ -103,6 +103,18 @@ def test_planned_marginal_on_degenerate_maps(D, case):
     assert np.array_equal(m_plan == 0, ref == 0)
 
 
+def test_a_plan_built_for_other_vocabularies_is_refused(D):
+    t2s = np.random.default_rng(0).integers(0, 1000, 5000).astype(np.int32)
+    plan = D.vocab_utils.MarginalPlan(t2s, 1000, DEV)
+    probs = torch.rand(2, 5000, device=DEV)
+    with pytest.raises(RuntimeError, match="the plan maps"):
+        D.vocab_utils.marginalise(probs, plan=plan, n_student=1008)
+    with pytest.raises(RuntimeError, match="the plan maps"):
+        D.vocab_utils.marginalise(torch.rand(2, 6000, device=DEV), plan=plan, n_student=1000)
+    with pytest.raises(RuntimeError, match="the plan maps"):
+        D.vocab_utils.rkl_marginalised(torch.randn(2, 1008, device=DEV), probs, plan)
+
+
 def test_marginal_of_16bit_probabilities(D):
     t2s, probs = _case(4, 512, 2048, 2)
     got = D.vocab_utils.marginalise(probs.to(torch.bfloat16).to(DEV), t2s=torch.tensor(t2s, device=DEV), n_student=512)
