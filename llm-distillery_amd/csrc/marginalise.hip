@@ -52,7 +52,6 @@ __host__ __device__ inline int64_t plan_slot_words(int64_t Vs, int n_extra) {
 // Plan entry: bit 31 = first entry of a run of one slot in its thread's list of the tile; bits
 // 15-30 = the slot on the last entry of the run, the lane's spare slot on the others; bits 0-14 =
 // byte offset of the probability inside the tile.  Padding is a first entry on the spare slot.
-constexpr unsigned PLAN_FIRST = 0x80000000u;
 constexpr int PLAN_SLOT_SHIFT = 15;
 constexpr unsigned PLAN_OFFSET_MASK = 0x7ffcu, PLAN_SLOT_MASK = 0xffffu;
 
@@ -76,7 +75,7 @@ __device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const
   for (int j = 0; j < PLAN_EB; ++j) base[j] = marg[(e[j] >> PLAN_SLOT_SHIFT) & PLAN_SLOT_MASK];
 #pragma unroll
   for (int j = 0; j < PLAN_EB; ++j) {
-    run = ((int)e[j] < 0 ? 0.f : run) + val[j];
+    run = ((int)e[j] < 0 ? 0.f : run) + val[j];          // bit 31: the run starts here
     marg[(e[j] >> PLAN_SLOT_SHIFT) & PLAN_SLOT_MASK] = base[j] + run;
   }
 }
