@@ -219,8 +219,8 @@ __device__ __forceinline__ float stage_teacher(const TopkParams& p, const TopkLd
 // Partial forward-KL sums over the ids inside [lo, hi):  B = sum q_k (t_k - z_k * inv_T)  and, over
 // all ids, Q = sum q_k.  The row value is  sum over parts of B  +  lse * Q.
 template <int NT>
-__device__ __forceinline__ void fkl_partials(const TopkParams& p, const TopkLds& s, float tlse, int lo,
-                                             int hi, float& B, float& Q) {
+__device__ __forceinline__ void fkl_partials(const TopkParams& p, const TopkLds& s, int lo, int hi, float& B,
+                                             float& Q) {
   B = 0.f; Q = 0.f;
   for (int k = threadIdx.x; k < s.Kp; k += NT) {
     const int id = s.idx[k];
@@ -364,7 +364,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
     return;
   }
   float B, Q;
-  fkl_partials<NT>(p, s, tlse, lo, hi, B, Q);
+  fkl_partials<NT>(p, s, lo, hi, B, Q);
 
   const float a = p.inv_T_s * LOG2E;
   float mx = -INFINITY;
@@ -528,7 +528,7 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
     return;
   }
   float B, Q;
-  fkl_partials<NT>(p, s, tlse, 0, (int)V, B, Q);
+  fkl_partials<NT>(p, s, 0, (int)V, B, Q);
   const float a = p.inv_T_s * LOG2E;
   float mx, sm;
   row_stats_streamed<Tag, NT, VEC>(row, V, a, s.red, mx, sm);
