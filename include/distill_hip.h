@@ -40,21 +40,19 @@ typedef enum {
 
 #define DL_MAX_TOPK 2048      /* entries per row a sparse teacher may hold        */
 #define DL_MAX_TEACHERS 8     /* teachers merged in one launch                    */
-#define DL_TOPK_UNIQUE_IDS 1   /* dl_div_topk flag: no id occurs twice in a row    */
+/* dl_div_topk flags (OR them together) */
+#define DL_TOPK_UNIQUE_IDS 1   /* no id occurs twice in a row                                          */
+#define DL_TOPK_NO_WAIT 2      /* parts of a split row never wait for their partners: every part that  */
+                               /* finds a record missing is finished by the second launch (exercises   */
+                               /* that path; same results, slower)                                      */
+#define DL_TOPK_PARTS_SHIFT 8  /* bits 8-11: column parts a row of 65537-131072 two-byte (half as many */
+#define DL_TOPK_PARTS(n) ((n) << DL_TOPK_PARTS_SHIFT)   /* four-byte) entries is cut into: 1, 2 or 4;   */
+                               /* 0 = automatic                                                         */
 
 /* Library ABI revision; bumped when a signature changes. */
 int dl_abi_version(void);
 /* Static, NUL-terminated description of a dl_status. */
 const char* dl_status_string(int status);
-
-/*
- * Process-wide tuning / test hooks (no reference counterpart).  Names:
- *   "split_parts"  0 = automatic (default), 1 / 2 / 4 = column parts a wide row is cut into;
- *   "spin_limit"   polls a part of a split row waits for its partners before it recomputes the
- *                  row statistics alone (default 20000; 0 = never wait, exercises that path).
- * Returns DL_ERR_DTYPE for an unknown name, DL_ERR_SHAPE for a value out of range.
- */
-int dl_set_option(const char* name, int value);
 
 /*
  * Forward or reverse KL against a sparse (top-K) teacher, loss and gradient in one sweep.
@@ -84,6 +82,8 @@ int dl_set_option(const char* name, int value);
  *            torch.topk and of dl_merge_remap_topk); the kernel then skips its check for repeated ids
  *            (a few instructions per entry in the register kernels, a scan in the streaming one).  With
  *            the flag set and duplicates present, the gradient at a duplicated id is wrong.
+ *            DL_TOPK_NO_WAIT and DL_TOPK_PARTS(n) are tuning / test hooks of the split-row kernels; they
+ *            change neither results nor requirements.  The library keeps no state between calls.
  * K <= DL_MAX_TOPK.
  * grad may be the logits buffer itself (same pointer and stride): every kernel holds, or has
  * consumed, what it still needs of a row before it writes there.  The same holds for dl_div_dense
@@ -191,10 +191,12 @@ int dl_composite_backward(const float* lse, const float* zk, const void* t_val, 
  *   classes/teacher/result_processor_worker.py:27-35  (content-row selection, via row_list)
  *   classes/data_manager.py:306,312  (cast to the storage dtypes: out_dtype DL_F16, out_itype DL_I32)
  * No temperature is applied at collection time.  row_list (int32 [n_out], may be NULL = rows
- * 0..n_out-1) names the logits row behind each output row.  Entries with equal log-prob are ordered
- * by ascending id (the reference leaves tie order to torch.topk).
- * K <= 1024, K <= V; V a multiple of 8 (4 for fp32), rows 16-byte aligned; V <= 262144 (131072 fp32);
- * K * parts <= 4096 with parts = ceil(V / 32768) (fp32: ceil(V / 16384)).
+ * 0..n_out-1) names the logits row behind each output row; an entry outside [0, n_rows) gives a
+ * masked output row (log-probs -inf, ids -1) and touches no logits.  Entries with equal log-prob are
+ * ordered by ascending id (the reference leaves tie order to torch.topk).
+ * K <= 1024, K <= V; V <= 262144 (131072 fp32); K * parts <= 4096 with parts = ceil(V / 32768)
+ * (fp32: ceil(V / 16384)).  Any V and any element-aligned row pitch are taken, as by the reference;
+ * V a multiple of 8 (4 for fp32) with 16-byte aligned rows selects the 16-byte loads.
  * workspace: device memory, 16-byte aligned, at least dl_teacher_topk_workspace_bytes(...) bytes
  * (per output row and 32768-column part: the part's best K candidates and its softmax statistics);
  * contents need no initialisation and mean nothing afterwards.  Two launches that may overlap in

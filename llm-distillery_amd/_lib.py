@@ -19,6 +19,8 @@ DL_FKL, DL_RKL, DL_JSD = 0, 1, 2
 DL_MAX_TOPK = 2048
 DL_MAX_TEACHERS = 8
 DL_TOPK_UNIQUE_IDS = 1
+DL_TOPK_NO_WAIT = 2
+DL_TOPK_PARTS_SHIFT = 8
 
 _P = c_void_p
 _SIGNATURES = {
@@ -50,7 +52,6 @@ _SIGNATURES = {
                                       _P]),
     "dl_teacher_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, c_int, _P, c_int, _P, c_int, _P, c_int64, _P]),
     "dl_teacher_topk_workspace_bytes": (c_int64, [c_int, c_int64, c_int64, c_int]),
-    "dl_set_option": (c_int, [c_char_p, c_int]),
     "dl_reduce_sum": (c_int, [_P, c_int64, c_float, _P, _P]),
     "dl_copy16": (c_int, [_P, _P, c_int64, _P]),
 }

@@ -21,8 +21,6 @@
 #include "distill_common.hpp"
 #include "distill_hip.h"
 #include <algorithm>
-#include <atomic>
-#include <cstring>
 
 namespace dl {
 
@@ -687,15 +685,12 @@ static hipError_t launch_split(TopkParams p, int parts, hipStream_t st) {
   return hipGetLastError();
 }
 
-// Library options (dl_set_option): tuning and test hooks, process-wide.
-static std::atomic<int> g_split_parts{0};       // 0 = automatic, else 1 / 2 / 4
-static std::atomic<int> g_spin_limit{20000};    // polls a part waits for a partner; 0 = never wait
-
 // Number of column parts a row of `nch` 16-byte chunks is cut into (1 = one workgroup per row).
-static int split_parts(int64_t nch) {
+// `forced` (the DL_TOPK_PARTS field of the call's flags): 1 / 2 / 4 override the choice for rows that
+// fit one workgroup of 1024 threads; anything else = automatic.
+static int split_parts(int64_t nch, int forced) {
   if (nch <= 512 * 16) return 1;
   if (nch > 1024 * 16) return (int)((nch + 256 * 16 - 1) / (256 * 16));      // 5 .. MAX_PARTS parts of 256 x 16 chunks
-  const int forced = g_split_parts.load();
   if (forced == 1 || forced == 2 || forced == 4) return forced;
   return 4;
 }
@@ -709,7 +704,7 @@ static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes
     // 4-byte logits: 8 chunks per thread from twice the threads keep the corrections in registers
     if (nch <= 256 * 16) return Tag::bytes == 4 ? launch_reg<Tag, 512, 8>(p, st) : launch_reg<Tag, 256, 16>(p, st);
     if (nch <= 512 * 16) return launch_reg<Tag, 512, 16>(p, st);
-    const int parts = split_parts(nch);
+    const int parts = split_parts(nch, (p.flags >> DL_TOPK_PARTS_SHIFT) & 15);
     const bool ws_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, parts) && p.n_rows * parts <= 0x7fffffffLL;
     if (parts == 2 && ws_ok) return launch_split<Tag, 512, 16>(p, 2, st);
     if (parts >= 4 && ws_ok) return launch_split<Tag, 256, 16>(p, parts, st);
@@ -736,24 +731,10 @@ static hipError_t launch_rkl(const TopkParams& p, bool aligned, hipStream_t st) 
   return hipGetLastError();
 }
 
-static int spin_limit() { return g_spin_limit.load(); }
+// Polls a part of a split row waits for its partners' records before it defers itself to the second launch.
+constexpr int SPIN_LIMIT = 20000;
 
 }  // namespace dl
-
-extern "C" int dl_set_option(const char* name, int value) {
-  if (!name) return DL_ERR_NULL;
-  if (!strcmp(name, "split_parts")) {
-    if (value != 0 && value != 1 && value != 2 && value != 4) return DL_ERR_SHAPE;
-    dl::g_split_parts.store(value);
-    return DL_OK;
-  }
-  if (!strcmp(name, "spin_limit")) {
-    if (value < 0) return DL_ERR_SHAPE;
-    dl::g_spin_limit.store(value);
-    return DL_OK;
-  }
-  return DL_ERR_DTYPE;
-}
 
 extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V) {
   if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
@@ -784,7 +765,8 @@ extern "C" int dl_div_topk(int kind, const void* logits, int logits_dtype, int64
                        (!grad || (reinterpret_cast<uintptr_t>(grad) % 16 == 0 && (grad_stride * eb) % 16 == 0));
   TopkParams p{logits, row_stride, n_rows, V, row_map, t_val, t_val_dtype, t_idx, t_idx_itype, K, n_teacher_rows,
                t_cnt, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride,
-               (reinterpret_cast<uintptr_t>(workspace) % 16 == 0) ? workspace : nullptr, 1, spin_limit(), flags};
+               (reinterpret_cast<uintptr_t>(workspace) % 16 == 0) ? workspace : nullptr, 1,
+               (flags & DL_TOPK_NO_WAIT) ? 0 : SPIN_LIMIT, flags};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   hipError_t e;
   if (kind == DL_FKL) {

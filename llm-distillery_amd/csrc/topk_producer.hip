@@ -38,7 +38,7 @@ typedef short i16x2 __attribute__((ext_vector_type(2)));
 struct PartHeader { float mx; float sm; int cnt; int pad; };     // 16 bytes, then cnt u64 entries
 
 struct ProducerParams {
-  const void* logits; int64_t row_stride; int64_t V;
+  const void* logits; int64_t row_stride; int64_t n_rows; int64_t V;
   const int32_t* row_list; int64_t n_out;
   int K; int parts;
   char* ws; int64_t part_stride;            // bytes per (row, part) record
@@ -248,9 +248,43 @@ __device__ __forceinline__ void wave_sort_emit(const typename Cand<Tag>::W* cand
   }
 }
 
+// Logits row behind output row ro, or -1 when the caller's row list names a row outside the logits
+// (negative padding entries, stale positions): such an output row is masked -- no logits are touched,
+// the merge kernel fills it with -inf log-probs and id -1.
+__device__ __forceinline__ int64_t producer_row(const ProducerParams& p, int64_t ro) {
+  const int64_t r = p.row_list ? (int64_t)p.row_list[ro] : ro;
+  return (r >= 0 && r < p.n_rows) ? r : -1;
+}
+
+// One 16-byte chunk of a row that keeps no alignment promise (odd vocabulary size, a cropped view
+// with an odd pitch): assembled from element-sized loads, columns at or beyond n_cols read as -inf.
+template <class Tag>
+__device__ __forceinline__ u32x4 load_chunk_elementwise(const char* part, int chunk, int n_cols) {
+  u32x4 v = Chunk<Tag>::neg_inf();
+  const int col0 = chunk * Chunk<Tag>::N;
+  if constexpr (Tag::bytes == 4) {
+    const unsigned* e = reinterpret_cast<const unsigned*>(part) + col0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) if (col0 + d < n_cols) v[d] = e[d];
+  } else {
+    const unsigned short* e = reinterpret_cast<const unsigned short*>(part) + col0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const unsigned lo = col0 + 2 * d < n_cols ? (unsigned)e[2 * d] : (v[d] & 0xffffu);
+      const unsigned hi = col0 + 2 * d + 1 < n_cols ? (unsigned)e[2 * d + 1] : (v[d] >> 16);
+      v[d] = lo | (hi << 16);
+    }
+  }
+  return v;
+}
+
 // G = chunk groups per thread whose maxima feed the threshold search: 256 * G groups per part must
 // be a few times K for the candidate set to stay close to K (4 for K <= 256, else 16).
-template <class Tag, int G>
+// ALIGNED: rows start on 16-byte boundaries and hold a whole number of chunks (16-byte loads);
+// otherwise the chunks are assembled element by element and the last one is padded with -inf,
+// which the collection leaves out (a padding entry has the lowest key and the highest columns of
+// its part, so the threshold searches, which only count, need no such test).
+template <class Tag, int G, bool ALIGNED>
 __global__ __launch_bounds__(PROD_NT) __attribute__((amdgpu_waves_per_eu(PROD_NT / 64, 8)))
 void topk_part_kernel(const ProducerParams p) {
   constexpr int NT = PROD_NT, NCH = PROD_NCH, NW = NT / WAVE, CPG = NCH / G;
@@ -273,11 +307,12 @@ void topk_part_kernel(const ProducerParams p) {
   const int64_t ro = (int64_t)grp * 8 + (t_in & 7u);
   const int h_part = (int)(t_in >> 3);
   if (ro >= p.n_out) return;
-  const int64_t r = p.row_list ? (int64_t)p.row_list[ro] : ro;
+  const int64_t r = producer_row(p, ro);
+  if (r < 0) return;                                                 // masked output row: the merge kernel fills it
   const int64_t c0 = (int64_t)h_part * NT * NCH;
-  const int nch = (int)min((int64_t)NT * NCH, p.V / C::N - c0);      // chunks of this part, >= 1
   const int lo = (int)(c0 * C::N);
-  const int n_elems = nch * C::N;
+  const int n_elems = (int)min((int64_t)NT * NCH * C::N, p.V - lo);  // columns of this part, >= 1
+  const int nch = (n_elems + C::N - 1) / C::N;                       // its chunks (the last one padded unless ALIGNED)
   const int Kp = min(p.K, n_elems);
   const char* rpart = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes + c0 * 16;
   char* rec = p.ws + (ro * P + h_part) * p.part_stride;
@@ -288,7 +323,8 @@ void topk_part_kernel(const ProducerParams p) {
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = i * NT + tid;
-    reg[i] = c < nch ? load16_stream(rpart + (int64_t)c * 16) : C::neg_inf();
+    if constexpr (ALIGNED) reg[i] = c < nch ? load16_stream(rpart + (int64_t)c * 16) : C::neg_inf();
+    else reg[i] = c < nch ? load_chunk_elementwise<Tag>(rpart, c, n_elems) : C::neg_inf();
   }
   if (tid == 0) s_n = 0;
 
@@ -397,7 +433,8 @@ void topk_part_kernel(const ProducerParams p) {
   if (L == 0) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      if (i < my_chunks) collect_entries<Tag, NT, NCH>(reg, i, cand, &s_n, [](unsigned, int) { return true; });
+      if (i < my_chunks)
+        collect_entries<Tag, NT, NCH>(reg, i, cand, &s_n, [n_elems](unsigned, int col) { return ALIGNED || col < n_elems; });
     }
   } else {
     const unsigned lm1 = KY::PER_DWORD == 2 ? (L - 1) * 0x00010001u : L - 1;
@@ -414,8 +451,8 @@ void topk_part_kernel(const ProducerParams p) {
 #pragma unroll
                 for (int h = 0; h < KY::PER_DWORD; ++h) {
                   const unsigned k = KY::key(reg[i][d], h);
-                  if (k >= L) {
-                    const int col = (i * NT + tid) * C::N + d * KY::PER_DWORD + h;
+                  const int col = (i * NT + tid) * C::N + d * KY::PER_DWORD + h;
+                  if (k >= L && (ALIGNED || col < n_elems)) {
                     const int slot = atomicAdd(&s_n, 1);
                     if (slot < PROD_CAP) cand[slot] = Cand<Tag>::make(k, col);
                   }
@@ -453,7 +490,9 @@ void topk_part_kernel(const ProducerParams p) {
     for (int i = 0; i < NCH; ++i) {
       if (i < my_chunks)
         collect_entries<Tag, NT, NCH>(reg, i, cand, &s_n,
-                                      [T, clo](unsigned k, int col) { return k > T || (k == T && col <= clo); });
+                                      [T, clo, n_elems](unsigned k, int col) {
+                                        return (k > T || (k == T && col <= clo)) && (ALIGNED || col < n_elems);
+                                      });
     }
     __syncthreads();
     n = s_n;                                                        // == Kp
@@ -528,6 +567,14 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p)
   const int sel_cap = producer_sel_cap(K);
   u64* sel = all + producer_merge_slots(K, P);                      // the selected words; sel_cap words
   const char* rec0 = p.ws + ro * P * p.part_stride;
+  if (producer_row(p, ro) < 0) {                                    // the row list names no logits row: masked output row
+    for (int k = tid; k < K; k += 256) {
+      store_from_float(p.out_val, p.out_dtype, ro * K + k, -INFINITY);
+      if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * K + k] = -1;
+      else reinterpret_cast<int64_t*>(p.out_idx)[ro * K + k] = -1;
+    }
+    return;
+  }
 
   float M = -INFINITY;
   for (int q = 0; q < P; ++q) M = fmaxf(M, reinterpret_cast<const PartHeader*>(rec0 + q * p.part_stride)->mx);
@@ -635,15 +682,21 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p)
 }
 
 static int producer_parts(int64_t V, int logits_dtype) {
-  const int64_t nch = V / (logits_dtype == DL_F32 ? 4 : 8);
+  const int epc = logits_dtype == DL_F32 ? 4 : 8;
+  const int64_t nch = (V + epc - 1) / epc;
   return (int)((nch + PROD_NT * PROD_NCH - 1) / (PROD_NT * PROD_NCH));
 }
 
 template <class Tag>
-static int launch_producer(const ProducerParams& p, hipStream_t st) {
+static int launch_producer(const ProducerParams& p, bool aligned, hipStream_t st) {
   const dim3 grid((unsigned)((p.n_out + 7) / 8 * 8 * p.parts));
-  if (p.K <= 256) hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_SMALL>), grid, dim3(PROD_NT), 0, st, p);
-  else hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_LARGE>), grid, dim3(PROD_NT), 0, st, p);
+  if (aligned) {
+    if (p.K <= 256) hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_SMALL, true>), grid, dim3(PROD_NT), 0, st, p);
+    else hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_LARGE, true>), grid, dim3(PROD_NT), 0, st, p);
+  } else {
+    if (p.K <= 256) hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_SMALL, false>), grid, dim3(PROD_NT), 0, st, p);
+    else hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_LARGE, false>), grid, dim3(PROD_NT), 0, st, p);
+  }
   const size_t lds = (size_t)(producer_merge_slots(p.K, p.parts) + producer_sel_cap(p.K)) * 8;      // <= 48 KiB
   hipLaunchKernelGGL((topk_merge_kernel<Tag>), dim3((unsigned)p.n_out), dim3(256), lds, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
@@ -673,16 +726,16 @@ extern "C" int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row
       n_out * parts > 0x7fffffffLL)
     return DL_ERR_LIMIT;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
-  if (V % (16 / eb) != 0 || reinterpret_cast<uintptr_t>(logits) % 16 != 0 || (row_stride * eb) % 16 != 0)
-    return DL_ERR_ALIGN;
+  if (reinterpret_cast<uintptr_t>(logits) % eb != 0) return DL_ERR_ALIGN;
+  const bool aligned = V % (16 / eb) == 0 && reinterpret_cast<uintptr_t>(logits) % 16 == 0 && (row_stride * eb) % 16 == 0;
   if (n_out == 0) return DL_OK;
   if (!workspace) return DL_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return DL_ERR_ALIGN;
   if (workspace_bytes < dl_teacher_topk_workspace_bytes(logits_dtype, n_out, V, K)) return DL_ERR_WORKSPACE;
-  ProducerParams p{logits, row_stride, V, row_list, n_out, K, parts, reinterpret_cast<char*>(workspace),
+  ProducerParams p{logits, row_stride, n_rows, V, row_list, n_out, K, parts, reinterpret_cast<char*>(workspace),
                    producer_part_stride(K, parts), out_val, out_dtype, out_idx, out_itype};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  return logits_dtype == DL_F32 ? launch_producer<TagF32>(p, st)
-         : logits_dtype == DL_BF16 ? launch_producer<TagBF16>(p, st)
-                                   : launch_producer<TagF16>(p, st);
+  return logits_dtype == DL_F32 ? launch_producer<TagF32>(p, aligned, st)
+         : logits_dtype == DL_BF16 ? launch_producer<TagBF16>(p, aligned, st)
+                                   : launch_producer<TagF16>(p, aligned, st);
 }

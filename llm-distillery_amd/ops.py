@@ -18,9 +18,24 @@ def _stream_ptr(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
-def _dev(t: torch.Tensor, name: str) -> None:
+def _dev(t: torch.Tensor, name: str, dev: torch.device | None = None) -> None:
+    """`t` must live on the GPU -- on `dev`, when given: the kernels take raw pointers and run on the
+    device of the logits, so a tensor on another GPU would be read through a foreign address."""
     if not t.is_cuda:
         raise RuntimeError(f"{name} must live on the GPU (got {t.device}); this library has no CPU path")
+    if dev is not None and t.device != dev:
+        raise RuntimeError(f"{name} lives on {t.device}, the logits on {dev}: all tensors of a call must share one device")
+
+
+def _grad_target(grad_out, R: int, V: int, dtype, dev) -> torch.Tensor:
+    """The gradient buffer of a launch over [R, V] logits: `grad_out` checked against what the kernel
+    will write (shape, dtype, dense along V, same device), or a fresh one."""
+    if grad_out is None:
+        return torch.empty((R, V), dtype=dtype, device=dev)
+    if grad_out.dim() != 2 or tuple(grad_out.shape) != (R, V) or grad_out.dtype != dtype or grad_out.stride(1) != 1 \
+            or grad_out.device != dev:
+        raise RuntimeError(f"grad_out must be a [{R}, {V}] {dtype} tensor on {dev}, dense along the vocabulary axis")
+    return grad_out
 
 
 def _rows_2d(logits: torch.Tensor) -> torch.Tensor:
@@ -58,22 +73,25 @@ def _opt_i32(t, n, name, dev):
 def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor, *,
              row_map: torch.Tensor | None = None, t_cnt: torch.Tensor | None = None,
              T: float = 1.0, teacher_T: float | None = None, grad_scale: float = 1.0,
-             want_grad: bool = True, grad_out: torch.Tensor | None = None, unique_ids: bool = False):
+             want_grad: bool = True, grad_out: torch.Tensor | None = None, unique_ids: bool = False,
+             no_wait: bool = False, parts: int = 0):
     """Per-token forward ("fkl") or reverse ("rkl") KL against a top-K teacher and,
     in the same launch, d(sum of row losses)/d(logits) * grad_scale.
 
     logits [..., V] bf16/fp16/fp32 (native model dtype, rows evenly strided);
     t_val/t_idx [N, K] stored teacher log-probs and ids; row_map int32 [rows]
     gives the teacher row of each logits row (negative = masked row).  `unique_ids=True` promises
-    that no id repeats within a row (skips the check for repeated ids).
+    that no id repeats within a row (skips the check for repeated ids).  `no_wait` / `parts` are the
+    library's per-call test hooks for rows cut into column parts (DL_TOPK_NO_WAIT, DL_TOPK_PARTS).
     Returns (row_loss fp32 [rows], grad like logits or None).
     """
     if kind not in ("fkl", "rkl"):
         raise ValueError("kind must be 'fkl' or 'rkl' for a top-K teacher")
-    _dev(logits, "logits"), _dev(t_val, "t_val"), _dev(t_idx, "t_idx")
+    _dev(logits, "logits")
     x = _rows_2d(logits)
     R, V = x.shape
     dev = x.device
+    _dev(t_val, "t_val", dev), _dev(t_idx, "t_idx", dev)
     if x.dtype not in _DT or t_val.dtype not in _DT or t_idx.dtype not in _IT:
         raise RuntimeError("unsupported dtype")
     if t_val.dim() != 2 or t_val.shape != t_idx.shape:
@@ -87,10 +105,12 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
     row_loss = torch.empty(R, dtype=torch.float32, device=dev)
     grad, g_ptr, g_stride = None, 0, V
     if want_grad:
-        grad = grad_out if grad_out is not None else torch.empty((R, V), dtype=x.dtype, device=dev)
-        if grad.shape != (R, V) or grad.dtype != x.dtype or grad.stride(1) != 1 or grad.device != dev:
-            raise RuntimeError("grad_out must match logits as a [rows, V] tensor")
+        grad = _grad_target(grad_out, R, V, x.dtype, dev)
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
+    if parts not in (0, 1, 2, 4):
+        raise ValueError("parts must be 0 (automatic), 1, 2 or 4")
+    flags = (_lib.DL_TOPK_UNIQUE_IDS if unique_ids else 0) | (_lib.DL_TOPK_NO_WAIT if no_wait else 0) | \
+        (parts << _lib.DL_TOPK_PARTS_SHIFT)
     lib = _lib.load()
     ws_bytes = lib.dl_div_topk_workspace_bytes(KINDS[kind], _DT[x.dtype], R, V) if want_grad else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
@@ -100,7 +120,7 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
                              cnt_ptr, 1.0 / T, 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
                              row_loss.data_ptr(), g_ptr, g_stride,
                              ws.data_ptr() if ws is not None else 0, ws_bytes,
-                             _lib.DL_TOPK_UNIQUE_IDS if unique_ids else 0, _stream_ptr(dev))
+                             flags, _stream_ptr(dev))
     _lib.check(st, "dl_div_topk")
     if grad is not None and logits.dim() != 2 and grad_out is None:
         grad = grad.view(logits.shape)
@@ -114,11 +134,12 @@ def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_ma
     d(sum of row losses)/d(logits) * grad_scale.  Returns (row_loss fp32 [rows], grad or None)."""
     if kind not in KINDS:
         raise ValueError("kind must be 'fkl', 'rkl' or 'jsd'")
-    _dev(logits, "logits"), _dev(t_logits, "t_logits")
+    _dev(logits, "logits")
     x = _rows_2d(logits)
     t = _rows_2d(t_logits)
     R, V = x.shape
     dev = x.device
+    _dev(t_logits, "t_logits", dev)
     if x.dtype not in _DT or t.dtype not in _DT:
         raise RuntimeError("unsupported dtype")
     if t.shape[1] != V:
@@ -130,9 +151,7 @@ def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_ma
     row_loss = torch.empty(R, dtype=torch.float32, device=dev)
     grad, g_ptr, g_stride = None, 0, V
     if want_grad:
-        grad = grad_out if grad_out is not None else torch.empty((R, V), dtype=x.dtype, device=dev)
-        if grad.shape != (R, V) or grad.dtype != x.dtype or grad.stride(1) != 1 or grad.device != dev:
-            raise RuntimeError("grad_out must match logits as a [rows, V] tensor")
+        grad = _grad_target(grad_out, R, V, x.dtype, dev)
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
     with torch.cuda.device(dev):
         st = _lib.load().dl_div_dense(KINDS[kind], x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr,
@@ -147,7 +166,7 @@ def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_ma
 
 def _rowstats_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float):
     """Phase 1 launch: (lse [N], zk [N, K]) for the valid rows of x [R, V]."""
-    _dev(x, "logits"), _dev(t_idx, "t_idx")
+    _dev(x, "logits"), _dev(t_idx, "t_idx", x.device)
     if x.dim() != 2 or x.stride(1) != 1 or x.dtype not in _DT:
         raise RuntimeError("logits must be [rows, V] bf16/fp16/fp32, dense along V")
     if t_idx.dim() != 2 or t_idx.dtype not in _IT:
@@ -177,9 +196,9 @@ def _rowcoef_grad_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: floa
     _, rm_ptr = _opt_i32(row_map, R, "row_map", x.device)
     g_lse = g_lse.to(torch.float32).contiguous()
     g_zk = g_zk.to(torch.float32).contiguous()
-    grad = grad_out if grad_out is not None else torch.empty((R, V), dtype=x.dtype, device=x.device)
-    if grad.shape != (R, V) or grad.dtype != x.dtype or grad.stride(1) != 1:
-        raise RuntimeError("grad_out must match the logits in shape and dtype and be dense along V")
+    for name, t in (("t_idx", t_idx), ("lse", lse), ("g_lse", g_lse), ("g_zk", g_zk)):
+        _dev(t, name, x.device)
+    grad = _grad_target(grad_out, R, V, x.dtype, x.device)
     with torch.cuda.device(x.device):
         st = _lib.load().dl_rowcoef_grad_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(),
                                               _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), g_lse.data_ptr(),
@@ -302,6 +321,8 @@ def composite_epilogue(lse: torch.Tensor, zk: torch.Tensor, t_val: torch.Tensor,
     `avoid` rows, and `offsets` int32 [3, C + 1] (first row, first label, first avoid entry of every
     conversation).  See dl_composite_forward."""
     _dev(zk, "zk")
+    for name, t in (("lse", lse), ("t_val", t_val), ("t_idx", t_idx), ("labels", labels), ("avoid", avoid), ("offsets", offsets)):
+        _dev(t, name, zk.device)
     if lse.dtype != torch.float32 or zk.dtype != torch.float32 or not (lse.is_contiguous() and zk.is_contiguous()):
         raise RuntimeError("lse / zk must be contiguous fp32 (phase 1's outputs)")
     if t_val.dtype not in _DT or t_idx.dtype not in _IT or labels.dtype != torch.int64 or avoid.dtype != torch.int32 \
@@ -328,15 +349,10 @@ def reduce_sum(values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
 
 def copy16(src: torch.Tensor, dst: torch.Tensor) -> None:
     """Streaming copy of src's bytes into dst (the calibration kernel for HBM counters)."""
-    _dev(src, "src"), _dev(dst, "dst")
+    _dev(src, "src"), _dev(dst, "dst", src.device)
     n = src.numel() * src.element_size()
     if not (src.is_contiguous() and dst.is_contiguous()) or dst.numel() * dst.element_size() != n:
         raise RuntimeError("copy16 needs two contiguous buffers of the same byte size")
     with torch.cuda.device(src.device):
         st = _lib.load().dl_copy16(src.data_ptr(), dst.data_ptr(), n, _stream_ptr(src.device))
     _lib.check(st, "dl_copy16")
-
-
-def set_option(name: str, value: int) -> None:
-    """Process-wide tuning / test hooks of the library ("split_parts", "spin_limit")."""
-    _lib.check(_lib.load().dl_set_option(name.encode(), int(value)), f"dl_set_option({name!r})")

@@ -33,13 +33,13 @@ def merge_remap_topk(vals: Sequence[torch.Tensor], idxs: Sequence[torch.Tensor],
     vals = [v.contiguous() for v in vals]
     idxs = [i.contiguous() for i in idxs]
     for v, i in zip(vals, idxs):
-        _dev(v, "vals"), _dev(i, "idxs")
+        _dev(v, "vals", vals[0].device), _dev(i, "idxs", vals[0].device)
         if v.shape != vals[0].shape or i.shape != vals[0].shape or v.dtype != vals[0].dtype or i.dtype != idxs[0].dtype:
             raise RuntimeError("all teachers must share shape [N, K] and dtypes")
     N, K = vals[0].shape
     dev = vals[0].device
     if id_map is not None:
-        _dev(id_map, "id_map")
+        _dev(id_map, "id_map", dev)
         if id_map.dtype != torch.int32 or id_map.dim() != 1 or not id_map.is_contiguous():
             raise RuntimeError("id_map must be a contiguous int32 vector")
         if student_vocab is None:
@@ -68,7 +68,7 @@ def merge_topk_pair(disk_val: torch.Tensor, disk_idx: torch.Tensor, new_val: tor
     (classes/data_manager.py:198-261): returns (log-mass fp32 [n, K], ids int64 [n, K]) in
     descending-mass order, n = the longer of the two inputs."""
     for t, name in ((disk_val, "disk_val"), (disk_idx, "disk_idx"), (new_val, "new_val"), (new_idx, "new_idx")):
-        _dev(t, name)
+        _dev(t, name, disk_val.device if disk_val.is_cuda else None)
     disk_val, disk_idx, new_val, new_idx = (t.contiguous() for t in (disk_val, disk_idx, new_val, new_idx))
     if disk_val.dtype != new_val.dtype or disk_idx.dtype != new_idx.dtype or disk_val.shape[1] != new_val.shape[1]:
         raise RuntimeError("both teachers must share K and dtypes")

@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .ops import _DT, _dev, _opt_i32, _rows_2d, _stream_ptr
+from .ops import _DT, _dev, _grad_target, _opt_i32, _rows_2d, _stream_ptr
 
 
 def _pack(vocab: Sequence[bytes]):
@@ -121,12 +121,14 @@ def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=Non
     if x.dtype not in _DT:
         raise RuntimeError("unsupported dtype")
     R, Vt = x.shape
+    if csr is None and plan is None and t2s is None:
+        raise ValueError("marginalise needs one of plan=, t2s= or csr=")
     out = torch.empty((R, n_student), dtype=torch.float32, device=x.device)
     lib = _lib.load()
     with torch.cuda.device(x.device):
         if csr is not None:
             off, ind = csr
-            _dev(off, "offsets"), _dev(ind, "indices")
+            _dev(off, "offsets", x.device), _dev(ind, "indices", x.device)
             if off.dtype != torch.int32 or ind.dtype != torch.int32 or off.numel() != n_student + 1:
                 raise RuntimeError("csr must be (int32 offsets [n_student + 1], int32 indices)")
             if int(off[-1].item()) > ind.numel():
@@ -155,11 +157,12 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
     (teacher_probs [N, Vt]) marginalised into the student vocabulary along `t2s`, loss and gradient
     in one launch; the marginal stays in LDS.  `t2s` is the int32 [Vt] map on the GPU or, better, a
     MarginalPlan built from it.  Returns (row_loss fp32 [rows], grad or None)."""
-    _dev(logits, "logits"), _dev(teacher_probs, "teacher_probs")
+    _dev(logits, "logits")
     x, tp = _rows_2d(logits), _rows_2d(teacher_probs)
     R, Vs = x.shape
     N, Vt = tp.shape
     dev = x.device
+    _dev(teacher_probs, "teacher_probs", dev)
     plan_args = (0, 0, 0, 0, 0, 0)
     if isinstance(t2s, MarginalPlan):
         t2s.check(Vs, Vt, dev)
@@ -174,7 +177,7 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
     row_loss = torch.empty(R, dtype=torch.float32, device=dev)
     grad, g_ptr, g_stride = None, 0, Vs
     if want_grad:
-        grad = grad_out if grad_out is not None else torch.empty((R, Vs), dtype=x.dtype, device=dev)
+        grad = _grad_target(grad_out, R, Vs, x.dtype, dev)
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
     with torch.cuda.device(dev):
         st = _lib.load().dl_rkl_marginalised(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vs, rm_ptr, tp.data_ptr(),

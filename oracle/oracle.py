@@ -24,6 +24,10 @@ Parity status (what pins each function besides reading the reference):
     with `indices=None` (it raises), so these follow the formula of
     `custom_kl_div` and reduce to the top-K functions at K=V    -> pinned by
     that reduction only.
+  * forward KL against a ragged, already-normalised sparse teacher
+    (`fwd_kl_sparse_rows`, the checker of the merged multi-teacher loss):
+    reduces to the golden-pinned top-K form on full rows, to `F.kl_div` on the
+    live prefix of ragged rows, gradient identity   -> pinned.
   * JSD, weighted multi-teacher merge, vocabulary remap, byte-trie map and CSR
     marginalisation have NO counterpart in the reference: "parity unpinned";
     they are pinned by textbook formulas, brute force and invariants.
@@ -236,6 +240,20 @@ def storage_tolerance(ref: torch.Tensor, storage_dtype, rtol: float) -> torch.Te
     half_ulp = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[storage_dtype]
     floor = {torch.float32: 1e-30, torch.bfloat16: 1e-30, torch.float16: 2.0 ** -25}[storage_dtype]
     return ref.abs() * (rtol + half_ulp) + floor + 1.2e-7 * ref.abs().max()
+
+
+def dense_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, t_logits: torch.Tensor, rows64: torch.Tensor,
+                             T: float, t_T: float, scale: float, storage_dtype, rtol: float) -> torch.Tensor:
+    """Element-wise bound for the gradient of a dense-teacher divergence, rows already selected
+    (`logits`, `t_logits`, `grad64` [n, V]; `rows64` [n] the per-row losses; `scale` the factor the
+    gradient carries, e.g. 1 / n_valid).  `storage_tolerance` plus 4e-6 of the terms a gradient entry
+    is a difference of, (p + q)(1 + |log p/q| + loss) * scale / T: where they cancel, fp32 evaluation
+    (the reference's as well) keeps ~1e-6 of the TERMS, not of the result."""
+    lp = torch.log_softmax(logits.double() / T, -1)
+    lq = torch.log_softmax(t_logits.double() / t_T, -1)
+    ratio = torch.nan_to_num((lp - lq).abs(), nan=0.0, posinf=0.0)
+    terms = (lp.exp() + lq.exp()) * (1 + ratio + rows64.unsqueeze(-1)) * (scale / T)
+    return storage_tolerance(grad64, storage_dtype, rtol) + 4e-6 * terms
 
 
 # ---------------------------------------------------------------------------

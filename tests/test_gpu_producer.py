@@ -90,8 +90,52 @@ def test_tie_plateaus_of_every_size(D, dtype, n_tied):
     np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype,V,K", [(torch.bfloat16, 50257, 200), (torch.float32, 50257, 400), (torch.float16, 1001, 10),
+                                       (torch.bfloat16, 131073, 64), (torch.float32, 7, 7)])
+def test_any_vocabulary_size(D, dtype, V, K):
+    """The reference's producer takes any `crop_distr_to_size` (classes/teacher/inference_worker.py:73-77):
+    vocabularies that are not a whole number of 16-byte chunks, rows on odd pitches."""
+    g = torch.Generator().manual_seed(V)
+    logits = (torch.randn(6, V, generator=g) * 3).to(dtype)
+    logits[2, V - 1] = 9.0                                   # the last column of the padded tail chunk wins a row
+    logits[4, V - 3:] = float("-inf")
+    val, idx = D.teacher_topk(logits.to(DEV), K, val_dtype=torch.float32, idx_dtype=torch.int64)
+    rv, ri = _ref(logits, V, K)
+    assert torch.equal(idx.cpu(), ri) and int(idx.max()) < V
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), rtol=0, atol=2e-6 * max(1.0, float(rv[torch.isfinite(rv)].abs().max())))
+
+
+def test_odd_crop_of_a_wider_vocabulary_and_tied_tails(D):
+    g = torch.Generator().manual_seed(12)
+    B, S, Vm, crop, K = 2, 7, 32003, 31999, 120
+    logits = (torch.randn(B, S, Vm, generator=g) * 2).to(torch.bfloat16)
+    logits[..., crop:] = 20.0                                # beyond the crop: must never be seen
+    logits[0, 3, crop - 40:crop] = 4.0                       # a tie plateau that runs into the padded tail
+    val, idx = D.teacher_topk(logits.to(DEV), K, crop_to_size=crop, val_dtype=torch.float32, idx_dtype=torch.int32)
+    rv, ri = _ref(logits.reshape(B * S, Vm), crop, K)
+    assert torch.equal(idx.cpu().long(), ri) and int(idx.max()) < crop
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), atol=1e-5)
+    # a constant row of odd width: every column ties, the first K ids win
+    const = torch.full((3, 4099), 0.25, dtype=torch.float16)
+    _, ci = D.teacher_topk(const.to(DEV), 300, idx_dtype=torch.int32)
+    assert ci[1].cpu().tolist() == list(range(300))
+
+
+def test_row_list_entries_outside_the_logits_give_masked_rows(D):
+    g = torch.Generator().manual_seed(5)
+    logits = (torch.randn(10, 4096, generator=g) * 2).to(torch.bfloat16)
+    rows = torch.tensor([3, -1, 9, 10, 0, 2 ** 31 - 1, -(2 ** 31)], dtype=torch.int32)
+    val, idx = D.teacher_topk(logits.to(DEV), 32, rows=rows.to(DEV), val_dtype=torch.float32)
+    good = torch.tensor([0, 2, 4])
+    rv, ri = _ref(logits[rows[good].long()], 4096, 32)
+    assert torch.equal(idx.cpu()[good].long(), ri)
+    np.testing.assert_allclose(val.cpu()[good].double().numpy(), rv.numpy(), atol=1e-5)
+    bad = torch.tensor([1, 3, 5, 6])
+    assert (idx.cpu()[bad] == -1).all() and torch.isneginf(val.cpu()[bad]).all()
+
+
 def test_producer_limits(D):
     with pytest.raises(RuntimeError):
         D.teacher_topk(torch.zeros(2, 4096, device=DEV), 2000)
     with pytest.raises(RuntimeError):
-        D.teacher_topk(torch.zeros(2, 1001, device=DEV), 10)
+        D.teacher_topk(torch.zeros(2, 100, device=DEV), 101)              # K > V

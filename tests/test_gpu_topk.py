@@ -26,7 +26,7 @@ def _case(R, V, K, dtype, seed, std=2.0, idx_dtype=torch.int32, val_dtype=torch.
     return logits, tv.to(val_dtype), ti.to(idx_dtype)
 
 
-def _check(D, kind, logits, tv, ti, T, valid=None, teacher_T=None, **tol_over):
+def _check(D, kind, logits, tv, ti, T, valid=None, teacher_T=None, hooks=None, **tol_over):
     R, V = logits.shape
     n_valid = R if valid is None else int(valid.sum())
     loss64, rows64, grad64 = O.mean_loss_and_grad(kind, logits, T, t_vals=tv, t_idx=ti, valid=valid, t_T=teacher_T,
@@ -37,7 +37,7 @@ def _check(D, kind, logits, tv, ti, T, valid=None, teacher_T=None, **tol_over):
         rm[valid] = torch.arange(n_valid, dtype=torch.int32)
         row_map = rm.to(DEV)
     rl, grad = D.div_topk(kind, logits.to(DEV), tv.to(DEV), ti.to(DEV), row_map=row_map, T=T, teacher_T=teacher_T,
-                          grad_scale=1.0 / n_valid)
+                          grad_scale=1.0 / n_valid, **(hooks or {}))
     loss = D.reduce_sum(rl, 1.0 / n_valid)
     torch.cuda.synchronize()
     rows_gpu = rl.cpu()
@@ -172,25 +172,18 @@ def test_errors_are_python_exceptions(D):
 def test_split_row_parts_agree_and_give_up_path(D, parts):
     """A 128256-wide row is cut into column parts that exchange statistics through the workspace.
     Every setting must give the oracle's numbers, also when no part waits for its partners
-    (spin_limit 0: every part that finds a record missing leaves and is finished by the retry
-    launch), and the same bits as with waiting."""
+    (the no-wait flag: every part that finds a record missing leaves and is finished by the second
+    launch), and the same bits as with waiting.  The hooks travel with the call: the library keeps
+    no state."""
     logits, tv, ti = _case(40, 128256, 200, torch.bfloat16, 12, std=3.0)
     valid = torch.ones(40, dtype=torch.bool)
     valid[[0, 7, 33]] = False
-    try:
-        D.set_option("split_parts", parts)
-        _check(D, "fkl", logits, tv[:37], ti[:37], T=1.0, valid=valid)
-        waited = _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid)
-        D.set_option("spin_limit", 0)
-        retried = _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid)
-        assert torch.equal(waited, retried)
-    finally:
-        D.set_option("split_parts", 0)
-        D.set_option("spin_limit", 20000)
-    with pytest.raises(RuntimeError):
-        D.set_option("split_parts", 3)
-    with pytest.raises(RuntimeError):
-        D.set_option("no_such_option", 1)
+    _check(D, "fkl", logits, tv[:37], ti[:37], T=1.0, valid=valid, hooks={"parts": parts})
+    waited = _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid, hooks={"parts": parts})
+    retried = _check(D, "fkl", logits, tv[:37], ti[:37], T=2.0, valid=valid, hooks={"parts": parts, "no_wait": True})
+    assert torch.equal(waited, retried)
+    with pytest.raises(ValueError):
+        D.div_topk("fkl", logits[:2].to(DEV), tv[:2].to(DEV), ti[:2].to(DEV), parts=3)
 
 
 @pytest.mark.parametrize("kind,V,dtype", [("fkl", 128256, torch.bfloat16), ("fkl", 32000, torch.bfloat16), ("fkl", 152064, torch.float16),
@@ -202,13 +195,9 @@ def test_gradient_may_overwrite_the_logits(D, kind, V, dtype):
     logits, tv, ti = _case(24, V, 64, dtype, 31)
     x = logits.to(DEV)
     rl, g = D.div_topk(kind, x, tv.to(DEV), ti.to(DEV), T=1.5)
-    for spin in (20000, 0):
-        try:
-            D.set_option("spin_limit", spin)
-            y = x.clone()
-            rl2, g2 = D.div_topk(kind, y, tv.to(DEV), ti.to(DEV), T=1.5, grad_out=y)
-        finally:
-            D.set_option("spin_limit", 20000)
+    for no_wait in (False, True):
+        y = x.clone()
+        rl2, g2 = D.div_topk(kind, y, tv.to(DEV), ti.to(DEV), T=1.5, grad_out=y, no_wait=no_wait)
         assert g2.data_ptr() == y.data_ptr() and torch.equal(rl, rl2) and torch.equal(g, y)
 
 
@@ -221,11 +210,7 @@ def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
     valid = torch.ones(10, dtype=torch.bool)
     valid[4] = False
     waited = _check(D, "fkl", logits, tv[:9], ti[:9], T=1.3, valid=valid)
-    try:
-        D.set_option("spin_limit", 0)
-        retried = _check(D, "fkl", logits, tv[:9], ti[:9], T=1.3, valid=valid)
-    finally:
-        D.set_option("spin_limit", 20000)
+    retried = _check(D, "fkl", logits, tv[:9], ti[:9], T=1.3, valid=valid, hooks={"no_wait": True})
     assert torch.equal(waited, retried)
 
 

@@ -7,6 +7,7 @@ import os
 import numpy as np
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import oracle as O
 
@@ -95,6 +96,49 @@ def test_merge_remap_all_dropped_row_and_padded_layout():
     ids, lq, cnt = O.merge_remap_padded(vals, idxs, (0.5, 0.5), id_map)
     assert cnt[1] == 0 and np.all(ids[1] == -1) and np.all(np.isneginf(lq[1]))
     assert ids.shape == (3, 8) and cnt[0] > 0
+
+
+def test_fwd_kl_sparse_rows_reduces_to_the_topk_form_and_to_the_library():
+    # (1) full rows (cnt == K, normalised log-probs): the value of fwd_kl_topk_rows, which the golden
+    #     vectors written from the reference's calculate_divergence pin
+    g = torch.Generator().manual_seed(11)
+    N, K, V = 9, 7, 41
+    z = torch.randn(N, V, generator=g, dtype=torch.float64) * 2
+    stored, idx = torch.topk(torch.log_softmax(torch.randn(N, V, generator=g, dtype=torch.float64), -1), K)
+    t = O.teacher_logprobs_topk(stored, 1.3, torch.float64)
+    full = O.fwd_kl_sparse_rows(z, idx.numpy().astype(np.int32), t.numpy(), np.full(N, K, dtype=np.int32))
+    np.testing.assert_allclose(full.numpy(), O.fwd_kl_topk_rows(z, t, idx).numpy(), rtol=1e-12)
+    # (2) ragged rows with padding behind the count: per row the library's kl_div on the live prefix;
+    #     the padding (-1 ids, -inf log-probs, and garbage behind a count of 0) must not be read
+    cnt = np.array([K, 3, 0, 1, 5, K, 2, 0, 4], dtype=np.int32)
+    ids = idx.numpy().astype(np.int32).copy()
+    lq = np.full((N, K), -np.inf)
+    for r in range(N):
+        n = int(cnt[r])
+        ids[r, n:] = -1
+        if n:
+            lq[r, :n] = torch.log_softmax(stored[r, :n], -1).numpy()
+    ids[2, :] = 12345                                        # count 0: whatever lies there is ignored
+    z.requires_grad_(True)
+    got = O.fwd_kl_sparse_rows(z, ids, lq, cnt)
+    s = torch.log_softmax(z.detach(), -1)
+    for r in range(N):
+        n = int(cnt[r])
+        if n == 0:
+            assert got[r].item() == 0.0
+            continue
+        want = F.kl_div(s[r, idx[r, :n]], torch.as_tensor(lq[r, :n]), reduction="none", log_target=True).sum()
+        np.testing.assert_allclose(got[r].item(), want.item(), rtol=1e-12)
+    # (3) gradient identity of the forward KL: softmax(z) - scatter(q) on rows with entries, 0 elsewhere
+    got.sum().backward()
+    want_g = torch.softmax(z.detach(), -1)
+    for r in range(N):
+        n = int(cnt[r])
+        if n == 0:
+            want_g[r] = 0
+        else:
+            want_g[r, idx[r, :n]] -= torch.exp(torch.as_tensor(lq[r, :n]))
+    np.testing.assert_allclose(z.grad.numpy(), want_g.numpy(), atol=1e-12)
 
 
 def _rand_vocab(rng, n, lo=1, hi=16, alphabet=256):
