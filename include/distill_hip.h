@@ -46,7 +46,8 @@ typedef enum {
                                /* finds a record missing is finished by the second launch (exercises   */
                                /* that path; same results, slower)                                      */
 #define DL_TOPK_PARTS_SHIFT 8  /* bits 8-11: column parts a row of 65537-131072 two-byte (half as many */
-#define DL_TOPK_PARTS(n) ((n) << DL_TOPK_PARTS_SHIFT)   /* four-byte) entries is cut into: 1, 2 or 4;   */
+#define DL_TOPK_PARTS(n) ((n) << DL_TOPK_PARTS_SHIFT)   /* four-byte) entries is cut into: 1, 2 or 4    */
+                               /* (4 only where four parts of 32768 two-byte entries all hold columns); */
                                /* 0 = automatic                                                         */
 
 /* Library ABI revision; bumped when a signature changes. */

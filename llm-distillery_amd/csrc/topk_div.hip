@@ -377,7 +377,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   mx = block_max<NT>(mx, s.red);
   // Second sweep: 2^(x a - max a + bias) takes the place of x in the registers; the gradient is
   // that value times a row constant, so each element costs one exp2, not two.
-  float mb = mx * a;
+  float mb = (mx == -INFINITY) ? 0.f : mx * a;      // a part that holds only -inf logits: every 2^(.) below is 0, not NaN
   const float mb_own = mb - C::stash_bias;
   float sm = 0.f;
 #pragma unroll
@@ -686,13 +686,15 @@ static hipError_t launch_split(TopkParams p, int parts, hipStream_t st) {
 }
 
 // Number of column parts a row of `nch` 16-byte chunks is cut into (1 = one workgroup per row).
-// `forced` (the DL_TOPK_PARTS field of the call's flags): 1 / 2 / 4 override the choice for rows that
-// fit one workgroup of 1024 threads; anything else = automatic.
+// Rows of up to 1024 x 16 chunks are cut into parts of 256 x 16 chunks, as many as hold columns (a
+// part without columns would have no maximum to publish); `forced` (the DL_TOPK_PARTS field of the
+// call's flags) = 1, 2 or 4 overrides that for such rows where every part still gets columns.
 static int split_parts(int64_t nch, int forced) {
   if (nch <= 512 * 16) return 1;
-  if (nch > 1024 * 16) return (int)((nch + 256 * 16 - 1) / (256 * 16));      // 5 .. MAX_PARTS parts of 256 x 16 chunks
-  if (forced == 1 || forced == 2 || forced == 4) return forced;
-  return 4;
+  const int parts = (int)((nch + 256 * 16 - 1) / (256 * 16));      // 3 .. MAX_PARTS parts of 256 x 16 chunks
+  if (nch > 1024 * 16) return parts;
+  if (forced == 1 || forced == 2 || (forced == 4 && parts == 4)) return forced;
+  return parts;
 }
 
 template <class Tag>
@@ -707,7 +709,7 @@ static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes
     const int parts = split_parts(nch, (p.flags >> DL_TOPK_PARTS_SHIFT) & 15);
     const bool ws_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, parts) && p.n_rows * parts <= 0x7fffffffLL;
     if (parts == 2 && ws_ok) return launch_split<Tag, 512, 16>(p, 2, st);
-    if (parts >= 4 && ws_ok) return launch_split<Tag, 256, 16>(p, parts, st);
+    if (parts >= 3 && ws_ok) return launch_split<Tag, 256, 16>(p, parts, st);
     if (nch <= 1024 * 16) return launch_reg<Tag, 1024, 16>(p, st);      // no workspace: one workgroup per row
   }
   if (aligned) {

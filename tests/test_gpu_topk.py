@@ -214,6 +214,35 @@ def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
     assert torch.equal(waited, retried)
 
 
+@pytest.mark.parametrize("V,dtype", [(40000, torch.float32), (70000, torch.bfloat16), (98304, torch.float16), (98312, torch.bfloat16)])
+def test_rows_cut_into_three_parts(D, V, dtype):
+    """Rows of 8193-12288 chunks fill three parts of 4096 chunks, not four: no part may be left
+    without columns."""
+    logits, tv, ti = _case(11, V, 48, dtype, 43, std=3.0)
+    waited = _check(D, "fkl", logits, tv, ti, T=1.1)
+    retried = _check(D, "fkl", logits, tv, ti, T=1.1, hooks={"no_wait": True})
+    forced = _check(D, "fkl", logits, tv, ti, T=1.1, hooks={"parts": 4})      # not honoured here: same launch, same bits
+    assert torch.equal(waited, retried) and torch.equal(waited, forced)
+    _check(D, "fkl", logits, tv, ti, T=1.1, hooks={"parts": 2})
+    _check(D, "fkl", logits, tv, ti, T=1.1, hooks={"parts": 1})
+
+
+def test_a_column_part_that_holds_only_minus_infinity(D):
+    """A masked stretch of the vocabulary (-inf logits) as wide as a whole column part: that part has
+    no finite maximum; its columns get zero gradient and the row's statistics come from the others."""
+    g = torch.Generator().manual_seed(44)
+    R, V, K = 9, 128256, 64
+    logits = torch.randn(R, V, generator=g) * 3
+    logits[:5, 65536:98304] = float("-inf")                   # part 2 of 4, whole
+    logits[5:, 120000:] = float("-inf")                       # the tail of the last part
+    logits = logits.to(torch.bfloat16)
+    tl = torch.log_softmax(logits.float() + torch.randn(R, V, generator=g), -1)
+    tv, ti = torch.topk(tl, K)
+    grad = _check(D, "fkl", logits, tv.to(torch.float16), ti.to(torch.int32), T=1.0)
+    assert torch.count_nonzero(grad[:5, 65536:98304]) == 0 and torch.isfinite(grad.float()).all()
+    _check(D, "fkl", logits, tv.to(torch.float16), ti.to(torch.int32), T=1.0, hooks={"no_wait": True})
+
+
 def test_repeated_ids_on_wide_four_byte_rows(D):
     # 16 chunks of fp32 per thread: the shapes that write their corrections behind the dense stores
     g = torch.Generator().manual_seed(78)
