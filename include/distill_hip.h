@@ -35,7 +35,8 @@ typedef enum {
   DL_ERR_LIMIT = -4,    /* a size exceeds what the kernels support         */
   DL_ERR_LAUNCH = -5,   /* the HIP runtime refused the launch              */
   DL_ERR_ALIGN = -6,    /* a pointer/stride breaks a stated alignment rule */
-  DL_ERR_WORKSPACE = -7 /* a required workspace is too small               */
+  DL_ERR_WORKSPACE = -7, /* a required workspace is too small              */
+  DL_ERR_SCRATCH = -8   /* dl_div_topk_static: the problem needs more scratch than the static array holds */
 } dl_status;
 
 #define DL_MAX_TOPK 2048      /* entries per row a sparse teacher may hold        */
@@ -103,6 +104,29 @@ int dl_div_topk(int kind,
 
 /* Scratch size dl_div_topk can make use of for this problem (0 = none needed).  Host-only. */
 int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V);
+
+/*
+ * dl_div_topk for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, results and kernels as dl_div_topk, without the workspace pair: the scratch of the
+ * split-row kernels lives in a static device array of DL_STATIC_SCRATCH_BYTES that every GPU the
+ * library runs on holds until the process ends.  The call allocates and frees nothing.
+ * Limit: dl_div_topk_workspace_bytes(kind, logits_dtype, n_rows, V) <= DL_STATIC_SCRATCH_BYTES
+ * (e.g. 52428 rows of 65537-131072 two-byte entries; narrower rows need no scratch and have no
+ * limit), else DL_ERR_SCRATCH and nothing is launched.
+ * All calls on one GPU share that GPU's array: calls that may overlap in time on one GPU (two
+ * streams, two threads) race on it and must use dl_div_topk with workspaces of their own.  Calls
+ * in stream order need no care: each call clears the part of the array it uses with a fill
+ * kernel before its main launch.
+ */
+#define DL_STATIC_SCRATCH_BYTES (4 << 20)
+int dl_div_topk_static(int kind,
+                       const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                       const int32_t* row_map,
+                       const void* t_val, int t_val_dtype, const void* t_idx, int t_idx_itype, int K,
+                       int64_t n_teacher_rows, const int32_t* t_cnt,
+                       float inv_T_student, float inv_T_teacher, float grad_scale,
+                       float* row_loss, void* grad, int64_t grad_stride, int flags, void* stream);
 
 /*
  * Forward KL (DL_FKL), reverse KL (DL_RKL) or Jensen-Shannon divergence (DL_JSD) against a dense

@@ -21,6 +21,7 @@ DL_MAX_TEACHERS = 8
 DL_TOPK_UNIQUE_IDS = 1
 DL_TOPK_NO_WAIT = 2
 DL_TOPK_PARTS_SHIFT = 8
+DL_STATIC_SCRATCH_BYTES = 4 << 20
 
 _P = c_void_p
 _SIGNATURES = {
@@ -29,6 +30,8 @@ _SIGNATURES = {
     "dl_div_topk": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, _P, c_int, c_int, c_int64, _P,
                             c_float, c_float, c_float, _P, _P, c_int64, _P, c_int64, c_int, _P]),
     "dl_div_topk_workspace_bytes": (c_int64, [c_int, c_int, c_int64, c_int64]),
+    "dl_div_topk_static": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, _P, c_int, c_int, c_int64, _P,
+                                   c_float, c_float, c_float, _P, _P, c_int64, c_int, _P]),
     "dl_div_dense": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int64, c_int64,
                              c_float, c_float, c_float, _P, _P, c_int64, _P]),
     "dl_rowstats_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int, c_int64, c_float,

@@ -43,6 +43,7 @@ extern "C" const char* dl_status_string(int status) {
     case DL_ERR_LAUNCH: return "the HIP runtime refused the launch";
     case DL_ERR_ALIGN: return "a pointer or stride breaks an alignment rule";
     case DL_ERR_WORKSPACE: return "a required workspace is too small";
+    case DL_ERR_SCRATCH: return "the problem needs more scratch than the static device array holds (use dl_div_topk with a workspace)";
     default: return "unknown status";
   }
 }

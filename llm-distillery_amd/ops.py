@@ -127,6 +127,48 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
     return row_loss, grad
 
 
+def div_topk_static(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor, row_loss: torch.Tensor,
+                    grad: torch.Tensor | None, *, row_map: torch.Tensor | None = None, t_cnt: torch.Tensor | None = None,
+                    T: float = 1.0, teacher_T: float | None = None, grad_scale: float = 1.0, unique_ids: bool = False,
+                    no_wait: bool = False, parts: int = 0) -> None:
+    """`div_topk` for callers that cannot allocate (dl_div_topk_static): the caller brings `row_loss`
+    fp32 [rows] and `grad` like the logits (or None), the split-row scratch is the library's static
+    device array, and neither this wrapper nor the library allocates.  Calls that may overlap in time
+    on one GPU must not use it (they would share the array); limit: DL_STATIC_SCRATCH_BYTES."""
+    if kind not in ("fkl", "rkl"):
+        raise ValueError("kind must be 'fkl' or 'rkl' for a top-K teacher")
+    if parts not in (0, 1, 2, 4):
+        raise ValueError("parts must be 0 (automatic), 1, 2 or 4")
+    _dev(logits, "logits")
+    x = _rows_2d(logits)
+    R, V = x.shape
+    dev = x.device
+    _dev(t_val, "t_val", dev), _dev(t_idx, "t_idx", dev), _dev(row_loss, "row_loss", dev)
+    if x.dtype not in _DT or t_val.dtype not in _DT or t_idx.dtype not in _IT:
+        raise RuntimeError("unsupported dtype")
+    if t_val.dim() != 2 or t_val.shape != t_idx.shape or not (t_val.is_contiguous() and t_idx.is_contiguous()):
+        raise RuntimeError("t_val and t_idx must both be contiguous [N, K]")
+    N, K = t_val.shape
+    if row_map is None and N < R:
+        raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
+    if row_loss.dtype != torch.float32 or row_loss.dim() != 1 or row_loss.numel() != R or not row_loss.is_contiguous():
+        raise RuntimeError(f"row_loss must be a contiguous fp32 vector of {R} entries")
+    _, rm_ptr = _opt_i32(row_map, R, "row_map", dev)
+    _, cnt_ptr = _opt_i32(t_cnt, N, "t_cnt", dev)
+    g_ptr, g_stride = 0, V
+    if grad is not None:
+        g = _grad_target(grad, R, V, x.dtype, dev)
+        g_ptr, g_stride = g.data_ptr(), g.stride(0)
+    flags = (_lib.DL_TOPK_UNIQUE_IDS if unique_ids else 0) | (_lib.DL_TOPK_NO_WAIT if no_wait else 0) | \
+        (parts << _lib.DL_TOPK_PARTS_SHIFT)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_div_topk_static(KINDS[kind], x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr,
+                                            t_val.data_ptr(), _DT[t_val.dtype], t_idx.data_ptr(), _IT[t_idx.dtype], K, N,
+                                            cnt_ptr, 1.0 / T, 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
+                                            row_loss.data_ptr(), g_ptr, g_stride, flags, _stream_ptr(dev))
+    _lib.check(st, "dl_div_topk_static")
+
+
 def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_map: torch.Tensor | None = None,
               T: float = 1.0, teacher_T: float | None = None, grad_scale: float = 1.0, want_grad: bool = True,
               grad_out: torch.Tensor | None = None):
