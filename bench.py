@@ -5,7 +5,7 @@
 One step = one pass of the fused loss + gradient over one batch of synthetic input followed by the
 deterministic mean reduction.  The default workload is the one the headline metric is quoted on
 (C3: 8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200 fp16/int32 teacher, T=1);
-`--workload c1|c2|c4|c5|producer|composite` measures the other configurations and the teacher producer with the
+`--workload c1|c2|c4|c4-merge|c5|producer|composite` measures the other configurations and the teacher producer with the
 same harness.  Inputs are
 resident in HBM before the timed region.  Prints ONE JSON line.
 """
@@ -49,6 +49,25 @@ def _wl_c3(D, S, dev, rows):
 
 
 def _wl_c4(D, S, dev, rows):
+    """dl_fkl_multi_teacher: K-wide preparation (map, weigh, renormalise, bucket per column part) + the loss kernel."""
+    import torch
+    rows = rows or 4 * 8192
+    V, Vt, K = 128256, 152064, 200
+    c = S.config4(dev, rows=rows, V=V, Vt=Vt, K=K)
+    grad = torch.empty_like(c["logits"])
+    scale = 1.0 / rows
+
+    def main():
+        return D.fkl_multi_teacher(c["logits"], c["t_vals"], c["t_idxs"], c["weights"], c["id_map"], T=1.0, grad_scale=scale,
+                                   grad_out=grad, fused=True)[0]
+
+    return (lambda: D.reduce_sum(main(), scale), main, rows * (V * 2 + V * 2 + 3 * K * 6) + Vt * 4, rows,
+            f"C4 3-teacher weighted merge + vocab remap ({Vt}->{V}) + forward-KL fwd+bwd, {rows} tokens, bf16",
+            "fkl_topk_reg_kernel<bf16,256,16,split,bucketed teachers> (4 column parts per row) fed by multi_prep_kernel", c, grad)
+
+
+def _wl_c4_merge(D, S, dev, rows):
+    """The two-launch form of C4: sorted merge through memory (bit-exact id output), then the loss kernel."""
     import torch
     rows = rows or 4 * 8192
     V, Vt, K = 128256, 152064, 200
@@ -70,7 +89,7 @@ def _wl_c4(D, S, dev, rows):
 
     merge()
     return (step, main, rows * (V * 2 + V * 2 + 3 * K * 6) + Vt * 4, rows,
-            f"C4 3-teacher weighted merge + vocab remap ({Vt}->{V}) + forward-KL fwd+bwd, {rows} tokens, bf16",
+            f"C4 in two launches: merge_kernel (3 teachers, remap {Vt}->{V}) feeding the forward-KL kernel, {rows} tokens, bf16",
             "fkl_topk_reg_kernel<bf16,256,16,split> fed by merge_kernel", c, grad)
 
 
@@ -176,7 +195,7 @@ def _wl_composite(D, S, dev, rows):
             "rowstats_kernel + composite epilogue + rowcoef_grad_kernel (two-phase, whole fwd+bwd)", {"logits": logits}, x)
 
 
-WORKLOADS = {"composite": _wl_composite, "producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c5": _wl_c5}
+WORKLOADS = {"composite": _wl_composite, "producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c4-merge": _wl_c4_merge, "c5": _wl_c5}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -193,7 +212,7 @@ def cpu_baseline(workload: str, rows: int, reps: int):
         c = S.config3("cpu", rows=rows, seed=3)
         fn = lambda: O.mean_loss_and_grad("fkl", c["logits"], 1.0, t_vals=c["t_val"], t_idx=c["t_idx"].long())
         what = f"{rows} of 32768 rows at V=128256, K=200"
-    elif workload == "c4":
+    elif workload in ("c4", "c4-merge"):
         c = S.config4("cpu", rows=rows)
         def fn():
             ids, lq, cnt = O.merge_remap_padded([v.numpy() for v in c["t_vals"]], [i.numpy() for i in c["t_idxs"]],
@@ -305,7 +324,7 @@ def main():
     kern_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
     achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
 
-    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048, "composite": 2048}[args.workload]
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c4-merge": 256, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048, "composite": 2048}[args.workload]
     out = {
         "metric": "tokens/sec fused KL fwd+bwd @ vocab 128256 bf16; % of HBM peak GB/s",
         "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,

@@ -70,7 +70,8 @@ const char* dl_status_string(int status);
  *            NULL = identity.
  * t_val      [*, K] stored teacher log-probs (dtype `t_val_dtype`), t_idx [*, K] vocabulary ids
  *            (`t_idx_itype`); both K-contiguous.  t_cnt: optional int32 per teacher row, only the
- *            first t_cnt entries count (NULL = all K).  Ids outside [0, V) are ignored.
+ *            first t_cnt entries count (NULL = all K).  Ids outside [0, V) are ignored, and so are entries
+ *            whose stored log-prob is -inf (zero mass: they do not belong to the teacher's support).
  *            The teacher is renormalised over its counted entries: log_softmax(t_val * inv_T_teacher).
  * row_loss   [n_rows] fp32 per-token divergence (optional, may be NULL).
  * grad       [n_rows, V] (stride `grad_stride`), same dtype as logits; receives
@@ -249,6 +250,42 @@ int dl_merge_remap_topk(int n_teachers, const void* const* t_vals, const void* c
                         int val_dtype, int idx_itype, int K, const float* weights, int64_t n_rows,
                         const int32_t* id_map, int64_t Vt, int64_t Vs,
                         int32_t* out_idx, float* out_logmass, int32_t* out_cnt, void* stream);
+
+/*
+ * Forward KL against the weighted mixture of n_teachers sparse teachers, loss and gradient:
+ * what dl_merge_remap_topk + dl_div_topk(DL_FKL) compute, without the sort and without the merged
+ * row going through memory for every column part (no reference counterpart for weights and id map;
+ * replaces, per training step, what the reference does at collection time in
+ * classes/data_manager.py:231-240 plus utils/finetuning_utils.py:88,91-92,104 and the autograd
+ * replay of classes/losses.py:77-78).
+ * Per row: mass_e = weights[j] * exp(t_vals[j][row, k]); the id goes through id_map (int32 [Vt],
+ * negative = dropped; NULL = identity); ids outside [0, V) are dropped; the teacher distribution is
+ * Q_id = (sum of the masses on id) / (sum of all surviving masses) -- the renormalisation of
+ * dl_div_topk at teacher temperature 1, the only one this entry point offers (for others merge first:
+ * the power 1/T applies to the summed mass of an id).  row_loss = sum_id Q_id (log Q_id - log p_id),
+ * grad = (softmax(logits * inv_T_student) - Q) * inv_T_student * grad_scale.  Sums over the entries of
+ * one id are taken in fixed point: results do not depend on the order the hardware met them in.
+ * Two launches: a K-wide one over the teacher rows (map, weigh, renormalise, deal the entries into
+ * one bucket per column part of the loss kernel's rows, in the workspace), then dl_div_topk's loss
+ * kernels, each workgroup reading only its own bucket.
+ * t_vals / t_idxs / weights are HOST arrays of n_teachers device pointers / non-negative floats;
+ * every teacher holds [n_teacher_rows, K] entries, K-contiguous.  flags: DL_TOPK_NO_WAIT,
+ * DL_TOPK_PARTS as for dl_div_topk.  workspace: at least dl_fkl_multi_teacher_workspace_bytes(...)
+ * bytes (same flags), 256-byte aligned, contents irrelevant on entry and on return; two launches
+ * that may overlap in time need different workspaces.
+ * Limits: n_teachers <= DL_MAX_TEACHERS, n_teachers * K <= DL_MAX_TOPK; rows 16-byte aligned with
+ * V % 8 == 0 (4 for fp32), else DL_ERR_ALIGN; V <= 262144 two-byte / 131072 four-byte columns, else
+ * DL_ERR_LIMIT (dl_fkl_multi_teacher_workspace_bytes then returns 0).  In those cases nothing was
+ * launched: call dl_merge_remap_topk + dl_div_topk.
+ */
+int dl_fkl_multi_teacher(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                         const int32_t* row_map, int n_teachers, const void* const* t_vals,
+                         const void* const* t_idxs, int val_dtype, int idx_itype, int K,
+                         int64_t n_teacher_rows, const float* weights, const int32_t* id_map, int64_t Vt,
+                         float inv_T_student, float grad_scale, float* row_loss, void* grad, int64_t grad_stride,
+                         void* workspace, int64_t workspace_bytes, int flags, void* stream);
+int64_t dl_fkl_multi_teacher_workspace_bytes(int logits_dtype, int64_t n_rows, int64_t V, int n_teachers, int K,
+                                             int64_t n_teacher_rows, int flags);
 
 /*
  * The dataset manager's pairwise merge, classes/data_manager.py:198-261 (merge_topk): exp both

@@ -38,6 +38,9 @@ _SIGNATURES = {
                                  _P, _P, _P]),
     "dl_rowcoef_grad_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int, c_int64, c_float,
                                      _P, _P, _P, _P, c_int64, _P]),
+    "dl_fkl_multi_teacher": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int, _P, _P, c_int, c_int, c_int, c_int64,
+                                     _P, _P, c_int64, c_float, c_float, _P, _P, c_int64, _P, c_int64, c_int, _P]),
+    "dl_fkl_multi_teacher_workspace_bytes": (c_int64, [c_int, c_int64, c_int64, c_int, c_int, c_int64, c_int]),
     "dl_merge_remap_topk": (c_int, [c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, c_int64, c_int64,
                                     _P, _P, _P, _P]),
     "dl_merge_topk_pair": (c_int, [_P, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int64, _P, _P, _P]),

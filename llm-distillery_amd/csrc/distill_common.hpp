@@ -175,11 +175,19 @@ __device__ __forceinline__ void correction_clear(int* head, unsigned* own) {
   own[threadIdx.x] = 0u;
 }
 
+// Index of the list head that serves the chunk holding column `offset` of the part.
+template <class Tag, int NT>
+__device__ __forceinline__ int correction_head_slot(int offset) {
+  const int c = offset / Chunk<Tag>::N;
+  const int owner = c % NT, i = c / NT;
+  return (i % (CORRECTION_HEADS / NT)) * NT + owner;
+}
+
 template <class Tag, int NT>
 __device__ __forceinline__ void correction_link(int* head, unsigned* own, int* next, int k, int offset) {
   const int c = offset / Chunk<Tag>::N;
   const int owner = c % NT, i = c / NT;
-  next[k] = atomicExch(&head[(i % (CORRECTION_HEADS / NT)) * NT + owner], k);
+  next[k] = atomicExch(&head[correction_head_slot<Tag, NT>(offset)], k);
   atomicOr(&own[owner], 1u << (i & 31));
 }
 

@@ -1,743 +1,7 @@
-// Forward / reverse KL against a sparse (top-K) teacher: loss and gradient in one sweep.
-//
-// Forward KL needs the full-vocabulary log-sum-exp of the student row, so the row is pulled
-// into registers with 16-byte non-temporal loads (read from HBM once), reduced, and the gradient
-//     d kl / d logit_j = (softmax(z)_j - sum_k q_k [j == idx_k]) * inv_T * scale
-// is produced from the same registers: a dense softmax sweep, then K sparse corrections after a
-// workgroup barrier.  The K teacher entries (id, log-prob, gathered student logit) live in LDS.
-//
-// A 128256-entry bf16 row is 250 KB, half of a CU's register file, so a workgroup that holds a
-// whole row runs alone on its CU and its load / arithmetic / store phases cannot overlap.  The
-// split kernel therefore cuts a row into P column parts, one workgroup each; several parts of
-// different rows share a CU and hide each other's phases.  The parts of a row exchange their
-// (max, sum-exp, partial loss) through a small workspace in global memory; the wait on the
-// partner is bounded, and a part that gives up recomputes the row statistics on its own.
-//
-// Reverse KL (student renormalised over the K ids) touches only the K gathered logits; its
-// gradient row is a zero fill plus K sparse values.
-//
-// Rows that do not fit (or break the 16-byte alignment rules) take the streaming kernel, which
-// reads the row twice.
-#include "distill_common.hpp"
-#include "distill_hip.h"
-#include <algorithm>
+// dl_div_topk, dl_div_topk_static: forward / reverse KL against one sparse (top-K) teacher.
+// The kernels live in topk_div.hpp.
+#include "topk_div.hpp"
 #include <mutex>
-
-namespace dl {
-
-struct TopkParams {
-  const void* logits; int64_t row_stride; int64_t n_rows; int64_t V;
-  const int32_t* row_map;
-  const void* t_val; int t_val_dtype; const void* t_idx; int t_idx_itype; int K;
-  int64_t n_trows; const int32_t* t_cnt;
-  float inv_T_s, inv_T_t, grad_scale;
-  float* row_loss; void* grad; int64_t grad_stride;
-  void* workspace; int parts; int spin_limit; int flags;
-};
-
-constexpr int MAX_PARTS = 8;
-
-// What one part of a split row tells the others: three floats and a tag that depends on all of
-// them.  The four words are written and read with relaxed device-scope accesses (they bypass the
-// non-coherent cache levels; no cache-wide flush or invalidate); a reader accepts a record only
-// when the tag matches, so no ordering between the words is needed.  A cleared record is invalid.
-struct PartStats { unsigned m, s, b, tag; };
-__device__ __forceinline__ unsigned part_tag(unsigned m, unsigned s, unsigned b) {
-  return m ^ ((s << 7) | (s >> 25)) ^ ((b << 13) | (b >> 19)) ^ 0x5eed1234u;
-}
-__device__ __forceinline__ void part_publish(PartStats* w, float m, float s, float b) {
-  const unsigned um = __float_as_uint(m), us = __float_as_uint(s), ub = __float_as_uint(b);
-  __hip_atomic_store(&w->m, um, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(&w->s, us, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(&w->b, ub, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(&w->tag, part_tag(um, us, ub), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// Bounded wait for a partner's record; false = gave up after `limit` polls.
-__device__ __forceinline__ bool part_collect(PartStats* w, int limit, float& m, float& s, float& b) {
-  for (int spins = 0; spins < limit; ++spins) {
-    const unsigned um = __hip_atomic_load(&w->m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned us = __hip_atomic_load(&w->s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned ub = __hip_atomic_load(&w->b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned ut = __hip_atomic_load(&w->tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (ut == part_tag(um, us, ub)) {
-      m = __uint_as_float(um); s = __uint_as_float(us); b = __uint_as_float(ub);
-      return true;
-    }
-    __builtin_amdgcn_s_sleep(4);
-  }
-  return false;
-}
-
-// Workspace of a split launch: n_rows * parts records, then a counter and the list of (row, part)
-// numbers that gave up waiting for a partner and are finished by a second launch.
-struct RetryList {
-  unsigned* count;
-  unsigned* entries;
-  __host__ __device__ RetryList(void* workspace, int64_t n_rows, int parts) {
-    char* base = reinterpret_cast<char*>(workspace) + n_rows * parts * (int64_t)sizeof(PartStats);
-    count = reinterpret_cast<unsigned*>(base);
-    entries = reinterpret_cast<unsigned*>(base + 16);
-  }
-  __host__ __device__ static int64_t bytes(int64_t n_rows, int parts) {
-    return n_rows * parts * (int64_t)(sizeof(PartStats) + 4) + 16;
-  }
-};
-
-// LDS carve-up shared by the kernels of this file.  The id array is padded to a multiple of 16
-// with -1 so that it can be scanned four ids per read.
-struct TopkLds {
-  float* red;        // reduction scratch, 64 floats
-  float* xm; float* xs; float* xb; int* xok;    // per-part statistics of a split row, MAX_PARTS each
-  int* idx;          // Kp  vocabulary id or -1
-  float* t;          // Kp  scaled teacher logit -> teacher log-probability over the K entries
-  float* q;          // Kp  teacher probability
-  float* z;          // Kp  gathered student logit
-  // in-register corrections (kernels that keep the row in registers; owners == 0 elsewhere):
-  float* val;        // Kp  final gradient value at the entry's column
-  int* next;         // Kp  next entry owned by the same thread, or -1
-  int* head;         // CORRECTION_HEADS list heads: first entry of a chunk's list, or -1
-  unsigned* own;     // one per thread: bit i set = chunk i of the thread holds an entry
-  int Kp;
-  __device__ TopkLds(unsigned char* base, int K, int owners = 0) {
-    Kp = (K + 15) & ~15;
-    red = reinterpret_cast<float*>(base);
-    xm = red + 64; xs = xm + MAX_PARTS; xb = xs + MAX_PARTS; xok = reinterpret_cast<int*>(xb + MAX_PARTS);
-    idx = reinterpret_cast<int*>(base + 512);
-    t = reinterpret_cast<float*>(idx + Kp);
-    q = t + Kp;
-    z = q + Kp;
-    val = z + Kp;
-    next = reinterpret_cast<int*>(val + Kp);
-    head = next + Kp;
-    own = reinterpret_cast<unsigned*>(head + (owners ? CORRECTION_HEADS : 0));
-  }
-  __host__ __device__ static size_t bytes(int K, int owners = 0) {
-    const size_t Kp = (size_t)((K + 15) & ~15);
-    return 512 + Kp * 16 + (owners ? Kp * 8 + (size_t)CORRECTION_HEADS * 4 + (size_t)owners * 4 : 0);
-  }
-};
-
-// Teacher entries of one row held in registers between issue and use: J entries per thread,
-// entry k = tid + j * NT.  Issuing their (tiny) loads before the row's 16 big ones, and the
-// dependent gathers right behind those, keeps three global-memory latencies off the critical path.
-template <int J>
-struct TeacherEntries {
-  int id[J];
-  float tv[J];
-  float z[J];
-};
-
-template <int NT, int J>
-__device__ __forceinline__ void teacher_issue(const TopkParams& p, int64_t trow, TeacherEntries<J>& t) {
-  const int K = p.K;
-  const int cnt = p.t_cnt ? min(p.t_cnt[trow], K) : K;
-#pragma unroll
-  for (int j = 0; j < J; ++j) {
-    const int k = threadIdx.x + j * NT;
-    int64_t id = -1;
-    float v = -INFINITY;
-    if (k < cnt) {
-      const int64_t at = trow * (int64_t)K + k;
-      id = load_index(p.t_idx, p.t_idx_itype, at);
-      v = load_as_float(p.t_val, p.t_val_dtype, at);       // independent of the id: both loads fly together
-    }
-    const bool ok = id >= 0 && id < p.V;
-    t.id[j] = ok ? (int)id : -1;
-    t.tv[j] = ok ? v * p.inv_T_t : -INFINITY;
-  }
-}
-
-template <class Tag, int J>
-__device__ __forceinline__ void teacher_gather(const char* row, int lo, int hi, TeacherEntries<J>& t) {
-#pragma unroll
-  for (int j = 0; j < J; ++j)
-    t.z[j] = (t.id[j] >= lo && t.id[j] < hi) ? load_as_float(row, Tag::id, t.id[j]) : 0.f;
-}
-
-// Registers -> LDS, then the teacher's log-sum-exp; same result layout as stage_teacher.
-template <int NT, int J>
-__device__ __forceinline__ float teacher_finish(const TopkLds& s, const TeacherEntries<J>& t) {
-  float tmax = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < J; ++j) {
-    const int k = threadIdx.x + j * NT;
-    if (k < s.Kp) { s.idx[k] = t.id[j]; s.z[k] = t.z[j]; }
-    tmax = fmaxf(tmax, t.tv[j]);
-  }
-  tmax = block_max<NT>(tmax, s.red);     // barrier inside: LDS entries visible afterwards
-  if (tmax == -INFINITY) return tmax;
-  float part = 0.f;
-#pragma unroll
-  for (int j = 0; j < J; ++j) part += expf(t.tv[j] - tmax);
-  const float tlse = tmax + logf(block_sum<NT>(part, s.red));
-#pragma unroll
-  for (int j = 0; j < J; ++j) {
-    const int k = threadIdx.x + j * NT;
-    if (k < s.Kp) {
-      const float lt = t.tv[j] - tlse;
-      s.t[k] = lt;
-      s.q[k] = expf(lt);
-    }
-  }
-  return tlse;
-}
-
-// Stage the teacher row: ids, scaled log-probs, and the student logits at the ids that fall into
-// the column range [lo, hi) this workgroup owns.  Returns the log-sum-exp of the scaled teacher
-// entries (-inf if the row has none); afterwards s.t holds the teacher log-probabilities and s.q
-// the probabilities (0 for padding and ignored entries).
-template <class Tag, int NT>
-__device__ __forceinline__ float stage_teacher(const TopkParams& p, const TopkLds& s, int64_t trow,
-                                               const char* row, int lo, int hi) {
-  const int K = p.K;
-  const int cnt = p.t_cnt ? min(p.t_cnt[trow], K) : K;
-  float tmax = -INFINITY;
-  for (int k = threadIdx.x; k < s.Kp; k += NT) {
-    const int64_t at = trow * (int64_t)K + k;
-    const int64_t id = k < cnt ? load_index(p.t_idx, p.t_idx_itype, at) : -1;
-    const bool ok = id >= 0 && id < p.V;
-    const float tv = ok ? load_as_float(p.t_val, p.t_val_dtype, at) * p.inv_T_t : -INFINITY;
-    s.idx[k] = ok ? (int)id : -1;
-    s.t[k] = tv;
-    s.z[k] = (ok && id >= lo && id < hi) ? load_as_float(row, Tag::id, id) : 0.f;
-    tmax = fmaxf(tmax, tv);
-  }
-  tmax = block_max<NT>(tmax, s.red);     // barrier inside: LDS entries visible afterwards
-  if (tmax == -INFINITY) return tmax;
-  float part = 0.f;
-  for (int k = threadIdx.x; k < s.Kp; k += NT) part += expf(s.t[k] - tmax);
-  const float tlse = tmax + logf(block_sum<NT>(part, s.red));
-  for (int k = threadIdx.x; k < s.Kp; k += NT) {      // own entries only: no barrier needed yet
-    const float lt = s.t[k] - tlse;
-    s.t[k] = lt;
-    s.q[k] = expf(lt);
-  }
-  return tlse;
-}
-
-// Partial forward-KL sums over the ids inside [lo, hi):  B = sum q_k (t_k - z_k * inv_T)  and, over
-// all ids, Q = sum q_k.  The row value is  sum over parts of B  +  lse * Q.
-template <int NT>
-__device__ __forceinline__ void fkl_partials(const TopkParams& p, const TopkLds& s, int lo, int hi, float& B,
-                                             float& Q) {
-  B = 0.f; Q = 0.f;
-  for (int k = threadIdx.x; k < s.Kp; k += NT) {
-    const int id = s.idx[k];
-    if (id >= 0) {
-      const float q = s.q[k];
-      Q += q;
-      if (id >= lo && id < hi) B += q * (s.t[k] - s.z[k] * p.inv_T_s);
-    }
-  }
-  block_sum2<NT>(B, Q, s.red);
-}
-
-// Teacher mass on the id of entry k, summed over every entry that carries the same id.
-__device__ __forceinline__ float mass_on_id(const TopkLds& s, int k, int id) {
-  int same = 0;
-  const int4* ids = reinterpret_cast<const int4*>(s.idx);
-#pragma unroll 4
-  for (int j = 0; j < s.Kp / 4; ++j) {
-    const int4 v = ids[j];
-    same += (v.x == id) + (v.y == id) + (v.z == id) + (v.w == id);
-  }
-  if (same == 1) return s.q[k];
-  float q = 0.f;                        // duplicates inside a row are rare: slow path
-  for (int j = 0; j < s.Kp; ++j) q += (s.idx[j] == id) ? s.q[j] : 0.f;
-  return q;
-}
-
-// Sparse corrections of the dense softmax row already written by this workgroup, for the ids
-// inside [lo, hi).  b is the row's log2-sum-exp2, a = inv_T * log2(e), c = inv_T * scale.
-template <class Tag, int NT>
-__device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int lo, int hi,
-                                               float a, float b, float c, bool ids_unique) {
-  for (int k = threadIdx.x; k < s.Kp; k += NT) {
-    const int id = s.idx[k];
-    if (id < lo || id >= hi) continue;
-    const float q = ids_unique ? s.q[k] : mass_on_id(s, k, id);
-    store_from_float(grow, Tag::id, id, (fast_exp2(fmaf(s.z[k], a, -b)) - q) * c);
-  }
-}
-
-// The same corrections for a row (part) held in registers, applied by the threads that hold the
-// columns before they store them (correction_link / correction_apply).  Entry threads leave the
-// student probability at the entry's column in s.val and link the entry into its owner's list; the
-// owner subtracts the teacher mass -- of all entries of that column, should ids repeat, which it
-// sees from the chunk's list: no scan over the row's ids.
-template <class Tag, int NT>
-__device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, int hi, float a, float b) {
-  for (int k = threadIdx.x; k < s.Kp; k += NT) {
-    const int id = s.idx[k];
-    if (id < lo || id >= hi) continue;
-    s.val[k] = fast_exp2(fmaf(s.z[k], a, -b));
-    correction_link<Tag, NT>(s.head, s.own, s.next, k, id - lo);
-  }
-}
-
-// Full-row statistics straight from global memory (two uses: the streaming kernel, and a split
-// part whose partner did not answer in time).  Returns the row maximum and sum 2^((x - max) a).
-template <class Tag, int NT, bool VEC>
-__device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, float a, float* red, float& mx,
-                                                   float& sm) {
-  using C = Chunk<Tag>;
-  float m = -INFINITY;
-  sm = 0.f;
-  if (VEC) {
-    for (int64_t ch = threadIdx.x; ch < V / C::N; ch += NT) {
-      float f[C::N];
-      C::unpack(*reinterpret_cast<const u32x4*>(row + ch * 16), f);
-      float cm = f[0];
-#pragma unroll
-      for (int e = 1; e < C::N; ++e) cm = fmaxf(cm, f[e]);
-      if (cm > m) { sm *= fast_exp2((m - cm) * a); m = cm; }
-      const float mb = m * a;
-#pragma unroll
-      for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[e], a, -mb));
-    }
-  } else {
-    for (int64_t j = threadIdx.x; j < V; j += NT) {
-      const float f = load_as_float(row, Tag::id, j);
-      if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
-      sm += fast_exp2(fmaf(f, a, -m * a));
-    }
-  }
-  mx = block_max<NT>(m, red);
-  sm = (m == -INFINITY) ? 0.f : sm * fast_exp2((m - mx) * a);
-  sm = block_sum<NT>(sm, red);
-}
-
-// ---------------------------------------------------------------------------------------
-// Forward KL, (part of) a row resident in registers: NT threads x NCH 16-byte chunks per thread.
-// SPLIT: P = p.parts workgroups per row.  Consecutive workgroup ids are dealt round-robin to the 8
-// XCDs, each of which dispatches its share in order, so the parts of a row are placed 8 ids apart:
-// they land on the same XCD back to back (partners start together and meet through one L2).
-// Within a group of 8*P ids, id t serves row 8*group + t % 8, part t / 8.
-// ---------------------------------------------------------------------------------------
-// J > 0: the K <= J * NT teacher entries travel in registers (loads issued ahead of the row's);
-// J == 0: any K, staged by a plain loop.
-// RETRY: second launch over the parts that gave up waiting in the first (see split_retry_list):
-// every record of the row is published by then, so nothing is waited for.
-template <class Tag, int NT, int NCH, bool SPLIT, int J, bool RETRY>
-__device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds& s, int64_t r, int h) {
-  using C = Chunk<Tag>;
-  const int tid = threadIdx.x;
-  const int P = SPLIT ? p.parts : 1;
-  const int64_t c0 = (int64_t)h * NT * NCH;                       // first chunk of this part
-  const int64_t nch = min((int64_t)NT * NCH, p.V / C::N - c0);    // chunks of this part
-  const int lo = (int)(c0 * C::N), hi = lo + (int)(nch * C::N);   // its column range
-  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
-  char* gpart = grow ? grow + c0 * 16 : nullptr;
-  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
-  if (trow < 0) {
-    if (gpart) zero_row<Tag, NT>(gpart, nch);
-    if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
-    return;
-  }
-  const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
-  const char* rpart = row + c0 * 16;
-
-  correction_clear<NT>(s.head, s.own);      // lists of corrections, filled after the row statistics
-  TeacherEntries<(J > 0 ? J : 1)> te;
-  if constexpr (J > 0) teacher_issue<NT, J>(p, trow, te);
-  u32x4 reg[NCH];
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int64_t c = (int64_t)i * NT + tid;
-    // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
-    // finds its lines in L2 instead of fetching them a second time (0.47 GB less per 32768 rows of K = 200)
-    reg[i] = c < nch ? *reinterpret_cast<const u32x4*>(rpart + c * 16) : C::neg_inf();
-  }
-
-  // teacher side while the row is in flight
-  float tlse;
-  if constexpr (J > 0) {
-    teacher_gather<Tag, J>(row, lo, hi, te);
-    tlse = teacher_finish<NT, J>(s, te);
-  } else {
-    tlse = stage_teacher<Tag, NT>(p, s, trow, row, lo, hi);
-  }
-  if (tlse == -INFINITY) {            // no usable teacher entry: the row contributes nothing
-    if (gpart) zero_row<Tag, NT>(gpart, nch);
-    if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
-    return;
-  }
-  float B, Q;
-  fkl_partials<NT>(p, s, lo, hi, B, Q);
-
-  const float a = p.inv_T_s * LOG2E;
-  float mx = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    float f[C::N];
-    forget(reg[i]);
-    C::unpack(reg[i], f);
-#pragma unroll
-    for (int e = 0; e < C::N; ++e) mx = fmaxf(mx, f[e]);
-  }
-  mx = block_max<NT>(mx, s.red);
-  // Second sweep: 2^(x a - max a + bias) takes the place of x in the registers; the gradient is
-  // that value times a row constant, so each element costs one exp2, not two.
-  float mb = (mx == -INFINITY) ? 0.f : mx * a;      // a part that holds only -inf logits: every 2^(.) below is 0, not NaN
-  const float mb_own = mb - C::stash_bias;
-  float sm = 0.f;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    float f[C::N];
-    forget(reg[i]);
-    C::unpack(reg[i], f);
-#pragma unroll
-    for (int e = 0; e < C::N; ++e) {
-      f[e] = fast_exp2(fmaf(f[e], a, -mb_own));
-      sm += f[e];
-    }
-    reg[i] = C::stash(f);
-    forget(reg[i]);         // pins the schedule chunk by chunk: no pile-up of unpacked values
-  }
-  sm = block_sum<NT>(sm * __builtin_exp2f(-C::stash_bias), s.red);      // exact: a power of two
-
-  if (SPLIT) {
-    // publish this part's statistics, collect the others'
-    PartStats* ws = reinterpret_cast<PartStats*>(p.workspace) + r * P;
-    if (tid == 0 && !RETRY) part_publish(ws + h, mx, sm, B);
-    if (tid < P) {
-      float om = mx, os = sm, ob = B;
-      const int ok = (tid == h) || part_collect(ws + tid, RETRY ? 0x7fffffff : p.spin_limit, om, os, ob);
-      s.xm[tid] = om; s.xs[tid] = os; s.xb[tid] = ob; s.xok[tid] = ok;
-    }
-    __syncthreads();
-    bool all_ok = true;
-    for (int j = 0; j < P; ++j) all_ok = all_ok && (s.xok[j] != 0);
-    if (!all_ok) {
-      // A partner did not answer in time.  Nothing has been written yet: this part puts itself on
-      // the retry list and leaves; its own record is published, so the partners can finish.
-      if (tid == 0) {
-        RetryList list(p.workspace, p.n_rows, P);
-        list.entries[atomicAdd(list.count, 1u)] = (unsigned)(r * P + h);
-      }
-      return;
-    }
-    float M = s.xm[0];
-    for (int j = 1; j < P; ++j) M = fmaxf(M, s.xm[j]);
-    float S = 0.f, Bt = 0.f;
-    for (int j = 0; j < P; ++j) { S += s.xs[j] * fast_exp2((s.xm[j] - M) * a); Bt += s.xb[j]; }
-    mb = M * a; sm = S; B = Bt;
-  }
-  const float b = mb + fast_log2(sm);      // log2-sum-exp2 of the scaled row
-  if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = B + (b * LN2) * Q;
-
-  if (gpart) {
-    const float c = p.inv_T_s * p.grad_scale;
-    const float kc = fast_exp2(mb_own - b) * c;       // stashed value -> gradient
-    // 16 chunks of 4-byte logits leave no registers for placing the corrections during the sweep
-    // (it spills): those shapes write them behind the dense stores instead.
-    constexpr bool IN_REGISTERS = !(Tag::bytes == 4 && NCH == 16);
-    if (IN_REGISTERS) {
-      fkl_link_corrections<Tag, NT>(s, lo, hi, a, b);
-      __syncthreads();
-    }
-    const unsigned mine = IN_REGISTERS ? s.own[tid] : 0u;
-    const bool may_repeat = (p.flags & DL_TOPK_UNIQUE_IDS) == 0;
-    const auto mass = [&](int k) { return s.q[k]; };
-    const auto value = [&](int k, float q) { return (s.val[k] - q) * c; };
-    unsigned repeats = 0u;            // chunks in which an id occurs more than once
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int64_t ch = (int64_t)i * NT + tid;
-      if (ch < nch) {
-        float f[C::N];
-        forget(reg[i]);
-        C::unstash(reg[i], f);
-#pragma unroll
-        for (int e = 0; e < C::N; ++e) f[e] *= kc;
-        if (mine & (1u << i))
-          if (correction_apply<Tag, NT>(s.head, s.next, s.idx, lo, i, f, mass, value)) repeats |= 1u << i;
-        store16_stream(gpart + ch * 16, C::pack(f));
-      }
-    }
-    if (may_repeat && repeats)
-      correction_repeats<Tag, NT>(s.head, s.next, s.idx, lo, repeats, NCH, mass, value,
-                                  [&](int column, float v) { store_from_float(grow, Tag::id, column, v); });
-    if (!IN_REGISTERS) {
-      __syncthreads();      // dense stores are ordered before the sparse corrections
-      fkl_sparse_fix<Tag, NT>(s, grow, lo, hi, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
-    }
-  }
-}
-
-template <class Tag, int NT, int NCH, bool SPLIT, int J>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
-void fkl_topk_reg_kernel(const TopkParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K, NT);
-  const int P = SPLIT ? p.parts : 1;
-  const unsigned grp = SPLIT ? blockIdx.x / (8u * P) : 0u, t_in = SPLIT ? blockIdx.x % (8u * P) : 0u;
-  const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : xcd_banded_row(blockIdx.x);
-  const int h = SPLIT ? (int)(t_in >> 3) : 0;
-  if (r >= p.n_rows) return;
-  fkl_topk_part<Tag, NT, NCH, SPLIT, J, false>(p, s, r, h);
-}
-
-// One listed part, as a real call: the loop around it then costs the body no registers.
-template <class Tag, int NT, int NCH, int J>
-__device__ __attribute__((noinline)) void fkl_topk_part_again(const TopkParams& p, const TopkLds& s, unsigned at) {
-  fkl_topk_part<Tag, NT, NCH, true, J, true>(p, s, (int64_t)(at / (unsigned)p.parts), (int)(at % (unsigned)p.parts));
-}
-
-// The parts on the retry list, a fixed grid striding over it (normally the list is empty and
-// every workgroup leaves after one load).
-template <class Tag, int NT, int NCH, int J>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
-void fkl_topk_retry_kernel(const TopkParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K, NT);
-  const RetryList list(p.workspace, p.n_rows, p.parts);
-  const unsigned n = *list.count;
-#pragma unroll 1
-  for (unsigned e = blockIdx.x; e < n; e += gridDim.x) {
-    fkl_topk_part_again<Tag, NT, NCH, J>(p, s, list.entries[e]);
-    __syncthreads();      // LDS is reused by the next entry
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// Forward KL, streaming: any V, any alignment; the row is read twice (second read mostly L2 / MALL).
-// ---------------------------------------------------------------------------------------
-template <class Tag, int NT, bool VEC>
-__global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K);
-  using C = Chunk<Tag>;
-  const int64_t r = xcd_banded_row(blockIdx.x);
-  if (r >= p.n_rows) return;
-  const int tid = threadIdx.x;
-  const int64_t V = p.V;
-  const int64_t nch = V / C::N;
-  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
-  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
-  const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
-  float tlse = -INFINITY;
-  if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
-  if (tlse == -INFINITY) {
-    if (grow) {
-      if (VEC) zero_row<Tag, NT>(grow, nch);
-      else for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
-    }
-    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
-    return;
-  }
-  float B, Q;
-  fkl_partials<NT>(p, s, 0, (int)V, B, Q);
-  const float a = p.inv_T_s * LOG2E;
-  float mx, sm;
-  row_stats_streamed<Tag, NT, VEC>(row, V, a, s.red, mx, sm);
-  const float b = mx * a + fast_log2(sm);
-  if (tid == 0 && p.row_loss) p.row_loss[r] = B + (b * LN2) * Q;
-
-  if (grow) {
-    const float c = p.inv_T_s * p.grad_scale;
-    if (VEC) {
-      for (int64_t ch = tid; ch < nch; ch += NT) {
-        float f[C::N];
-        C::unpack(*reinterpret_cast<const u32x4*>(row + ch * 16), f);
-#pragma unroll
-        for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * c;
-        store16_stream(grow + ch * 16, C::pack(f));
-      }
-    } else {
-      for (int64_t j = tid; j < V; j += NT)
-        store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * c);
-    }
-    __syncthreads();
-    fkl_sparse_fix<Tag, NT>(s, grow, 0, (int)V, a, b, c, (p.flags & DL_TOPK_UNIQUE_IDS) != 0);
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// Reverse KL on the teacher's support: K gathered logits per row, gradient = zero row + K values.
-// ---------------------------------------------------------------------------------------
-template <class Tag, int NT, bool VEC>
-__global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const TopkLds s(smem, p.K, NT);
-  using C = Chunk<Tag>;
-  const int64_t r = xcd_banded_row(blockIdx.x);
-  if (r >= p.n_rows) return;
-  const int tid = threadIdx.x;
-  const int64_t V = p.V;
-  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
-  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
-  const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
-  correction_clear<NT>(s.head, s.own);
-  float tlse = -INFINITY;
-  if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
-  // Every store comes after the K logits have been gathered (stage_teacher ends in barriers), so
-  // the gradient may be written over the logits.
-  if (grow && (!VEC || tlse == -INFINITY)) {
-    if (VEC) zero_row<Tag, NT>(grow, V / C::N);
-    else for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
-  }
-  if (tlse == -INFINITY) {
-    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
-    return;
-  }
-  // student renormalised over the staged ids
-  float zm = -INFINITY;
-  for (int k = tid; k < s.Kp; k += NT)
-    if (s.idx[k] >= 0) zm = fmaxf(zm, s.z[k] * p.inv_T_s);
-  zm = block_max<NT>(zm, s.red);
-  float part = 0.f;
-  for (int k = tid; k < s.Kp; k += NT)
-    if (s.idx[k] >= 0) part += expf(s.z[k] * p.inv_T_s - zm);
-  const float slse = zm + logf(block_sum<NT>(part, s.red));
-  part = 0.f;
-  for (int k = tid; k < s.Kp; k += NT) {
-    if (s.idx[k] >= 0) {
-      const float sp = s.z[k] * p.inv_T_s - slse;
-      const float d = sp - s.t[k];
-      const float rk = expf(sp);
-      part += rk * d;
-      s.q[k] = rk;      // student mass on the support
-      s.z[k] = d;       // log ratio
-    }
-  }
-  const float rkl = block_sum<NT>(part, s.red);     // barriers inside publish s.t / s.z
-  if (tid == 0 && p.row_loss) p.row_loss[r] = rkl;
-  if (grow) {
-    const float c = p.inv_T_s * p.grad_scale;
-    __syncthreads();    // zero fill precedes the sparse values (scalar path); s.q / s.z complete
-    for (int k = tid; k < s.Kp; k += NT) {
-      const int id = s.idx[k];
-      if (id < 0) continue;
-      if (VEC) {
-        correction_link<Tag, NT>(s.head, s.own, s.next, k, id);     // placed by the thread that writes the column's chunk
-      } else {
-        float g = 0.f;
-        for (int j = 0; j < s.Kp; ++j) g += (s.idx[j] == id) ? s.q[j] * (s.z[j] - rkl) : 0.f;
-        store_from_float(grow, Tag::id, id, g * c);
-      }
-    }
-    if (VEC) {
-      // the row of zeros, each chunk written once with the support's values already in place
-      __syncthreads();
-      const unsigned mine = s.own[tid];
-      const int64_t nch = V / C::N;
-      const auto term = [&](int k) { return s.q[k] * (s.z[k] - rkl); };
-      const auto value = [&](int, float g) { return g * c; };
-      unsigned repeats = 0u;
-      int n_own = 0;
-      for (int64_t ch = tid, i = 0; ch < nch; ch += NT, ++i) {
-        float f[C::N];
-#pragma unroll
-        for (int e = 0; e < C::N; ++e) f[e] = 0.f;
-        if (mine & (1u << (i & 31)))
-          if (correction_apply<Tag, NT>(s.head, s.next, s.idx, 0, (int)i, f, term, value)) repeats |= 1u << (i & 31);
-        store16_stream(grow + ch * 16, C::pack(f));
-        n_own = (int)i + 1;
-      }
-      if (repeats)
-        correction_repeats<Tag, NT>(s.head, s.next, s.idx, 0, repeats, n_own, term, value,
-                                    [&](int column, float v) { store_from_float(grow, Tag::id, column, v); });
-    }
-  }
-}
-
-// clears the `ready` words of the split kernel's workspace
-__global__ __launch_bounds__(256) void clear_workspace_kernel(u32x4* ws, int64_t n16) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n16) ws[i] = u32x4{0u, 0u, 0u, 0u};
-}
-
-// ---------------------------------------------------------------------------------------
-// host dispatch
-// ---------------------------------------------------------------------------------------
-template <class Tag, int NT, int NCH, bool SPLIT>
-static void launch_reg_j(const TopkParams& p, unsigned grid, hipStream_t st) {
-  const int Kp = (p.K + 15) & ~15;
-  const size_t lds = TopkLds::bytes(p.K, NT);
-  if (Kp <= NT) hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 1>), dim3(grid), dim3(NT), lds, st, p);
-  else if (Kp <= 3 * NT) hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 3>), dim3(grid), dim3(NT), lds, st, p);
-  else hipLaunchKernelGGL((fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, 0>), dim3(grid), dim3(NT), lds, st, p);
-}
-
-template <class Tag, int NT, int NCH>
-static void launch_retry_j(const TopkParams& p, unsigned grid, hipStream_t st) {
-  const int Kp = (p.K + 15) & ~15;
-  const size_t lds = TopkLds::bytes(p.K, NT);
-  if (Kp <= NT) hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 1>), dim3(grid), dim3(NT), lds, st, p);
-  else if (Kp <= 3 * NT) hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 3>), dim3(grid), dim3(NT), lds, st, p);
-  else hipLaunchKernelGGL((fkl_topk_retry_kernel<Tag, NT, NCH, 0>), dim3(grid), dim3(NT), lds, st, p);
-}
-
-template <class Tag, int NT, int NCH>
-static hipError_t launch_reg(const TopkParams& p, hipStream_t st) {
-  launch_reg_j<Tag, NT, NCH, false>(p, xcd_banded_grid(p.n_rows), st);
-  return hipGetLastError();
-}
-
-template <class Tag, int NT, int NCH>
-static hipError_t launch_split(TopkParams p, int parts, hipStream_t st) {
-  p.parts = parts;
-  const int64_t n16 = p.n_rows * parts + 1;      // one 16-byte PartStats per (row, part), then the retry counter
-  hipLaunchKernelGGL(clear_workspace_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
-                     reinterpret_cast<u32x4*>(p.workspace), n16);
-  launch_reg_j<Tag, NT, NCH, true>(p, (unsigned)((p.n_rows + 7) / 8 * 8 * parts), st);
-  launch_retry_j<Tag, NT, NCH>(p, (unsigned)std::min<int64_t>(p.n_rows * parts, 256), st);
-  return hipGetLastError();
-}
-
-// Number of column parts a row of `nch` 16-byte chunks is cut into (1 = one workgroup per row).
-// Rows of up to 1024 x 16 chunks are cut into parts of 256 x 16 chunks, as many as hold columns (a
-// part without columns would have no maximum to publish); `forced` (the DL_TOPK_PARTS field of the
-// call's flags) = 1, 2 or 4 overrides that for such rows where every part still gets columns.
-static int split_parts(int64_t nch, int forced) {
-  if (nch <= 512 * 16) return 1;
-  const int parts = (int)((nch + 256 * 16 - 1) / (256 * 16));      // 3 .. MAX_PARTS parts of 256 x 16 chunks
-  if (nch > 1024 * 16) return parts;
-  if (forced == 1 || forced == 2 || (forced == 4 && parts == 4)) return forced;
-  return parts;
-}
-
-template <class Tag>
-static hipError_t launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipStream_t st) {
-  const int64_t nch = p.V / Tag::epc;
-  if (aligned && nch <= (int64_t)MAX_PARTS * 256 * 16) {
-    if (nch <= 256 * 4) return launch_reg<Tag, 256, 4>(p, st);
-    if (nch <= 256 * 8) return launch_reg<Tag, 256, 8>(p, st);
-    // 4-byte logits: 8 chunks per thread from twice the threads keep the corrections in registers
-    if (nch <= 256 * 16) return Tag::bytes == 4 ? launch_reg<Tag, 512, 8>(p, st) : launch_reg<Tag, 256, 16>(p, st);
-    if (nch <= 512 * 16) return launch_reg<Tag, 512, 16>(p, st);
-    const int parts = split_parts(nch, (p.flags >> DL_TOPK_PARTS_SHIFT) & 15);
-    const bool ws_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, parts) && p.n_rows * parts <= 0x7fffffffLL;
-    if (parts == 2 && ws_ok) return launch_split<Tag, 512, 16>(p, 2, st);
-    if (parts >= 3 && ws_ok) return launch_split<Tag, 256, 16>(p, parts, st);
-    if (nch <= 1024 * 16) return launch_reg<Tag, 1024, 16>(p, st);      // no workspace: one workgroup per row
-  }
-  if (aligned) {
-    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
-                       TopkLds::bytes(p.K), st, p);
-  } else {
-    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, false>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
-                       TopkLds::bytes(p.K), st, p);
-  }
-  return hipGetLastError();
-}
-
-template <class Tag>
-static hipError_t launch_rkl(const TopkParams& p, bool aligned, hipStream_t st) {
-  if (aligned)
-    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
-                       TopkLds::bytes(p.K, 256), st, p);
-  else
-    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, false>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
-                       TopkLds::bytes(p.K, 256), st, p);
-  return hipGetLastError();
-}
-
-// Polls a part of a split row waits for its partners' records before it defers itself to the second launch.
-constexpr int SPIN_LIMIT = 20000;
-
-}  // namespace dl
 
 extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V) {
   if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
@@ -772,16 +36,13 @@ static int div_topk_checked(int kind, const void* logits, int logits_dtype, int6
                (reinterpret_cast<uintptr_t>(workspace) % 16 == 0) ? workspace : nullptr, 1,
                (flags & DL_TOPK_NO_WAIT) ? 0 : SPIN_LIMIT, flags};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  hipError_t e;
-  if (kind == DL_FKL) {
-    e = logits_dtype == DL_F32 ? launch_fkl<TagF32>(p, aligned, workspace_bytes, st)
-        : logits_dtype == DL_BF16 ? launch_fkl<TagBF16>(p, aligned, workspace_bytes, st)
-                                  : launch_fkl<TagF16>(p, aligned, workspace_bytes, st);
-  } else {
-    e = logits_dtype == DL_F32 ? launch_rkl<TagF32>(p, aligned, st)
-        : logits_dtype == DL_BF16 ? launch_rkl<TagBF16>(p, aligned, st)
-                                  : launch_rkl<TagF16>(p, aligned, st);
-  }
+  if (kind == DL_FKL)
+    return logits_dtype == DL_F32 ? launch_fkl<TagF32, false>(p, aligned, workspace_bytes, st)
+           : logits_dtype == DL_BF16 ? launch_fkl<TagBF16, false>(p, aligned, workspace_bytes, st)
+                                     : launch_fkl<TagF16, false>(p, aligned, workspace_bytes, st);
+  const hipError_t e = logits_dtype == DL_F32 ? launch_rkl<TagF32>(p, aligned, st)
+                       : logits_dtype == DL_BF16 ? launch_rkl<TagBF16>(p, aligned, st)
+                                                 : launch_rkl<TagF16>(p, aligned, st);
   return e == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 

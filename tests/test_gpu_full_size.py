@@ -82,6 +82,17 @@ def test_config4_full(D):
     np.testing.assert_allclose(rl[sd].cpu().double().numpy(), ref.detach().numpy(), rtol=3e-5, atol=3e-6)
     g = grad[sd].cpu().double() * rows
     assert ((g - z.grad).abs() <= O.storage_tolerance(z.grad, torch.bfloat16, 2e-3)).all()
+    # the bucketed form (no sort; the loss kernel's workgroups read their own share of the entries) on the same input
+    rl1, grad1 = D.fkl_multi_teacher(c["logits"], c["t_vals"], c["t_idxs"], c["weights"], c["id_map"], grad_scale=1.0 / rows,
+                                     fused=True)
+    assert _row_sums(grad1).abs().max().item() * rows < 2e-2
+    np.testing.assert_allclose(rl1[sd].cpu().double().numpy(), ref.detach().numpy(), rtol=3e-5, atol=3e-6)
+    np.testing.assert_allclose(rl1.cpu().numpy(), rl.cpu().numpy(), rtol=3e-5, atol=3e-6)
+    g1 = grad1[sd].cpu().double() * rows
+    assert ((g1 - z.grad).abs() <= O.storage_tolerance(z.grad, torch.bfloat16, 2e-3)).all()
+    rl2, grad2 = D.fkl_multi_teacher(c["logits"], c["t_vals"], c["t_idxs"], c["weights"], c["id_map"], grad_scale=1.0 / rows,
+                                     fused=True)
+    assert torch.equal(rl1, rl2) and torch.equal(grad1, grad2)              # bit-reproducible
 
 
 def test_config1_and_config2_full(D):

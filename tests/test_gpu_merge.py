@@ -116,6 +116,140 @@ def test_fused_multi_teacher_loss_against_oracle(D):
     assert np.allclose(np.exp(lq.astype(np.float64)).sum(-1)[cnt > 0], 1.0, atol=1e-5)
 
 
+def _oracle_multi(logits, vals, idxs, weights, id_map, T, valid=None):
+    """Loss rows and gradient of the mixture against the dict/loop merge + the pinned ragged forward KL."""
+    V = logits.shape[1]
+    ids, lq, cnt = O.merge_remap_padded([v.float().numpy() for v in vals], [i.numpy() for i in idxs], weights,
+                                        None if id_map is None else id_map.numpy(), 1.0, n_student=V)
+    sel = torch.arange(logits.shape[0]) if valid is None else torch.nonzero(valid).squeeze(-1)
+    z = (logits[sel].double() / T).requires_grad_(True)
+    rows = O.fwd_kl_sparse_rows(z, ids, lq.astype(np.float64), cnt)
+    rows.sum().backward()
+    grad = torch.zeros(logits.shape, dtype=torch.float64)
+    grad[sel] = z.grad / T
+    return rows.detach(), grad, cnt
+
+
+@pytest.mark.parametrize("V,dtype,n,K,Vt,T", [
+    (128256, torch.bfloat16, 3, 200, 152064, 1.0),      # rows cut into 4 parts, 3 slots of 256 entries
+    (32000, torch.bfloat16, 3, 200, 40000, 2.0),        # one workgroup per row
+    (2048, torch.float16, 2, 100, 3000, 1.0),           # narrowest shape
+    (40000, torch.float32, 2, 400, 50000, 1.3),         # 3 parts of fp32 (corrections behind the dense stores), 2 slots per teacher
+    (16000, torch.float32, 3, 200, 20000, 1.0),         # 512 threads x 8 chunks
+    (152064, torch.float16, 1, 200, 152064, 1.0),       # a single teacher through the map, 5 parts
+    (65536, torch.bfloat16, 4, 128, 70000, 0.7),        # 512 x 16, one workgroup per row
+    (100000, torch.bfloat16, 8, 64, 120000, 1.0),       # 8 teachers: 8 slots
+])
+def test_bucketed_multi_teacher_against_oracle(D, V, dtype, n, K, Vt, T):
+    """dl_fkl_multi_teacher (entries mapped, renormalised and dealt into per-part buckets by a K-wide
+    launch, shared ids summed inside the loss kernel) against the dict/loop merge + ragged forward KL
+    of the oracle, and against the sorting form of the library, with masked rows; waiting and
+    deferred parts give the same bits."""
+    g = torch.Generator().manual_seed(V + n)
+    R = 14
+    logits = (torch.randn(R, V, generator=g) * 3).to(dtype)
+    valid = torch.ones(R, dtype=torch.bool)
+    valid[[1, 9]] = False
+    nv = int(valid.sum())
+    vals, idxs = _teachers(nv, K, Vt, n, V + 1)
+    weights = [0.5, 0.3, 0.2, 0.1, 0.25, 0.05, 0.4, 0.15][:n]
+    id_map = torch.randint(0, V, (Vt,), generator=g, dtype=torch.int32)
+    id_map[torch.rand(Vt, generator=g) < 0.05] = -1
+    id_map[idxs[0][0, :40].long()] = 7                      # forty entries of one row land on one student id
+    if n > 1:
+        id_map[idxs[1][2, :3].long()] = id_map[idxs[0][2, :3].long()]
+    rm = torch.full((R,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(nv, dtype=torch.int32)
+    args = (logits.to(DEV), [v.to(DEV) for v in vals], [i.to(DEV) for i in idxs], weights, id_map.to(DEV))
+    rl, grad = D.fkl_multi_teacher(*args, row_map=rm.to(DEV), T=T, teacher_T=1.0, grad_scale=1.0 / nv, fused=True)
+    rows64, grad64, cnt = _oracle_multi(logits, vals, idxs, weights, id_map, T, valid)
+    assert (cnt > 0).all()
+    np.testing.assert_allclose(D.reduce_sum(rl, 1.0 / nv).item(), rows64.mean().item(), rtol=1e-5)
+    np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+    assert torch.count_nonzero(rl.cpu()[~valid]) == 0 and torch.count_nonzero(grad.cpu()[~valid]) == 0
+    grad64 = grad64 / nv                                    # the scale the kernel stored its gradient with
+    err = (grad.cpu().double() - grad64).abs()
+    bound = O.storage_tolerance(grad64, dtype, 1e-4 if dtype == torch.float32 else 2e-3)
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+    rl2, grad2 = D.fkl_multi_teacher(*args, row_map=rm.to(DEV), T=T, teacher_T=1.0, grad_scale=1.0 / nv, fused=True, no_wait=True)
+    assert torch.equal(rl, rl2) and torch.equal(grad, grad2)
+    # the two-launch form (sorted merge through memory, then the loss kernel) agrees to rounding
+    rl3, grad3 = D.fkl_multi_teacher(*args, row_map=rm.to(DEV), T=T, teacher_T=1.0, grad_scale=1.0 / nv, fused=False)
+    np.testing.assert_allclose(rl.cpu().numpy(), rl3.cpu().numpy(), rtol=2e-5, atol=2e-6)
+    assert ((grad3.cpu().double() - grad64).abs() <= bound).all()
+
+
+def test_bucketed_multi_teacher_edge_rows(D):
+    """Rows whose entries are all dropped (loss 0, zero gradient), a teacher of weight 0, ids outside
+    the teacher vocabulary, int64 ids with fp32 values, no map at all."""
+    g = torch.Generator().manual_seed(91)
+    R, V, Vt, K = 6, 4096, 6000, 48
+    logits = torch.randn(R, V, generator=g) * 2
+    vals, idxs = _teachers(R, K, Vt, 3, 92, idx_dtype=torch.int64, val_dtype=torch.float32)
+    id_map = torch.randint(0, V, (Vt,), generator=g, dtype=torch.int32)
+    for i in idxs:
+        id_map[i[1].long()] = -1                              # row 1: nothing survives
+    idxs[0][3, :5] = Vt + 11                                  # outside the map: dropped
+    idxs[1][3, 5] = -4
+    weights = [0.7, 0.0, 0.3]
+    rl, grad = D.fkl_multi_teacher(logits.to(DEV), [v.to(DEV) for v in vals], [i.to(DEV) for i in idxs], weights,
+                                   id_map.to(DEV), fused=True)
+    assert rl[1].item() == 0 and torch.count_nonzero(grad[1]) == 0
+    rows64, grad64, cnt = _oracle_multi(logits, [vals[0], vals[2]], [idxs[0], idxs[2]], [0.7, 0.3], id_map, 1.0)
+    assert cnt[1] == 0
+    np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+    assert ((grad.cpu().double() - grad64).abs() <= O.storage_tolerance(grad64, torch.float32, 1e-4)).all()
+    # same vocabulary, no map: ids collide only where two teachers chose the same token
+    small = [i.clamp(0, V - 1) for i in idxs]
+    rl, grad = D.fkl_multi_teacher(logits.to(DEV), [v.to(DEV) for v in vals], [i.to(DEV) for i in small], [1.0, 1.0, 1.0], None,
+                                   fused=True)
+    rows64, grad64, _ = _oracle_multi(logits, vals, small, [1.0, 1.0, 1.0], None, 1.0)
+    np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+    assert ((grad.cpu().double() - grad64).abs() <= O.storage_tolerance(grad64, torch.float32, 1e-4)).all()
+
+
+def test_bucketed_multi_teacher_crowded_buckets_and_many_entries(D):
+    """Every entry of a row inside one column part (its bucket overflows the slots laid out for an
+    even share), 7 teachers x 290 entries, the largest entry count the library takes."""
+    g = torch.Generator().manual_seed(94)
+    R, V, Vt = 6, 128256, 140000
+    logits = (torch.randn(R, V, generator=g) * 3).to(torch.bfloat16)
+    for n, K in ((3, 200), (7, 290), (8, 256)):
+        vals, idxs = _teachers(R, K, Vt, n, 95 + n)
+        id_map = torch.randint(0, V, (Vt,), generator=g, dtype=torch.int32)
+        crowd = torch.randint(70000, 75000, (Vt,), generator=g, dtype=torch.int32)      # part 2 of 4, many shared ids
+        for i in idxs:
+            id_map[i[1].long()] = crowd[i[1].long()]
+            id_map[i[4].long()] = crowd[i[4].long()] % 16 + 98300                       # sixteen ids astride the boundary of parts 2 and 3
+        weights = [1.0 / (j + 1) for j in range(n)]
+        args = (logits.to(DEV), [v.to(DEV) for v in vals], [i.to(DEV) for i in idxs], weights, id_map.to(DEV))
+        rl, grad = D.fkl_multi_teacher(*args, fused=True)
+        rows64, grad64, _ = _oracle_multi(logits, vals, idxs, weights, id_map, 1.0)
+        np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+        err = (grad.cpu().double() - grad64).abs()
+        bound = O.storage_tolerance(grad64, torch.bfloat16, 2e-3)
+        assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+        rl2, grad2 = D.fkl_multi_teacher(*args, fused=True, no_wait=True)
+        assert torch.equal(rl, rl2) and torch.equal(grad, grad2)
+
+
+def test_bucketed_multi_teacher_refuses_what_it_cannot_take(D):
+    vals, idxs = _teachers(4, 32, 5000, 2, 93)
+    x = torch.randn(4, 4096, device=DEV)
+    args = ([v.to(DEV) for v in vals], [i.to(DEV) for i in idxs], [1.0, 1.0], None)
+    with pytest.raises(RuntimeError, match="bucketed"):       # teacher temperature other than 1
+        D.fkl_multi_teacher(x, *args, T=2.0, fused=True)
+    with pytest.raises(RuntimeError, match="bucketed"):       # odd vocabulary
+        D.fkl_multi_teacher(torch.randn(4, 4097, device=DEV), *args, fused=True)
+    rl, _ = D.fkl_multi_teacher(torch.randn(4, 4097, device=DEV), *args)      # automatic: the sorting form
+    assert torch.isfinite(rl).all()
+    with pytest.raises(RuntimeError):
+        D.fkl_multi_teacher(x, *args[:2], [1.0, -0.5], None, fused=True)      # negative weight
+    lib = D._lib.load()
+    assert lib.dl_fkl_multi_teacher_workspace_bytes(1, 64, 128256, 3, 200, 64, 0) > 0
+    assert lib.dl_fkl_multi_teacher_workspace_bytes(1, 64, 300000, 3, 200, 64, 0) == 0      # too wide for the register kernels
+
+
 def test_merge_is_bit_reproducible(D):
     vals, idxs = _teachers(64, 200, 152064, 3, 5)
     m = torch.randint(0, 128256, (152064,), dtype=torch.int32)

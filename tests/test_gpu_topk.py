@@ -243,6 +243,24 @@ def test_a_column_part_that_holds_only_minus_infinity(D):
     _check(D, "fkl", logits, tv.to(torch.float16), ti.to(torch.int32), T=1.0, hooks={"no_wait": True})
 
 
+@pytest.mark.parametrize("kind", ["fkl", "rkl"])
+@pytest.mark.parametrize("V,K", [(4096, 24), (128256, 300), (32000, 900)])
+def test_entries_of_zero_mass_are_no_entries(D, kind, V, K):
+    """A stored log-prob of -inf (a teacher that masks part of its vocabulary) carries no mass: the
+    entry counts neither for the loss nor for the support, exactly as if it were not there."""
+    logits, tv, ti = _case(7, V, K, torch.bfloat16, 51)
+    tv = tv.float()
+    dead = torch.zeros(7, K, dtype=torch.bool)
+    dead[:, 3::4] = True
+    dead[5, 1:] = True                                        # one live entry
+    tv_dead = tv.masked_fill(dead, float("-inf"))
+    rl, g = D.div_topk(kind, logits.to(DEV), tv_dead.to(DEV), ti.to(DEV), T=1.2)
+    # the same rows with the dead entries pointed outside the vocabulary (ignored by contract)
+    ti_out = ti.masked_fill(dead, -1)
+    rl2, g2 = D.div_topk(kind, logits.to(DEV), tv.to(DEV), ti_out.to(DEV), T=1.2)
+    assert torch.isfinite(rl).all() and torch.equal(rl, rl2) and torch.equal(g, g2)
+
+
 def test_repeated_ids_on_wide_four_byte_rows(D):
     # 16 chunks of fp32 per thread: the shapes that write their corrections behind the dense stores
     g = torch.Generator().manual_seed(78)
