@@ -5,7 +5,7 @@
 One step = one pass of the fused loss + gradient over one batch of synthetic input followed by the
 deterministic mean reduction.  The default workload is the one the headline metric is quoted on
 (C3: 8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200 fp16/int32 teacher, T=1);
-`--workload c1|c2|c4|c4-merge|c5|producer|composite` measures the other configurations and the teacher producer with the
+`--workload c1|c2|c4|c4-merge|c5|producer|composite|dropin|dropin-batch` measures the other configurations and the teacher producer with the
 same harness.  Inputs are
 resident in HBM before the timed region.  Prints ONE JSON line.
 """
@@ -195,7 +195,79 @@ def _wl_composite(D, S, dev, rows):
             "rowstats_kernel + composite epilogue + rowcoef_grad_kernel (two-phase, whole fwd+bwd)", {"logits": logits}, x)
 
 
-WORKLOADS = {"composite": _wl_composite, "producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c4-merge": _wl_c4_merge, "c5": _wl_c5}
+def _wl_dropin(batched):
+    """The reference's own call pattern at its default shape (config.json: context_len 2048, crop 32000,
+    save_topK 400, batch 4): per conversation `calculate_divergence` on fp32 logits + `Losses.add_losses`,
+    then one `Losses.backward` for the batch (classes/student/model.py:415-441) -- or, `batched`, the same
+    batch through `distill_loss_batch` + `Losses.add_batch`.  The dominant-kernel figure is the library's
+    launches alone (phase 1, epilogue, its backward, phase 2 per conversation) on preallocated buffers."""
+    def build(D, S, dev, rows):
+        import torch
+        from llm_distillery_amd import ops
+        B, N, V, K, alpha = 4, (rows // 4) if rows else 2048, 32000, 400, 2.0
+        g = torch.Generator(device=dev)
+        g.manual_seed(11)
+        xs, tvs, tis, labs = [], [], [], []
+        for _ in range(B):
+            x = torch.randn(N, V, generator=g, device=dev) * 2
+            tl = torch.log_softmax(x + torch.randn(N, V, generator=g, device=dev), -1)
+            tv, ti = torch.topk(tl, K)
+            xs.append(x.requires_grad_(True)); tvs.append(tv.contiguous()); tis.append(ti.contiguous())
+            labs.append(ti[:-1, 1].contiguous())
+        avoid = torch.tensor([N // 2], dtype=torch.long, device=dev)
+        xb = torch.stack([x.detach() for x in xs]).requires_grad_(True)
+        rows_all = torch.arange(N, device=dev)
+
+        def step():
+            L = D.Losses(None)
+            if batched:
+                xb.grad = None
+                L.add_batch(D.distill_loss_batch(xb, [(rows_all, tvs[i], tis[i], labs[i], avoid) for i in range(B)], alpha))
+            else:
+                for i in range(B):
+                    xs[i].grad = None
+                    L.add_losses(D.calculate_divergence(xs[i], tvs[i], tis[i], labs[i], alpha, avoid))
+            total = L.loss_dict["train_loss"].detach()
+            L.backward(divisor=1)
+            return total
+
+        lib = D._lib.load()
+        bufs = [dict(lse=torch.empty(N, device=dev), zk=torch.empty(N, K, device=dev), rec=torch.empty(N, 8, device=dev),
+                     coef=torch.empty(N, 4, device=dev), out=torch.empty(1, 9, device=dev), g=torch.ones(1, device=dev),
+                     g_lse=torch.empty(N, device=dev), g_zk=torch.empty(N, K, device=dev), grad=torch.empty(N, V, device=dev))
+                for _ in range(B)]
+        import ctypes
+        arr = ctypes.c_int32 * 2
+        offs = (arr(0, N), arr(0, N - 1), arr(0, 1))
+
+        def launches():
+            st = torch.cuda.current_stream().cuda_stream
+            for i in range(B):
+                x, b = xs[i].detach(), bufs[i]
+                lib.dl_rowstats_topk(x.data_ptr(), 0, V, N, V, 0, tis[i].data_ptr(), 1, K, N, 1.0, b["lse"].data_ptr(),
+                                     b["zk"].data_ptr(), st)
+                lib.dl_composite_forward(b["lse"].data_ptr(), b["zk"].data_ptr(), tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
+                                         labs[i].data_ptr(), avoid.data_ptr(), 1, offs[0], offs[1], offs[2], 1, 1, N, alpha,
+                                         b["rec"].data_ptr(), b["coef"].data_ptr(), b["out"].data_ptr(), st)
+            for i in range(B):
+                x, b = xs[i].detach(), bufs[i]
+                lib.dl_composite_backward(b["lse"].data_ptr(), b["zk"].data_ptr(), tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
+                                          offs[0], 1, 1, N, b["rec"].data_ptr(), b["coef"].data_ptr(), b["g"].data_ptr(),
+                                          b["g_lse"].data_ptr(), b["g_zk"].data_ptr(), st)
+                lib.dl_rowcoef_grad_topk(x.data_ptr(), 0, V, N, V, 0, tis[i].data_ptr(), 1, K, N, 1.0, b["lse"].data_ptr(),
+                                         b["g_lse"].data_ptr(), b["g_zk"].data_ptr(), b["grad"].data_ptr(), V, st)
+            return bufs[0]["out"]
+
+        algo = B * (N * V * 4 * 3 + N * K * (4 + 8 + 4 + 4 + 4))
+        return (step, launches, algo, B * N,
+                f"the reference's call pattern at its default shape: {B} conversations x {N} tokens x {V} vocab fp32, K={K}: "
+                + ("distill_loss_batch + Losses.add_batch" if batched else "calculate_divergence + Losses.add_losses per conversation")
+                + " + Losses.backward", "library launches alone: rowstats + composite epilogue + its backward + rowcoef_grad, per conversation",
+                {"logits": xb.detach()}, torch.empty_like(xb))
+    return build
+
+
+WORKLOADS = {"dropin": _wl_dropin(False), "dropin-batch": _wl_dropin(True), "composite": _wl_composite, "producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c4-merge": _wl_c4_merge, "c5": _wl_c5}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -324,12 +396,12 @@ def main():
     kern_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
     achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
 
-    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c4-merge": 256, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048, "composite": 2048}[args.workload]
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c4-merge": 256, "dropin": 0, "dropin-batch": 0, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048, "composite": 2048}[args.workload]
     out = {
         "metric": "tokens/sec fused KL fwd+bwd @ vocab 128256 bf16; % of HBM peak GB/s",
         "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "fp32" if args.workload == "c1" else "bf16", "data": "synthetic",
+        "vs_baseline": None, "dtype": "fp32" if args.workload in ("c1", "dropin", "dropin-batch") else "bf16", "data": "synthetic",
         "config": {"workload": desc, "rows": tokens},
         "loss": loss.item(),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -337,6 +409,8 @@ def main():
                      "kernel": kernel, "kernel_ms": kern_ms, "algorithmic_bytes": algo_bytes},
         "cpu_baseline": cpu_baseline(args.workload, cpu_rows, 7 if args.workload == "c3" else 3) if cpu_rows > 0 else None,
     }
+    if args.workload.startswith("dropin"):
+        out["step_over_launches"] = ms_per_step / kern_ms
     print(json.dumps(out))
 
 

@@ -41,6 +41,7 @@ typedef enum {
 
 #define DL_MAX_TOPK 2048      /* entries per row a sparse teacher may hold        */
 #define DL_MAX_TEACHERS 8     /* teachers merged in one launch                    */
+#define DL_MAX_HOST_CONVOS 64 /* conversations whose offsets may travel with a launch (dl_composite_*) */
 /* dl_div_topk flags (OR them together) */
 #define DL_TOPK_UNIQUE_IDS 1   /* no id occurs twice in a row                                          */
 #define DL_TOPK_NO_WAIT 2      /* parts of a split row never wait for their partners: every part that  */
@@ -184,8 +185,12 @@ int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_strid
  * [label_off[c], label_off[c+1]) of `labels` (row i of the conversation carries label i; the caller
  * guarantees #labels == #rows - 1, the only case the reference's code runs without raising) and
  * entries [avoid_off[c], avoid_off[c+1]) of `avoid` (conversation-local rows excluded from the cross
- * entropy; entries outside [0, #labels) are ignored).  The teacher rows are renormalised over their
- * K entries after scaling by inv_T_teacher.
+ * entropy; entries outside [0, #labels) are ignored; avoid_itype DL_I32 or DL_I64).  The teacher rows
+ * are renormalised over their K entries after scaling by inv_T_teacher.
+ * row_off / label_off / avoid_off: [n_convos + 1] each; DEVICE arrays, or with offsets_on_host != 0
+ * HOST arrays of at most DL_MAX_HOST_CONVOS conversations that are copied into the launch (no upload:
+ * the reference calls its loss once per conversation, classes/student/model.py:415-427; labels /
+ * avoid may then be NULL where a conversation set has none).
  * out [n_convos, 9] in the reference's key order: train_loss, custom loss, CE loss, kl_div,
  * reverse kl_div, weighted kl_div, weighted rev. kl_div, teacher CE loss, CE diff.
  * row_records (32 bytes per row) and row_coef (16 bytes per row, may be NULL when no gradient is
@@ -194,8 +199,8 @@ int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_strid
  */
 int dl_composite_forward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
                          float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
-                         const int64_t* labels, const int32_t* avoid, const int32_t* row_off,
-                         const int32_t* label_off, const int32_t* avoid_off, int n_convos,
+                         const int64_t* labels, const void* avoid, int avoid_itype, const int32_t* row_off,
+                         const int32_t* label_off, const int32_t* avoid_off, int offsets_on_host, int n_convos,
                          int64_t n_rows, float alpha, void* row_records, void* row_coef, float* out,
                          void* stream);
 
@@ -203,12 +208,13 @@ int dl_composite_forward(const float* lse, const float* zk, const void* t_val, i
  * Backward of dl_composite_forward for upstream gradients g_train [n_convos] on each conversation's
  * train_loss: g_lse [n_rows] = dL/dlse and g_zk [n_rows, K] = dL/dzk, the inputs of
  * dl_rowcoef_grad_topk.  Replaces the autograd replay started at classes/losses.py:77-78.
+ * row_off / offsets_on_host as for dl_composite_forward.
  */
 int dl_composite_backward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
                           float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
-                          const int32_t* row_off, int n_convos, int64_t n_rows, const void* row_records,
-                          const void* row_coef, const float* g_train, float* g_lse, float* g_zk,
-                          void* stream);
+                          const int32_t* row_off, int offsets_on_host, int n_convos, int64_t n_rows,
+                          const void* row_records, const void* row_coef, const float* g_train, float* g_lse,
+                          float* g_zk, void* stream);
 
 /*
  * Teacher producer: per selected row, log_softmax over the V (cropped) columns, then the K largest

@@ -18,6 +18,7 @@ DL_I32, DL_I64 = 0, 1
 DL_FKL, DL_RKL, DL_JSD = 0, 1, 2
 DL_MAX_TOPK = 2048
 DL_MAX_TEACHERS = 8
+DL_MAX_HOST_CONVOS = 64
 DL_TOPK_UNIQUE_IDS = 1
 DL_TOPK_NO_WAIT = 2
 DL_TOPK_PARTS_SHIFT = 8
@@ -52,10 +53,10 @@ _SIGNATURES = {
     "dl_marginalise_csr": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int64, _P, c_int64, c_int, _P]),
     "dl_rkl_marginalised": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int64, c_int64, c_int64, _P,
                                     _P, _P, c_int, _P, c_int, c_int, c_float, c_float, c_float, _P, _P, c_int64, _P]),
-    "dl_composite_forward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, _P, _P, _P, _P, c_int, c_int64,
-                                     c_float, _P, _P, _P, _P]),
-    "dl_composite_backward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, c_int, c_int64, _P, _P, _P, _P, _P,
-                                      _P]),
+    "dl_composite_forward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, _P, c_int, _P, _P, _P, c_int, c_int,
+                                     c_int64, c_float, _P, _P, _P, _P]),
+    "dl_composite_backward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, c_int, c_int, c_int64, _P, _P, _P, _P,
+                                      _P, _P]),
     "dl_teacher_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, c_int, _P, c_int, _P, c_int, _P, c_int64, _P]),
     "dl_teacher_topk_workspace_bytes": (c_int64, [c_int, c_int64, c_int64, c_int]),
     "dl_reduce_sum": (c_int, [_P, c_int64, c_float, _P, _P]),

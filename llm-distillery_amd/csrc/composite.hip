@@ -25,12 +25,23 @@ struct RowRec { float kl, rkl, own_s, own_t, t_lse, s_lse; int kstar; int valid;
 // per-row coefficients for a unit upstream gradient on the conversation's train loss
 struct RowCoef { float g_kl, g_rkl, g_own; float pad; };                                  // 16 bytes
 
+// First row / label / ignore entry of every conversation, [C + 1] each: device arrays, or -- for up to
+// DL_MAX_HOST_CONVOS conversations -- copies that travel with the launch (a caller with one
+// conversation, or a handful, then needs no upload of three tiny arrays per call).
+struct ConvoOffsets {
+  const int32_t* dev[3];                          // row, label, avoid; NULL = use `inl`
+  int32_t inl[3][DL_MAX_HOST_CONVOS + 1];
+  __device__ __forceinline__ int row(int c) const { return dev[0] ? dev[0][c] : inl[0][c]; }
+  __device__ __forceinline__ int label(int c) const { return dev[1] ? dev[1][c] : inl[1][c]; }
+  __device__ __forceinline__ int avoid(int c) const { return dev[2] ? dev[2][c] : inl[2][c]; }
+};
+
 struct CompositeParams {
   const float* lse; const float* zk;
   const void* t_val; int t_val_dtype; float inv_T_t;
   const void* t_idx; int t_idx_itype; int K;
-  const int64_t* labels; const int32_t* avoid;
-  const int32_t* row_off; const int32_t* label_off; const int32_t* avoid_off;   // [C + 1] each
+  const int64_t* labels; const void* avoid; int avoid_itype;
+  ConvoOffsets off;
   int n_convos; int64_t n_rows; float alpha;
   RowRec* rec; RowCoef* coef; float* out;         // out [C, 9]
   const float* g_train; float* g_lse; float* g_zk;
@@ -42,17 +53,22 @@ __device__ __forceinline__ int wave_min_int(int v) {
   return v;
 }
 
-// conversation that holds row i: last c with row_off[c] <= i
-__device__ __forceinline__ int convo_of_row(const int32_t* row_off, int n_convos, int64_t i) {
+// conversation that holds row i: last c whose first row is <= i
+__device__ __forceinline__ int convo_of_row(const ConvoOffsets& off, int n_convos, int64_t i) {
   int lo = 0, hi = n_convos - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
-    if (row_off[mid] <= i) lo = mid; else hi = mid - 1;
+    if (off.row(mid) <= i) lo = mid; else hi = mid - 1;
   }
   return lo;
 }
 
 // ---- rows, forward ---------------------------------------------------------------------------------
+// One wave per token row.  R > 0: K <= 64 * R and the storage types are known at compile time: the
+// row's teacher values, ids and gathered logits are fetched once, all loads in flight together, and
+// stay in registers for the three passes (maxima, sums, divergences).  R == 0: any K, any types,
+// three passes over memory.
+template <int VD, int IT, int R>
 __global__ __launch_bounds__(CMP_NT) void composite_rows_fwd_kernel(const CompositeParams p) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int64_t i = (int64_t)blockIdx.x * CMP_ROWS_PER_WG + threadIdx.x / WAVE;
@@ -60,42 +76,87 @@ __global__ __launch_bounds__(CMP_NT) void composite_rows_fwd_kernel(const Compos
   const int K = p.K;
   const float* z = p.zk + i * K;
   const float lse = p.lse[i];
+  constexpr int RR = R > 0 ? R : 1;
+  float tv[RR], zv[RR];
+  int64_t id[RR];
+  if constexpr (R > 0) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int k = lane + j * WAVE;
+      const int64_t at = i * K + (k < K ? k : 0);      // lanes beyond K read entry 0 and discard it: no branch between the loads
+      float t;
+      if constexpr (VD == F32) t = reinterpret_cast<const float*>(p.t_val)[at];
+      else if constexpr (VD == BF16) t = __uint_as_float((unsigned)reinterpret_cast<const unsigned short*>(p.t_val)[at] << 16);
+      else t = (float)reinterpret_cast<const _Float16*>(p.t_val)[at];
+      if constexpr (IT == I32) id[j] = reinterpret_cast<const int32_t*>(p.t_idx)[at];
+      else id[j] = reinterpret_cast<const int64_t*>(p.t_idx)[at];
+      const float zz = z[k < K ? k : 0];
+      tv[j] = k < K ? t * p.inv_T_t : -INFINITY;
+      zv[j] = k < K ? zz : -INFINITY;
+      id[j] = k < K ? id[j] : -1;
+    }
+  }
   // maxima
   float tmax = -INFINITY, zmax = -INFINITY;
-  for (int k = lane; k < K; k += WAVE) {
-    tmax = fmaxf(tmax, load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t);
-    zmax = fmaxf(zmax, z[k]);
+  if constexpr (R > 0) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) { tmax = fmaxf(tmax, tv[j]); zmax = fmaxf(zmax, zv[j]); }
+  } else {
+    for (int k = lane; k < K; k += WAVE) {
+      tmax = fmaxf(tmax, load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t);
+      zmax = fmaxf(zmax, z[k]);
+    }
   }
   tmax = wave_max(tmax);
   zmax = wave_max(zmax);
   float tsum = 0.f, zsum = 0.f;
-  for (int k = lane; k < K; k += WAVE) {
-    tsum += expf(load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t - tmax);
-    zsum += expf(z[k] - zmax);
+  if constexpr (R > 0) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) { tsum += expf(tv[j] - tmax); zsum += expf(zv[j] - zmax); }      // exp(-inf) = 0 beyond K
+  } else {
+    for (int k = lane; k < K; k += WAVE) {
+      tsum += expf(load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t - tmax);
+      zsum += expf(z[k] - zmax);
+    }
   }
   const float t_lse = tmax + logf(wave_sum(tsum));          // teacher renormalised over its K entries
   const float z_lse = zmax + logf(wave_sum(zsum));          // log-sum-exp of the student over the support
   const float s_lse = z_lse - lse;                          // = logsumexp_k(s_k), s_k = z_k - lse
 
   // label of this row, if it has one: conversation-local row li carries label li, for li < #labels
-  const int c = convo_of_row(p.row_off, p.n_convos, i);
-  const int li = (int)(i - p.row_off[c]);
-  const int n_lab = p.label_off[c + 1] - p.label_off[c];
+  const int c = convo_of_row(p.off, p.n_convos, i);
+  const int li = (int)(i - p.off.row(c));
+  const int n_lab = p.off.label(c + 1) - p.off.label(c);
   bool want = li < n_lab;
   int64_t label = -1;
   if (want) {
-    label = p.labels[p.label_off[c] + li];
-    for (int a = p.avoid_off[c]; a < p.avoid_off[c + 1]; ++a) want = want && (p.avoid[a] != li);
+    label = p.labels[p.off.label(c) + li];
+    for (int a = p.off.avoid(c); a < p.off.avoid(c + 1); ++a) want = want && (load_index(p.avoid, p.avoid_itype, a) != li);
   }
   float kl = 0.f, rkl = 0.f;
   int kfound = 0x7fffffff;
-  for (int k = lane; k < K; k += WAVE) {
-    const float t = load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t - t_lse;
-    const float s = z[k] - lse;
-    const float s2 = s - s_lse;
-    kl += expf(t) * (t - s);
-    rkl += expf(s2) * (s2 - t);
-    if (want && load_index(p.t_idx, p.t_idx_itype, i * K + k) == label) kfound = min(kfound, k);
+  if constexpr (R > 0) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int k = lane + j * WAVE;
+      if (k < K) {
+        const float t = tv[j] - t_lse;
+        const float s = zv[j] - lse;
+        const float s2 = s - s_lse;
+        kl += expf(t) * (t - s);
+        rkl += expf(s2) * (s2 - t);
+        if (want && id[j] == label) kfound = min(kfound, k);
+      }
+    }
+  } else {
+    for (int k = lane; k < K; k += WAVE) {
+      const float t = load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t - t_lse;
+      const float s = z[k] - lse;
+      const float s2 = s - s_lse;
+      kl += expf(t) * (t - s);
+      rkl += expf(s2) * (s2 - t);
+      if (want && load_index(p.t_idx, p.t_idx_itype, i * K + k) == label) kfound = min(kfound, k);
+    }
   }
   kl = wave_sum(kl);
   rkl = wave_sum(rkl);
@@ -141,15 +202,27 @@ __device__ __forceinline__ void weight_powers(float x, float alpha, float& pa, f
   else { pa1 = powf(x, alpha - 1.f); pa = powf(x, alpha); }
 }
 
-constexpr int CONVO_NT = 256;
+constexpr int CONVO_NT = 512;
+constexpr int CONVO_R = 4;      // rows per thread kept in registers between the passes: conversations of up to 2048 rows are read once
+
+// f(i, record of row i) for the rows this thread serves: the first CONVO_R of them from registers
+template <class F>
+__device__ __forceinline__ void convo_rows(const RowRec (&mine)[CONVO_R], const RowRec* rec, int n, F f) {
+#pragma unroll
+  for (int j = 0; j < CONVO_R; ++j) {
+    const int i = threadIdx.x + j * CONVO_NT;
+    if (i < n) f(i, mine[j]);
+  }
+  for (int i = threadIdx.x + CONVO_R * CONVO_NT; i < n; i += CONVO_NT) f(i, rec[i]);
+}
 
 __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const CompositeParams p) {
   constexpr int CMP_NT = CONVO_NT;  // (shadows the row kernels' size inside this kernel)
   __shared__ float red[64];
   __shared__ double dred[10 * CMP_NT / WAVE];
   const int c = blockIdx.x, tid = threadIdx.x;
-  const int r0 = p.row_off[c], n = p.row_off[c + 1] - r0;
-  const int m = p.label_off[c + 1] - p.label_off[c];          // labels; the host guarantees m == n - 1
+  const int r0 = p.off.row(c), n = p.off.row(c + 1) - r0;
+  const int m = p.off.label(c + 1) - p.off.label(c);          // labels; the host guarantees m == n - 1
   const RowRec* rec = p.rec + r0;
   float* out = p.out + (int64_t)c * 9;
   if (n <= 0) {
@@ -157,18 +230,23 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
     return;
   }
   const float alpha = p.alpha;
+  RowRec mine[CONVO_R];
+#pragma unroll
+  for (int j = 0; j < CONVO_R; ++j) {
+    const int i = tid + j * CMP_NT;
+    mine[j] = rec[i < n ? i : 0];
+  }
 
   // maxima (with their multiplicity: the gradient of max() is shared evenly among ties), valid sums
   float mk = -INFINITY, mr = -INFINITY;
-  for (int i = tid; i < n; i += CMP_NT) { mk = fmaxf(mk, rec[i].kl); mr = fmaxf(mr, rec[i].rkl); }
+  convo_rows(mine, rec, n, [&](int, const RowRec& r) { mk = fmaxf(mk, r.kl); mr = fmaxf(mr, r.rkl); });
   block_max2<CMP_NT>(mk, mr, red);
   double nv = 0.0, sum_s = 0.0, sum_t = 0.0, tie_k = 0.0, tie_r = 0.0;
-  for (int i = tid; i < n; i += CMP_NT) {
-    const RowRec r = rec[i];
+  convo_rows(mine, rec, n, [&](int i, const RowRec& r) {
     if (i < m && r.valid) { nv += 1.0; sum_s += (double)r.own_s; sum_t += (double)r.own_t; }
     tie_k += r.kl == mk ? 1.0 : 0.0;
     tie_r += r.rkl == mr ? 1.0 : 0.0;
-  }
+  });
   {
     double v[5] = {nv, sum_s, sum_t, tie_k, tie_r};
     block_sums_f64<CMP_NT>(v, dred);
@@ -180,8 +258,7 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
   double a_wkl = 0.0, a_wrkl = 0.0, a_kl = 0.0, a_rkl = 0.0, a_ces = 0.0, a_cet = 0.0, a_d = 0.0;
   double a_gmk = 0.0, a_gmr = 0.0, a_ginv = 0.0;
   const float inv_n = 1.f / (float)n;
-  for (int i = tid; i < n; i += CMP_NT) {
-    const RowRec r = rec[i];
+  convo_rows(mine, rec, n, [&](int i, const RowRec& r) {
     float cpos = 0.f;
     if (i < m) {
       const float ce_s = -(r.valid ? r.own_s : mean_s), ce_t = -(r.valid ? r.own_t : mean_t);
@@ -200,7 +277,7 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
     a_kl += (double)r.kl; a_rkl += (double)r.rkl;
     a_gmk += (double)(r.kl * alpha * pk1 * (-r.kl / (mk * mk)));
     a_gmr += (double)(r.rkl * alpha * pr1 * (-r.rkl / (mr * mr)));
-  }
+  });
   {
     double v[10] = {a_wkl, a_wrkl, a_kl, a_rkl, a_ces, a_cet, a_d, a_gmk, a_gmr, a_ginv};
     block_sums_f64<CMP_NT>(v, dred);
@@ -225,8 +302,7 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
   const float gmk = 0.5f * inv_n * (float)a_gmk / (float)tie_k, gmr = 0.5f * inv_n * (float)a_gmr / (float)tie_r;
   const float ginv_share = (float)(a_ginv / nv);
   RowCoef* coef = p.coef + r0;
-  for (int i = tid; i < n; i += CMP_NT) {
-    const RowRec r = rec[i];
+  convo_rows(mine, rec, n, [&](int i, const RowRec& r) {
     float cpos = 0.f, g_own = 0.f;
     if (i < m) {
       const float d = -(r.valid ? r.own_s : mean_s) + (r.valid ? r.own_t : mean_t);
@@ -246,7 +322,7 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
     o.g_own = g_own;
     o.pad = 0.f;
     coef[i] = o;
-  }
+  });
 }
 
 // ---- rows, backward ----------------------------------------------------------------------------------
@@ -255,7 +331,7 @@ __global__ __launch_bounds__(CMP_NT) void composite_rows_bwd_kernel(const Compos
   const int64_t i = (int64_t)blockIdx.x * CMP_ROWS_PER_WG + threadIdx.x / WAVE;
   if (i >= p.n_rows) return;
   const int K = p.K;
-  const int c = convo_of_row(p.row_off, p.n_convos, i);
+  const int c = convo_of_row(p.off, p.n_convos, i);
   const float up = p.g_train[c];
   const RowRec r = p.rec[i];
   const RowCoef g = p.coef[i];
@@ -279,55 +355,96 @@ __global__ __launch_bounds__(CMP_NT) void composite_rows_bwd_kernel(const Compos
 
 }  // namespace dl
 
+namespace dl {
+template <int VD, int IT>
+static void launch_rows_fwd_k(const CompositeParams& p, hipStream_t st) {
+  const dim3 grid((unsigned)((p.n_rows + CMP_ROWS_PER_WG - 1) / CMP_ROWS_PER_WG)), block(CMP_NT);
+  if (p.K <= 2 * WAVE) hipLaunchKernelGGL((composite_rows_fwd_kernel<VD, IT, 2>), grid, block, 0, st, p);
+  else if (p.K <= 4 * WAVE) hipLaunchKernelGGL((composite_rows_fwd_kernel<VD, IT, 4>), grid, block, 0, st, p);
+  else if (p.K <= 8 * WAVE) hipLaunchKernelGGL((composite_rows_fwd_kernel<VD, IT, 8>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((composite_rows_fwd_kernel<VD, IT, 0>), grid, block, 0, st, p);
+}
+template <int VD>
+static void launch_rows_fwd_v(const CompositeParams& p, hipStream_t st) {
+  if (p.t_idx_itype == DL_I32) launch_rows_fwd_k<VD, I32>(p, st);
+  else launch_rows_fwd_k<VD, I64>(p, st);
+}
+static void launch_rows_fwd(const CompositeParams& p, hipStream_t st) {
+  if (p.t_val_dtype == DL_F32) launch_rows_fwd_v<F32>(p, st);
+  else if (p.t_val_dtype == DL_BF16) launch_rows_fwd_v<BF16>(p, st);
+  else launch_rows_fwd_v<F16>(p, st);
+}
+}  // namespace dl
+
 static int composite_check(const float* lse, const float* zk, const void* t_val, int t_val_dtype, const void* t_idx,
                            int t_idx_itype, int K, const int32_t* row_off, const int32_t* label_off,
-                           const int32_t* avoid_off, int n_convos, int64_t n_rows, const void* rec) {
+                           const int32_t* avoid_off, int offsets_on_host, int n_convos, int64_t n_rows, const void* rec) {
   if (!lse || !zk || !t_val || !t_idx || !row_off || !label_off || !avoid_off || !rec) return DL_ERR_NULL;
   if (t_val_dtype < DL_F32 || t_val_dtype > DL_F16 || (t_idx_itype != DL_I32 && t_idx_itype != DL_I64)) return DL_ERR_DTYPE;
   if (K <= 0 || n_convos <= 0 || n_rows < 0) return DL_ERR_SHAPE;
-  if (n_rows > 0x7fffffffLL) return DL_ERR_LIMIT;
+  if (n_rows > 0x7fffffffLL || (offsets_on_host && n_convos > DL_MAX_HOST_CONVOS)) return DL_ERR_LIMIT;
+  if (offsets_on_host) {
+    // host arrays can be checked here: non-decreasing, rows cover exactly n_rows
+    if (row_off[0] != 0 || row_off[n_convos] != n_rows || label_off[0] < 0 || avoid_off[0] < 0) return DL_ERR_SHAPE;
+    for (int c = 0; c < n_convos; ++c)
+      if (row_off[c + 1] < row_off[c] || label_off[c + 1] < label_off[c] || avoid_off[c + 1] < avoid_off[c]) return DL_ERR_SHAPE;
+  }
   return DL_OK;
+}
+
+static void set_offsets(dl::ConvoOffsets& off, const int32_t* row_off, const int32_t* label_off, const int32_t* avoid_off,
+                        int offsets_on_host, int n_convos) {
+  const int32_t* src[3] = {row_off, label_off, avoid_off};
+  for (int a = 0; a < 3; ++a) {
+    off.dev[a] = offsets_on_host ? nullptr : src[a];
+    if (offsets_on_host)
+      for (int c = 0; c <= n_convos; ++c) off.inl[a][c] = src[a][c];
+  }
 }
 
 extern "C" int dl_composite_forward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
                                     float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
-                                    const int64_t* labels, const int32_t* avoid, const int32_t* row_off,
-                                    const int32_t* label_off, const int32_t* avoid_off, int n_convos,
+                                    const int64_t* labels, const void* avoid, int avoid_itype, const int32_t* row_off,
+                                    const int32_t* label_off, const int32_t* avoid_off, int offsets_on_host, int n_convos,
                                     int64_t n_rows, float alpha, void* row_records, void* row_coef, float* out,
                                     void* stream) {
   using namespace dl;
   const int st0 = composite_check(lse, zk, t_val, t_val_dtype, t_idx, t_idx_itype, K, row_off, label_off, avoid_off,
-                                  n_convos, n_rows, row_records);
+                                  offsets_on_host, n_convos, n_rows, row_records);
   if (st0 != DL_OK) return st0;
-  if (!out || !labels) return DL_ERR_NULL;
+  if (!out) return DL_ERR_NULL;
+  if (avoid_itype != DL_I32 && avoid_itype != DL_I64) return DL_ERR_DTYPE;
+  if (offsets_on_host && ((label_off[n_convos] > label_off[0] && !labels) || (avoid_off[n_convos] > avoid_off[0] && !avoid)))
+    return DL_ERR_NULL;                       // without labels / ignore entries the pointers may be NULL
+  if (!offsets_on_host && (!labels || !avoid)) return DL_ERR_NULL;
   CompositeParams p{};
   p.lse = lse; p.zk = zk; p.t_val = t_val; p.t_val_dtype = t_val_dtype; p.inv_T_t = inv_T_teacher;
-  p.t_idx = t_idx; p.t_idx_itype = t_idx_itype; p.K = K; p.labels = labels; p.avoid = avoid;
-  p.row_off = row_off; p.label_off = label_off; p.avoid_off = avoid_off; p.n_convos = n_convos; p.n_rows = n_rows;
+  p.t_idx = t_idx; p.t_idx_itype = t_idx_itype; p.K = K; p.labels = labels; p.avoid = avoid; p.avoid_itype = avoid_itype;
+  set_offsets(p.off, row_off, label_off, avoid_off, offsets_on_host, n_convos);
+  p.n_convos = n_convos; p.n_rows = n_rows;
   p.alpha = alpha; p.rec = reinterpret_cast<RowRec*>(row_records); p.coef = reinterpret_cast<RowCoef*>(row_coef);
   p.out = out;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (n_rows > 0)
-    hipLaunchKernelGGL(composite_rows_fwd_kernel, dim3((unsigned)((n_rows + CMP_ROWS_PER_WG - 1) / CMP_ROWS_PER_WG)),
-                       dim3(CMP_NT), 0, st, p);
+  if (n_rows > 0) launch_rows_fwd(p, st);
   hipLaunchKernelGGL(composite_convo_kernel, dim3((unsigned)n_convos), dim3(CONVO_NT), 0, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
 extern "C" int dl_composite_backward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
                                      float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
-                                     const int32_t* row_off, int n_convos, int64_t n_rows, const void* row_records,
-                                     const void* row_coef, const float* g_train, float* g_lse, float* g_zk,
-                                     void* stream) {
+                                     const int32_t* row_off, int offsets_on_host, int n_convos, int64_t n_rows,
+                                     const void* row_records, const void* row_coef, const float* g_train, float* g_lse,
+                                     float* g_zk, void* stream) {
   using namespace dl;
   const int st0 = composite_check(lse, zk, t_val, t_val_dtype, t_idx, t_idx_itype, K, row_off, row_off, row_off,
-                                  n_convos, n_rows, row_records);
+                                  offsets_on_host, n_convos, n_rows, row_records);
   if (st0 != DL_OK) return st0;
   if (!row_coef || !g_train || !g_lse || !g_zk) return DL_ERR_NULL;
   if (n_rows == 0) return DL_OK;
   CompositeParams p{};
   p.lse = lse; p.zk = zk; p.t_val = t_val; p.t_val_dtype = t_val_dtype; p.inv_T_t = inv_T_teacher;
-  p.t_idx = t_idx; p.t_idx_itype = t_idx_itype; p.K = K; p.row_off = row_off; p.n_convos = n_convos; p.n_rows = n_rows;
+  p.t_idx = t_idx; p.t_idx_itype = t_idx_itype; p.K = K; p.n_convos = n_convos; p.n_rows = n_rows;
+  set_offsets(p.off, row_off, row_off, row_off, offsets_on_host, n_convos);
   p.rec = reinterpret_cast<RowRec*>(const_cast<void*>(row_records));
   p.coef = reinterpret_cast<RowCoef*>(const_cast<void*>(row_coef));
   p.g_train = g_train; p.g_lse = g_lse; p.g_zk = g_zk;

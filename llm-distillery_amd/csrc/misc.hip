@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void copy16_kernel(const u32x4* __restrict__ s
 
 }  // namespace dl
 
-extern "C" int dl_abi_version(void) { return 1; }
+extern "C" int dl_abi_version(void) { return 2; }
 
 extern "C" const char* dl_status_string(int status) {
   switch (status) {

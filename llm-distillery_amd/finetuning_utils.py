@@ -20,6 +20,7 @@ import torch.nn.functional as F
 from torch import Tensor
 
 from . import ops
+from .losses import LossDict
 
 LOSS_KEYS = ("train_loss", "custom loss", "CE loss", "kl_div", "reverse kl_div",
              "weighted kl_div", "weighted rev. kl_div", "teacher CE loss", "CE diff")
@@ -88,28 +89,35 @@ def _fusable(counts, labels, alpha) -> bool:
     return not isinstance(alpha, Tensor) and all(lab.dim() == 1 and lab.numel() == n - 1 for n, lab in zip(counts, labels))
 
 
-def _fused_dicts(lse: Tensor, zk: Tensor, counts, t_vals, t_idxs, labels, avoids, inv_T_teacher: float, alpha):
-    """Nine-key dicts of all conversations from one forward launch pair; `train_loss` / `custom loss`
-    carry the autograd history, the seven logged values do not (the reference's `Losses.add_losses`
-    detaches them before any use, classes/losses.py:35-37)."""
-    dev = zk.device
+def _fused_dicts(x: Tensor, row_map, inv_T: float, crop: int, counts, t_vals, t_idxs, labels, avoids,
+                 inv_T_teacher: float, alpha):
+    """Nine-key dicts of all conversations from one autograd node (`ops.composite_loss`: one phase-1
+    launch over the logits, the K-wide epilogue, and in backward their two counterparts);
+    `train_loss` / `custom loss` carry the autograd history, the seven logged values do not (the
+    reference's `Losses.add_losses` detaches them before any use, classes/losses.py:35-37).
+    The conversations' row / label / ignore offsets travel with the launch: nothing is uploaded."""
+    dev = x.device
+    C = len(counts)
     n_lab = [int(lab.numel()) for lab in labels]
     n_avoid = [int(a.numel()) for a in avoids]
-    offs = torch.tensor([[0] + list(_cumsum(counts)), [0] + list(_cumsum(n_lab)), [0] + list(_cumsum(n_avoid))],
-                        dtype=torch.int32)
-    offs = (offs.pin_memory() if dev.type == "cuda" else offs).to(dev, non_blocking=True)
-    lab_cat = torch.cat([lab.to(torch.int64) for lab in labels]) if len(labels) > 1 else labels[0].to(torch.int64)
-    avoid_cat = torch.cat([a.to(torch.int32) for a in avoids]) if len(avoids) > 1 else avoids[0].to(torch.int32)
-    if lab_cat.numel() == 0:
-        lab_cat = torch.zeros(1, dtype=torch.int64, device=dev)
-    if avoid_cat.numel() == 0:
-        avoid_cat = torch.zeros(1, dtype=torch.int32, device=dev)
-    train, nine = ops.composite_epilogue(lse, zk, _packed_rows(t_vals), _packed_rows(t_idxs), lab_cat, avoid_cat, offs,
-                                         inv_T_teacher, alpha)
+    if C <= ops._lib.DL_MAX_HOST_CONVOS:
+        offs = ([0] + list(_cumsum(counts)), [0] + list(_cumsum(n_lab)), [0] + list(_cumsum(n_avoid)))
+    else:
+        offs = torch.tensor([[0] + list(_cumsum(counts)), [0] + list(_cumsum(n_lab)), [0] + list(_cumsum(n_avoid))],
+                            dtype=torch.int32).to(dev)
+    lab_cat = (torch.cat([lab.to(torch.int64) for lab in labels]) if C > 1 else labels[0].to(torch.int64)).contiguous()
+    if C > 1:
+        avoid_cat = torch.cat([a.to(torch.int64) for a in avoids])
+    else:
+        avoid_cat = avoids[0] if avoids[0].dtype in ops._IT else avoids[0].to(torch.int64)
+    train, nine = ops.composite_loss(x, _packed_rows(t_vals), _packed_rows(t_idxs), lab_cat, avoid_cat.contiguous(), offs,
+                                     row_map, inv_T, inv_T_teacher, alpha, crop)
     out = []
-    for c in range(len(counts)):
-        d = {k: nine[c, j] for j, k in enumerate(LOSS_KEYS)}
-        d["train_loss"] = d["custom loss"] = train[c]
+    for c in range(C):
+        row = nine[c]
+        d = LossDict(zip(LOSS_KEYS, row.unbind(0)))
+        d["train_loss"] = train[c]          # the one value with a graph; "custom loss" is the same number without
+        d.packed, d.keys_packed = row, LOSS_KEYS
         out.append(d)
     return out
 
@@ -141,10 +149,11 @@ def calculate_divergence(student_logits: Tensor, teacher_logits: Tensor, indices
     if n < student_logits.size(0):
         row_map = torch.full((student_logits.size(0),), -1, dtype=torch.int32, device=student_logits.device)
         row_map[:n] = torch.arange(n, dtype=torch.int32, device=student_logits.device)
-    lse, zk = ops.rowstats_topk(student_logits, idx, row_map, 1.0)
     labels = convo_CE_tokens[:n]
     if _fusable([n], [labels], alpha) and teacher_logits.dtype in ops._DT:
-        return _fused_dicts(lse, zk, [n], [teacher_logits[:n]], [idx], [labels], [avoid_indices], 1.0, alpha)[0]
+        return _fused_dicts(student_logits, row_map, 1.0, 0, [n], [teacher_logits[:n]], [idx], [labels], [avoid_indices], 1.0,
+                            alpha)[0]
+    lse, zk = ops.rowstats_topk(student_logits, idx, row_map, 1.0)
     s_sup = zk - lse.unsqueeze(-1)                       # log_softmax over V, gathered at the ids
     t = F.log_softmax(teacher_logits[:n].float(), dim=-1)
     return _assemble(s_sup, t, idx, labels, alpha, avoid_indices)
@@ -166,12 +175,12 @@ def distill_loss(model_logits: Tensor, content_rows: Tensor, teacher_logprobs: T
     n = min(content_rows.numel(), teacher_logprobs.size(0), indices.size(0))
     row_map = torch.full((S,), -1, dtype=torch.int32, device=x.device)
     row_map[content_rows[:n].long()] = torch.arange(n, dtype=torch.int32, device=x.device)
-    lse, zk = ops.rowstats_topk(x, indices[:n], row_map, 1.0 / temperature, int(crop_to_size or 0))
     tT = temperature if teacher_temperature is None else teacher_temperature
     labels = convo_CE_tokens[:n]
     if _fusable([n], [labels], alpha) and teacher_logprobs.dtype in ops._DT:
-        return _fused_dicts(lse, zk, [n], [teacher_logprobs[:n]], [indices[:n]], [labels], [avoid_indices], 1.0 / tT,
-                            alpha)[0]
+        return _fused_dicts(x, row_map, 1.0 / temperature, int(crop_to_size or 0), [n], [teacher_logprobs[:n]], [indices[:n]],
+                            [labels], [avoid_indices], 1.0 / tT, alpha)[0]
+    lse, zk = ops.rowstats_topk(x, indices[:n], row_map, 1.0 / temperature, int(crop_to_size or 0))
     s_sup = zk - lse.unsqueeze(-1)
     t = F.log_softmax(teacher_logprobs[:n].float() / tT, dim=-1)
     return _assemble(s_sup, t, indices[:n], labels, alpha, avoid_indices)
@@ -209,12 +218,13 @@ def distill_loss_batch(model_logits: Tensor, convos, alpha, temperature: float =
         where = torch.cat([rows[:n].long() + b * S for b, ((rows, *_), n) in enumerate(zip(convos, counts))])
         row_map[where] = torch.arange(where.numel(), dtype=torch.int32, device=dev)      # one scatter for the batch
     idx_cat = _packed_rows([idx[:n] for (_, _, idx, _, _), n in zip(convos, counts)])
-    lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature, int(crop_to_size or 0))
     tT = temperature if teacher_temperature is None else teacher_temperature
     labels_all = [labels[:n] for (_, _, _, labels, _), n in zip(convos, counts)]
     if _fusable(counts, labels_all, alpha) and all(c[1].dtype in ops._DT for c in convos):
-        return _fused_dicts(lse, zk, counts, [t_lp[:n] for (_, t_lp, _, _, _), n in zip(convos, counts)],
-                            [idx_cat], labels_all, [c[4] for c in convos], 1.0 / tT, alpha)
+        return _fused_dicts(ops._rows_2d(x), row_map, 1.0 / temperature, int(crop_to_size or 0), counts,
+                            [t_lp[:n] for (_, t_lp, _, _, _), n in zip(convos, counts)], [idx_cat], labels_all,
+                            [c[4] for c in convos], 1.0 / tT, alpha)
+    lse, zk = ops.rowstats_topk(ops._rows_2d(x), idx_cat, row_map, 1.0 / temperature, int(crop_to_size or 0))
     out, base = [], 0
     for (rows, t_lp, idx, labels, avoid), n in zip(convos, counts):
         s_sup = zk[base:base + n] - lse[base:base + n].unsqueeze(-1)

@@ -3,6 +3,7 @@ stream; all arithmetic happens in the HIP kernels.  No fallbacks: a CPU tensor o
 a missing library raises."""
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Tuple
 
 import torch
@@ -219,8 +220,10 @@ def _rowstats_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float):
     if row_map is None and N < R:
         raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
     _, rm_ptr = _opt_i32(row_map, R, "row_map", x.device)
-    lse = torch.zeros(N, dtype=torch.float32, device=x.device)
-    zk = torch.zeros((N, K), dtype=torch.float32, device=x.device)
+    # every teacher row is written by the kernel unless a row map leaves some out: no zero fill then
+    make = torch.empty if row_map is None else torch.zeros
+    lse = make(N, dtype=torch.float32, device=x.device)
+    zk = make((N, K), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         st = _lib.load().dl_rowstats_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(),
                                           _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), zk.data_ptr(),
@@ -311,69 +314,129 @@ def _rowstats_backward(ctx, g_lse, g_zk):
 rowstats_topk.register_autograd(_rowstats_backward, setup_context=_rowstats_setup)
 
 
-class _CompositeEpilogue(torch.autograd.Function):
-    """K-wide composite loss of a batch of conversations (dl_composite_forward / _backward).
-    Returns (train_loss [C], the nine values [C, 9]); only train_loss is differentiable."""
+def _offsets_arg(offsets):
+    """(row, label, avoid) offsets for dl_composite_*: three ctypes int32 arrays that travel with the
+    launch when `offsets` is a host list of three lists (at most DL_MAX_HOST_CONVOS conversations), or
+    the rows of a device int32 [3, C + 1] tensor."""
+    if isinstance(offsets, torch.Tensor):
+        return (offsets[0].data_ptr(), offsets[1].data_ptr(), offsets[2].data_ptr()), 0, offsets.shape[1] - 1
+    C = len(offsets[0]) - 1
+    arr = ctypes.c_int32 * (C + 1)
+    return (arr(*offsets[0]), arr(*offsets[1]), arr(*offsets[2])), 1, C
+
+
+class _CompositeLoss(torch.autograd.Function):
+    """The reference's composite loss of C conversations as ONE autograd node: phase 1 over the logits
+    (dl_rowstats_topk), the K-wide epilogue (dl_composite_forward), and in backward their two
+    counterparts (dl_composite_backward, dl_rowcoef_grad_topk).  Returns (train_loss [C], the nine
+    values [C, 9]); only train_loss is differentiable, and only with respect to the logits."""
 
     @staticmethod
-    def forward(ctx, lse, zk, t_val, t_idx, labels, avoid, offsets, inv_T_teacher: float, alpha: float):
-        dev = zk.device
-        N, K = zk.shape
-        C = offsets.shape[1] - 1
-        need_grad = lse.requires_grad or zk.requires_grad
+    def forward(ctx, logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T: float, inv_T_teacher: float,
+                alpha: float, crop: int):
+        x = _cropped(logits, crop)
+        dev = x.device
+        R, V = x.shape
+        N, K = t_idx.shape
+        lib = _lib.load()
+        offs, on_host, C = _offsets_arg(offsets)
+        need_grad = ctx.needs_input_grad[0]          # False under torch.no_grad() (the validation loop) and for detached logits
+        # every teacher row is written by phase 1 unless a row map leaves some out
+        make = torch.empty if row_map is None else torch.zeros
+        lse = make(N, dtype=torch.float32, device=dev)
+        zk = make((N, K), dtype=torch.float32, device=dev)
         rec = torch.empty((N, 8), dtype=torch.float32, device=dev)
         coef = torch.empty((N, 4), dtype=torch.float32, device=dev) if need_grad else None
         out = torch.empty((C, 9), dtype=torch.float32, device=dev)
+        rm_ptr = row_map.data_ptr() if row_map is not None else 0
+        stream = _stream_ptr(dev)
         with torch.cuda.device(dev):
-            st = _lib.load().dl_composite_forward(
+            st = lib.dl_rowstats_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(), _IT[t_idx.dtype],
+                                      K, N, inv_T, lse.data_ptr(), zk.data_ptr(), stream)
+            _lib.check(st, "dl_rowstats_topk")
+            st = lib.dl_composite_forward(
                 lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
-                _IT[t_idx.dtype], K, labels.data_ptr(), avoid.data_ptr(), offsets[0].data_ptr(), offsets[1].data_ptr(),
-                offsets[2].data_ptr(), C, N, float(alpha), rec.data_ptr(), coef.data_ptr() if need_grad else 0,
-                out.data_ptr(), _stream_ptr(dev))
-        _lib.check(st, "dl_composite_forward")
+                _IT[t_idx.dtype], K, labels.data_ptr() if labels.numel() else 0, avoid.data_ptr() if avoid.numel() else 0,
+                _IT[avoid.dtype], offs[0], offs[1], offs[2], on_host, C, N, alpha, rec.data_ptr(),
+                coef.data_ptr() if need_grad else 0, out.data_ptr(), stream)
+            _lib.check(st, "dl_composite_forward")
         if need_grad:
-            ctx.save_for_backward(lse, zk, t_val, t_idx, offsets, rec, coef)
-        ctx.inv_T_teacher = inv_T_teacher
-        train = out[:, 0].contiguous()
+            ctx.save_for_backward(logits, t_val, t_idx, lse, zk, rec, coef, *([row_map] if row_map is not None else []),
+                                  *([offsets] if on_host == 0 else []))
+            ctx.host_offsets = offsets if on_host else None
+            ctx.has_map = row_map is not None
+            ctx.scalars = (inv_T, inv_T_teacher, crop)
+        train = out[:, 0].clone()      # its own storage: the differentiable output must not alias the logged one
         ctx.mark_non_differentiable(out)
         return train, out
 
     @staticmethod
     def backward(ctx, g_train, _g_logged):
-        lse, zk, t_val, t_idx, offsets, rec, coef = ctx.saved_tensors
-        dev = zk.device
-        N, K = zk.shape
+        saved = ctx.saved_tensors
+        logits, t_val, t_idx, lse, zk, rec, coef = saved[:7]
+        row_map = saved[7] if ctx.has_map else None
+        offsets = ctx.host_offsets if ctx.host_offsets is not None else saved[-1]
+        inv_T, inv_T_teacher, crop = ctx.scalars
+        x = _cropped(logits, crop)
+        dev = x.device
+        R, V = x.shape
+        N, K = t_idx.shape
+        lib = _lib.load()
+        offs, on_host, C = _offsets_arg(offsets)
         g = g_train.to(torch.float32).contiguous()
         g_lse = torch.empty_like(lse)
         g_zk = torch.empty_like(zk)
+        grad = torch.empty_like(logits)                      # full width; the kernel fills [:, :crop]
+        if x is not logits:
+            grad[:, crop:].zero_()
+        gx = _cropped(grad, crop)
+        stream = _stream_ptr(dev)
         with torch.cuda.device(dev):
-            st = _lib.load().dl_composite_backward(
-                lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], ctx.inv_T_teacher, t_idx.data_ptr(),
-                _IT[t_idx.dtype], K, offsets[0].data_ptr(), offsets.shape[1] - 1, N, rec.data_ptr(), coef.data_ptr(),
-                g.data_ptr(), g_lse.data_ptr(), g_zk.data_ptr(), _stream_ptr(dev))
-        _lib.check(st, "dl_composite_backward")
-        return g_lse, g_zk, None, None, None, None, None, None, None
+            st = lib.dl_composite_backward(
+                lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
+                _IT[t_idx.dtype], K, offs[0], on_host, C, N, rec.data_ptr(), coef.data_ptr(), g.data_ptr(),
+                g_lse.data_ptr(), g_zk.data_ptr(), stream)
+            _lib.check(st, "dl_composite_backward")
+            st = lib.dl_rowcoef_grad_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V,
+                                          row_map.data_ptr() if row_map is not None else 0, t_idx.data_ptr(),
+                                          _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), g_lse.data_ptr(), g_zk.data_ptr(),
+                                          gx.data_ptr(), gx.stride(0), stream)
+            _lib.check(st, "dl_rowcoef_grad_topk")
+        return (grad,) + (None,) * 10
 
 
-def composite_epilogue(lse: torch.Tensor, zk: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor,
-                       labels: torch.Tensor, avoid: torch.Tensor, offsets: torch.Tensor, inv_T_teacher: float,
-                       alpha: float) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(train_loss [C], nine values [C, 9]) of C conversations from phase 1's `lse` [N] / `zk` [N, K],
-    the stored teacher rows `t_val` / `t_idx` [N, K], the concatenated int64 `labels` and int32
-    `avoid` rows, and `offsets` int32 [3, C + 1] (first row, first label, first avoid entry of every
-    conversation).  See dl_composite_forward."""
-    _dev(zk, "zk")
-    for name, t in (("lse", lse), ("t_val", t_val), ("t_idx", t_idx), ("labels", labels), ("avoid", avoid), ("offsets", offsets)):
-        _dev(t, name, zk.device)
-    if lse.dtype != torch.float32 or zk.dtype != torch.float32 or not (lse.is_contiguous() and zk.is_contiguous()):
-        raise RuntimeError("lse / zk must be contiguous fp32 (phase 1's outputs)")
-    if t_val.dtype not in _DT or t_idx.dtype not in _IT or labels.dtype != torch.int64 or avoid.dtype != torch.int32 \
-            or offsets.dtype != torch.int32:
+def composite_loss(logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor, labels: torch.Tensor,
+                   avoid: torch.Tensor, offsets, row_map: Optional[torch.Tensor], inv_T: float, inv_T_teacher: float,
+                   alpha: float, crop: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(train_loss [C], nine values [C, 9]) of C conversations straight from the logits [rows, V]:
+    `t_val` / `t_idx` [N, K] the stored teacher rows of all conversations back to back, `labels` int64
+    and `avoid` int32 / int64 concatenated, `offsets` = three host lists (first row, first label,
+    first ignore entry of every conversation, C + 1 entries each; C <= DL_MAX_HOST_CONVOS) or a device
+    int32 [3, C + 1] tensor, `row_map` as for `div_topk`.  See dl_rowstats_topk / dl_composite_forward."""
+    _dev(logits, "logits")
+    dev = logits.device
+    for name, t in (("t_val", t_val), ("t_idx", t_idx), ("labels", labels), ("avoid", avoid)):
+        _dev(t, name, dev)
+    if logits.dim() != 2 or logits.stride(1) != 1 or logits.dtype not in _DT:
+        raise RuntimeError("logits must be [rows, V] bf16/fp16/fp32, dense along V")
+    if t_val.dtype not in _DT or t_idx.dtype not in _IT or labels.dtype != torch.int64 or avoid.dtype not in _IT:
         raise RuntimeError("unsupported dtype")
-    if t_val.shape != zk.shape or t_idx.shape != zk.shape or offsets.dim() != 2 or offsets.shape[0] != 3:
-        raise RuntimeError("shape mismatch")
-    return _CompositeEpilogue.apply(lse, zk, t_val.contiguous(), t_idx.contiguous(), labels.contiguous(),
-                                    avoid.contiguous(), offsets.contiguous(), float(inv_T_teacher), float(alpha))
+    if t_idx.dim() != 2 or t_val.shape != t_idx.shape or not (t_val.is_contiguous() and t_idx.is_contiguous()
+                                                             and labels.is_contiguous() and avoid.is_contiguous()):
+        raise RuntimeError("t_val / t_idx must be contiguous [N, K], labels and avoid contiguous vectors")
+    N = t_idx.shape[0]
+    if row_map is None and N < logits.shape[0]:
+        raise RuntimeError(f"{logits.shape[0]} logits rows but only {N} teacher rows and no row_map")
+    if row_map is not None:
+        _opt_i32(row_map, logits.shape[0], "row_map", dev)
+    if isinstance(offsets, torch.Tensor):
+        _dev(offsets, "offsets", dev)
+        if offsets.dtype != torch.int32 or offsets.dim() != 2 or offsets.shape[0] != 3 or not offsets.is_contiguous():
+            raise RuntimeError("device offsets must be a contiguous int32 [3, C + 1] tensor")
+    elif len(offsets) != 3 or len(offsets[0]) - 1 > _lib.DL_MAX_HOST_CONVOS or offsets[0][-1] != N:
+        raise RuntimeError("host offsets: three lists of C + 1 entries, C <= DL_MAX_HOST_CONVOS, rows ending at N")
+    return _CompositeLoss.apply(logits, t_val, t_idx, labels, avoid, offsets, row_map, float(inv_T), float(inv_T_teacher),
+                                float(alpha), int(crop))
 
 
 def reduce_sum(values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:

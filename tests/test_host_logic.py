@@ -81,6 +81,49 @@ def test_losses_validation_prefix_and_scaling_operators():
     assert "Validation Losses" in str(L)
 
 
+def test_losses_packed_dicts_accumulate_like_plain_ones():
+    """`calculate_divergence` hands out dicts whose values are views of one [9] tensor; `Losses` sums
+    those with one addition per conversation.  Totals, step count, backward and logging must be what
+    the key-by-key form gives, also when packed and plain dicts are mixed."""
+    from llm_distillery_amd.losses import LossDict
+    keys = D.LOSS_KEYS
+    leafs = [torch.tensor(float(i + 1), requires_grad=True) for i in range(3)]
+
+    def make(i, packed):
+        row = torch.arange(9, dtype=torch.float32) * (i + 1)
+        train = leafs[i] * 2
+        d = LossDict(zip(keys, row.unbind(0))) if packed else dict(zip(keys, row.clone().unbind(0)))
+        d["train_loss"] = train
+        if packed:
+            d.packed, d.keys_packed = row, keys
+        return d
+
+    for pattern in ((True, True, True), (False, False, False), (True, False, True), (False, True, True)):
+        for leaf in leafs:
+            leaf.grad = None
+        L = D.Losses(_Log())
+        for i, packed in enumerate(pattern):
+            L.add_losses(make(i, packed))
+        assert L.num_steps_accumulated == 3
+        got = L.loss_dict
+        assert list(got)[0] == "train_loss" and set(got) == set(keys)
+        assert got["train_loss"].item() == 2 * (1 + 2 + 3)
+        for j, k in enumerate(keys[1:], start=1):
+            assert got[k].item() == j * (1 + 2 + 3) and not got[k].requires_grad
+        L.backward(divisor=2)
+        assert all(leaf.grad.item() == 1.0 for leaf in leafs) and "train_loss" not in L.loss_dict
+        L.log(step=3)
+        assert L.logger.rows[0][0]["Loss/custom loss"].item() == pytest.approx(1 * 6 / 3)
+        L.empty()
+        assert L.loss_dict == {} and L.num_steps_accumulated == 0
+    # the batch form: stack + sum
+    L = D.Losses(None)
+    L.add_batch([make(i, True) for i in range(3)])
+    assert L.num_steps_accumulated == 3 and L.loss_dict["kl_div"].item() == 3 * 6 and L.loss_dict["train_loss"].item() == 12
+    half = L / 2
+    assert half.loss_dict["kl_div"].item() == 9.0
+
+
 def test_library_exports_every_symbol_the_header_declares():
     header = open(os.path.join(ROOT, "include", "distill_hip.h")).read()
     declared = set(re.findall(r"\b(dl_[a-z0-9_]+)\s*\(", header))
@@ -90,6 +133,42 @@ def test_library_exports_every_symbol_the_header_declares():
     assert declared == set(D._lib.exported_symbols())
     assert lib.dl_abi_version() >= 1
     assert lib.dl_status_string(0) == b"ok" and b"NULL" in lib.dl_status_string(-1)
+
+
+def test_argument_errors_are_reported_before_any_gpu_work():
+    """Host-side validation of the entry points that take host arrays: every call below returns its
+    status before the first HIP call, so the (never dereferenced) device pointers can be anything."""
+    import ctypes
+    lib = D._lib.load()
+    fake = ctypes.c_void_p(4096)
+    i32 = lambda *v: (ctypes.c_int32 * len(v))(*v)
+    # composite: offsets that travel with the launch are checked on the host
+    def fwd(row, lab, av, C, N):
+        return lib.dl_composite_forward(fake, fake, fake, 2, 1.0, fake, 0, 8, fake, fake, 1, row, lab, av, 1, C, N, 2.0, fake, fake,
+                                        fake, None)
+    assert fwd(i32(0, 5, 3), i32(0, 4, 6), i32(0, 0, 0), 2, 3) == -3            # rows not non-decreasing
+    assert fwd(i32(0, 5, 9), i32(0, 4, 7), i32(0, 0, 0), 2, 10) == -3           # rows do not end at n_rows
+    assert fwd(i32(1, 5), i32(0, 4), i32(0, 0), 1, 5) == -3                     # rows do not start at 0
+    many = i32(*range(66))
+    assert fwd(many, many, many, 65, 65) == -4                                  # more conversations than a launch carries
+    assert lib.dl_composite_forward(fake, fake, fake, 2, 1.0, fake, 0, 8, fake, fake, 7, i32(0, 5), i32(0, 4), i32(0, 0), 1, 1, 5,
+                                    2.0, fake, fake, fake, None) == -2          # ignore entries of an unknown integer type
+    assert lib.dl_composite_backward(fake, fake, fake, 2, 1.0, fake, 0, 8, i32(0, 4), 1, 1, 5, fake, fake, fake, fake, fake,
+                                     None) == -3
+    # multi-teacher loss: limits, weights, workspace
+    ptrs = (ctypes.c_void_p * 3)(4096, 4096, 4096)
+    w = lambda *v: (ctypes.c_float * len(v))(*v)
+    def multi(V=128256, n=3, K=200, ws=fake, ws_bytes=1 << 40, weights=w(0.5, 0.3, 0.2), stride=None):
+        return lib.dl_fkl_multi_teacher(fake, 1, stride or V, 64, V, None, n, ptrs, ptrs, 2, 0, K, 64, weights, None, 0, 1.0, 1.0,
+                                        fake, fake, V, ws, ws_bytes, 0, None)
+    assert multi(n=3, K=700) == -4                                              # more than DL_MAX_TOPK entries per row
+    assert multi(V=300000) == -4                                                # rows too wide for the register kernels
+    assert multi(V=128257, stride=128264) == -6                                 # odd vocabulary
+    assert multi(ws=None) == -7 and multi(ws_bytes=1000) == -7                  # no / too small a workspace
+    assert multi(weights=w(0.5, -0.1, 0.2)) == -3 and multi(weights=w(0.5, float("nan"), 0.2)) == -3
+    need = lib.dl_fkl_multi_teacher_workspace_bytes(1, 64, 128256, 3, 200, 64, 0)
+    assert need > 64 * 4 * 256 * 8 and multi(ws_bytes=need - 1) == -7
+    assert lib.dl_fkl_multi_teacher_workspace_bytes(1, 64, 300000, 3, 200, 64, 0) == 0
 
 
 def test_no_cpu_fallback():
