@@ -5,7 +5,7 @@
 One step = one pass of the fused loss + gradient over one batch of synthetic input followed by the
 deterministic mean reduction.  The default workload is the one the headline metric is quoted on
 (C3: 8 x 4096 tokens x 128256-vocabulary bf16 student logits, top-K=200 fp16/int32 teacher, T=1);
-`--workload c1|c2|c4|c4-merge|c5|producer|composite|dropin|dropin-batch` measures the other configurations and the teacher producer with the
+`--workload c1|c2|c4|c4-merge|c5|producer|composite|dropin|dropin-batch|copyshape` measures the other configurations and the teacher producer with the
 same harness.  Inputs are
 resident in HBM before the timed region.  Prints ONE JSON line.
 """
@@ -29,6 +29,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 # step_fn runs the whole step and returns the loss tensor; main_launch_fn launches only the dominant kernel.
 # ---------------------------------------------------------------------------------------------
 INPLACE = False        # --inplace: the gradient is written over the logits (C3 only; see main)
+PARTS = 0              # --parts: column parts per row of the C3 loss kernel (0 = the library's choice)
 
 
 def _wl_c3(D, S, dev, rows):
@@ -40,12 +41,14 @@ def _wl_c3(D, S, dev, rows):
     scale = 1.0 / rows
 
     def main():
-        return D.div_topk("fkl", c["logits"], c["t_val"], c["t_idx"], T=1.0, grad_scale=scale, grad_out=grad)[0]
+        return D.div_topk("fkl", c["logits"], c["t_val"], c["t_idx"], T=1.0, grad_scale=scale, grad_out=grad, parts=PARTS)[0]
 
+    shape = {0: "256,16,split> (4 column parts per row)", 1: "1024,16> (one workgroup per row)", 2: "512,16,split> (2 column parts per row)",
+             4: "256,16,split> (4 column parts per row)", 16: "256,4,split> (16 column parts per row)"}[PARTS]
     return (lambda: D.reduce_sum(main(), scale), main, rows * (V * 2 + V * 2 + K * 6), rows,
             f"C3 forward-KL fwd+bwd, top-K={K} fp16/int32 teacher, {rows} tokens x {V} vocab bf16 logits, T=1, "
             "bf16 gradient" + (" written over the logits" if INPLACE else ""),
-            "fkl_topk_reg_kernel<bf16,256,16,split> (4 column parts per row)", c, grad)
+            "fkl_topk_reg_kernel<bf16," + shape, c, grad)
 
 
 def _wl_c4(D, S, dev, rows):
@@ -267,7 +270,33 @@ def _wl_dropin(batched):
     return build
 
 
-WORKLOADS = {"dropin": _wl_dropin(False), "dropin-batch": _wl_dropin(True), "composite": _wl_composite, "producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c4-merge": _wl_c4_merge, "c5": _wl_c5}
+COPY_SHAPE = {"threads": 256, "chunks": 16, "one_xcd": True, "wave_major": True, "lds_kb": 0}      # --workload copyshape: see main
+
+
+def _wl_copyshape(D, S, dev, rows):
+    """A bare copy of the C3 logits buffer in the access shape of a row kernel: what the memory system gives
+    a kernel that moves `--chunks` 16-byte chunks per thread between its loads and its stores."""
+    import torch
+    rows = rows or 8 * 4096
+    V = 128256
+    src = torch.empty((rows, V), dtype=torch.bfloat16, device=dev).normal_()
+    dst = torch.empty_like(src)
+    cs = COPY_SHAPE
+
+    def main():
+        D.copy_rows(src, dst, cs["threads"], cs["chunks"], cs["one_xcd"], cs["wave_major"], cs["lds_kb"])
+        return dst[0, :1].float().sum()
+
+    parts = -(-(V * 2 // 16) // (cs["threads"] * cs["chunks"]))
+    return (main, main, rows * V * 2 * 2, rows,
+            f"bare copy of {rows} x {V} bf16 rows, {cs['threads']} threads x {cs['chunks']} chunks per workgroup ({parts} parts per row, "
+            + ("parts of a row on one XCD" if cs["one_xcd"] else "row-major workgroup order") + ", "
+            + ("wave-major" if cs["wave_major"] else "striped") + " chunks"
+            + (f", at most {160 // cs['lds_kb']} workgroups per CU" if cs["lds_kb"] else "") + ")",
+            f"copy_rows_kernel<{cs['threads']},{cs['chunks']}>", {"logits": src}, dst)
+
+
+WORKLOADS = {"copyshape": _wl_copyshape, "dropin": _wl_dropin(False), "dropin-batch": _wl_dropin(True), "composite": _wl_composite, "producer": _wl_producer, "c1": _wl_dense("c1"), "c2": _wl_dense("c2"), "c3": _wl_c3, "c4": _wl_c4, "c4-merge": _wl_c4_merge, "c5": _wl_c5}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -351,13 +380,25 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's plain copy kernel over the logits buffer (known traffic: its "
                          "byte size each way), the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--threads", type=int, default=256, help="copyshape: threads per workgroup (256 / 512 / 1024)")
+    ap.add_argument("--chunks", type=int, default=16, help="copyshape: 16-byte chunks per thread (2 / 4 / 8 / 12 / 16)")
+    ap.add_argument("--row-major", action="store_true", help="copyshape: workgroups in row-major order instead of a row's "
+                                                              "parts on one XCD")
+    ap.add_argument("--striped", action="store_true", help="copyshape: chunk c of a part belongs to thread c %% threads "
+                                                            "instead of every wave owning `chunks` KiB in one piece")
+    ap.add_argument("--lds-kb", type=int, default=0, help="copyshape: LDS held per workgroup (bounds workgroups per CU at 160 / n)")
+    ap.add_argument("--parts", type=int, default=0, choices=(0, 1, 2, 4, 16),
+                    help="c3 only: column parts per row of the loss kernel (0 = the library's choice)")
     ap.add_argument("--inplace", action="store_true",
                     help="c3 only: write the gradient over the logits (same DRAM pages: about 4 %% faster).  After the "
                          "first step the buffer holds gradients, not logits, so the printed loss means nothing; the "
                          "traffic and the arithmetic per step are unchanged.  Not the default for that reason")
     args = ap.parse_args()
-    global INPLACE
+    global INPLACE, PARTS
+    PARTS = args.parts if args.workload == "c3" else 0
     INPLACE = bool(args.inplace and args.workload == "c3")
+    COPY_SHAPE.update(threads=args.threads, chunks=args.chunks, one_xcd=not args.row_major, wave_major=not args.striped,
+                      lds_kb=args.lds_kb)
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is row-parallel and every configuration fits one "
                  "MI355X; run with --gpus 1")
@@ -396,7 +437,7 @@ def main():
     kern_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
     achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
 
-    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c4-merge": 256, "dropin": 0, "dropin-batch": 0, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048, "composite": 2048}[args.workload]
+    cpu_rows = args.cpu_rows if args.cpu_rows >= 0 else {"c3": 4096, "c4": 256, "c4-merge": 256, "dropin": 0, "dropin-batch": 0, "copyshape": 0, "c1": 512, "c2": 4096, "c5": 512, "producer": 2048, "composite": 2048}[args.workload]
     out = {
         "metric": "tokens/sec fused KL fwd+bwd @ vocab 128256 bf16; % of HBM peak GB/s",
         "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,

@@ -47,6 +47,9 @@ typedef enum {
 #define DL_TOPK_NO_WAIT 2      /* parts of a split row never wait for their partners: every part that  */
                                /* finds a record missing is finished by the second launch (exercises   */
                                /* that path; same results, slower)                                      */
+#define DL_TOPK_FINE_PARTS 4   /* rows of 1025-16384 16-byte chunks are cut into parts of 1024 chunks   */
+                               /* (up to 16 per row) where the workspace holds 20 bytes per row and    */
+                               /* part + 16; else ignored                                               */
 #define DL_TOPK_PARTS_SHIFT 8  /* bits 8-11: column parts a row of 65537-131072 two-byte (half as many */
 #define DL_TOPK_PARTS(n) ((n) << DL_TOPK_PARTS_SHIFT)   /* four-byte) entries is cut into: 1, 2 or 4    */
                                /* (4 only where four parts of 32768 two-byte entries all hold columns); */
@@ -399,6 +402,27 @@ int dl_reduce_sum(const float* values, int64_t n, float scale, float* out, void*
  * counters (FETCH_SIZE / WRITE_SIZE) of the loss kernels are scaled by.
  */
 int dl_copy16(const void* src, void* dst, int64_t n_bytes, void* stream);
+
+/*
+ * Copy of n_rows rows of row_bytes (a multiple of 16; both pointers 16-byte aligned, rows dense) in
+ * the access shape of the row kernels: every row is cut into column parts of threads x chunks
+ * 16-byte chunks, one workgroup per part, each thread issuing all its loads and then all its stores.
+ * No reference counterpart: the yardstick that says what a bare copy reaches in a kernel's shape.
+ * (threads, chunks) one of (256, 2 / 4 / 8 / 12 / 16), (512, 4 / 8 / 16), (1024, 4 / 16), else
+ * DL_ERR_LIMIT.  flags:
+ *   DL_COPY_PARTS_ON_ONE_XCD  the parts of a row are placed 8 workgroup ids apart (as the split loss
+ *                             kernels do); else row-major
+ *   DL_COPY_WAVE_MAJOR        every wave owns `chunks` KiB in one piece (the loss kernels' layout);
+ *                             else chunk c of a part belongs to thread c % threads
+ *   DL_COPY_LDS_KB(n)         every workgroup also holds n KiB of LDS (n <= 64), which bounds the
+ *                             workgroups per CU at 160 / n
+ */
+#define DL_COPY_PARTS_ON_ONE_XCD 1
+#define DL_COPY_WAVE_MAJOR 2
+#define DL_COPY_LDS_KB_SHIFT 8
+#define DL_COPY_LDS_KB(n) ((n) << DL_COPY_LDS_KB_SHIFT)
+int dl_copy_rows(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int threads, int chunks,
+                 int flags, void* stream);
 
 #ifdef __cplusplus
 }

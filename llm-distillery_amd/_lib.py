@@ -21,6 +21,7 @@ DL_MAX_TEACHERS = 8
 DL_MAX_HOST_CONVOS = 64
 DL_TOPK_UNIQUE_IDS = 1
 DL_TOPK_NO_WAIT = 2
+DL_TOPK_FINE_PARTS = 4
 DL_TOPK_PARTS_SHIFT = 8
 DL_STATIC_SCRATCH_BYTES = 4 << 20
 
@@ -61,6 +62,7 @@ _SIGNATURES = {
     "dl_teacher_topk_workspace_bytes": (c_int64, [c_int, c_int64, c_int64, c_int]),
     "dl_reduce_sum": (c_int, [_P, c_int64, c_float, _P, _P]),
     "dl_copy16": (c_int, [_P, _P, c_int64, _P]),
+    "dl_copy_rows": (c_int, [_P, _P, c_int64, c_int64, c_int, c_int, c_int, _P]),
 }
 
 _lib = None

@@ -6,8 +6,8 @@
 extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V) {
   if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
   const int64_t nch = V / (logits_dtype == DL_F32 ? 4 : 8);
-  if (nch <= 512 * 16 || nch > (int64_t)dl::MAX_PARTS * 256 * 16) return 0;
-  return dl::RetryList::bytes(n_rows, nch <= 1024 * 16 ? 4 : dl::MAX_PARTS);
+  if (nch <= 512 * 16 || nch > (int64_t)dl::MAX_COARSE_PARTS * 256 * 16) return 0;
+  return dl::RetryList::bytes(n_rows, nch <= 1024 * 16 ? 4 : dl::MAX_COARSE_PARTS);
 }
 
 // Argument checks and dispatch shared by dl_div_topk and dl_div_topk_static.

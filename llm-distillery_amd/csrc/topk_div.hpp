@@ -60,7 +60,8 @@ struct TopkParams {
   TeacherBuckets bk;    // MULTI kernels only; K is then the number of entries a bucket may hold, rounded up to whole slots
 };
 
-constexpr int MAX_PARTS = 8;
+constexpr int MAX_PARTS = 16;             // parts a row may be cut into (parts of 256 x 4 chunks)
+constexpr int MAX_COARSE_PARTS = 8;       // of 256 x 16 chunks
 
 // What one part of a split row tells the others: three floats and a tag that depends on all of
 // them.  The four words are written and read with relaxed device-scope accesses (they bypass the
@@ -316,7 +317,7 @@ __device__ __forceinline__ float mass_on_column(const int* next, const int* col,
 // row crowd into one part) are fetched here, from the row's overflow share.
 // Leaves q in s.q, Q_id(k) in s.val[k], z in s.z[k]; returns the number of LDS entry slots in use
 // (a multiple of NT); B as fkl_partials.
-template <class Tag, int NT, int J>
+template <class Tag, int NT, int NCH, int J>
 __device__ __forceinline__ int bucket_finish(const TopkParams& p, const TopkLds& s, const TeacherEntries<J>& te,
                                              const BucketHead& hd, int64_t trow, const char* row, int lo, int hi, float& B) {
   const int nk = max(J * NT, (hd.n + NT - 1) / NT * NT);
@@ -345,14 +346,14 @@ __device__ __forceinline__ int bucket_finish(const TopkParams& p, const TopkLds&
   }
   for (int k = threadIdx.x; k < nk; k += NT) {
     const int id = s.idx[k];                               // this thread's own store
-    if (id >= 0) correction_link<Tag, NT>(s.head, s.own, s.next, k, id - lo);
+    if (id >= 0) correction_link<Tag, NT, NCH>(s.head, s.own, s.next, k, id - lo);
   }
   __syncthreads();
   B = 0.f;
   for (int k = threadIdx.x; k < nk; k += NT) {
     const int id = s.idx[k];
     if (id < 0) continue;
-    const int first = s.head[correction_head_slot<Tag, NT>(id - lo)];
+    const int first = s.head[correction_head_slot<Tag, NT, NCH>(id - lo)];
     int same = 0;
     float big = 0.f;
     for (int e = first; e >= 0; e = s.next[e]) {
@@ -406,13 +407,13 @@ __device__ __forceinline__ void fkl_sparse_fix(const TopkLds& s, void* grow, int
 // student probability at the entry's column in s.val and link the entry into its owner's list; the
 // owner subtracts the teacher mass -- of all entries of that column, should ids repeat, which it
 // sees from the chunk's list: no scan over the row's ids.
-template <class Tag, int NT>
+template <class Tag, int NT, int NCH>
 __device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, int hi, float a, float b) {
   for (int k = threadIdx.x; k < s.Kp; k += NT) {
     const int id = s.idx[k];
     if (id < lo || id >= hi) continue;
     s.val[k] = fast_exp2(fmaf(s.z[k], a, -b));
-    correction_link<Tag, NT>(s.head, s.own, s.next, k, id - lo);
+    correction_link<Tag, NT, NCH>(s.head, s.own, s.next, k, id - lo);
   }
 }
 
@@ -488,7 +489,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   u32x4 reg[NCH];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int64_t c = (int64_t)i * NT + tid;
+    const int64_t c = ChunkMap<NT, NCH>::chunk(i, tid);
     // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
     // finds its lines in L2 instead of fetching them a second time (0.47 GB less per 32768 rows of K = 200)
     reg[i] = c < nch ? *reinterpret_cast<const u32x4*>(rpart + c * 16) : C::neg_inf();
@@ -499,7 +500,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   int nk = s.Kp;                      // LDS entry slots in use
   if constexpr (MULTI) {
     teacher_gather<Tag, J>(row, lo, hi, te);
-    if (hd.total > 0) nk = bucket_finish<Tag, NT, J>(p, s, te, hd, trow, row, lo, hi, B);
+    if (hd.total > 0) nk = bucket_finish<Tag, NT, NCH, J>(p, s, te, hd, trow, row, lo, hi, B);
     tlse = hd.total > 0 ? 0.f : -INFINITY;
     Q = hd.qsum;
   } else if constexpr (J > 0) {
@@ -591,7 +592,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
       }
       __syncthreads();
     } else if (IN_REGISTERS) {
-      fkl_link_corrections<Tag, NT>(s, lo, hi, a, b);
+      fkl_link_corrections<Tag, NT, NCH>(s, lo, hi, a, b);
       __syncthreads();
     }
     const unsigned mine = IN_REGISTERS ? s.own[tid] : 0u;
@@ -601,7 +602,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
     unsigned repeats = 0u;            // chunks in which an id occurs more than once
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int64_t ch = (int64_t)i * NT + tid;
+      const int64_t ch = ChunkMap<NT, NCH>::chunk(i, tid);
       if (ch < nch) {
         float f[C::N];
         forget(reg[i]);
@@ -609,12 +610,12 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
         if (mine & (1u << i))
-          if (correction_apply<Tag, NT>(s.head, s.next, s.idx, lo, i, f, mass, value)) repeats |= 1u << i;
+          if (correction_apply<Tag, NT, NCH>(s.head, s.next, s.idx, lo, i, f, mass, value)) repeats |= 1u << i;
         store16_stream(gpart + ch * 16, C::pack(f));
       }
     }
     if (may_repeat && repeats)
-      correction_repeats<Tag, NT>(s.head, s.next, s.idx, lo, repeats, NCH, mass, value,
+      correction_repeats<Tag, NT, NCH>(s.head, s.next, s.idx, lo, repeats, NCH, mass, value,
                                   [&](int column, float v) { store_from_float(grow, Tag::id, column, v); });
     if (!IN_REGISTERS) {
       __syncthreads();      // dense stores are ordered before the sparse corrections
@@ -885,9 +886,10 @@ static int launch_split(TopkParams p, int parts, hipStream_t st) {
 // Rows of up to 1024 x 16 chunks are cut into parts of 256 x 16 chunks, as many as hold columns (a
 // part without columns would have no maximum to publish); `forced` (the DL_TOPK_PARTS field of the
 // call's flags) = 1, 2 or 4 overrides that for such rows where every part still gets columns.
-static int split_parts(int64_t nch, int forced) {
+static int split_parts(int64_t nch, int forced, bool fine = false) {
+  if (fine && nch > 256 * 4 && nch <= (int64_t)MAX_PARTS * 256 * 4) return (int)((nch + 256 * 4 - 1) / (256 * 4));
   if (nch <= 512 * 16) return 1;
-  const int parts = (int)((nch + 256 * 16 - 1) / (256 * 16));      // 3 .. MAX_PARTS parts of 256 x 16 chunks
+  const int parts = (int)((nch + 256 * 16 - 1) / (256 * 16));      // 3 .. MAX_COARSE_PARTS parts of 256 x 16 chunks
   if (nch > 1024 * 16) return parts;
   if (forced == 1 || forced == 2 || (forced == 4 && parts == 4)) return forced;
   return parts;
@@ -897,8 +899,9 @@ static int split_parts(int64_t nch, int forced) {
 // workgroup, chunks per thread, column parts per row (parts > 1: the split kernels, which need the
 // exchange workspace: `split_ok`).  NT == 0: none (rows too wide: the streaming kernel).
 struct FklShape { int NT, NCH, parts; };
-static FklShape fkl_shape(int64_t nch, int bytes, int forced_parts, bool split_ok) {
-  if (nch > (int64_t)MAX_PARTS * 256 * 16) return {0, 0, 0};
+static FklShape fkl_shape(int64_t nch, int bytes, int forced_parts, bool split_ok, bool fine = false) {
+  if (nch > (int64_t)MAX_COARSE_PARTS * 256 * 16) return {0, 0, 0};
+  if (fine && split_ok && nch > 256 * 4 && nch <= (int64_t)MAX_PARTS * 256 * 4) return {256, 4, split_parts(nch, forced_parts, true)};
   if (nch <= 256 * 4) return {256, 4, 1};
   if (nch <= 256 * 8) return {256, 8, 1};
   // 4-byte logits: 8 chunks per thread from twice the threads keep the corrections in registers
@@ -916,11 +919,16 @@ template <class Tag, bool MULTI>
 static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipStream_t st) {
   const int64_t nch = p.V / Tag::epc;
   const int forced = (p.flags >> DL_TOPK_PARTS_SHIFT) & 15;
-  const int want = split_parts(nch, forced);
+  const bool fine = !MULTI && (p.flags & DL_TOPK_FINE_PARTS) != 0 &&
+                    ws_bytes >= RetryList::bytes(p.n_rows, split_parts(nch, forced, true));
+  const int want = split_parts(nch, forced, fine);
   const bool split_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, want) && p.n_rows * want <= 0x7fffffffLL;
-  const FklShape sh = aligned ? fkl_shape(nch, Tag::bytes, forced, split_ok) : FklShape{0, 0, 0};
+  const FklShape sh = aligned ? fkl_shape(nch, Tag::bytes, forced, split_ok, fine) : FklShape{0, 0, 0};
   switch (sh.NT * 100 + sh.NCH) {
-    case 256 * 100 + 4: return launch_reg<Tag, 256, 4, MULTI>(p, st);
+    case 256 * 100 + 4:
+      if constexpr (!MULTI)
+        if (sh.parts > 1) return launch_split<Tag, 256, 4, MULTI>(p, sh.parts, st);
+      return launch_reg<Tag, 256, 4, MULTI>(p, st);
     case 256 * 100 + 8: return launch_reg<Tag, 256, 8, MULTI>(p, st);
     case 512 * 100 + 8:
       if constexpr (Tag::bytes == 4) return launch_reg<Tag, 512, 8, MULTI>(p, st);

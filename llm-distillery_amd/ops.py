@@ -108,12 +108,14 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
     if want_grad:
         grad = _grad_target(grad_out, R, V, x.dtype, dev)
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
-    if parts not in (0, 1, 2, 4):
-        raise ValueError("parts must be 0 (automatic), 1, 2 or 4")
+    if parts not in (0, 1, 2, 4, 16):
+        raise ValueError("parts must be 0 (automatic), 1, 2, 4 or 16 (parts of 1024 chunks, up to 16 per row)")
     flags = (_lib.DL_TOPK_UNIQUE_IDS if unique_ids else 0) | (_lib.DL_TOPK_NO_WAIT if no_wait else 0) | \
-        (parts << _lib.DL_TOPK_PARTS_SHIFT)
+        (_lib.DL_TOPK_FINE_PARTS if parts == 16 else parts << _lib.DL_TOPK_PARTS_SHIFT)
     lib = _lib.load()
     ws_bytes = lib.dl_div_topk_workspace_bytes(KINDS[kind], _DT[x.dtype], R, V) if want_grad else 0
+    if parts == 16 and want_grad:
+        ws_bytes = R * 16 * 20 + 16
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     with torch.cuda.device(dev):
         st = lib.dl_div_topk(KINDS[kind], x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr,
@@ -461,3 +463,21 @@ def copy16(src: torch.Tensor, dst: torch.Tensor) -> None:
     with torch.cuda.device(src.device):
         st = _lib.load().dl_copy16(src.data_ptr(), dst.data_ptr(), n, _stream_ptr(src.device))
     _lib.check(st, "dl_copy16")
+
+
+def copy_rows(src: torch.Tensor, dst: torch.Tensor, threads: int, chunks: int, parts_on_one_xcd: bool = True,
+              wave_major: bool = True, lds_kb: int = 0) -> None:
+    """Copy of a contiguous [rows, width] tensor in the access shape of the row kernels (dl_copy_rows):
+    the yardstick for what a bare copy reaches with `threads` x `chunks` 16-byte chunks per workgroup.
+    `wave_major`: every wave owns `chunks` KiB in one piece; `lds_kb`: LDS held per workgroup, which
+    bounds the workgroups per CU at 160 / lds_kb."""
+    _dev(src, "src"), _dev(dst, "dst", src.device)
+    if src.dim() != 2 or not (src.is_contiguous() and dst.is_contiguous()) or src.shape != dst.shape or src.dtype != dst.dtype:
+        raise RuntimeError("copy_rows needs two contiguous [rows, width] tensors of one shape and dtype")
+    if not 0 <= int(lds_kb) <= 64:
+        raise ValueError("lds_kb must be 0..64")
+    flags = (1 if parts_on_one_xcd else 0) | (2 if wave_major else 0) | (int(lds_kb) << 8)
+    with torch.cuda.device(src.device):
+        st = _lib.load().dl_copy_rows(src.data_ptr(), dst.data_ptr(), src.shape[0], src.shape[1] * src.element_size(), int(threads),
+                                      int(chunks), flags, _stream_ptr(src.device))
+    _lib.check(st, "dl_copy_rows")

@@ -97,3 +97,17 @@ def test_topk_divergence_index_handling(D, case):
         gref = gref[0] / T
         err = (grad[r].double() - gref).abs()
         assert (err <= O.storage_tolerance(gref, torch.float32, 2e-4)).all(), float(err.max())
+
+
+@pytest.mark.parametrize("threads,chunks", [(256, 2), (256, 4), (256, 8), (256, 12), (256, 16), (512, 4), (512, 8), (512, 16),
+                                            (1024, 4), (1024, 16)])
+@pytest.mark.parametrize("one_xcd,wave_major,lds_kb", [(True, True, 0), (False, False, 0), (True, False, 40), (False, True, 64)])
+def test_row_shaped_copy_is_a_copy(D, threads, chunks, one_xcd, wave_major, lds_kb):
+    # the bandwidth yardstick moves every byte exactly once: ragged last part, a row count that is not a multiple of 8
+    g = torch.Generator().manual_seed(threads + chunks)
+    src = torch.randint(-2 ** 31, 2 ** 31 - 1, (13, 4 * 5003), generator=g, dtype=torch.int32).to(DEV)
+    dst = torch.full_like(src, 7)
+    D.copy_rows(src, dst, threads, chunks, one_xcd, wave_major, lds_kb)
+    assert torch.equal(src, dst)
+    with pytest.raises(RuntimeError):
+        D.copy_rows(src, dst, 128, 3, one_xcd)

@@ -227,6 +227,21 @@ def test_rows_cut_into_three_parts(D, V, dtype):
     _check(D, "fkl", logits, tv, ti, T=1.1, hooks={"parts": 1})
 
 
+@pytest.mark.parametrize("V,dtype,K", [(128256, torch.bfloat16, 200), (32000, torch.bfloat16, 400), (32000, torch.float32, 300),
+                                       (8200, torch.float16, 64), (40000, torch.float32, 700), (131072, torch.float16, 32)])
+def test_rows_cut_into_parts_of_1024_chunks(D, V, dtype, K):
+    """The finer cut (up to 16 parts of 256 threads x 4 chunks per row): the oracle's numbers, with
+    repeated ids, masked rows, waiting or not."""
+    logits, tv, ti = _case(21, V, K, dtype, 47, std=3.0)
+    ti[3, 5] = ti[3, 9]
+    ti[6, :] = ti[6, 0]
+    valid = torch.ones(21, dtype=torch.bool)
+    valid[[2, 20]] = False
+    waited = _check(D, "fkl", logits, tv[:19], ti[:19], T=1.2, valid=valid, hooks={"parts": 16})
+    retried = _check(D, "fkl", logits, tv[:19], ti[:19], T=1.2, valid=valid, hooks={"parts": 16, "no_wait": True})
+    assert torch.equal(waited, retried)
+
+
 def test_a_column_part_that_holds_only_minus_infinity(D):
     """A masked stretch of the vocabulary (-inf logits) as wide as a whole column part: that part has
     no finite maximum; its columns get zero gradient and the row's statistics come from the others."""
