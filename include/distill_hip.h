@@ -337,16 +337,24 @@ int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_student, in
  * get replica slots (n_student rounded up to 4, + j), *n_extra_out in all, folded into the id's
  * slot after the last tile as listed in `fold` (int32 triples: id, first replica slot, replica
  * count).  The teacher vocabulary is cut into tiles of *tile_out ids; for tile k and wave w, rows
- * row_off[16k + w] .. row_off[16k + w + 1] of `ent` hold 64 entries each (one per lane), per thread
- * sorted by (slot, t).  A thread adds up runs of entries of one slot and stores slot + running sum
- * after every entry: bit 31 of an entry = first of its run, bits 15-30 = the slot on the run's last
- * entry and the lane's spare slot (64 of them behind the replicas) on the others, bits 0-14 =
- * 4 * (t - k * tile).  Padding = a first entry on the spare slot with offset 0; every (tile, wave)
- * list is padded to a multiple of 8 rows, at least 8.  Between tiles a slot may change hands.
+ * (row_off[16k + w] & ~3) .. (row_off[16k + w + 1] & ~3) of `ent` (64 dwords per row) hold the
+ * entries of the wave's 64 threads, per thread sorted by (slot, t), in one of two formats:
+ *   general (bit 0 of row_off[16k + w] clear): batches of 8 entries per lane, 8 rows each, the
+ *     entries of lane l in dwords [8l, 8l + 8) of the batch.  A thread adds up runs of entries of one
+ *     slot and stores slot + running sum after every entry: bit 31 of an entry = first of its run,
+ *     bits 15-30 = the slot on the run's last entry and the lane's spare slot (64 of them behind the
+ *     replicas) on the others, bits 0-14 = 4 * (t - k * tile).  Padding = a first entry on the spare
+ *     slot with offset 0, ahead of the lane's entries.
+ *   packed (bit 0 set: every lane holds at most one run of at most 8 entries): 4 rows, the lane's 4
+ *     dwords at [4l, 4l + 4), two 16-bit fields per dword, entries in order from the low field of
+ *     dword 0; bits 2-15 of a field = 4 * (t - k * tile), or 4 * tile (words the kernels keep at
+ *     zero) for padding, which comes first; the low two bits of the eight fields together are the
+ *     slot: field 2j carries its bits 2j, 2j + 1, field 2j + 1 its bits 8 + 2j, 9 + 2j.
+ * Between tiles a slot may change hands.
  * Call once with row_off = ent = fold = NULL to learn *tile_out, *ent_rows_out, *n_fold_out and
  * *n_extra_out, allocate row_off int32 [16 * ceil(n_teacher / tile) + 1], ent uint32
  * [64 * ent_rows] and fold int32 [3 * n_fold], call again.
- * DL_ERR_LIMIT: the student vocabulary is too wide for a plan (fp32 marginal + 64 spare slots + 16 KiB tile must fit 159 KiB).
+ * DL_ERR_LIMIT: the student vocabulary is too wide for a plan (fp32 marginal + 64 spare slots + 16 KiB tile + 16 bytes must fit 159 KiB).
  */
 int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int64_t n_student, int* tile_out,
                            int32_t* row_off, uint32_t* ent, int64_t ent_rows_capacity, int64_t* ent_rows_out,

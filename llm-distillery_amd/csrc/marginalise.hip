@@ -49,11 +49,27 @@ __host__ __device__ inline int64_t plan_slot_words(int64_t Vs, int n_extra) {
   return ((Vs + 3) & ~(int64_t)3) + (((int64_t)n_extra + 3) & ~(int64_t)3) + PLAN_SPARE_SLOTS;
 }
 
-// Plan entry: bit 31 = first entry of a run of one slot in its thread's list of the tile; bits
-// 15-30 = the slot on the last entry of the run, the lane's spare slot on the others; bits 0-14 =
-// byte offset of the probability inside the tile.  Padding is a first entry on the spare slot.
+// Plan entry of a general list: bit 31 = first entry of a run of one slot in its thread's list of
+// the tile; bits 15-30 = the slot on the last entry of the run, the lane's spare slot on the others;
+// bits 0-14 = byte offset of the probability inside the tile.  Padding is a first entry on the spare
+// slot.  A batch is 8 entries per lane, lane-major: the entries of lane l are dwords [8l, 8l + 8) of
+// the batch's 512, fetched with two 16-byte loads.
 constexpr int PLAN_SLOT_SHIFT = 15;
 constexpr unsigned PLAN_OFFSET_MASK = 0x7ffcu, PLAN_SLOT_MASK = 0xffffu;
+constexpr int PLAN_EB = 8;           // entries per batch
+// Packed list (every lane holds at most one run, at most 8 entries): 4 dwords per lane, lane-major, one
+// 16-byte load.  Every dword holds two 16-bit fields; bits 2-15 of a field are the byte offset of a
+// probability inside the tile, or of the zero words behind the tile for padding (first in the lane's
+// list); the low two bits of the eight fields together are the lane's slot: field 2j carries slot bits
+// 2j and 2j + 1, field 2j + 1 bits 8 + 2j and 9 + 2j.
+constexpr int PLAN_PACKED_ROWS = 4;  // rows of 64 dwords a packed list takes in the entry array
+constexpr int PLAN_ZERO_WORDS = 4;   // LDS words behind the tile that stay 0
+
+struct PlanBatch { u32x4 lo, hi; };
+
+__device__ __forceinline__ float plan_tile_value(const float* tile, unsigned byte_offset) {
+  return *reinterpret_cast<const float*>(reinterpret_cast<const char*>(tile) + byte_offset);
+}
 
 // Marginal of one teacher row into marg[0, Vs) (LDS, zeroed here) along a plan; `tile` is LDS
 // scratch of plan_tile floats.  fp32 probabilities, 16-byte aligned rows.
@@ -64,13 +80,11 @@ constexpr unsigned PLAN_OFFSET_MASK = 0x7ffcu, PLAN_SLOT_MASK = 0xffffu;
 // slot, which nobody reads for its value.  A slot belongs to one thread inside a tile and has one
 // run per thread and tile, so reading all slots of a batch before its stores changes nothing.
 // The run totals are added as slot + (0 + v0 + v1 + ...), in list order.
-constexpr int PLAN_EB = 8;           // entries per batch
-
-__device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const float* tile, float* marg, float& run) {
+__device__ __forceinline__ void plan_consume(const PlanBatch& b, const float* tile, float* marg, float& run) {
+  const unsigned e[PLAN_EB] = {b.lo.x, b.lo.y, b.lo.z, b.lo.w, b.hi.x, b.hi.y, b.hi.z, b.hi.w};
   float val[PLAN_EB], base[PLAN_EB];
 #pragma unroll
-  for (int j = 0; j < PLAN_EB; ++j)
-    val[j] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(tile) + (e[j] & PLAN_OFFSET_MASK));
+  for (int j = 0; j < PLAN_EB; ++j) val[j] = plan_tile_value(tile, e[j] & PLAN_OFFSET_MASK);
 #pragma unroll
   for (int j = 0; j < PLAN_EB; ++j) base[j] = marg[(e[j] >> PLAN_SLOT_SHIFT) & PLAN_SLOT_MASK];
 #pragma unroll
@@ -80,11 +94,38 @@ __device__ __forceinline__ void plan_consume(const unsigned (&e)[PLAN_EB], const
   }
 }
 
-// Teacher tiles (and the first batch of their lists) are fetched PLAN_DEPTH tiles ahead, into
-// registers.  Measured at depths 1-5 on 8192 rows of 152064 -> 32000: 1.40, 1.44, 1.48, 1.51, 1.55 ms.
-// One tile ahead is enough: the consume phase of a tile outlasts the memory latency.
-constexpr int PLAN_DEPTH = 1;
+// A packed list: the same sum in the same order as plan_consume gives for a lane with one run (its
+// padding adds zeros ahead of the run), the slot read and written once.
+__device__ __forceinline__ void plan_consume_packed(const u32x4& d, const float* tile, float* marg) {
+  const unsigned w[4] = {d.x, d.y, d.z, d.w};
+  float val[PLAN_EB];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    val[2 * j] = plan_tile_value(tile, w[j] & 0xfffcu);
+    val[2 * j + 1] = plan_tile_value(tile, (w[j] >> 16) & 0xfffcu);
+  }
+  unsigned u = w[0] & 0x00030003u;
+#pragma unroll
+  for (int j = 1; j < 4; ++j) u |= (w[j] & 0x00030003u) << (2 * j);
+  const unsigned slot = (u & 0xffu) | ((u >> 8) & 0xff00u);
+  const float base = marg[slot];
+  float run = 0.f;
+#pragma unroll
+  for (int j = 0; j < PLAN_EB; ++j) run += val[j];
+  marg[slot] = base + run;
+}
 
+// The loop over the tiles keeps two kinds of loads in flight, always issued in the same order: the
+// first batch of the next tile's list (into the entry registers the current tile does not use) and,
+// behind it, the 16-byte loads of the tile after the next (into the registers the current tile's data
+// has just left for LDS); the loop is unrolled by two so that both register sets are addressed
+// statically.  Loads complete in issue order and the hardware counts them per wave, so every wait
+// names how many younger loads may stay in flight: the wait for a tile's entries, issued ahead of the
+// data of the tile behind it, leaves that data in flight, which gives every tile two iterations to
+// arrive.  That only works out if the order is the same on every path into the loop, which the
+// scheduling barriers pin.  (With the entries of the first tile issued ahead of its data, as the
+// compiler had it, every wait in the loop became a wait for all but one or none of the loads: one
+// tile in flight whatever the depth, and the entries' trip to L2 and back waited for in full.)
 __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p, const char* prow, float* marg,
                                                             float* tile) {
   const int tid = threadIdx.x, lane = tid & (WAVE - 1);
@@ -98,72 +139,92 @@ __device__ __forceinline__ void accumulate_marginal_planned(const MargParams& p,
   const int64_t n4 = p.Vt / 4;
   const int n_slots = (int)plan_slot_words(p.Vs, p.plan_n_extra);
   for (int j = tid; j < n_slots; j += MARG_NT) marg[j] = 0.f;
-  u32x4 tbuf[PLAN_DEPTH][2];
+  if (tid < PLAN_ZERO_WORDS) tile[TS + tid] = 0.f;  // the tile's stores never reach these
+  // Byte offsets inside a tile are 32-bit and the tile's base is uniform: loads with a scalar base.
+  // Unconditional load from a clamped offset: with branch-free loads the compiler knows how many are
+  // in flight and never has to drain the whole queue.  What a clamped load brings is never used: no
+  // entry points behind the end of the row, and a select on the value here would make the thread
+  // wait for the load right away instead of two tiles later.
+  u32x4 tbuf[2][2];
   auto fetch_tile = [&](int k, u32x4 (&buf)[2]) {
+    const bool in_row = k < ntiles;
+    const char* base = prow + (in_row ? (int64_t)k * TS * 4 : 0);
+    const int left = in_row ? (int)(n4 - (int64_t)k * q_tile) : 0;      // 16-byte units from the tile's start to the row's end
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      // Unconditional load from a clamped address: with branch-free loads the compiler knows how
-      // many are in flight and never has to drain the whole queue.  What a clamped load brings is
-      // never used: no entry points behind the end of the row, and a select on the value here
-      // would make the thread wait for the load right away instead of PLAN_DEPTH tiles later.
-      const int64_t c = (int64_t)k * q_tile + (int64_t)u * MARG_NT + tid;
-      const bool live = u * MARG_NT + tid < q_tile && c < n4;
-      buf[u] = load16_stream(prow + (live ? c : 0) * 16);
+      const int c = u * MARG_NT + tid;
+      const unsigned off = (c < q_tile && c < left) ? (unsigned)c * 16u : 0u;
+      buf[u] = load16_stream(base + off);
     }
-  };
-  // every (tile, wave) list of the plan is a whole number of batches (padding entries included)
-  auto fetch_entries = [&](int r_first, unsigned (&e)[PLAN_EB]) {
-    const unsigned* at = p.plan_ent + (int64_t)r_first * WAVE + lane;
-#pragma unroll
-    for (int j = 0; j < PLAN_EB; ++j) e[j] = at[j * WAVE];
   };
   // the constant address space tells the compiler that nothing in this kernel writes the offsets:
   // only then does it fetch them with scalar loads
   typedef const __attribute__((address_space(4))) int32_t* ConstI32;
   ConstI32 row_off = (ConstI32)p.plan_row_off;
-  // Per buffer in flight: the tile's data and the first batch of its list, both fetched PLAN_DEPTH
-  // tiles ahead.  Loads complete in issue order, so a thread that waits for the batch of the next
-  // tile also waits for everything issued before it: fetching the batches as far ahead as the
-  // tiles is what lets the tile loads stay in flight for several tiles.
-  unsigned ebuf[PLAN_DEPTH][PLAN_EB];
-  int r_first[PLAN_DEPTH], r_end[PLAN_DEPTH];
-  auto list_of = [&](int k, int& first, int& end) {  // behind the last tile: the plan's first batch, fetched and dropped
-    first = end = 0;
+  // Row numbers are multiples of 4; bit 0 of a list's first row number says that the list is packed.
+  // Behind the last tile: the plan's first list, fetched and dropped.
+  struct List { int first, end, packed; };
+  auto list_of = [&](int k) {
+    List l{0, 0, 0};
     if (k < ntiles) {
-      first = row_off[k * NW + w];
-      end = row_off[k * NW + w + 1];
+      const int a = row_off[k * NW + w], b = row_off[k * NW + w + 1];
+      l.first = a & ~3;
+      l.end = b & ~3;
+      l.packed = a & 1;
+    }
+    return l;
+  };
+  // (the first batch of) a list: one 16-byte load per lane if packed, else two
+  auto fetch_batch = [&](int r_first, int packed, PlanBatch& b) {
+    const unsigned* at = p.plan_ent + (int64_t)r_first * WAVE;          // uniform
+    if (packed) {
+      b.lo = *reinterpret_cast<const u32x4*>(at + (unsigned)lane * 4u);
+    } else {
+      b.lo = *reinterpret_cast<const u32x4*>(at + (unsigned)lane * 8u);
+      b.hi = *reinterpret_cast<const u32x4*>(at + (unsigned)lane * 8u + 4u);
     }
   };
-#pragma unroll
-  for (int d = 0; d < PLAN_DEPTH; ++d) {
-    fetch_tile(d, tbuf[d]);
-    list_of(d, r_first[d], r_end[d]);
-    fetch_entries(r_first[d], ebuf[d]);
-  }
+  PlanBatch e_even, e_odd;
+  List cur = list_of(0), next = list_of(1);           // the descriptors run two tiles ahead of the entries
+  fetch_tile(0, tbuf[0]);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_batch(cur.first, cur.packed, e_even);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_tile(1, tbuf[1]);
+  __builtin_amdgcn_sched_barrier(0);
   float run = 0.f;
-  auto do_tile = [&](int k, u32x4 (&buf)[2], unsigned (&e)[PLAN_EB], int& first, int& end) {
+  auto do_tile = [&](int k, u32x4 (&buf)[2], PlanBatch& e, PlanBatch& e_next) {
     __syncthreads();                                 // previous tile fully consumed (first pass: marg zeroed)
 #pragma unroll
     for (int u = 0; u < 2; ++u)
       if (u * MARG_NT + tid < q_tile) *reinterpret_cast<u32x4*>(tile + ((int64_t)u * MARG_NT + tid) * 4) = buf[u];
     __syncthreads();
-    fetch_tile(k + PLAN_DEPTH, buf);                 // refill this buffer, PLAN_DEPTH tiles ahead
-    int n_first, n_end;
-    list_of(k + PLAN_DEPTH, n_first, n_end);
-    plan_consume(e, tile, marg, run);
-    for (int r = first + PLAN_EB; r < end; r += PLAN_EB) {     // a list longer than one batch (rare: not enough LDS
-      fetch_entries(r, e);                                     // for replicas): fetched on the spot
+    fetch_batch(next.first, next.packed, e_next);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch_tile(k + 2, buf);
+    __builtin_amdgcn_sched_barrier(0);
+    const List after = list_of(k + 2);
+    if (cur.packed) {                                          // wave-uniform: the flag came by a scalar load
+      plan_consume_packed(e.lo, tile, marg);
+    } else {
       plan_consume(e, tile, marg, run);
+      for (int r = cur.first + PLAN_EB; r < cur.end; r += PLAN_EB) {   // a list longer than one batch (rare: not enough LDS
+        fetch_batch(r, 0, e);                                          // for replicas): fetched on the spot
+        plan_consume(e, tile, marg, run);
+      }
     }
-    fetch_entries(n_first, e);
-    first = n_first;
-    end = n_end;
+    cur = next;
+    next = after;
   };
-  for (int k = 0; k < ntiles; k += PLAN_DEPTH) {     // unrolled by the depth: buffers are addressed statically
-#pragma unroll
-    for (int d = 0; d < PLAN_DEPTH; ++d)
-      if (k + d < ntiles) do_tile(k + d, tbuf[d], ebuf[d], r_first[d], r_end[d]);
+  // unrolled by two: the registers are addressed statically.  No path may enter the loop body with a
+  // different set of loads in flight than the others, or every wait falls back to the worst case: an
+  // odd last tile is therefore a third copy behind the loop, not a skipped second half.
+  int k = 0;
+  for (; k + 1 < ntiles; k += 2) {
+    do_tile(k, tbuf[0], e_even, e_odd);
+    do_tile(k + 1, tbuf[1], e_odd, e_even);
   }
+  if (k < ntiles) do_tile(k, tbuf[0], e_even, e_odd);
   __syncthreads();
   // replicas into their id's slot: own slot first, then the replicas in ascending order
   for (int f = tid; f < p.plan_n_fold; f += MARG_NT) {
@@ -243,7 +304,7 @@ __global__ __launch_bounds__(MARG_NT) void marginalise_map_kernel(const MargPara
   const char* prow = reinterpret_cast<const char*>(p.probs) + r * p.p_stride * pb;
   float* out = p.marg + r * p.marg_stride;
   if (VEC && p.plan_ent) {
-    float* marg = acc + p.plan_tile;                // the tile sits first: its addresses are then plain offsets
+    float* marg = acc + p.plan_tile + PLAN_ZERO_WORDS;      // the tile sits first: its addresses are then plain offsets
     accumulate_marginal_planned(p, prow, marg, acc);
     for (int j = threadIdx.x; j < p.Vs; j += MARG_NT) out[j] = p.out_log ? logf(marg[j]) : marg[j];
     return;
@@ -325,7 +386,7 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
   const char* prow = reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb;
   float* marg = acc;
   if (VEC && p.plan_ent) {
-    marg = acc + p.plan_tile;                    // the tile sits first: its addresses are then plain offsets
+    marg = acc + p.plan_tile + PLAN_ZERO_WORDS;  // the tile sits first: its addresses are then plain offsets
     rows.load(srow, p.Vs / 8);                   // in flight during the accumulation
     accumulate_marginal_planned(p, prow, marg, acc);
   } else {
@@ -379,7 +440,7 @@ static size_t attach_plan(dl::MargParams& p, const int32_t* plan_row_off, const 
   if (!plan_row_off || !plan_ent || !vec) return lds_without_plan;
   if (plan_tile < 4096 || plan_tile > 8192 || plan_tile % 1024) return lds_without_plan;
   if (plan_n_fold < 0 || plan_n_extra < 0 || (plan_n_fold > 0 && !plan_fold)) return lds_without_plan;
-  const size_t need = (size_t)dl::plan_slot_words(p.Vs, plan_n_extra) * 4 + (size_t)plan_tile * 4;
+  const size_t need = (size_t)dl::plan_slot_words(p.Vs, plan_n_extra) * 4 + (size_t)(plan_tile + dl::PLAN_ZERO_WORDS) * 4;
   if (need > (size_t)dl::MARG_MAX_DYN_LDS) return lds_without_plan;
   p.plan_row_off = plan_row_off; p.plan_ent = plan_ent; p.plan_tile = plan_tile;
   p.plan_fold = plan_fold; p.plan_n_fold = plan_n_fold; p.plan_n_extra = plan_n_extra;

@@ -120,20 +120,30 @@ extern "C" int dl_csr_from_map(const int32_t* t2s, int64_t n_teacher, int64_t n_
 // come out level, which matters because every wave of the workgroup waits for the longest one.
 // The tile size is chosen among the multiples of 1024 ids from 8192 down to 4096: a smaller tile
 // leaves more LDS for replicas (shorter lists when a few ids are very hot) but costs more barriers.
-// For tile k and wave w, rows row_off[k*16 + w] .. row_off[k*16 + w + 1] of `ent` hold, 64 entries
-// per row (one per lane), the entries of the wave's threads, each thread's entries sorted by
-// (slot, t).  A thread adds up a run of entries of one slot and stores slot + running sum after
-// every entry, so only the run's last entry may name the slot: bits 15-30 hold the slot there and
-// the lane's spare slot (behind the replicas, one per lane) on the other entries; bit 31 marks the
-// first entry of a run (the running sum restarts); bits 0-14 hold 4 * (t - k*tile), the byte offset
-// inside the tile.  Padding is a first entry on the spare slot with offset 0.  Every (tile, wave)
-// list is padded to whole batches of PLAN_BATCH rows, at least one, so the kernels fetch batches
-// without looking at the list's end.
+// For tile k and wave w, rows (row_off[k*16 + w] & ~3) .. (row_off[k*16 + w + 1] & ~3) of `ent` (64
+// dwords per row) hold the entries of the wave's threads, each thread's entries sorted by (slot, t).
+// Threads that hold at most one run in a tile are given the low thread numbers of that tile, the
+// others the high ones, so most waves consist of one-run threads only.  Two list formats:
+//   * general (bit 0 of row_off[k*16 + w] clear): batches of PLAN_BATCH entries per lane, 8 rows each,
+//     lane-major (the entries of lane l are dwords [8l, 8l + 8) of the batch), at least one batch.  A
+//     thread adds up a run of entries of one slot and stores slot + running sum after every entry, so
+//     only the run's last entry may name the slot: bits 15-30 hold the slot there and the lane's spare
+//     slot (behind the replicas, one per lane) on the other entries; bit 31 marks the first entry of a
+//     run (the running sum restarts); bits 0-14 hold 4 * (t - k*tile), the byte offset inside the tile.
+//     Padding is a first entry on the spare slot with offset 0; a thread's padding comes first and
+//     its entries last.
+//   * packed (bit 0 set; every lane holds at most one run of at most 8 entries): 4 rows, 4 dwords per
+//     lane, lane-major.  A dword holds two 16-bit fields, the lane's entries in order from the low
+//     field of dword 0 on; bits 2-15 of a field are the byte offset 4 * (t - k*tile), padding (first)
+//     points at the zero words behind the tile, 4 * tile; the low two bits of the eight fields
+//     together are the run's slot (the lane's spare slot if it has no entries): field 2j carries slot
+//     bits 2j and 2j + 1, field 2j + 1 bits 8 + 2j and 9 + 2j.
 namespace {
 
 constexpr int PLAN_NT = 1024, PLAN_WAVE = 64, PLAN_NW = PLAN_NT / PLAN_WAVE;
 constexpr int PLAN_BATCH = 8;                                 // entries per batch in the kernels
-constexpr int64_t PLAN_LDS_BUDGET = 160 * 1024 - 1024 - 64 * 4;   // dynamic LDS one workgroup may use, less the spare slots
+constexpr int64_t PLAN_LDS_BUDGET = 160 * 1024 - 1024 - 64 * 4 - 16;   // dynamic LDS one workgroup may use, less the spare slots and the zero words behind the tile
+constexpr int PLAN_PACKED_ROWS = 4;                           // rows a packed list takes
 constexpr int PLAN_SLOT_SHIFT = 15;
 
 struct PlanLayout {
@@ -233,6 +243,21 @@ void plan_deal_tile(const PlanLayout& L, const std::vector<std::pair<int32_t, in
     std::push_heap(th.begin(), th.end(), heavier);
   }
   for (auto& b : bucket) std::sort(b.begin(), b.end());       // (slot, t) ascending: slot in the high bits
+  // threads with at most one run first (in the order they were dealt), the others behind them
+  auto one_run = [&](const std::vector<uint32_t>& b) {
+    return b.empty() || (b.front() >> L.tile_bits) == (b.back() >> L.tile_bits);
+  };
+  std::stable_partition(bucket.begin(), bucket.end(), one_run);
+}
+
+// True if every thread of wave w holds at most one run and no more than one batch of entries.
+bool plan_wave_is_uniform(const PlanLayout& L, const std::vector<std::vector<uint32_t>>& bucket, int w) {
+  for (int l = 0; l < PLAN_WAVE; ++l) {
+    const auto& b = bucket[w * PLAN_WAVE + l];
+    if (b.size() > (size_t)PLAN_BATCH) return false;
+    if (!b.empty() && (b.front() >> L.tile_bits) != (b.back() >> L.tile_bits)) return false;
+  }
+  return true;
 }
 
 }  // namespace
@@ -290,25 +315,43 @@ extern "C" int dl_marginal_plan_build(const int32_t* t2s, int64_t n_teacher, int
     tile_entries(t2s, n_teacher, L, k, entries);
     plan_deal_tile(L, entries, bucket);
     for (int w = 0; w < PLAN_NW; ++w) {
+      const bool packed = plan_wave_is_uniform(L, bucket, w);
       size_t longest = 0;
       for (int l = 0; l < PLAN_WAVE; ++l) longest = std::max(longest, bucket[w * PLAN_WAVE + l].size());
       longest = std::max<size_t>(PLAN_BATCH, (longest + PLAN_BATCH - 1) / PLAN_BATCH * PLAN_BATCH);   // whole batches, at least one
+      const size_t list_rows = packed ? (size_t)PLAN_PACKED_ROWS : longest;
       if (ent) {
-        if (rows + (int64_t)longest > ent_rows_capacity) return DL_ERR_SHAPE;
-        for (size_t j = 0; j < longest; ++j)
-          for (int l = 0; l < PLAN_WAVE; ++l) {
-            const auto& b = bucket[w * PLAN_WAVE + l];
+        if (rows + (int64_t)list_rows > ent_rows_capacity) return DL_ERR_SHAPE;
+        uint32_t* out = ent + rows * PLAN_WAVE;
+        for (int l = 0; l < PLAN_WAVE; ++l) {
+          const auto& b = bucket[w * PLAN_WAVE + l];
+          if (packed) {
+            const uint32_t slot = b.empty() ? spare + (uint32_t)l : b.front() >> L.tile_bits;
+            for (int f = 0; f < PLAN_BATCH; ++f) {                              // padding first, the entries last
+              const int j = f - (PLAN_BATCH - (int)b.size());
+              const uint32_t offset = j >= 0 ? (b[j] & ((1u << L.tile_bits) - 1u)) : (uint32_t)L.tile;
+              const int slot_bit = (f & 1) ? 8 + (f & ~1) : f;                   // where the field's two slot bits come from
+              const uint32_t field = offset << 2 | ((slot >> slot_bit) & 3u);
+              uint32_t& d = out[l * 4 + f / 2];
+              d = (f & 1) ? (d | field << 16) : field;
+            }
+            continue;
+          }
+          for (size_t row = 0; row < longest; ++row) {
             uint32_t e = FIRST | (spare + (uint32_t)l) << PLAN_SLOT_SHIFT;
-            if (j < b.size()) {
+            if (row >= longest - b.size()) {                                    // padding first, the entries last
+              const size_t j = row - (longest - b.size());
               const uint32_t slot = b[j] >> L.tile_bits, offset = b[j] & ((1u << L.tile_bits) - 1u);
               const bool first = j == 0 || (b[j - 1] >> L.tile_bits) != slot;
               const bool last = j + 1 == b.size() || (b[j + 1] >> L.tile_bits) != slot;
               e = (first ? FIRST : 0u) | (last ? slot : spare + (uint32_t)l) << PLAN_SLOT_SHIFT | offset << 2;
             }
-            ent[(rows + (int64_t)j) * PLAN_WAVE + l] = e;
+            out[(row / PLAN_BATCH) * PLAN_BATCH * PLAN_WAVE + l * PLAN_BATCH + row % PLAN_BATCH] = e;
           }
+        }
       }
-      rows += (int64_t)longest;
+      if (row_off && packed) row_off[k * PLAN_NW + w] |= 1;
+      rows += (int64_t)list_rows;
       if (rows > 0x7fffffffLL) return DL_ERR_LIMIT;
       if (row_off) row_off[k * PLAN_NW + w + 1] = (int32_t)rows;
     }

@@ -57,6 +57,49 @@ def test_config5_vocabularies_at_full_size():
     assert off[-1] == 152064 and np.array_equal(np.sort(ind), np.arange(152064))
 
 
+ZERO = -1        # tile index of a packed list's padding: the words the kernels keep at zero behind the tile
+
+
+def _plan_lists(plan, Vs):
+    """Decodes a plan into what the kernels do with it: for every (tile, wave, lane) the list of steps
+    (restart, tile index or ZERO, slot stored to or None), for both list formats, with the format's own
+    invariants checked on the way.  Yields (k, w, lane, packed, steps, rows of the list)."""
+    tile = plan.tile
+    raw_off = plan.row_off.numpy()
+    assert ((raw_off & 2) == 0).all() and raw_off[-1] & 1 == 0
+    packed_flag, row_off = raw_off & 1, raw_off & ~3
+    ent = plan.ent.numpy().view(np.uint32).astype(np.int64)
+    assert row_off[0] == 0 and row_off[-1] == ent.shape[0]
+    n_pad = (Vs + 3) & ~3
+    spare0 = n_pad + ((plan.n_extra + 3) & ~3)
+    for kw in range(len(row_off) - 1):
+        k, w = divmod(kw, 16)
+        rows = ent[row_off[kw]:row_off[kw + 1]]
+        if packed_flag[kw]:
+            assert rows.shape[0] == 4                                        # 4 dwords per lane, lane-major
+            words = rows.reshape(64, 4)
+            for lane in range(64):
+                fields = [(int(words[lane, f // 2]) >> (16 * (f & 1))) & 0xffff for f in range(8)]
+                slot = 0
+                for f, v in enumerate(fields):
+                    slot |= (v & 3) << ((8 + (f & ~1)) if f & 1 else f)
+                offs = [v >> 2 for v in fields]
+                n_padding = sum(o == tile for o in offs)
+                assert all(o == tile for o in offs[:n_padding]) and all(o < tile for o in offs[n_padding:])   # padding first
+                assert n_padding < 8 or slot == spare0 + lane               # an idle lane parks on its spare slot
+                steps = [(f == 0, ZERO if o == tile else o, slot if f == 7 else None) for f, o in enumerate(offs)]
+                yield k, w, lane, True, steps, 4
+        else:
+            assert rows.shape[0] >= 8 and rows.shape[0] % 8 == 0            # whole batches of 8 entries per lane
+            batches = rows.reshape(-1, 64, 8)                                # [batch, lane, entry]
+            for lane in range(64):
+                col = batches[:, lane, :].reshape(-1)
+                first, slot, offset = (col >> 31).astype(bool), (col >> 15) & 0xffff, col & 0x7fff
+                assert (offset % 4 == 0).all() and (offset // 4 < tile).all()
+                steps = [(bool(f), int(o) // 4, None if sl == spare0 + lane else int(sl)) for f, o, sl in zip(first, offset, slot)]
+                yield k, w, lane, False, steps, rows.shape[0]
+
+
 def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     rng = np.random.default_rng(7)
     Vt, Vs = 20000, 3000
@@ -65,11 +108,9 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     plan = D.vocab_utils.MarginalPlan(t2s, Vs, "cpu")
     tile = plan.tile
     assert 4096 <= tile <= 8192 and tile % 1024 == 0
-    row_off = plan.row_off.numpy()
-    ent = plan.ent.numpy().view(np.uint32)
     fold = plan.fold.numpy()[:plan.n_fold]
     ntiles = -(-Vt // tile)
-    assert row_off.shape == (16 * ntiles + 1,) and row_off[0] == 0 and row_off[-1] == ent.shape[0]
+    assert plan.row_off.shape == (16 * ntiles + 1,)
     # replica slots sit behind the padded marginal, each belongs to exactly one hot id
     n_pad = (Vs + 3) & ~3
     slot_id = np.arange(n_pad + plan.n_extra)
@@ -82,32 +123,42 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
         cursor += cnt
     assert cursor == n_pad + plan.n_extra and plan.n_fold > 0       # the hot ids did get replicas
     seen = np.zeros(Vt, dtype=np.int32)
-    longest = []
-    for k in range(ntiles):
-        owner = {}                                                        # slots may change hands between tiles
-        for w in range(16):
-            rows = ent[row_off[16 * k + w]:row_off[16 * k + w + 1]]
-            longest.append(rows.shape[0])
-            assert rows.shape[0] >= 8 and rows.shape[0] % 8 == 0            # whole batches of the kernels
-            for lane in range(64):
-                col = rows[:, lane].astype(np.int64)
-                first, slot, offset = (col >> 31).astype(bool), (col >> 15) & 0xffff, col & 0x7fff
-                assert (offset % 4 == 0).all()
-                spare = n_pad + ((plan.n_extra + 3) & ~3) + lane          # where unfinished run totals are parked
-                ends = np.nonzero(slot != spare)[0]                      # the last entry of every run names the run's slot
-                n_live = ends[-1] + 1 if len(ends) else 0
-                assert (col[n_live:] == (1 << 31 | spare << 15)).all()   # padding only at the tail: restarts, parks, offset 0
-                starts = np.concatenate(([0], ends[:-1] + 1)) if len(ends) else ends
-                assert np.array_equal(np.nonzero(first[:n_live])[0], starts)        # the running sum restarts exactly at run starts
-                run_slot = slot[ends]
-                assert (np.diff(run_slot) > 0).all() and (run_slot < n_pad + plan.n_extra).all()   # one run per slot, ascending
-                for a, z, sl in zip(starts, ends, run_slot):
-                    t = offset[a:z + 1] // 4 + k * tile
-                    assert (np.diff(t) > 0).all() and (t < Vt).all()
-                    assert (t2s[t] == slot_id[sl]).all()                  # the entries land on a slot of their own id
-                    assert owner.setdefault(int(sl), w * 64 + lane) == w * 64 + lane      # one thread per LDS word inside a tile
-                    seen[t] += 1
+    longest, n_packed = [], 0
+    owner = {}                                                            # (tile, slot) -> thread: slots may change hands between tiles
+    runs_in_wave = {}
+    for k, w, lane, packed, steps, n_rows in _plan_lists(plan, Vs):
+        if lane == 0:
+            longest.append(n_rows)
+            n_packed += packed
+        # cut the steps into runs: a run starts where the running sum restarts and ends where a real slot is stored
+        runs, at = [], None
+        for restart, t, slot in steps:
+            if restart:
+                at = []
+            assert at is not None                                         # every list starts with a restart
+            at.append(t)
+            if slot is not None:
+                runs.append((slot, at))
+                at = None                                                 # the next entry must restart
+        live = [(slot, [t for t in ts if t != ZERO]) for slot, ts in runs if slot < n_pad + plan.n_extra]
+        live = [(slot, ts) for slot, ts in live if ts]
+        if not packed:
+            runs_in_wave[(k, w)] = (max(runs_in_wave.get((k, w), (0, 0))[0], len(live)), n_rows)
+        assert [sl for sl, _ in live] == sorted({sl for sl, _ in live})    # one run per slot, ascending
+        if live:
+            assert steps[-1][2] == live[-1][0]                            # padding comes first: the last run ends on the last row
+        for slot, ts in live:
+            t = np.asarray(ts) + k * tile
+            assert (np.diff(t) > 0).all() and (t < Vt).all()
+            assert (t2s[t] == slot_id[slot]).all()                        # the entries land on a slot of their own id
+            assert owner.setdefault((k, slot), w * 64 + lane) == w * 64 + lane      # one thread per LDS word inside a tile
+            seen[t] += 1
+        if packed:
+            assert len(live) <= 1
     assert np.array_equal(seen, (t2s >= 0).astype(np.int32))
+    # a list is packed exactly when every lane of the wave holds at most one run and no more than 8 entries
+    assert all(most > 1 or n_rows > 8 for most, n_rows in runs_in_wave.values())
+    assert n_packed >= 4 * ntiles                 # one-run threads are gathered in the low waves: half the entries sit on 8 ids
     # half of the entries sit on 8 ids: without replicas one thread would hold > 1200 entries of a tile
     assert max(longest) <= 4 * (tile // 1024)
     # too wide a student vocabulary: no plan, the atomic form remains
@@ -116,33 +167,26 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
 
 
 def _apply_plan(plan, probs, Vs):
-    """What the planned kernels compute, entry by entry in numpy: per tile and thread the running sum
-    restarts on bit 31, every entry stores slot + running sum into the slot its bits 15-30 name (spare
-    slots on unfinished runs), replicas are folded into their id after the last tile."""
+    """What the planned kernels compute, step by step in numpy: per tile and thread the running sum
+    restarts where the list says so, a general list stores slot + running sum after every entry (spare
+    slots on unfinished runs), a packed list once, behind its last entry; replicas are folded into their
+    id after the last tile."""
     tile = plan.tile
-    row_off = plan.row_off.numpy()
-    ent = plan.ent.numpy().view(np.uint32).astype(np.int64)
     n_pad = (Vs + 3) & ~3
     slots = np.zeros(n_pad + ((plan.n_extra + 3) & ~3) + 64, dtype=np.float32)
-    ntiles = -(-probs.size // tile)
-    for k in range(ntiles):
-        seg = np.zeros(tile, dtype=np.float32)
-        part = probs[k * tile:(k + 1) * tile]
-        seg[:part.size] = part
-        touched = {}
-        for w in range(16):
-            rows = ent[row_off[16 * k + w]:row_off[16 * k + w + 1]]
-            assert rows.shape[0] % 8 == 0 and rows.shape[0] >= 8
-            for lane in range(64):
-                run = np.float32(0)
-                for e in rows[:, lane]:
-                    slot, offset = (e >> 15) & 0xffff, (e & 0x7fff) >> 2
-                    assert slot < slots.size and offset < tile
-                    run = np.float32((0 if e >> 31 else run) + seg[offset])
-                    if slot < n_pad + plan.n_extra:      # a real slot: only this thread may touch it in this tile
-                        assert touched.setdefault(int(slot), (w, lane)) == (w, lane)
-                        slots[slot] = slots[slot] + run   # one store per run: slot value read before the batch == before the run
-                    # spare slots: value never used
+    touched, seg, seg_k = {}, None, -1
+    for k, w, lane, packed, steps, _ in _plan_lists(plan, Vs):
+        if k != seg_k:
+            seg = np.zeros(tile, dtype=np.float32)
+            part = probs[k * tile:(k + 1) * tile]
+            seg[:part.size] = part
+            seg_k, touched = k, {}
+        run = np.float32(0)
+        for restart, t, slot in steps:
+            run = np.float32((0 if restart else run) + (np.float32(0) if t == ZERO else seg[t]))
+            if slot is not None and slot < n_pad + plan.n_extra:   # a real slot: only this thread may touch it in this tile
+                assert touched.setdefault(int(slot), (w, lane)) == (w, lane)
+                slots[slot] = slots[slot] + run                    # one store per run: slot value read before the batch == before the run
     for sid, first, cnt in plan.fold.numpy()[:plan.n_fold]:
         for j in range(cnt):
             slots[sid] = slots[sid] + slots[first + j]
