@@ -366,6 +366,93 @@ struct LdsTeacherRows {
   }
 };
 
+// Reverse KL of the student row (in registers) against a marginal that sits in LDS as probabilities,
+// with its gradient; the same quantities as dense_stats<DL_RKL> + dense_grad_sweep<DL_RKL> on the
+// logarithm of the marginal, in three passes of fewer instructions (with one 1024-thread workgroup per
+// CU these passes run on the vector ALUs alone, no memory traffic to hide behind: 31 % of the
+// kernel's time before).  Log2 domain throughout:
+//   xt_j = log2(m_j) / T_t - bt        bt from the largest marginal (xt = -inf off the support)
+//   xs_j = s_j a_s - bs                bs from the largest student logit on the support
+//   S = sum_on 2^xs, T = sum 2^xt, W = sum_on 2^xs (xs - xt)
+//   RKL = (W / S - log2 S + log2 T) ln 2
+//   d RKL / d s_j = 2^xs_j (ln 2 / (T_s S)) ((xs_j - xt_j) - W / S)      on the support, else 0
+// Pass A: maxima.  Pass B: xt (written over the marginal), the three sums.  Pass C: gradient.
+template <class TagS, int NU>
+__device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float* red,
+                                                     const MargParams& p, int64_t r, char* grow) {
+  const int tid = threadIdx.x;
+  const float a_s = p.inv_T_s * LOG2E;
+  const auto marginal_of = [&](int64_t u, float (&m)[8]) {
+    const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
+    m[0] = m0.x; m[1] = m0.y; m[2] = m0.z; m[3] = m0.w; m[4] = m1.x; m[5] = m1.y; m[6] = m1.z; m[7] = m1.w;
+  };
+  float mmax = 0.f, ms = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NU; ++i) {
+    const int64_t u = (int64_t)i * MARG_NT + tid;
+    if (u < nunits) {
+      float sv[8], m[8];
+      s[i].unpack(sv);
+      marginal_of(u, m);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        mmax = fmaxf(mmax, m[e]);
+        ms = fmaxf(ms, m[e] > 0.f ? sv[e] : -INFINITY);
+      }
+    }
+  }
+  block_max2<MARG_NT>(mmax, ms, red);
+  if (!(mmax > 0.f)) {                              // the teacher row carried no mass at all
+    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    if (grow) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
+    return;
+  }
+  const float bt = fast_log2(mmax) * p.inv_T_t, bs = ms * a_s;
+  float ss = 0.f, stt = 0.f, w = 0.f;
+#pragma unroll
+  for (int i = 0; i < NU; ++i) {
+    const int64_t u = (int64_t)i * MARG_NT + tid;
+    if (u < nunits) {
+      float sv[8], m[8];
+      s[i].unpack(sv);
+      marginal_of(u, m);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xt = fmaf(fast_log2(m[e]), p.inv_T_t, -bt), xs = fmaf(sv[e], a_s, -bs);
+        const float es = fast_exp2(xs);
+        stt += fast_exp2(xt);
+        const bool on = m[e] > 0.f;
+        ss += on ? es : 0.f;
+        w += (on && es > 0.f) ? es * (xs - xt) : 0.f;
+        m[e] = xt;
+      }
+      *reinterpret_cast<float4*>(marg + u * 8) = float4{m[0], m[1], m[2], m[3]};        // own columns only: no barrier needed
+      *reinterpret_cast<float4*>(marg + u * 8 + 4) = float4{m[4], m[5], m[6], m[7]};
+    }
+  }
+  block_sum2<MARG_NT>(ss, stt, red);
+  w = block_sum<MARG_NT>(w, red);
+  const float wbar = w / ss;
+  if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - fast_log2(ss) + fast_log2(stt)) * LN2;
+  if (!grow) return;
+  const float k1 = p.inv_T_s * p.grad_scale * LN2 / ss;
+#pragma unroll
+  for (int i = 0; i < NU; ++i) {
+    const int64_t u = (int64_t)i * MARG_NT + tid;
+    if (u < nunits) {
+      float sv[8], xt[8], g[8];
+      s[i].unpack(sv);
+      marginal_of(u, xt);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xs = fmaf(sv[e], a_s, -bs);
+        g[e] = xt[e] > -INFINITY ? fast_exp2(xs) * k1 * ((xs - xt[e]) - wbar) : 0.f;
+      }
+      Unit<TagS>::store(grow, u, g);
+    }
+  }
+}
+
 template <class TagS, int NU, bool VEC>
 __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargParams p) {
   extern __shared__ __align__(16) float acc[];
@@ -393,16 +480,7 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
     rows.load(srow, p.Vs / 8);                   // in flight during the scatter
     accumulate_marginal<VEC>(p, prow, acc, 0, (int)p.Vs);
   }
-  for (int j = tid; j < p.Vs; j += MARG_NT) marg[j] = fast_log2(marg[j]) * LN2;    // log 0 = -inf: off the support
-  __syncthreads();
-  rows.lt = marg;
-  const DenseStats st = dense_stats<DL_RKL, MARG_NT>(rows, p.inv_T_s, p.inv_T_t, red);
-  const bool empty = st.tmax == -INFINITY;        // the teacher row carried no mass at all
-  if (tid == 0 && p.row_loss) p.row_loss[r] = empty ? 0.f : st.loss;
-  if (grow) {
-    if (empty) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
-    else dense_grad_sweep<DL_RKL, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
-  }
+  rkl_against_marginal<TagS, NU>(rows.s, rows.nunits, marg, red, p, r, grow);
 }
 
 static bool ok16(const void* ptr, int64_t stride, int eb) {
