@@ -40,9 +40,9 @@ struct MultiTeacher {
 // The same teachers prepared for the loss kernels (multi_prep_kernel): per teacher row the surviving
 // entries as (student id, log of the renormalised mass), dealt into one bucket per column part of
 // the loss kernel's row split, in stored order (teacher 0 first).  Bucket h of a row holds its first
-// `cap0` entries in first[(row * parts + h) * cap0 ...], padded with (-1, -inf) -- so the part's
-// workgroup fetches them by lane without knowing the count -- and whatever exceeds cap0 in the row's
-// share of `more`, buckets back to back.  head[row * 16 + h] = entries of bucket h (h < 8),
+// `cap0` entries in first[(row * parts + h) * cap0 ...] -- the part's workgroup fetches all cap0 slots
+// by lane before it knows the count, and keeps what lies below it: the slots behind are never written
+// -- and whatever exceeds cap0 in the row's share of `more`, buckets back to back.  head[row * 16 + h] = entries of bucket h (h < 8),
 // [8] = entries of the row, [9] = float bits of the sum of the renormalised masses (1 up to rounding).
 struct TeacherBuckets {
   const uint2* first; const uint2* more; const int* head;
@@ -181,7 +181,7 @@ __device__ __forceinline__ void teacher_gather(const char* row, int lo, int hi, 
 }
 
 // Prepared teachers (TeacherBuckets): the first J * NT = cap0 entries of this part's bucket, one per
-// lane and slot, fetched by position alone (padding reads as id -1); the bucket's and the row's entry
+// lane and slot, fetched by position alone (slots behind the count hold whatever was there); the bucket's and the row's entry
 // counts and the row's mass sum come along as same-address loads.
 struct BucketHead { int n; int total; float qsum; int more_at; };
 
@@ -324,7 +324,7 @@ __device__ __forceinline__ int bucket_finish(const TopkParams& p, const TopkLds&
 #pragma unroll
   for (int j = 0; j < J; ++j) {
     const int k = threadIdx.x + j * NT;
-    const bool ok = te.id[j] >= lo && te.id[j] < hi;      // anything else in a bucket is padding
+    const bool ok = k < hd.n && te.id[j] >= lo && te.id[j] < hi;      // what lies behind the bucket's count was never written
     s.idx[k] = ok ? te.id[j] : -1;
     s.t[k] = te.tv[j];
     s.q[k] = ok ? expf(te.tv[j]) : 0.f;

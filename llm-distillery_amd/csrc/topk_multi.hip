@@ -157,32 +157,46 @@ __global__ __launch_bounds__(PREP_ROWS * WAVE) void multi_prep_kernel(const Prep
   if (P > 4) at_lane[1] = wave_scan_packed(mine[1], total[1]);
   const auto field = [](const unsigned long long (&w)[2], int h) { return (int)((w[h >> 2] >> (16 * (h & 3))) & 0xffffull); };
 
-  uint2* first = p.first + trow * (int64_t)P * p.cap0;
-  uint2* more = p.more + trow * (int64_t)p.E;
+  // The entries go to the wave's own stretch of LDS first, bucket after bucket, and from there to
+  // memory in order: a lane's entries of one bucket lie up to J slots apart, so storing them straight
+  // from the registers is J instructions of 64 lanes in 64 different lines each, and the vector memory
+  // path takes a cycle per line; out of LDS a bucket leaves in whole 512-byte pieces.
+  extern __shared__ __align__(16) uint2 staged_rows[];
+  uint2* staged = staged_rows + (threadIdx.x / WAVE) * p.E;
+  unsigned long long start[2] = {0ull, 0ull};          // where bucket h begins in `staged`, packed like the counters
+  {
+    int run = 0;
+    for (int h = 0; h < P; ++h) {
+      start[h >> 2] |= (unsigned long long)run << (16 * (h & 3));
+      run += field(total, h);
+    }
+  }
 #pragma unroll
   for (int j = 0; j < J; ++j) {
     if (id[j] < 0) continue;
     const int h = P == 1 ? 0 : min(id[j] >> p.part_shift, P - 1);
-    int at = field(at_lane, h);
+    const int at = field(start, h) + field(at_lane, h);
     at_lane[h >> 2] += 1ull << (16 * (h & 3));
-    const uint2 e{(unsigned)id[j], __float_as_uint(tv[j] - tlse)};
-    if (at < p.cap0) {
-      first[(int64_t)h * p.cap0 + at] = e;
-    } else {
-      // rare: a bucket holds more than cap0 entries.  The overflow shares of the buckets lie back to
-      // back in the row's share of `more`.
-      at -= p.cap0;
-      for (int g = 0; g < h; ++g) at += max(field(total, g) - p.cap0, 0);
-      more[at] = e;
-    }
+    staged[at] = uint2{(unsigned)id[j], __float_as_uint(tv[j] - tlse)};
   }
-  // padding: what a part's workgroup reads beyond its entries says "no entry"
-  int n_row = 0;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  uint2* first = p.first + trow * (int64_t)P * p.cap0;
+  uint2* more = p.more + trow * (int64_t)p.E;
+  int spilled = 0;                                     // entries of lower buckets beyond their cap0: they lie back to back in `more`
   for (int h = 0; h < P; ++h) {
-    const int n = field(total, h);
-    n_row += n;
-    for (int k = n + lane; k < p.cap0; k += WAVE) first[(int64_t)h * p.cap0 + k] = uint2{0xffffffffu, 0xff800000u};
+    const int n = field(total, h), from = field(start, h);
+    for (int k = lane; k < n; k += WAVE) {
+      const uint2 e = staged[from + k];
+      if (k < p.cap0) first[(int64_t)h * p.cap0 + k] = e;
+      else more[spilled + k - p.cap0] = e;             // rare: a bucket holds more than cap0 entries
+    }
+    spilled += max(n - p.cap0, 0);
   }
+  // no padding: a part's workgroup reads cap0 slots of its bucket and goes by the count in the header
+  int n_row = 0;
+  for (int h = 0; h < P; ++h) n_row += field(total, h);
   if (lane < 16) {
     int v = lane < P ? field(total, lane & 7) : 0;
     if (lane == 8) v = n_row;
@@ -222,8 +236,9 @@ static bool multi_plan(int logits_dtype, int64_t n_rows, int64_t V, int E, int64
 template <int J, int VD, bool VEC>
 static void launch_prep_it(const PrepParams& p, hipStream_t st) {
   const dim3 grid((unsigned)((p.n_trows + PREP_ROWS - 1) / PREP_ROWS)), block(PREP_ROWS * WAVE);
-  if (p.idx_itype == DL_I32) hipLaunchKernelGGL((multi_prep_kernel<J, VD, I32, VEC>), grid, block, 0, st, p);
-  else hipLaunchKernelGGL((multi_prep_kernel<J, VD, I64, VEC>), grid, block, 0, st, p);
+  const size_t lds = (size_t)PREP_ROWS * p.E * sizeof(uint2);      // <= 64 KiB: E <= DL_MAX_TOPK
+  if (p.idx_itype == DL_I32) hipLaunchKernelGGL((multi_prep_kernel<J, VD, I32, VEC>), grid, block, lds, st, p);
+  else hipLaunchKernelGGL((multi_prep_kernel<J, VD, I64, VEC>), grid, block, lds, st, p);
 }
 
 template <int J, bool VEC>
