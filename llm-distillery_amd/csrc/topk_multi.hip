@@ -53,7 +53,9 @@ __device__ __forceinline__ unsigned long long wave_scan_packed(unsigned long lon
 // lane) + j % 4 of teacher j / 4 / S, S = ceil(Kt / 256); J a multiple of 4) -- a quarter of the load
 // instructions, which is what bounds this kernel: the CU's vector memory path takes about as long
 // for a 4-byte-per-lane load as for a 16-byte one.
-template <int J, int VD, int IT, bool VEC>
+// WIDE: more than four buckets per row (a second packed word of counters; with four or fewer every
+// reference to it folds away).
+template <int J, int VD, int IT, bool VEC, bool WIDE>
 __global__ __launch_bounds__(PREP_ROWS * WAVE) void multi_prep_kernel(const PrepParams p) {
   const MultiTeacher& m = p.mt;
   const int lane = threadIdx.x & (WAVE - 1);
@@ -140,8 +142,8 @@ __global__ __launch_bounds__(PREP_ROWS * WAVE) void multi_prep_kernel(const Prep
   if (tmax > -INFINITY) {
     float part = 0.f;
 #pragma unroll
-    for (int j = 0; j < J; ++j) part += expf(tv[j] - tmax);
-    tlse = tmax + logf(wave_sum(part));
+    for (int j = 0; j < J; ++j) part += fast_exp2((tv[j] - tmax) * LOG2E);
+    tlse = tmax + fast_log2(wave_sum(part)) * LN2;
   }
 
   // buckets: counters of four buckets share a 64-bit word, 16 bits each
@@ -150,12 +152,12 @@ __global__ __launch_bounds__(PREP_ROWS * WAVE) void multi_prep_kernel(const Prep
   for (int j = 0; j < J; ++j) {
     if (id[j] < 0) continue;
     const int h = P == 1 ? 0 : min(id[j] >> p.part_shift, P - 1);
-    mine[h >> 2] += 1ull << (16 * (h & 3));
+    mine[WIDE ? h >> 2 : 0] += 1ull << (16 * (h & 3));
   }
   unsigned long long total[2] = {0ull, 0ull}, at_lane[2] = {0ull, 0ull};
   at_lane[0] = wave_scan_packed(mine[0], total[0]);
-  if (P > 4) at_lane[1] = wave_scan_packed(mine[1], total[1]);
-  const auto field = [](const unsigned long long (&w)[2], int h) { return (int)((w[h >> 2] >> (16 * (h & 3))) & 0xffffull); };
+  if (WIDE) at_lane[1] = wave_scan_packed(mine[1], total[1]);
+  const auto field = [](const unsigned long long (&w)[2], int h) { return (int)((w[WIDE ? h >> 2 : 0] >> (16 * (h & 3))) & 0xffffull); };
 
   // The entries go to the wave's own stretch of LDS first, bucket after bucket, and from there to
   // memory in order: a lane's entries of one bucket lie up to J slots apart, so storing them straight
@@ -167,7 +169,7 @@ __global__ __launch_bounds__(PREP_ROWS * WAVE) void multi_prep_kernel(const Prep
   {
     int run = 0;
     for (int h = 0; h < P; ++h) {
-      start[h >> 2] |= (unsigned long long)run << (16 * (h & 3));
+      start[WIDE ? h >> 2 : 0] |= (unsigned long long)run << (16 * (h & 3));
       run += field(total, h);
     }
   }
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(PREP_ROWS * WAVE) void multi_prep_kernel(const Prep
     if (id[j] < 0) continue;
     const int h = P == 1 ? 0 : min(id[j] >> p.part_shift, P - 1);
     const int at = field(start, h) + field(at_lane, h);
-    at_lane[h >> 2] += 1ull << (16 * (h & 3));
+    at_lane[WIDE ? h >> 2 : 0] += 1ull << (16 * (h & 3));
     staged[at] = uint2{(unsigned)id[j], __float_as_uint(tv[j] - tlse)};
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -237,8 +239,13 @@ template <int J, int VD, bool VEC>
 static void launch_prep_it(const PrepParams& p, hipStream_t st) {
   const dim3 grid((unsigned)((p.n_trows + PREP_ROWS - 1) / PREP_ROWS)), block(PREP_ROWS * WAVE);
   const size_t lds = (size_t)PREP_ROWS * p.E * sizeof(uint2);      // <= 64 KiB: E <= DL_MAX_TOPK
-  if (p.idx_itype == DL_I32) hipLaunchKernelGGL((multi_prep_kernel<J, VD, I32, VEC>), grid, block, lds, st, p);
-  else hipLaunchKernelGGL((multi_prep_kernel<J, VD, I64, VEC>), grid, block, lds, st, p);
+  if (p.parts > 4) {
+    if (p.idx_itype == DL_I32) hipLaunchKernelGGL((multi_prep_kernel<J, VD, I32, VEC, true>), grid, block, lds, st, p);
+    else hipLaunchKernelGGL((multi_prep_kernel<J, VD, I64, VEC, true>), grid, block, lds, st, p);
+  } else {
+    if (p.idx_itype == DL_I32) hipLaunchKernelGGL((multi_prep_kernel<J, VD, I32, VEC, false>), grid, block, lds, st, p);
+    else hipLaunchKernelGGL((multi_prep_kernel<J, VD, I64, VEC, false>), grid, block, lds, st, p);
+  }
 }
 
 template <int J, bool VEC>
