@@ -335,11 +335,10 @@ __global__ __launch_bounds__(256) void marginalise_csr_kernel(const void* probs,
 }
 
 // ---- fused: marginal in LDS -> reverse KL against the student row in registers -----------------
+// The student row of the fused kernel: NU units of 8 columns per thread, in registers.
 template <class TagS, int NU>
-struct LdsTeacherRows {
-  static constexpr bool ONLINE = false;
+struct StudentRow {
   Unit<TagS> s[NU];
-  const float* lt;      // log marginal, LDS
   int64_t nunits;
   __device__ __forceinline__ void load(const char* srow, int64_t nu) {
     nunits = nu;
@@ -347,21 +346,6 @@ struct LdsTeacherRows {
     for (int i = 0; i < NU; ++i) {
       const int64_t u = (int64_t)i * MARG_NT + threadIdx.x;
       if (u < nunits) s[i].load(srow, u); else s[i].fill_neg_inf();
-    }
-  }
-  template <class F>
-  __device__ __forceinline__ void sweep(F f) {
-#pragma unroll
-    for (int i = 0; i < NU; ++i) {
-      const int64_t u = (int64_t)i * MARG_NT + threadIdx.x;
-      if (u < nunits) {
-        float a[8], b[8];
-        s[i].unpack(a);
-        const float4 b0 = *reinterpret_cast<const float4*>(lt + u * 8);
-        const float4 b1 = *reinterpret_cast<const float4*>(lt + u * 8 + 4);
-        b[0] = b0.x; b[1] = b0.y; b[2] = b0.z; b[3] = b0.w; b[4] = b1.x; b[5] = b1.y; b[6] = b1.z; b[7] = b1.w;
-        f(u, a, b);
-      }
     }
   }
 };
@@ -467,7 +451,7 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
-  LdsTeacherRows<TagS, NU> rows;
+  StudentRow<TagS, NU> rows;
   const char* srow = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes;
   const int pb = p.p_dtype == F32 ? 4 : 2;
   const char* prow = reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb;
