@@ -467,7 +467,9 @@ def merge_remap_padded(vals, idxs, weights, id_map, T: float = 1.0, n_student: i
 
 def fwd_kl_sparse_rows(z: torch.Tensor, ids: np.ndarray, logq: np.ndarray, cnt: np.ndarray):
     """Forward KL against an already-normalised ragged sparse teacher
-    (utils/finetuning_utils.py:92,104 with a per-row entry count)."""
+    (utils/finetuning_utils.py:92,104 with a per-row entry count).  An entry of zero mass
+    (log-probability -inf: a merged id all of whose teachers carry weight 0) contributes 0,
+    the convention of this build for forward KL (the library routine would give 0 * inf = NaN)."""
     s = F.log_softmax(z, dim=-1)
     rows = []
     for r in range(z.shape[0]):
@@ -477,7 +479,8 @@ def fwd_kl_sparse_rows(z: torch.Tensor, ids: np.ndarray, logq: np.ndarray, cnt: 
             continue
         sk = s[r, torch.as_tensor(ids[r, :n].astype(np.int64))]
         t = torch.as_tensor(logq[r, :n]).to(z.dtype)
-        rows.append((torch.exp(t) * (t - sk)).sum())
+        live = ~torch.isneginf(t)
+        rows.append((torch.exp(t[live]) * (t[live] - sk[live])).sum())
     return torch.stack(rows)
 
 

@@ -208,6 +208,25 @@ def test_bucketed_multi_teacher_edge_rows(D):
     assert ((grad.cpu().double() - grad64).abs() <= O.storage_tolerance(grad64, torch.float32, 1e-4)).all()
 
 
+def test_multi_teacher_with_a_teacher_of_weight_zero(D):
+    """A teacher of weight 0 contributes no entries (its ids stay in the merged id list with mass 0, which the
+    loss takes as no entry): both forms against the oracle, whose forward KL follows the same convention."""
+    g = torch.Generator().manual_seed(91)
+    R, V, Vt, K = 6, 40000, 45000, 100
+    logits = (torch.randn(R, V, generator=g) * 3).to(torch.bfloat16)
+    vals, idxs = _teachers(R, K, Vt, 3, 92)
+    weights = [0.6, 0.0, 0.4]
+    id_map = torch.randint(0, V, (Vt,), generator=g, dtype=torch.int32)
+    rows64, grad64, _ = _oracle_multi(logits, vals, idxs, weights, id_map, 1.0)
+    assert torch.isfinite(rows64).all()
+    args = (logits.to(DEV), [v.to(DEV) for v in vals], [i.to(DEV) for i in idxs], weights, id_map.to(DEV))
+    bound = O.storage_tolerance(grad64 / R, torch.bfloat16, 2e-3)
+    for fused in (True, False):
+        rl, grad = D.fkl_multi_teacher(*args, T=1.0, teacher_T=1.0, grad_scale=1.0 / R, fused=fused)
+        np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+        assert ((grad.cpu().double() - grad64 / R).abs() <= bound).all()
+
+
 def test_bucketed_multi_teacher_crowded_buckets_and_many_entries(D):
     """Every entry of a row inside one column part (its bucket overflows the slots laid out for an
     even share), 7 teachers x 290 entries, the largest entry count the library takes."""
