@@ -441,7 +441,8 @@ def merge_remap_rows(vals: Sequence[np.ndarray], idxs: Sequence[np.ndarray],
         ids = np.asarray(sorted(acc), dtype=np.int32)
         mass = np.asarray([acc[i] for i in ids], dtype=np.float32)
         if ids.size:
-            lg = np.log(mass.astype(np.float64)) / T
+            with np.errstate(divide="ignore"):                    # an id all of whose entries carry zero mass: log 0 = -inf
+                lg = np.log(mass.astype(np.float64)) / T
             lg = lg - (lg.max() + math.log(np.exp(lg - lg.max()).sum()))
         else:
             lg = np.zeros(0, dtype=np.float64)
