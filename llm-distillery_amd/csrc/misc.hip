@@ -4,20 +4,32 @@
 
 namespace dl {
 
-// One workgroup, fixed association order: thread t adds values t, t+NT, ... in double,
-// then a fixed LDS tree.  Same input => same bits.
+// One workgroup, fixed association order: thread t adds values t, t+NT, ... in double (eight loads
+// in flight at a time), then the lanes of a wave fold by shuffles and thread 0 adds the waves' sums
+// in order.  Same input => same bits.
 template <int NT>
 __global__ __launch_bounds__(NT) void reduce_sum_kernel(const float* v, int64_t n, float scale, float* out) {
-  __shared__ double sh[NT];
+  __shared__ double sh[NT / WAVE];
   double acc = 0.0;
-  for (int64_t i = threadIdx.x; i < n; i += NT) acc += (double)v[i];
-  sh[threadIdx.x] = acc;
-  __syncthreads();
-  for (int o = NT / 2; o > 0; o >>= 1) {
-    if ((int)threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
-    __syncthreads();
+  int64_t i = threadIdx.x;
+  for (; i + 7 * NT < n; i += 8 * NT) {
+    float x[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) x[k] = v[i + k * NT];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc += (double)x[k];
   }
-  if (threadIdx.x == 0) out[0] = (float)(sh[0] * (double)scale);
+  for (; i < n; i += NT) acc += (double)v[i];
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) acc += __shfl_down(acc, o, WAVE);
+  if ((threadIdx.x & (WAVE - 1)) == 0) sh[threadIdx.x / WAVE] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double total = 0.0;
+#pragma unroll
+    for (int w = 0; w < NT / WAVE; ++w) total += sh[w];
+    out[0] = (float)(total * (double)scale);
+  }
 }
 
 

@@ -871,12 +871,18 @@ static int launch_reg(const TopkParams& p, hipStream_t st) {
   return launch_status();
 }
 
+// 16-byte words at the head of the exchange workspace that must be zero when the split kernels start:
+// one PartStats per (row, part), then the retry counter
+static int64_t split_clear_words(int64_t n_rows, int parts) { return n_rows * parts + 1; }
+
+// `cleared`: an earlier launch on the same stream has already zeroed those words
 template <class Tag, int NT, int NCH, bool MULTI>
-static int launch_split(TopkParams p, int parts, hipStream_t st) {
+static int launch_split(TopkParams p, int parts, hipStream_t st, bool cleared) {
   p.parts = parts;
-  const int64_t n16 = p.n_rows * parts + 1;      // one 16-byte PartStats per (row, part), then the retry counter
-  hipLaunchKernelGGL(clear_workspace_kernel<256>, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
-                     reinterpret_cast<u32x4*>(p.workspace), n16);
+  const int64_t n16 = split_clear_words(p.n_rows, parts);
+  if (!cleared)
+    hipLaunchKernelGGL(clear_workspace_kernel<256>, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
+                       reinterpret_cast<u32x4*>(p.workspace), n16);
   launch_reg_j<Tag, NT, NCH, true, MULTI>(p, (unsigned)((p.n_rows + 7) / 8 * 8 * parts), st);
   launch_retry_j<Tag, NT, NCH, MULTI>(p, (unsigned)std::min<int64_t>(p.n_rows * parts, 256), st);
   return launch_status();
@@ -916,7 +922,7 @@ static FklShape fkl_shape(int64_t nch, int bytes, int forced_parts, bool split_o
 
 // MULTI has no streaming form: the caller checks fkl_shape first.
 template <class Tag, bool MULTI>
-static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipStream_t st) {
+static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipStream_t st, bool ws_cleared = false) {
   const int64_t nch = p.V / Tag::epc;
   const int forced = (p.flags >> DL_TOPK_PARTS_SHIFT) & 15;
   const bool fine = !MULTI && (p.flags & DL_TOPK_FINE_PARTS) != 0 &&
@@ -927,18 +933,18 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
   switch (sh.NT * 100 + sh.NCH) {
     case 256 * 100 + 4:
       if constexpr (!MULTI)
-        if (sh.parts > 1) return launch_split<Tag, 256, 4, MULTI>(p, sh.parts, st);
+        if (sh.parts > 1) return launch_split<Tag, 256, 4, MULTI>(p, sh.parts, st, ws_cleared);
       return launch_reg<Tag, 256, 4, MULTI>(p, st);
     case 256 * 100 + 8: return launch_reg<Tag, 256, 8, MULTI>(p, st);
     case 512 * 100 + 8:
       if constexpr (Tag::bytes == 4) return launch_reg<Tag, 512, 8, MULTI>(p, st);
       break;
     case 256 * 100 + 16:
-      if (sh.parts > 1) return launch_split<Tag, 256, 16, MULTI>(p, sh.parts, st);
+      if (sh.parts > 1) return launch_split<Tag, 256, 16, MULTI>(p, sh.parts, st, ws_cleared);
       if constexpr (Tag::bytes != 4) return launch_reg<Tag, 256, 16, MULTI>(p, st);
       break;
     case 512 * 100 + 16:
-      return sh.parts > 1 ? launch_split<Tag, 512, 16, MULTI>(p, sh.parts, st) : launch_reg<Tag, 512, 16, MULTI>(p, st);
+      return sh.parts > 1 ? launch_split<Tag, 512, 16, MULTI>(p, sh.parts, st, ws_cleared) : launch_reg<Tag, 512, 16, MULTI>(p, st);
     case 1024 * 100 + 16: return launch_reg<Tag, 1024, 16, MULTI>(p, st);
     default: break;
   }

@@ -22,6 +22,7 @@ struct PrepParams {
   int parts; int part_shift;      // bucket of student id s: s >> part_shift (parts == 1: everything in bucket 0)
   int cap0; int E;
   uint2* first; uint2* more; int* head;
+  u32x4* clear; int64_t clear_n16;      // the loss kernels' exchange records, zeroed on the way (clear_n16 == 0: nothing to clear)
 };
 
 // Exclusive prefix sum over the lanes of a wave of four 16-bit counters packed into 64 bits (no field
@@ -59,6 +60,8 @@ template <int J, int VD, int IT, bool VEC, bool WIDE>
 __global__ __launch_bounds__(PREP_ROWS * WAVE) void multi_prep_kernel(const PrepParams p) {
   const MultiTeacher& m = p.mt;
   const int lane = threadIdx.x & (WAVE - 1);
+  for (int64_t i = (int64_t)blockIdx.x * (PREP_ROWS * WAVE) + threadIdx.x; i < p.clear_n16; i += (int64_t)gridDim.x * (PREP_ROWS * WAVE))
+    p.clear[i] = u32x4{0u, 0u, 0u, 0u};
   const int64_t trow = (int64_t)blockIdx.x * PREP_ROWS + threadIdx.x / WAVE;
   if (trow >= p.n_trows) return;
   const int S = (m.Kt + (VEC ? 4 : 1) * WAVE - 1) / ((VEC ? 4 : 1) * WAVE);
@@ -313,6 +316,7 @@ extern "C" int dl_fkl_multi_teacher(const void* logits, int logits_dtype, int64_
   p.bk.more = reinterpret_cast<const uint2*>(ws + plan.exchange_bytes + plan.first_bytes + plan.head_bytes);
   p.bk.cap0 = plan.cap0; p.bk.E = E;
 
+  bool ws_cleared = false;
   if (n_teacher_rows > 0) {
     PrepParams q{};
     q.mt.n = n_teachers; q.mt.Kt = K; q.mt.id_map = id_map; q.mt.Vt = Vt;
@@ -326,6 +330,10 @@ extern "C" int dl_fkl_multi_teacher(const void* logits, int logits_dtype, int64_
     q.parts = plan.shape.parts;
     q.part_shift = __builtin_ctzll((uint64_t)plan.shape.NT * plan.shape.NCH * (16 / eb));      // columns per part: a power of two
     q.cap0 = plan.cap0; q.E = E;
+    if (plan.shape.parts > 1) {      // saves the split kernels' own fill launch
+      q.clear = reinterpret_cast<u32x4*>(ws); q.clear_n16 = split_clear_words(n_rows, plan.shape.parts);
+      ws_cleared = true;
+    }
     q.first = const_cast<uint2*>(p.bk.first); q.more = const_cast<uint2*>(p.bk.more); q.head = const_cast<int*>(p.bk.head);
     bool vec = K % 4 == 0;
     for (int j = 0; j < n_teachers; ++j)
@@ -343,7 +351,7 @@ extern "C" int dl_fkl_multi_teacher(const void* logits, int logits_dtype, int64_
       else launch_prep<40, false>(q, st);
     }
   }
-  return logits_dtype == DL_F32 ? launch_fkl<TagF32, true>(p, true, plan.exchange_bytes, st)
-         : logits_dtype == DL_BF16 ? launch_fkl<TagBF16, true>(p, true, plan.exchange_bytes, st)
-                                   : launch_fkl<TagF16, true>(p, true, plan.exchange_bytes, st);
+  return logits_dtype == DL_F32 ? launch_fkl<TagF32, true>(p, true, plan.exchange_bytes, st, ws_cleared)
+         : logits_dtype == DL_BF16 ? launch_fkl<TagBF16, true>(p, true, plan.exchange_bytes, st, ws_cleared)
+                                   : launch_fkl<TagF16, true>(p, true, plan.exchange_bytes, st, ws_cleared);
 }
