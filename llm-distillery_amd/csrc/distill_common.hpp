@@ -358,6 +358,24 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* scratch) {
   a = ra; b = rb;
 }
 
+// Three sums in one pair of barriers (scratch: 3 * NT / 64 floats).
+template <int NT>
+__device__ __forceinline__ void block_sum3(float& a, float& b, float& c, float* scratch) {
+  constexpr int NW = NT / WAVE;
+  a = wave_sum(a);
+  b = wave_sum(b);
+  c = wave_sum(c);
+  if constexpr (NW == 1) return;
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  if (lane == 0) { scratch[w] = a; scratch[NW + w] = b; scratch[2 * NW + w] = c; }
+  __syncthreads();
+  float ra = scratch[0], rb = scratch[NW], rc = scratch[2 * NW];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) { ra += scratch[i]; rb += scratch[NW + i]; rc += scratch[2 * NW + i]; }
+  __syncthreads();
+  a = ra; b = rb; c = rc;
+}
+
 // Teacher row feeding logits row r: row_map[r] (identity without a map); anything outside
 // [0, n_trows) means "masked row".
 __device__ __forceinline__ int64_t teacher_row(const int32_t* row_map, int64_t r, int64_t n_trows) {

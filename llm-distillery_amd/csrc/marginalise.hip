@@ -352,89 +352,204 @@ struct StudentRow {
 
 // Reverse KL of the student row (in registers) against a marginal that sits in LDS as probabilities,
 // with its gradient; the same quantities as dense_stats<DL_RKL> + dense_grad_sweep<DL_RKL> on the
-// logarithm of the marginal, in three passes of fewer instructions (with one 1024-thread workgroup per
-// CU these passes run on the vector ALUs alone, no memory traffic to hide behind: 31 % of the
-// kernel's time before).  Log2 domain throughout:
-//   xt_j = log2(m_j) / T_t - bt        bt from the largest marginal (xt = -inf off the support)
-//   xs_j = s_j a_s - bs                bs from the largest student logit on the support
+// logarithm of the marginal, in fewer instructions (with one 1024-thread workgroup per CU these
+// passes run on the vector ALUs alone, no memory traffic to hide behind).  Log2 domain throughout:
+//   xt_j = log2(m_j) / T_t - bt        (off the support: XT_OFF, standing for -inf)
+//   xs_j = s_j a_s - bs
 //   S = sum_on 2^xs, T = sum 2^xt, W = sum_on 2^xs (xs - xt)
 //   RKL = (W / S - log2 S + log2 T) ln 2
 //   d RKL / d s_j = 2^xs_j (ln 2 / (T_s S)) ((xs_j - xt_j) - W / S)      on the support, else 0
-// Pass A: maxima.  Pass B: xt (written over the marginal), the three sums.  Pass C: gradient.
-template <class TagS, int NU>
-__device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float* red,
-                                                     const MargParams& p, int64_t r, char* grow) {
+// None of these depends on the biases bs, bt; they only keep the sums in range.  The usual choice, the
+// largest marginal and the largest student logit ON THE SUPPORT, costs a pass over the marginal before
+// the sums can start.  Instead: bt = 0 (a marginal of probabilities is at most 1, and its largest entry
+// is rarely below 2^-20) and bs from the largest student logit of the whole row, which needs the
+// registers only.  Pass B: xt (written over the marginal; a log-domain value, exact whatever the
+// bias), the three sums.  If T or S then lies outside [2^-64, 2^64] -- the row carries no or hardly any
+// mass, an unnormalised teacher, or a student whose mass sits far off the support -- the maxima are
+// taken after all, from the stored xt, and the sums are redone on them.  Pass C: gradient.
+// What stands for log2(0) in the stored xt and for a student logit of -inf: finite, so that differences
+// of two such values are finite (0 * finite = 0 needs no select), and far below anything a sum notices.
+constexpr float XT_OFF = -1e30f;
+
+// WITH_T: T is summed here; else the caller sums it in the gradient pass (see rkl_against_marginal).
+template <class TagS, int NU, bool UNIT_T, bool WITH_T>
+__device__ __forceinline__ void rkl_sums_optimistic(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float a_s, float bs,
+                                                    float inv_T_t, float& ss, float& stt, float& w) {
   const int tid = threadIdx.x;
-  const float a_s = p.inv_T_s * LOG2E;
-  const auto marginal_of = [&](int64_t u, float (&m)[8]) {
-    const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
-    m[0] = m0.x; m[1] = m0.y; m[2] = m0.z; m[3] = m0.w; m[4] = m1.x; m[5] = m1.y; m[6] = m1.z; m[7] = m1.w;
-  };
-  float mmax = 0.f, ms = -INFINITY;
 #pragma unroll
   for (int i = 0; i < NU; ++i) {
     const int64_t u = (int64_t)i * MARG_NT + tid;
     if (u < nunits) {
       float sv[8], m[8];
       s[i].unpack(sv);
-      marginal_of(u, m);
+      const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
+      m[0] = m0.x; m[1] = m0.y; m[2] = m0.z; m[3] = m0.w; m[4] = m1.x; m[5] = m1.y; m[6] = m1.z; m[7] = m1.w;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        mmax = fmaxf(mmax, m[e]);
-        ms = fmaxf(ms, m[e] > 0.f ? sv[e] : -INFINITY);
-      }
-    }
-  }
-  block_max2<MARG_NT>(mmax, ms, red);
-  if (!(mmax > 0.f)) {                              // the teacher row carried no mass at all
-    if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
-    if (grow) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
-    return;
-  }
-  const float bt = fast_log2(mmax) * p.inv_T_t, bs = ms * a_s;
-  float ss = 0.f, stt = 0.f, w = 0.f;
-#pragma unroll
-  for (int i = 0; i < NU; ++i) {
-    const int64_t u = (int64_t)i * MARG_NT + tid;
-    if (u < nunits) {
-      float sv[8], m[8];
-      s[i].unpack(sv);
-      marginal_of(u, m);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float xt = fmaf(fast_log2(m[e]), p.inv_T_t, -bt), xs = fmaf(sv[e], a_s, -bs);
-        const float es = fast_exp2(xs);
-        stt += fast_exp2(xt);
-        const bool on = m[e] > 0.f;
-        ss += on ? es : 0.f;
-        w += (on && es > 0.f) ? es * (xs - xt) : 0.f;
+        const float l2 = fast_log2(m[e]);
+        const float xt = fmaxf(UNIT_T ? l2 : l2 * inv_T_t, XT_OFF), xs = fmaxf(fmaf(sv[e], a_s, -bs), XT_OFF);
+        const float eon = m[e] > 0.f ? fast_exp2(xs) : 0.f;
+        if (WITH_T) stt += UNIT_T ? m[e] : fast_exp2(xt);      // 2^xt; 0 off the support
+        ss += eon;
+        w = fmaf(eon, xs - xt, w);                 // the difference is finite: no 0 * inf
         m[e] = xt;
       }
       *reinterpret_cast<float4*>(marg + u * 8) = float4{m[0], m[1], m[2], m[3]};        // own columns only: no barrier needed
       *reinterpret_cast<float4*>(marg + u * 8 + 4) = float4{m[4], m[5], m[6], m[7]};
     }
   }
-  block_sum2<MARG_NT>(ss, stt, red);
-  w = block_sum<MARG_NT>(w, red);
-  const float wbar = w / ss;
-  if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - fast_log2(ss) + fast_log2(stt)) * LN2;
-  if (!grow) return;
-  const float k1 = p.inv_T_s * p.grad_scale * LN2 / ss;
+}
+
+// Pass C.  WITH_T: T = sum 2^xt is taken along (into stt, this thread's share).
+template <class TagS, int NU, bool WITH_T>
+__device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t nunits, const float* marg, float a_s, float bs,
+                                                  float k1, float wbar, char* grow, float& stt) {
+  const int tid = threadIdx.x;
 #pragma unroll
   for (int i = 0; i < NU; ++i) {
     const int64_t u = (int64_t)i * MARG_NT + tid;
     if (u < nunits) {
       float sv[8], xt[8], g[8];
       s[i].unpack(sv);
-      marginal_of(u, xt);
+      const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
+      xt[0] = m0.x; xt[1] = m0.y; xt[2] = m0.z; xt[3] = m0.w; xt[4] = m1.x; xt[5] = m1.y; xt[6] = m1.z; xt[7] = m1.w;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float xs = fmaf(sv[e], a_s, -bs);
-        g[e] = xt[e] > -INFINITY ? fast_exp2(xs) * k1 * ((xs - xt[e]) - wbar) : 0.f;
+        g[e] = xt[e] > 0.5f * XT_OFF ? fast_exp2(xs) * k1 * ((xs - xt[e]) - wbar) : 0.f;
+        if (WITH_T) stt += fast_exp2(xt[e]);
       }
       Unit<TagS>::store(grow, u, g);
     }
   }
+}
+
+// The sums' pass is bound by its three transcendentals per column (2^xs, log2 m, 2^xt), the gradient
+// pass, with one, by its other instructions: when a gradient is asked for and T_t != 1, 2^xt moves to
+// the gradient pass -- T enters the loss only, not the gradient -- and the row's loss is written last.
+template <class TagS, int NU>
+__device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float* red,
+                                                     const MargParams& p, int64_t r, char* grow) {
+  const int tid = threadIdx.x;
+  const float a_s = p.inv_T_s * LOG2E;
+  const auto stored_of = [&](int64_t u, float (&m)[8]) {
+    const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
+    m[0] = m0.x; m[1] = m0.y; m[2] = m0.z; m[3] = m0.w; m[4] = m1.x; m[5] = m1.y; m[6] = m1.z; m[7] = m1.w;
+  };
+  const auto in_range = [](float v) { return v > 0x1p-64f && v < 0x1p64f; };
+  float ms = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NU; ++i) {      // units beyond the row hold -inf
+    float sv[8];
+    s[i].unpack(sv);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ms = fmaxf(ms, sv[e]);
+  }
+  ms = block_max<MARG_NT>(ms, red);
+  float bs = ms > -INFINITY ? ms * a_s : 0.f;
+  float ss = 0.f, stt = 0.f, w = 0.f;
+  bool t_known = true;
+  if (p.inv_T_t == 1.f) {
+    rkl_sums_optimistic<TagS, NU, true, true>(s, nunits, marg, a_s, bs, 1.f, ss, stt, w);
+  } else if (!grow) {
+    rkl_sums_optimistic<TagS, NU, false, true>(s, nunits, marg, a_s, bs, p.inv_T_t, ss, stt, w);
+  } else {
+    rkl_sums_optimistic<TagS, NU, false, false>(s, nunits, marg, a_s, bs, p.inv_T_t, ss, stt, w);
+    t_known = false;
+  }
+  block_sum3<MARG_NT>(ss, stt, w, red);
+  if (!(in_range(ss) && (!t_known || in_range(stt)))) {      // the same for every thread
+    float tmax = -INFINITY;
+    ms = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + tid;
+      if (u < nunits) {
+        float sv[8], xt[8];
+        s[i].unpack(sv);
+        stored_of(u, xt);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          tmax = fmaxf(tmax, xt[e]);
+          ms = fmaxf(ms, xt[e] > 0.5f * XT_OFF ? sv[e] : -INFINITY);
+        }
+      }
+    }
+    block_max2<MARG_NT>(tmax, ms, red);
+    if (!(tmax > 0.5f * XT_OFF)) {                    // the teacher row carried no mass at all
+      if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
+      if (grow) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
+      return;
+    }
+    bs = ms * a_s;
+    ss = 0.f, stt = 0.f, w = 0.f;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + tid;
+      if (u < nunits) {
+        float sv[8], xt[8];
+        s[i].unpack(sv);
+        stored_of(u, xt);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const bool on = xt[e] > 0.5f * XT_OFF;
+          xt[e] = on ? xt[e] - tmax : XT_OFF;
+          const float xs = fmaxf(fmaf(sv[e], a_s, -bs), XT_OFF);
+          const float eon = on ? fast_exp2(xs) : 0.f;
+          stt += fast_exp2(xt[e]);
+          ss += eon;
+          w = fmaf(eon, xs - xt[e], w);
+        }
+        *reinterpret_cast<float4*>(marg + u * 8) = float4{xt[0], xt[1], xt[2], xt[3]};
+        *reinterpret_cast<float4*>(marg + u * 8 + 4) = float4{xt[4], xt[5], xt[6], xt[7]};
+      }
+    }
+    block_sum3<MARG_NT>(ss, stt, w, red);
+    t_known = true;
+  }
+  const float wbar = w / ss, l2s = fast_log2(ss);
+  if (t_known) {
+    if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - l2s + fast_log2(stt)) * LN2;
+    if (!grow) return;
+  }
+  const float k1 = p.inv_T_s * p.grad_scale * LN2 / ss;
+  if (t_known) {
+    rkl_gradient_pass<TagS, NU, false>(s, nunits, marg, a_s, bs, k1, wbar, grow, stt);
+    return;
+  }
+  stt = 0.f;
+  rkl_gradient_pass<TagS, NU, true>(s, nunits, marg, a_s, bs, k1, wbar, grow, stt);
+  if (!p.row_loss) return;
+  stt = block_sum<MARG_NT>(stt, red);
+  float l2t = fast_log2(stt);
+  if (!in_range(stt)) {      // hardly any teacher mass, or an unnormalised teacher: T on the largest entry after all
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + tid;
+      if (u < nunits) {
+        float xt[8];
+        stored_of(u, xt);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) tmax = fmaxf(tmax, xt[e]);
+      }
+    }
+    tmax = block_max<MARG_NT>(tmax, red);
+    stt = 0.f;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + tid;
+      if (u < nunits) {
+        float xt[8];
+        stored_of(u, xt);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) stt += fast_exp2(xt[e] - tmax);
+      }
+    }
+    stt = block_sum<MARG_NT>(stt, red);
+    l2t = tmax + fast_log2(stt);
+  }
+  if (tid == 0) p.row_loss[r] = (wbar - l2s + l2t) * LN2;
 }
 
 template <class TagS, int NU, bool VEC>

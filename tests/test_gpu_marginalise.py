@@ -158,6 +158,44 @@ def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T, planne
     assert torch.count_nonzero(grad.cpu()[valid][:, (marg.sum(0) == 0)]) == 0
 
 
+@pytest.mark.parametrize("planned", [False, True])
+@pytest.mark.parametrize("T", [1.0, 2.0, 0.5])
+def test_fused_reverse_kl_on_rows_whose_sums_leave_the_range(D, T, planned):
+    """Rows for which a bias of 0 for the teacher and the row's largest logit for the student do not keep
+    the sums in range: hardly any teacher mass, an unnormalised teacher, a student whose mass sits on a
+    column outside the marginal's support, and a teacher row without mass (zero loss, zero gradient)."""
+    R, Vs, Vt = 6, 2048, 9000
+    t2s, probs = _case(R, Vs, Vt, 5, 4, drop=0.01)
+    g = torch.Generator().manual_seed(11)
+    logits = torch.randn(R, Vs, generator=g) * 2
+    probs = probs.clone()
+    probs[0] *= 1e-25
+    probs[1] *= 1e25
+    off = int(t2s[t2s >= 0][0])                      # a student column that is taken off the support of row 2
+    probs[2, torch.tensor(t2s == off)] = 0.0
+    logits[2, off] = 300.0
+    probs[3] = 0.0
+    tmap = D.vocab_utils.MarginalPlan(t2s, Vs, DEV) if planned else torch.tensor(t2s, device=DEV)
+    with_mass = torch.tensor([0, 1, 2, 4, 5])
+    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, T=T, grad_scale=1.0 / len(with_mass))
+    rl, grad = rl.cpu(), grad.cpu()
+    assert rl[3] == 0 and torch.count_nonzero(grad[3]) == 0
+    marg = torch.tensor(O.marginalise_map(probs.double().numpy(), t2s, Vs))[with_mass]
+    assert marg[2, off] == 0
+    with np.errstate(divide="ignore"):
+        t_logits = O.marginal_to_teacher_logits(marg)
+    _, rows64, grad64 = O.mean_loss_and_grad("rkl", logits[with_mass], T, t_logits=t_logits, dtype=torch.float64)
+    np.testing.assert_allclose(rl[with_mass].double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    err = (grad[with_mass].double() - grad64).abs()
+    bound = 1e-4 * grad64.abs() + 2e-6 * grad64.abs().amax(-1, keepdim=True)
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+    assert torch.count_nonzero(grad[with_mass][marg == 0]) == 0
+    # without a gradient the loss takes other passes over the row: the same values to rounding
+    rl_only, none = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, T=T, want_grad=False)
+    assert none is None
+    np.testing.assert_allclose(rl_only.cpu().numpy(), rl.numpy(), rtol=1e-5, atol=1e-6)
+
+
 def test_fused_path_limits_are_reported(D):
     with pytest.raises(RuntimeError, match="exceeds"):
         D.vocab_utils.rkl_marginalised(torch.zeros(2, 40000, device=DEV), torch.zeros(2, 64, device=DEV),
