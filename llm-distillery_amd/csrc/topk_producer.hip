@@ -135,6 +135,22 @@ __device__ __forceinline__ int block_sum_int(int v, int* scratch) {
   return r;
 }
 
+// Largest of a per-thread integer over the workgroup; two barriers, scratch reusable at once.
+template <int NT>
+__device__ __forceinline__ int block_max_int(int v, int* scratch) {
+  constexpr int NW = NT / WAVE;
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, WAVE));
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  if (lane == 0) scratch[w] = v;
+  __syncthreads();
+  int r = scratch[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) r = max(r, scratch[i]);
+  __syncthreads();
+  return r;
+}
+
 // ---- candidate words -----------------------------------------------------------------------------
 // A candidate is one word that sorts ascending = key descending, column ascending.  Inside a part
 // the column needs 15 bits, so 16-bit keys give 31-bit words; fp32 keys need 64 bits.  The part
@@ -330,15 +346,35 @@ void topk_part_kernel(const ProducerParams p) {
 
   // max and sum-exp of the part (natural log-softmax; no temperature at collection time)
   float mx = -INFINITY;
+  bool have_max = false;
+  if constexpr (Tag::bytes == 2) {
+    // Non-negative 16-bit floats order like their bit patterns read as signed integers, and every
+    // negative one reads as a negative integer: the packed integer maximum of the raw pairs is the
+    // row maximum whenever that is not negative (half an instruction per element instead of two).
+    i16x2 pm = {(short)-32768, (short)-32768};
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    float f[C::N];
-    forget(reg[i]);
-    C::unpack(reg[i], f);
+    for (int i = 0; i < NCH; ++i) {
+      forget(reg[i]);
 #pragma unroll
-    for (int e = 0; e < C::N; ++e) mx = fmaxf(mx, f[e]);
+      for (int d = 0; d < 4; ++d) pm = __builtin_elementwise_max(pm, __builtin_bit_cast(i16x2, reg[i][d]));
+    }
+    const int top = block_max_int<NT>(max((int)pm.x, (int)pm.y), ired);
+    if (top >= 0) {
+      mx = Tag::id == BF16 ? __uint_as_float((unsigned)top << 16) : (float)__builtin_bit_cast(_Float16, (unsigned short)top);
+      have_max = true;
+    }
   }
-  mx = block_max<NT>(mx, red);
+  if (!have_max) {                        // the same for every thread
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      float f[C::N];
+      forget(reg[i]);
+      C::unpack(reg[i], f);
+#pragma unroll
+      for (int e = 0; e < C::N; ++e) mx = fmaxf(mx, f[e]);
+    }
+    mx = block_max<NT>(mx, red);
+  }
   const float mb = (mx == -INFINITY) ? 0.f : mx * LOG2E;
   float sm = 0.f;
 #pragma unroll

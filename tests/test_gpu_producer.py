@@ -39,6 +39,26 @@ def test_topk_ids_bit_exact_values_close(D, dtype, V, K):
     np.testing.assert_allclose(val.cpu().numpy(), ov.numpy(), rtol=0, atol=3e-6 * max(1.0, float(ov.abs().max())))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_rows_whose_largest_logit_is_negative_or_zero(D, dtype):
+    """16-bit rows take their maximum from the raw bit patterns when it is not negative, else from the
+    values: rows of negative logits only, rows whose maximum is +0 or -0, and ordinary rows between them."""
+    g = torch.Generator().manual_seed(5)
+    V, K = 40000, 64
+    logits = torch.randn(8, V, generator=g) * 3
+    logits[0] = -logits[0].abs() - 0.5
+    logits[1] = -logits[1].abs() - 20.0
+    logits[2] = torch.minimum(logits[2], torch.zeros(()))                    # maximum +0, many times
+    logits[3] = -logits[3].abs() - 1.0
+    logits[3, 777] = -0.0
+    logits[5, :] = -7.25
+    logits = logits.to(dtype)
+    val, idx = D.teacher_topk(logits.to(DEV), K, val_dtype=torch.float32, idx_dtype=torch.int64)
+    rv, ri = _ref(logits, V, K)
+    assert torch.equal(idx.cpu(), ri)
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), rtol=0, atol=2e-6 * max(1.0, float(rv.abs().max())))
+
+
 def test_storage_layout_crop_and_content_rows(D):
     g = torch.Generator().manual_seed(3)
     B, S, Vm, crop, K = 2, 40, 32064, 32000, 100
