@@ -41,6 +41,36 @@ struct RegRows {
       }
     }
   }
+  // Maxima of both rows from the raw bit patterns, for two 16-bit rows: non-negative 16-bit floats
+  // order like their patterns read as signed integers and every negative one reads as a negative
+  // integer, so the packed integer maximum is the row's maximum whenever that is not negative (half
+  // an instruction per element instead of two).  False -- for every thread alike -- when a row's
+  // maximum is negative or the types are not 16-bit: the caller then takes the maxima from the values.
+  static constexpr bool RAW_MAXIMA = TagS::bytes == 2 && TagT::bytes == 2;
+  __device__ __forceinline__ bool raw_maxima(float& ms, float& mt, float* red) {
+    if constexpr (!RAW_MAXIMA) return false;
+    typedef short i16x2 __attribute__((ext_vector_type(2)));
+    i16x2 a = {(short)-32768, (short)-32768}, b = a;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {      // units beyond the row hold -inf: negative patterns
+      forget(s[i].c[0]);
+      forget(t[i].c[0]);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        a = __builtin_elementwise_max(a, __builtin_bit_cast(i16x2, s[i].c[0][d]));
+        b = __builtin_elementwise_max(b, __builtin_bit_cast(i16x2, t[i].c[0][d]));
+      }
+    }
+    float fa = (float)max((int)a.x, (int)a.y), fb = (float)max((int)b.x, (int)b.y);      // exact, order-preserving
+    block_max2<NT>(fa, fb, red);
+    if (fa < 0.f || fb < 0.f) return false;
+    const auto value = [](int id, unsigned bits) {
+      return id == BF16 ? __uint_as_float(bits << 16) : (float)__builtin_bit_cast(_Float16, (unsigned short)bits);
+    };
+    ms = value(TagS::id, (unsigned)(int)fa);
+    mt = value(TagT::id, (unsigned)(int)fb);
+    return true;
+  }
 };
 
 template <int KIND, class TagS, class TagT, int NT, int NU>

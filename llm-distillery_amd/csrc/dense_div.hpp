@@ -136,14 +136,18 @@ __device__ __forceinline__ DenseStats dense_stats(Rows& rows, float inv_T_s, flo
     block_max2<NT>(gs, gt, red);
     carry(gs, gt);                          // this thread's sums on the row's biases
   } else {
-    rows.sweep([&](int64_t, const float* s, const float* t) {
+    bool have = false;
+    if constexpr (KIND != DL_RKL && Rows::RAW_MAXIMA) have = rows.raw_maxima(ms, mt, red);      // RKL: the student's maximum is over the support
+    if (!have) {
+      rows.sweep([&](int64_t, const float* s, const float* t) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        mt = fmaxf(mt, t[e]);
-        ms = fmaxf(ms, (KIND == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
-      }
-    });
-    block_max2<NT>(ms, mt, red);
+        for (int e = 0; e < 8; ++e) {
+          mt = fmaxf(mt, t[e]);
+          ms = fmaxf(ms, (KIND == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
+        }
+      });
+      block_max2<NT>(ms, mt, red);
+    }
     const float bs = ms * a_s, bt = mt * a_t;
     rows.sweep([&](int64_t, const float* s, const float* t) {
 #pragma unroll

@@ -61,6 +61,23 @@ def test_dense_small(D, kind, dtype, t_dtype):
     _check(D, kind, s, t, T=1.0)
 
 
+@pytest.mark.parametrize("kind", ["fkl", "jsd"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dense_16bit_rows_whose_maximum_is_negative_or_zero(D, kind, dtype):
+    """16-bit rows take non-negative maxima from the raw bit patterns, else from the values: student or
+    teacher rows of negative logits only, and maxima of exactly +0 and -0."""
+    s, t = _pair(12, 4096, dtype, 7)
+    s, t = s.float(), t.float()
+    s[0] = -s[0].abs() - 0.25
+    t[1] = -t[1].abs() - 3.0
+    s[2] = -s[2].abs() - 1.0
+    t[2] = -t[2].abs() - 1.0
+    s[3] = torch.minimum(s[3], torch.zeros(()))
+    t[4] = -t[4].abs()
+    t[4, 17] = -0.0
+    _check(D, kind, s.to(dtype), t.to(dtype), T=1.0)
+
+
 @pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
 def test_dense_vocab_32000_bf16_temperature_ragged_mask(D, kind):
     s, t = _pair(48, 32000, torch.bfloat16, 2, noise=1.5)
