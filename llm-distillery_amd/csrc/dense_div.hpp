@@ -56,12 +56,14 @@ __device__ __forceinline__ void rkl_term(float lp, float lq, float& acc) {
   acc += (lq > -INFINITY && r > 0.f) ? r * (lp - lq) : 0.f;
 }
 // Three transcendentals per column: the mixture's logarithm is taken of the probabilities themselves.
-// Columns where both probabilities underflow contribute nothing (they are skipped by the guards).
+// Columns where a probability underflows contribute nothing for it: the logarithms are held at a
+// finite floor, so their differences are finite and 0 * difference is 0 without a select.
+constexpr float LOG_FLOOR = -1e30f;
 __device__ __forceinline__ void jsd_term(float lp, float lq, float& kl_pm, float& kl_qm) {
   const float pr = fast_exp2(lp), q = fast_exp2(lq);
-  const float lm = fast_log2(0.5f * pr + 0.5f * q);
-  kl_pm += pr > 0.f ? pr * (lp - lm) : 0.f;
-  kl_qm += q > 0.f ? q * (lq - lm) : 0.f;
+  const float lm = fmaxf(fast_log2(0.5f * pr + 0.5f * q), LOG_FLOOR);
+  kl_pm = fmaf(pr, fmaxf(lp, LOG_FLOOR) - lm, kl_pm);
+  kl_qm = fmaf(q, fmaxf(lq, LOG_FLOOR) - lm, kl_qm);
 }
 
 // Gradient of one column (before the common factor c = inv_T * scale).
