@@ -370,6 +370,9 @@ struct StudentRow {
 // What stands for log2(0) in the stored xt and for a student logit of -inf: finite, so that differences
 // of two such values are finite (0 * finite = 0 needs no select), and far below anything a sum notices.
 constexpr float XT_OFF = -1e30f;
+// 2^24 lifts every positive fp32 value, denormals included (>= 2^-149), into the normal range; marginal
+// entries above 2^103 would overflow (probabilities are at most 1).
+constexpr float MARG_LOG_SCALE = 0x1p24f, MARG_LOG_SHIFT = 24.f;
 
 // WITH_T: T is summed here; else the caller sums it in the gradient pass (see rkl_against_marginal).
 template <class TagS, int NU, bool UNIT_T, bool WITH_T>
@@ -386,8 +389,10 @@ __device__ __forceinline__ void rkl_sums_optimistic(Unit<TagS> (&s)[NU], int64_t
       m[0] = m0.x; m[1] = m0.y; m[2] = m0.z; m[3] = m0.w; m[4] = m1.x; m[5] = m1.y; m[6] = m1.z; m[7] = m1.w;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float l2 = fast_log2(m[e]);
-        const float xt = fmaxf(UNIT_T ? l2 : l2 * inv_T_t, XT_OFF), xs = fmaxf(fmaf(sv[e], a_s, -bs), XT_OFF);
+        // the hardware logarithm takes a denormal for zero: the marginal is scaled into the normal range first
+        const float l2 = fast_log2(m[e] * MARG_LOG_SCALE);
+        const float xt = fmaxf(UNIT_T ? l2 - MARG_LOG_SHIFT : fmaf(l2, inv_T_t, -MARG_LOG_SHIFT * inv_T_t), XT_OFF);
+        const float xs = fmaxf(fmaf(sv[e], a_s, -bs), XT_OFF);
         const float eon = m[e] > 0.f ? fast_exp2(xs) : 0.f;
         if (WITH_T) stt += UNIT_T ? m[e] : fast_exp2(xt);      // 2^xt; 0 off the support
         ss += eon;

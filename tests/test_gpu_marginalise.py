@@ -162,8 +162,9 @@ def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T, planne
 @pytest.mark.parametrize("T", [1.0, 2.0, 0.5])
 def test_fused_reverse_kl_on_rows_whose_sums_leave_the_range(D, T, planned):
     """Rows for which a bias of 0 for the teacher and the row's largest logit for the student do not keep
-    the sums in range: hardly any teacher mass, an unnormalised teacher, a student whose mass sits on a
-    column outside the marginal's support, and a teacher row without mass (zero loss, zero gradient)."""
+    the sums in range: hardly any teacher mass (down to denormal entries), an unnormalised teacher, a student
+    whose mass sits on a column outside the marginal's support, and a teacher row without mass (zero loss,
+    zero gradient)."""
     R, Vs, Vt = 6, 2048, 9000
     t2s, probs = _case(R, Vs, Vt, 5, 4, drop=0.01)
     g = torch.Generator().manual_seed(11)
@@ -171,6 +172,7 @@ def test_fused_reverse_kl_on_rows_whose_sums_leave_the_range(D, T, planned):
     probs = probs.clone()
     probs[0] *= 1e-25
     probs[1] *= 1e25
+    probs[5] *= 1e-33                                # most of the marginal's entries are denormal: their logarithms still count
     off = int(t2s[t2s >= 0][0])                      # a student column that is taken off the support of row 2
     probs[2, torch.tensor(t2s == off)] = 0.0
     logits[2, off] = 300.0
