@@ -228,7 +228,8 @@ int dl_composite_backward(const float* lse, const float* zk, const void* t_val, 
  * No temperature is applied at collection time.  row_list (int32 [n_out], may be NULL = rows
  * 0..n_out-1) names the logits row behind each output row; an entry outside [0, n_rows) gives a
  * masked output row (log-probs -inf, ids -1) and touches no logits.  Entries with equal log-prob are
- * ordered by ascending id (the reference leaves tie order to torch.topk).
+ * ordered by ascending id (the reference leaves tie order to torch.topk); logits are ranked by their
+ * bit patterns, so a -0 ranks just below a +0.
  * K <= 1024, K <= V; V <= 262144 (131072 fp32); K * parts <= 4096 with parts = ceil(V / 32768)
  * (fp32: ceil(V / 16384)).  Any V and any element-aligned row pitch are taken, as by the reference;
  * V a multiple of 8 (4 for fp32) with 16-byte aligned rows selects the 16-byte loads.

@@ -18,7 +18,7 @@
 // register and every branch taken by whole waves (votes instead of atomics): no LDS atomics left, but
 // 12 % more vector instructions (each vote costs a select and a compare) and 10 % more time.
 // Ties go to the smaller id, deterministically; torch.topk, which the reference calls, leaves tie
-// order open.  Rows with more than 2048 entries at or above L (constant or coarsely quantised rows)
+// order open.  (Values are ordered by their bit patterns: -0 ranks just below +0, not level with it.)  Rows with more than 2048 entries at or above L (constant or coarsely quantised rows)
 // take an exact but slow select by bisection over key bits and then over columns.
 #include "distill_common.hpp"
 #include "distill_hip.h"
