@@ -139,6 +139,8 @@ def _oracle_multi(logits, vals, idxs, weights, id_map, T, valid=None):
     (152064, torch.float16, 1, 200, 152064, 1.0),       # a single teacher through the map, 5 parts
     (65536, torch.bfloat16, 4, 128, 70000, 0.7),        # 512 x 16, one workgroup per row
     (100000, torch.bfloat16, 8, 64, 120000, 1.0),       # 8 teachers: 8 slots
+    (128256, torch.float32, 2, 100, 152064, 1.0),       # 4 parts of 512 threads x 16 chunks
+    (262144, torch.bfloat16, 2, 100, 152064, 1.0),      # the same for two-byte rows
 ])
 def test_bucketed_multi_teacher_against_oracle(D, V, dtype, n, K, Vt, T):
     """dl_fkl_multi_teacher (entries mapped, renormalised and dealt into per-part buckets by a K-wide

@@ -202,10 +202,12 @@ def test_gradient_may_overwrite_the_logits(D, kind, V, dtype):
 
 
 
-@pytest.mark.parametrize("V,dtype", [(152064, torch.bfloat16), (128256, torch.float32), (262144, torch.float16)])
+@pytest.mark.parametrize("V,dtype", [(152064, torch.bfloat16), (128256, torch.float32), (262144, torch.float16),
+                                     (100000, torch.float32), (98304, torch.float32), (229376, torch.bfloat16)])
 def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
     """Vocabularies beyond 131072 two-byte (65536 four-byte) entries are cut into 5..8 parts of 4096
-    chunks; with and without waiting for the partners the oracle's numbers and the same bits."""
+    chunks, or (four-byte rows of 6 parts and more, two-byte rows of 8) into 3..4 parts of 8192; with and
+    without waiting for the partners the oracle's numbers and the same bits."""
     logits, tv, ti = _case(10, V, 48, dtype, 41, std=3.0)
     valid = torch.ones(10, dtype=torch.bool)
     valid[4] = False
