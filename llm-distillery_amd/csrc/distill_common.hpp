@@ -461,6 +461,27 @@ __device__ __forceinline__ void block_sort(W (&c)[EPL], W* xch) {
   }
 }
 
+// A row that starts or ends off the 16-byte grid, seen as head | body | tail: the body is made of the
+// 16-byte chunks that lie wholly inside the row (vector loads and stores), head and tail are the at
+// most N - 1 elements on either side (element-wise).  peel == false: the row is on the grid and a whole
+// number of chunks long; everything is body.
+template <class Tag>
+struct RowSplit {
+  int head; int64_t nbody; int tail;
+  __device__ __forceinline__ RowSplit(const void* row, int64_t V, bool peel) {
+    constexpr int N = 16 / Tag::bytes;
+    const int mis = peel ? (int)(reinterpret_cast<uintptr_t>(row) & 15) : 0;
+    int64_t h = mis ? (16 - mis) / Tag::bytes : 0;
+    if (h > V) h = V;
+    head = (int)h;
+    nbody = (V - h) / N;
+    tail = (int)(V - h - nbody * N);
+  }
+  __device__ __forceinline__ int leftovers() const { return head + tail; }
+  // column of leftover i, 0 <= i < leftovers()
+  __device__ __forceinline__ int64_t column(int i) const { return i < head ? i : head + nbody * (16 / Tag::bytes) + (i - head); }
+};
+
 // zero-fill one gradient row (masked / padded token positions)
 template <class Tag, int NT>
 __device__ __forceinline__ void zero_row(void* grad_row, int64_t nchunks) {

@@ -19,7 +19,10 @@ struct StatsParams {
 };
 
 // ---- phase 1: lse_r = logsumexp_j(x_rj * inv_T),  zk_rk = x[r, idx_rk] * inv_T ------------------
-template <class Tag, int NT, bool VEC>
+// MODE 0: element-wise loads (rows that are not even element-aligned never get here; kept for reference
+// and for rows shorter than a chunk).  MODE 1: rows on the 16-byte grid, a whole number of chunks long.
+// MODE 2: any other row: its 16-byte chunks by vector loads, the elements before and behind them one by one.
+template <class Tag, int NT, int MODE>
 __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
   __shared__ float red[64];
   using C = Chunk<Tag>;
@@ -34,14 +37,20 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
   }
   const float a = p.inv_T * LOG2E;
   float m = -INFINITY, sm = 0.f;
-  if (VEC) {
-    const int64_t nch = p.V / C::N;
+  const auto one = [&](float f) {
+    if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
+    if (f > -INFINITY) sm += fast_exp2(fmaf(f, a, -m * a));
+  };
+  if (MODE != 0) {
+    const RowSplit<Tag> sp(row, p.V, MODE == 2);
+    const char* body = row + (int64_t)sp.head * Tag::bytes;
+    const int64_t nch = sp.nbody;
     for (int64_t c0 = 0; c0 < nch; c0 += 4 * NT) {          // four 16-byte loads in flight per thread
       u32x4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int64_t ch = c0 + (int64_t)u * NT + tid;
-        v[u] = ch < nch ? load16_stream(row + ch * 16) : C::neg_inf();
+        v[u] = ch < nch ? load16_stream(body + ch * 16) : C::neg_inf();
       }
       float cm = -INFINITY;
       float f[4][C::N];
@@ -60,12 +69,9 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
           for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[u][e], a, -mb));
       }
     }
+    if (MODE == 2 && tid < sp.leftovers()) one(load_as_float(row, Tag::id, sp.column(tid)));
   } else {
-    for (int64_t j = tid; j < p.V; j += NT) {
-      const float f = load_as_float(row, Tag::id, j);
-      if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
-      sm += fast_exp2(fmaf(f, a, -m * a));
-    }
+    for (int64_t j = tid; j < p.V; j += NT) one(load_as_float(row, Tag::id, j));
   }
   const float mx = block_max<NT>(m, red);
   sm = (m == -INFINITY) ? 0.f : sm * fast_exp2((m - mx) * a);
@@ -91,9 +97,13 @@ __device__ __forceinline__ float coef_on_id(const int* s_idx, const float* s_c, 
   return cs;
 }
 
-template <class Tag, int NT, int NCH, bool VEC>
+// MODE as for phase 1.  MODE 2 needs the gradient row to sit on the 16-byte grid exactly as the logits row does
+// (same address modulo 16): the kernel then works on the rows' bodies, with the teacher ids counted
+// from the body's first column, and part 0 adds the few columns before and behind the body one by one.
+template <class Tag, int NT, int NCH, int MODE>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void rowcoef_grad_kernel(const StatsParams p, int parts) {
+  constexpr bool VEC = MODE != 0;
   extern __shared__ __align__(16) unsigned char smem[];
   using C = Chunk<Tag>;
   const int Kp = (p.K + 15) & ~15;
@@ -112,13 +122,20 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
   if (r >= p.n_rows) return;
   const int tid = threadIdx.x;
   const int64_t per_part = (int64_t)NT * NCH * C::N;                 // columns per part
-  const int64_t lo = h * per_part, hi = min(p.V, lo + per_part);
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
-  char* grow = reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes;
-  const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  char* grow_all = reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes;
+  const char* row_all = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  // what the sweeps below see as the row: all of it, or (MODE 2) its body
+  const RowSplit<Tag> sp(row_all, p.V, MODE == 2);
+  const int64_t V = MODE == 2 ? sp.nbody * C::N : p.V;
+  const int shift = MODE == 2 ? sp.head : 0;                         // column of the row that is column 0 of the sweeps
+  char* grow = grow_all + (int64_t)shift * Tag::bytes;
+  const char* row = row_all + (int64_t)shift * Tag::bytes;
+  const int64_t lo = min(V, h * per_part), hi = min(V, lo + per_part);
   if (trow < 0) {
     if (VEC) zero_row<Tag, NT>(grow + lo * Tag::bytes, (hi - lo) / C::N);
     else for (int64_t j = lo + tid; j < hi; j += NT) store_from_float(grow, Tag::id, j, 0.f);
+    if (MODE == 2 && h == 0 && tid < sp.leftovers()) store_from_float(grow_all, Tag::id, sp.column(tid), 0.f);
     return;
   }
   const float a = p.inv_T * LOG2E;
@@ -130,11 +147,22 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     for (int k = tid; k < Kp; k += NT) {
       int64_t id = -1;
       float cv = 0.f;
+      bool in_row = false;                                           // ids outside the row name no column
       if (k < p.K) {
         id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
+        in_row = id >= 0 && id < p.V;
+        id -= shift;
         cv = p.coef_zk[trow * p.K + k];
       }
-      const bool mine = id >= lo && id < hi;
+      const bool mine = in_row && id >= lo && id < hi;
+      if (MODE == 2 && h == 0 && in_row && (id < 0 || id >= V)) {
+        // a column before or behind the body: leftover number li is kept as -2 - li for part 0's last step
+        const int64_t li = id < 0 ? id + shift : sp.head + (id - V);
+        s_idx[k] = -2 - (int)li;
+        s_c[k] = cv;
+        s_z[k] = 0.f;
+        continue;
+      }
       s_idx[k] = mine ? (int)id : -1;
       s_c[k] = cv;
       s_z[k] = mine ? load_as_float(row, Tag::id, id) : 0.f;
@@ -181,6 +209,13 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     if (repeats)
       correction_repeats<Tag, NT>(s_head, s_next, s_idx, (int)lo, repeats, NCH, coef, value,
                                   [&](int column, float g) { store_from_float(grow, Tag::id, column, g); });
+    if (MODE == 2 && h == 0 && tid < sp.leftovers()) {
+      // a column before or behind the body: dense value plus the coefficients of every entry that names it
+      const int64_t j = sp.column(tid);
+      float cs = 0.f;
+      for (int k = 0; k < Kp; ++k) cs += s_idx[k] == -2 - tid ? s_c[k] : 0.f;
+      store_from_float(grow_all, Tag::id, j, fast_exp2(fmaf(load_as_float(row_all, Tag::id, j), a, -b)) * w + cs * p.inv_T);
+    }
     return;
   } else {
     stage();
@@ -200,15 +235,22 @@ static bool aligned16(const void* ptr, int64_t stride, int eb) {
   return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (stride * eb) % 16 == 0;
 }
 
+// Rows whose addresses differ by a multiple of 16 bytes, row for row: what the kernels that sweep the
+// 16-byte chunks inside unaligned rows need of a (logits, gradient) pair.
+static bool same_phase16(const void* a, int64_t stride_a, const void* b, int64_t stride_b, int eb) {
+  return reinterpret_cast<uintptr_t>(a) % 16 == reinterpret_cast<uintptr_t>(b) % 16 && ((stride_a - stride_b) * eb) % 16 == 0;
+}
+
 template <class Tag>
-static hipError_t launch_stats(const StatsParams& p, bool vec, hipStream_t st) {
-  if (vec) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, true>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((rowstats_kernel<Tag, 256, false>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
+static hipError_t launch_stats(const StatsParams& p, int mode, hipStream_t st) {
+  if (mode == 1) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 1>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
+  else if (mode == 2) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 2>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 0>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
   return hipGetLastError();
 }
 
 template <class Tag>
-static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
+static hipError_t launch_coef(const StatsParams& p, int mode, hipStream_t st) {
   // 4 chunks per thread: this kernel keeps nothing of the row beyond the chunk it is converting, and a
   // stream that moves few chunks per thread between its loads and its stores runs 6-9 % faster on this
   // device than one that moves 16 (measured on a plain copy as well: 78 % against 70 % of peak)
@@ -217,8 +259,9 @@ static hipError_t launch_coef(const StatsParams& p, bool vec, hipStream_t st) {
   const int parts = (int)((p.V + per_part - 1) / per_part);
   const size_t lds = (size_t)((p.K + 15) & ~15) * 20 + (size_t)CORRECTION_HEADS * 4 + (size_t)NT * 4;   // ids, coefficients, logits, values, links; list heads, chunk masks
   const dim3 grid((unsigned)((p.n_rows + 7) / 8 * 8 * parts));
-  if (vec) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, true>), grid, dim3(NT), lds, st, p, parts);
-  else hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, false>), grid, dim3(NT), lds, st, p, parts);
+  if (mode == 1) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 1>), grid, dim3(NT), lds, st, p, parts);
+  else if (mode == 2) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 2>), grid, dim3(NT), lds, st, p, parts);
+  else hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 0>), grid, dim3(NT), lds, st, p, parts);
   return hipGetLastError();
 }
 
@@ -242,7 +285,8 @@ extern "C" int dl_rowstats_topk(const void* logits, int logits_dtype, int64_t ro
   if ((!lse || !zk) && n_teacher_rows > 0) return DL_ERR_NULL;
   if (n_rows == 0) return DL_OK;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
-  const bool vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb);
+  if (reinterpret_cast<uintptr_t>(logits) % eb != 0) return DL_ERR_ALIGN;
+  const int vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb) ? 1 : 2;
   StatsParams p{logits, row_stride, n_rows, V, row_map, t_idx, t_idx_itype, K, n_teacher_rows, inv_T, lse, zk,
                 nullptr, nullptr, nullptr, 0};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -263,7 +307,9 @@ extern "C" int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_
   if (grad_stride < V) return DL_ERR_SHAPE;
   if (n_rows == 0) return DL_OK;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
-  const bool vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb) && aligned16(grad, grad_stride, eb);
+  if (reinterpret_cast<uintptr_t>(logits) % eb != 0 || reinterpret_cast<uintptr_t>(grad) % eb != 0) return DL_ERR_ALIGN;
+  const int vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb) && aligned16(grad, grad_stride, eb) ? 1
+                  : same_phase16(logits, row_stride, grad, grad_stride, eb) ? 2 : 0;
   StatsParams p{logits, row_stride, n_rows, V, row_map, t_idx, t_idx_itype, K, n_teacher_rows, inv_T,
                 const_cast<float*>(lse), nullptr, coef_lse, coef_zk, grad, grad_stride};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);

@@ -28,6 +28,7 @@ static int div_topk_checked(int kind, const void* logits, int logits_dtype, int6
   if (n_rows == 0 || !launch) return DL_OK;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
   const int epc = 16 / eb;
+  if (reinterpret_cast<uintptr_t>(logits) % eb != 0 || (grad && reinterpret_cast<uintptr_t>(grad) % eb != 0)) return DL_ERR_ALIGN;
   const bool aligned = (V % epc == 0) && (reinterpret_cast<uintptr_t>(logits) % 16 == 0) &&
                        ((row_stride * eb) % 16 == 0) &&
                        (!grad || (reinterpret_cast<uintptr_t>(grad) % 16 == 0 && (grad_stride * eb) % 16 == 0));

@@ -419,30 +419,37 @@ __device__ __forceinline__ void fkl_link_corrections(const TopkLds& s, int lo, i
 
 // Full-row statistics straight from global memory (two uses: the streaming kernel, and a split
 // part whose partner did not answer in time).  Returns the row maximum and sum 2^((x - max) a).
-template <class Tag, int NT, bool VEC>
+// MODE 0: element by element.  MODE 1: rows on the 16-byte grid, a whole number of chunks long.
+// MODE 2: any row: its 16-byte chunks by vector loads, the elements before and behind them one by one.
+template <class Tag, int NT, int MODE>
 __device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, float a, float* red, float& mx,
                                                    float& sm) {
   using C = Chunk<Tag>;
   float m = -INFINITY;
   sm = 0.f;
-  if (VEC) {
-    for (int64_t ch = threadIdx.x; ch < V / C::N; ch += NT) {
+  const auto one = [&](float f) {
+    if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
+    if (f > -INFINITY) sm += fast_exp2(fmaf(f, a, -m * a));
+  };
+  if (MODE != 0) {
+    const RowSplit<Tag> sp(row, V, MODE == 2);
+    const char* body = row + (int64_t)sp.head * Tag::bytes;
+    for (int64_t ch = threadIdx.x; ch < sp.nbody; ch += NT) {
       float f[C::N];
-      C::unpack(*reinterpret_cast<const u32x4*>(row + ch * 16), f);
+      C::unpack(*reinterpret_cast<const u32x4*>(body + ch * 16), f);
       float cm = f[0];
 #pragma unroll
       for (int e = 1; e < C::N; ++e) cm = fmaxf(cm, f[e]);
       if (cm > m) { sm *= fast_exp2((m - cm) * a); m = cm; }
       const float mb = m * a;
+      if (m > -INFINITY) {
 #pragma unroll
-      for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[e], a, -mb));
+        for (int e = 0; e < C::N; ++e) sm += fast_exp2(fmaf(f[e], a, -mb));
+      }
     }
+    if (MODE == 2 && (int)threadIdx.x < sp.leftovers()) one(load_as_float(row, Tag::id, sp.column(threadIdx.x)));
   } else {
-    for (int64_t j = threadIdx.x; j < V; j += NT) {
-      const float f = load_as_float(row, Tag::id, j);
-      if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
-      sm += fast_exp2(fmaf(f, a, -m * a));
-    }
+    for (int64_t j = threadIdx.x; j < V; j += NT) one(load_as_float(row, Tag::id, j));
   }
   mx = block_max<NT>(m, red);
   sm = (m == -INFINITY) ? 0.f : sm * fast_exp2((m - mx) * a);
@@ -668,8 +675,10 @@ void fkl_topk_retry_kernel(const TopkParams p) {
 
 // ---------------------------------------------------------------------------------------
 // Forward KL, streaming: any V, any alignment; the row is read twice (second read mostly L2 / MALL).
+// MODE as for row_stats_streamed; MODE 2 needs the gradient row to sit on the 16-byte grid as the
+// logits row does (same address modulo 16), so that the chunks of both line up.
 // ---------------------------------------------------------------------------------------
-template <class Tag, int NT, bool VEC>
+template <class Tag, int NT, int MODE>
 __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const TopkLds s(smem, p.K);
@@ -678,16 +687,20 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
   if (r >= p.n_rows) return;
   const int tid = threadIdx.x;
   const int64_t V = p.V;
-  const int64_t nch = V / C::N;
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  const RowSplit<Tag> sp(row, V, MODE == 2);
   float tlse = -INFINITY;
   if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
   if (tlse == -INFINITY) {
     if (grow) {
-      if (VEC) zero_row<Tag, NT>(grow, nch);
-      else for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
+      if (MODE != 0) {
+        zero_row<Tag, NT>(grow + (int64_t)sp.head * Tag::bytes, sp.nbody);
+        if (MODE == 2 && tid < sp.leftovers()) store_from_float(grow, Tag::id, sp.column(tid), 0.f);
+      } else {
+        for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
+      }
     }
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
@@ -696,19 +709,25 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
   fkl_partials<NT>(p, s, 0, (int)V, B, Q);
   const float a = p.inv_T_s * LOG2E;
   float mx, sm;
-  row_stats_streamed<Tag, NT, VEC>(row, V, a, s.red, mx, sm);
+  row_stats_streamed<Tag, NT, MODE>(row, V, a, s.red, mx, sm);
   const float b = mx * a + fast_log2(sm);
   if (tid == 0 && p.row_loss) p.row_loss[r] = B + (b * LN2) * Q;
 
   if (grow) {
     const float c = p.inv_T_s * p.grad_scale;
-    if (VEC) {
-      for (int64_t ch = tid; ch < nch; ch += NT) {
+    if (MODE != 0) {
+      const char* body = row + (int64_t)sp.head * Tag::bytes;
+      char* gbody = grow + (int64_t)sp.head * Tag::bytes;
+      for (int64_t ch = tid; ch < sp.nbody; ch += NT) {
         float f[C::N];
-        C::unpack(*reinterpret_cast<const u32x4*>(row + ch * 16), f);
+        C::unpack(*reinterpret_cast<const u32x4*>(body + ch * 16), f);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * c;
-        store16_stream(grow + ch * 16, C::pack(f));
+        store16_stream(gbody + ch * 16, C::pack(f));
+      }
+      if (MODE == 2 && tid < sp.leftovers()) {
+        const int64_t j = sp.column(tid);
+        store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * c);
       }
     } else {
       for (int64_t j = tid; j < V; j += NT)
@@ -722,8 +741,12 @@ __global__ __launch_bounds__(NT) void fkl_topk_stream_kernel(const TopkParams p)
 // ---------------------------------------------------------------------------------------
 // Reverse KL on the teacher's support: K gathered logits per row, gradient = zero row + K values.
 // ---------------------------------------------------------------------------------------
-template <class Tag, int NT, bool VEC>
+// MODE 0: element-wise stores.  MODE 1: gradient rows on the 16-byte grid, a whole number of chunks long.
+// MODE 2: any other gradient row: its 16-byte chunks by vector stores (the teacher ids counted from the
+// first of them), the columns before and behind them one by one.
+template <class Tag, int NT, int MODE>
 __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
+  constexpr bool VEC = MODE != 0;
   extern __shared__ __align__(16) unsigned char smem[];
   const TopkLds s(smem, p.K, NT);
   using C = Chunk<Tag>;
@@ -734,14 +757,20 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+  const RowSplit<Tag> sp(grow, V, MODE == 2 && grow);              // the row that is written decides
+  char* gbody = grow + (int64_t)sp.head * Tag::bytes;
   correction_clear<NT>(s.head, s.own);
   float tlse = -INFINITY;
   if (trow >= 0) tlse = stage_teacher<Tag, NT>(p, s, trow, row, 0, (int)V);
   // Every store comes after the K logits have been gathered (stage_teacher ends in barriers), so
   // the gradient may be written over the logits.
   if (grow && (!VEC || tlse == -INFINITY)) {
-    if (VEC) zero_row<Tag, NT>(grow, V / C::N);
-    else for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
+    if (VEC) {
+      zero_row<Tag, NT>(gbody, sp.nbody);
+      if (MODE == 2 && tid < sp.leftovers()) store_from_float(grow, Tag::id, sp.column(tid), 0.f);
+    } else {
+      for (int64_t j = tid; j < V; j += NT) store_from_float(grow, Tag::id, j, 0.f);
+    }
   }
   if (tlse == -INFINITY) {
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
@@ -776,7 +805,9 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
       const int id = s.idx[k];
       if (id < 0) continue;
       if (VEC) {
-        correction_link<Tag, NT>(s.head, s.own, s.next, k, id);     // placed by the thread that writes the column's chunk
+        // placed by the thread that writes the column's chunk; columns beside the body are left to the last step
+        const int64_t idb = (int64_t)id - sp.head;
+        if (idb >= 0 && idb < sp.nbody * C::N) correction_link<Tag, NT>(s.head, s.own, s.next, k, (int)idb);
       } else {
         float g = 0.f;
         for (int j = 0; j < s.Kp; ++j) g += (s.idx[j] == id) ? s.q[j] * (s.z[j] - rkl) : 0.f;
@@ -787,7 +818,7 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
       // the row of zeros, each chunk written once with the support's values already in place
       __syncthreads();
       const unsigned mine = s.own[tid];
-      const int64_t nch = V / C::N;
+      const int64_t nch = sp.nbody;
       const auto term = [&](int k) { return s.q[k] * (s.z[k] - rkl); };
       const auto value = [&](int, float g) { return g * c; };
       unsigned repeats = 0u;
@@ -797,13 +828,19 @@ __global__ __launch_bounds__(NT) void rkl_topk_kernel(const TopkParams p) {
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = 0.f;
         if (mine & (1u << (i & 31)))
-          if (correction_apply<Tag, NT>(s.head, s.next, s.idx, 0, (int)i, f, term, value)) repeats |= 1u << (i & 31);
-        store16_stream(grow + ch * 16, C::pack(f));
+          if (correction_apply<Tag, NT>(s.head, s.next, s.idx, sp.head, (int)i, f, term, value)) repeats |= 1u << (i & 31);
+        store16_stream(gbody + ch * 16, C::pack(f));
         n_own = (int)i + 1;
       }
       if (repeats)
-        correction_repeats<Tag, NT>(s.head, s.next, s.idx, 0, repeats, n_own, term, value,
+        correction_repeats<Tag, NT>(s.head, s.next, s.idx, sp.head, repeats, n_own, term, value,
                                     [&](int column, float v) { store_from_float(grow, Tag::id, column, v); });
+      if (MODE == 2 && tid < sp.leftovers()) {
+        const int64_t j = sp.column(tid);
+        float g = 0.f;
+        for (int k = 0; k < s.Kp; ++k) g += (s.idx[k] == j) ? term(k) : 0.f;
+        store_from_float(grow, Tag::id, j, g * c);
+      }
     }
   }
 }
@@ -954,11 +991,18 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
     default: break;
   }
   if (MULTI) return aligned ? DL_ERR_LIMIT : DL_ERR_ALIGN;
+  // rows off the 16-byte grid: their chunks by vector accesses if logits and gradient rows share their
+  // address modulo 16 (the same pitch from 16-byte aligned bases, or the gradient written over the logits)
+  const bool same_phase = !p.grad || (reinterpret_cast<uintptr_t>(p.logits) % 16 == reinterpret_cast<uintptr_t>(p.grad) % 16 &&
+                                      ((p.row_stride - p.grad_stride) * Tag::bytes) % 16 == 0);
   if (aligned) {
-    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
+    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, 1>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
+                       TopkLds::bytes(p.K), st, p);
+  } else if (same_phase) {
+    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, 2>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
                        TopkLds::bytes(p.K), st, p);
   } else {
-    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, false>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
+    hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, 0>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
                        TopkLds::bytes(p.K), st, p);
   }
   return launch_status();
@@ -966,11 +1010,12 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
 
 template <class Tag>
 static hipError_t launch_rkl(const TopkParams& p, bool aligned, hipStream_t st) {
+  // the logits are only gathered from; what is written decides: MODE 2 takes any gradient row
   if (aligned)
-    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, true>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
+    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, 1>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
                        TopkLds::bytes(p.K, 256), st, p);
   else
-    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, false>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
+    hipLaunchKernelGGL((rkl_topk_kernel<Tag, 256, 2>), dim3(xcd_banded_grid(p.n_rows)), dim3(256),
                        TopkLds::bytes(p.K, 256), st, p);
   return hipGetLastError();
 }

@@ -28,10 +28,20 @@ def _dev(t: torch.Tensor, name: str, dev: torch.device | None = None) -> None:
         raise RuntimeError(f"{name} lives on {t.device}, the logits on {dev}: all tensors of a call must share one device")
 
 
-def _grad_target(grad_out, R: int, V: int, dtype, dev) -> torch.Tensor:
+def _grad_target(grad_out, R: int, V: int, dtype, dev, like: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The gradient buffer of a launch over [R, V] logits: `grad_out` checked against what the kernel
-    will write (shape, dtype, dense along V, same device), or a fresh one."""
+    will write (shape, dtype, dense along V, same device), or a fresh one.  A fresh buffer for logits
+    `like` whose rows do not all start on 16-byte boundaries (a column slice, an odd pitch) copies their
+    pitch and their offset on the 16-byte grid: the kernels use vector accesses inside such rows only when
+    logits and gradient rows line up."""
     if grad_out is None:
+        if like is not None and like.dim() == 2:
+            eb = like.element_size()
+            phase = (like.data_ptr() % 16) // eb
+            if phase or (like.stride(0) * eb) % 16 or (V * eb) % 16:
+                pitch = like.stride(0)
+                buf = torch.empty(R * pitch + phase + 8, dtype=dtype, device=dev)      # torch allocations start on 16-byte boundaries
+                return buf.as_strided((R, V), (pitch, 1), phase)
         return torch.empty((R, V), dtype=dtype, device=dev)
     if grad_out.dim() != 2 or tuple(grad_out.shape) != (R, V) or grad_out.dtype != dtype or grad_out.stride(1) != 1 \
             or grad_out.device != dev:
@@ -106,7 +116,7 @@ def div_topk(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.
     row_loss = torch.empty(R, dtype=torch.float32, device=dev)
     grad, g_ptr, g_stride = None, 0, V
     if want_grad:
-        grad = _grad_target(grad_out, R, V, x.dtype, dev)
+        grad = _grad_target(grad_out, R, V, x.dtype, dev, like=x)
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
     if parts not in (0, 1, 2, 4, 16):
         raise ValueError("parts must be 0 (automatic), 1, 2, 4 or 16 (parts of 1024 chunks, up to 16 per row)")
@@ -245,7 +255,7 @@ def _rowcoef_grad_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: floa
     g_zk = g_zk.to(torch.float32).contiguous()
     for name, t in (("t_idx", t_idx), ("lse", lse), ("g_lse", g_lse), ("g_zk", g_zk)):
         _dev(t, name, x.device)
-    grad = _grad_target(grad_out, R, V, x.dtype, x.device)
+    grad = _grad_target(grad_out, R, V, x.dtype, x.device, like=x)
     with torch.cuda.device(x.device):
         st = _lib.load().dl_rowcoef_grad_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(),
                                               _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), g_lse.data_ptr(),

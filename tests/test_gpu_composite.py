@@ -52,7 +52,7 @@ def _convo(N, V, K, seed, dtype=torch.float32):
     return student, tv, ti, labels
 
 
-@pytest.mark.parametrize("V,K,N", [(32000, 200, 130), (128256, 64, 21), (1000, 16, 50)])
+@pytest.mark.parametrize("V,K,N", [(32000, 200, 130), (128256, 64, 21), (1000, 16, 50), (32003, 200, 40), (1001, 16, 50), (5, 3, 9)])
 def test_calculate_divergence_against_oracle_fp32(D, V, K, N):
     student, tv, ti, labels = _convo(N, V, K, 5)
     avoid = torch.tensor([3, N // 2])
@@ -170,6 +170,46 @@ def test_rowstats_raw_outputs_and_losses_accumulator_on_gpu(D):
     L.backward(divisor=2)
     assert all(s.grad is not None and torch.isfinite(s.grad).all() for s in leafs)
     assert total > 0 and L.num_steps_accumulated == 2
+
+
+@pytest.mark.parametrize("dtype,V,pitch,offset", [(torch.bfloat16, 32003, 32003, 0), (torch.float32, 1003, 1003, 0),
+                                                  (torch.bfloat16, 5001, 5120, 3), (torch.float16, 7, 7, 0)])
+@pytest.mark.parametrize("grad_mode", ["fresh", "other_phase"])
+def test_two_phase_kernels_on_rows_off_the_16_byte_grid(D, dtype, V, pitch, offset, grad_mode):
+    """Phase 1 and phase 2 on rows that do not start or end on 16-byte boundaries (vector accesses to the
+    chunks inside them, element-wise beside; element-wise throughout when the gradient buffer sits on
+    another phase of the grid), with repeated ids, ids in the first and last columns and masked rows."""
+    from llm_distillery_amd import ops
+    R, K = 9, min(12, V)
+    g = torch.Generator().manual_seed(V)
+    xs = (torch.randn(R, V, generator=g) * 3).to(dtype)
+    idx = torch.randint(0, V, (R - 2, K), generator=g, dtype=torch.int32)
+    idx[:, 0] = 0
+    idx[:, 1] = V - 1
+    idx[:, 2] = idx[:, 1]                                         # a repeated id in the last column
+    rm = torch.tensor([0, 1, -1, 2, 3, 4, -1, 5, 6], dtype=torch.int32)
+    full = torch.zeros(R, pitch + 8, dtype=dtype, device=DEV)
+    x = full[:, offset:offset + V] if pitch != V else xs.to(DEV)
+    if pitch != V:
+        x.copy_(xs.to(DEV))
+    inv_T = 0.7
+    lse, zk = ops._rowstats_raw(x, idx.to(DEV), rm.to(DEV), inv_T)
+    sel = rm >= 0
+    ref_lse = torch.logsumexp(xs[sel].double() * inv_T, -1)
+    np.testing.assert_allclose(lse.cpu().double().numpy(), ref_lse.numpy(), rtol=2e-6, atol=2e-6)
+    assert torch.equal(zk.cpu(), torch.gather(xs[sel].float(), 1, idx.long()) * inv_T)
+    g_lse = torch.randn(R - 2, generator=g)
+    g_zk = torch.randn(R - 2, K, generator=g)
+    out = None if grad_mode == "fresh" else torch.empty(R, x.stride(0) + 1, dtype=dtype, device=DEV)[:, 1:1 + V]
+    grad = ops._rowcoef_grad_raw(x, idx.to(DEV), rm.to(DEV), inv_T, lse, g_lse.to(DEV), g_zk.to(DEV), grad_out=out)
+    ref = torch.zeros(R, V, dtype=torch.float64)
+    p = torch.softmax(xs[sel].double() * inv_T, -1) * g_lse.double().unsqueeze(-1)
+    p.scatter_add_(1, idx.long(), g_zk.double())
+    ref[sel] = p * inv_T
+    err = (grad.cpu().double() - ref).abs()
+    bound = O.storage_tolerance(ref, dtype, 1e-4 if dtype == torch.float32 else 2e-3) + 1e-6
+    assert (err <= bound).all(), f"worst {(err / bound).max():.2f}"
+    assert torch.count_nonzero(grad.cpu()[~sel]) == 0
 
 
 def test_batched_caller_equals_the_per_conversation_loop(D):

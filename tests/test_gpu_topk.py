@@ -94,6 +94,54 @@ def test_streaming_path_odd_vocab_and_int64_fp32_teacher(D, V):
     _check(D, "rkl", logits, tv, ti, T=1.3)
 
 
+@pytest.mark.parametrize("dtype,V,pitch,offset", [(torch.bfloat16, 32003, 32003, 0),      # contiguous odd rows: every row starts elsewhere on the grid
+                                                  (torch.float32, 1003, 1003, 0),
+                                                  (torch.bfloat16, 5001, 5120, 3),          # a column slice of aligned rows: one phase for all rows
+                                                  (torch.float16, 7, 7, 0),                 # rows shorter than a chunk
+                                                  (torch.float32, 4099, 4104, 2)])
+@pytest.mark.parametrize("grad_mode", ["fresh", "in_place", "other_phase"])
+@pytest.mark.parametrize("kind", ["fkl", "rkl"])
+def test_rows_off_the_16_byte_grid(D, kind, dtype, V, pitch, offset, grad_mode):
+    """Rows that do not start on 16-byte boundaries or do not end on one: their 16-byte chunks go through
+    vector accesses when logits and gradient rows share their address modulo 16 (a fresh gradient of the
+    same pitch, or the gradient written over the logits), the few elements on either side one by one;
+    a gradient buffer on another phase takes the element-wise kernel (reverse KL, which only gathers from
+    the logits, goes by the gradient rows alone).  All three against the oracle."""
+    R, K = 7, min(24, V)
+    logits, tv, ti = _case(R, V, K, dtype, 61, std=3.0)
+    valid = torch.ones(R, dtype=torch.bool)
+    valid[2] = False
+    rm = torch.full((R,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(R - 1, dtype=torch.int32)
+    tv, ti = tv[valid], ti[valid]
+    ti[:, 0] = 0                                                  # entries in the first and the last column
+    ti[:, 1] = V - 1
+    if K > 3:
+        ti[:, 2] = V - 1                                          # and a repeated id there
+    tl = torch.log_softmax(logits[valid].float() * 1.1, -1)       # teacher values that belong to those ids
+    tv = torch.gather(tl, 1, ti.long()).to(tv.dtype)
+    loss64, rows64, grad64 = O.mean_loss_and_grad(kind, logits, 1.3, t_vals=tv, t_idx=ti, valid=valid, dtype=torch.float64)
+    full = torch.zeros(R, pitch + 8, dtype=dtype, device=DEV)
+    x = full[:, offset:offset + V] if pitch != V else logits.to(DEV)
+    if pitch != V:
+        x.copy_(logits.to(DEV))
+    assert x.stride(0) == (pitch + 8 if pitch != V else V)
+    if grad_mode == "fresh":
+        out = None
+    elif grad_mode == "in_place":
+        out = x
+    else:
+        out = torch.empty(R, x.stride(0) + 1, dtype=dtype, device=DEV)[:, 1:1 + V]
+    rl, grad = D.div_topk(kind, x, tv.to(DEV), ti.to(DEV), row_map=rm.to(DEV), T=1.3, grad_scale=1.0 / (R - 1), grad_out=out)
+    assert grad_mode == "fresh" or grad.data_ptr() == out.data_ptr()
+    np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+    assert rl[2].item() == 0 and torch.count_nonzero(grad[2]) == 0
+    err = (grad.cpu().double() - grad64).abs()
+    assert (err <= O.storage_tolerance(grad64, dtype, TOL[dtype])).all(), f"worst {(err / O.storage_tolerance(grad64, dtype, TOL[dtype])).max():.2f}"
+    if pitch != V and grad_mode != "in_place":      # nothing outside the slice was touched
+        assert torch.count_nonzero(full[:, :offset]) == 0 and torch.count_nonzero(full[:, offset + V:]) == 0
+
+
 def test_streaming_path_rows_larger_than_register_file(D):
     logits, tv, ti = _case(6, 152064, 200, torch.bfloat16, 6)
     _check(D, "fkl", logits, tv, ti, T=1.0)
