@@ -57,8 +57,9 @@ struct RegRows {
       forget(t[i].c[0]);
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
-        a = __builtin_elementwise_max(a, __builtin_bit_cast(i16x2, s[i].c[0][d]));
-        b = __builtin_elementwise_max(b, __builtin_bit_cast(i16x2, t[i].c[0][d]));
+        const unsigned ws = s[i].c[0][d], wt = t[i].c[0][d];      // by value: a bit cast straight from a vector element reads element 0
+        a = __builtin_elementwise_max(a, __builtin_bit_cast(i16x2, ws));
+        b = __builtin_elementwise_max(b, __builtin_bit_cast(i16x2, wt));
       }
     }
     float fa = (float)max((int)a.x, (int)a.y), fb = (float)max((int)b.x, (int)b.y);      // exact, order-preserving

@@ -356,7 +356,10 @@ void topk_part_kernel(const ProducerParams p) {
     for (int i = 0; i < NCH; ++i) {
       forget(reg[i]);
 #pragma unroll
-      for (int d = 0; d < 4; ++d) pm = __builtin_elementwise_max(pm, __builtin_bit_cast(i16x2, reg[i][d]));
+      for (int d = 0; d < 4; ++d) {
+        const unsigned w16 = reg[i][d];      // by value: a bit cast straight from a vector element reads element 0
+        pm = __builtin_elementwise_max(pm, __builtin_bit_cast(i16x2, w16));
+      }
     }
     const int top = block_max_int<NT>(max((int)pm.x, (int)pm.y), ired);
     if (top >= 0) {

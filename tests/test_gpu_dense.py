@@ -78,6 +78,19 @@ def test_dense_16bit_rows_whose_maximum_is_negative_or_zero(D, kind, dtype):
     _check(D, kind, s.to(dtype), t.to(dtype), T=1.0)
 
 
+@pytest.mark.parametrize("kind", ["fkl", "jsd"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dense_16bit_rows_with_one_towering_logit(D, kind, dtype):
+    """A logit far above the rest of its row, at every position inside a 16-byte chunk in turn: a maximum
+    that missed it would let the sums of exponentials overflow."""
+    s, t = _pair(8, 4096, dtype, 9)
+    s, t = s.float(), t.float()
+    for r in range(8):
+        s[r, 8 * (3 + 17 * r) + r] = 150.0
+        t[r, 8 * (5 + 11 * r) + (7 - r)] = 140.0
+    _check(D, kind, s.to(dtype), t.to(dtype), T=1.0)
+
+
 @pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
 def test_dense_vocab_32000_bf16_temperature_ragged_mask(D, kind):
     s, t = _pair(48, 32000, torch.bfloat16, 2, noise=1.5)

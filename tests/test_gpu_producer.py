@@ -59,6 +59,22 @@ def test_rows_whose_largest_logit_is_negative_or_zero(D, dtype):
     np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), rtol=0, atol=2e-6 * max(1.0, float(rv.abs().max())))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rows_with_one_towering_logit(D, dtype):
+    """A logit far above the rest of its row, at every position inside a 16-byte chunk in turn: a maximum
+    that missed it would let the sum of exponentials overflow."""
+    g = torch.Generator().manual_seed(6)
+    V, K = 40000, 32
+    logits = torch.randn(8, V, generator=g) * 2
+    for r in range(8):
+        logits[r, 8 * (100 + 37 * r) + r] = 150.0
+    logits = logits.to(dtype)
+    val, idx = D.teacher_topk(logits.to(DEV), K, val_dtype=torch.float32, idx_dtype=torch.int64)
+    rv, ri = _ref(logits, V, K)
+    assert torch.equal(idx.cpu(), ri) and torch.isfinite(val).all()
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), rtol=0, atol=3e-6 * float(rv.abs().max()))
+
+
 def test_storage_layout_crop_and_content_rows(D):
     g = torch.Generator().manual_seed(3)
     B, S, Vm, crop, K = 2, 40, 32064, 32000, 100
