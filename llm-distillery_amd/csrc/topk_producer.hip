@@ -336,11 +336,18 @@ void topk_part_kernel(const ProducerParams p) {
   const int select_wave = (int)((blockIdx.x >> 3) & (NW - 1));
 
   u32x4 reg[NCH];
+  const bool on_grid = (reinterpret_cast<uintptr_t>(rpart) & 15) == 0;      // the same for the whole workgroup
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = i * NT + tid;
-    if constexpr (ALIGNED) reg[i] = c < nch ? load16_stream(rpart + (int64_t)c * 16) : C::neg_inf();
-    else reg[i] = c < nch ? load_chunk_elementwise<Tag>(rpart, c, n_elems) : C::neg_inf();
+    if constexpr (ALIGNED) {
+      reg[i] = c < nch ? load16_stream(rpart + (int64_t)c * 16) : C::neg_inf();
+    } else {
+      // rows that start on the 16-byte grid but end off it (a crop of padded rows): only the last chunk
+      // has to be put together element by element
+      const bool whole = on_grid && (c + 1) * C::N <= n_elems;
+      reg[i] = c >= nch ? C::neg_inf() : whole ? load16_stream(rpart + (int64_t)c * 16) : load_chunk_elementwise<Tag>(rpart, c, n_elems);
+    }
   }
   if (tid == 0) s_n = 0;
 
