@@ -94,11 +94,12 @@ const char* dl_status_string(int status);
  * K <= DL_MAX_TOPK.
  * Alignment: any V and any element-aligned pointers and row strides are taken (else DL_ERR_ALIGN).  Rows
  * on the 16-byte grid (16-byte aligned pointers; row strides and V whole numbers of 16-byte chunks)
- * take the register kernels.  Other rows (an odd vocabulary, a column slice) take a streaming kernel
- * that still moves the 16-byte chunks inside each row with vector accesses, provided that logits and
- * gradient rows share their address modulo 16 (the same stride from 16-byte aligned bases, or the
- * gradient written over the logits; reverse KL: any gradient row), and element by element otherwise.
- * dl_rowstats_topk and dl_rowcoef_grad_topk follow the same rule.
+ * take the aligned register kernels.  Other rows (an odd vocabulary, a column slice) are still moved
+ * 16 bytes at a time: forward-KL rows of up to 4096 16-byte chunks by unaligned accesses in the register
+ * kernels; wider ones, and dl_rowstats_topk / dl_rowcoef_grad_topk, by the aligned chunks inside each
+ * row, provided that logits and gradient rows share their address modulo 16 (the same stride from
+ * 16-byte aligned bases, or the gradient written over the logits; reverse KL: any gradient row), and
+ * element by element otherwise.
  * grad may be the logits buffer itself (same pointer and stride): every kernel holds, or has
  * consumed, what it still needs of a row before it writes there.  The same holds for dl_div_dense
  * and dl_rkl_marginalised, not for dl_rowcoef_grad_topk.

@@ -138,6 +138,14 @@ __device__ __forceinline__ int64_t load_index(const void* base, int itype, int64
 __device__ __forceinline__ u32x4 load16_stream(const void* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
+// 16 bytes from any address: the compiler lowers the copy to one unaligned 16-byte load, which global
+// memory accesses of this target allow.
+__device__ __forceinline__ u32x4 load16_unaligned(const void* p) {
+  u32x4 v;
+  __builtin_memcpy(&v, p, 16);
+  return v;
+}
+__device__ __forceinline__ void store16_unaligned(void* p, const u32x4& v) { __builtin_memcpy(p, &v, 16); }
 // Non-temporal stores: a bare copy kernel runs ~4 % faster with the default policy, but in the
 // loss kernels (sparse corrections follow the dense row) the non-temporal hint measured faster.
 __device__ __forceinline__ void store16_stream(void* p, const u32x4& v) {
@@ -481,6 +489,45 @@ struct RowSplit {
   // column of leftover i, 0 <= i < leftovers()
   __device__ __forceinline__ int64_t column(int i) const { return i < head ? i : head + nbody * (16 / Tag::bytes) + (i - head); }
 };
+
+// One 16-byte chunk of a row that keeps no alignment promise and may end inside the chunk: assembled
+// from element-sized loads, columns at or beyond n_cols read as -inf.
+template <class Tag>
+__device__ __forceinline__ u32x4 load_chunk_elementwise(const char* part, int chunk, int n_cols) {
+  u32x4 v = Chunk<Tag>::neg_inf();
+  const int col0 = chunk * Chunk<Tag>::N;
+  if constexpr (Tag::bytes == 4) {
+    const unsigned* e = reinterpret_cast<const unsigned*>(part) + col0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) if (col0 + d < n_cols) v[d] = e[d];
+  } else {
+    const unsigned short* e = reinterpret_cast<const unsigned short*>(part) + col0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const unsigned lo = col0 + 2 * d < n_cols ? (unsigned)e[2 * d] : (v[d] & 0xffffu);
+      const unsigned hi = col0 + 2 * d + 1 < n_cols ? (unsigned)e[2 * d + 1] : (v[d] >> 16);
+      v[d] = lo | (hi << 16);
+    }
+  }
+  return v;
+}
+// The counterpart for stores: the elements of chunk `chunk` that lie before column n_cols.
+template <class Tag>
+__device__ __forceinline__ void store_chunk_elementwise(char* part, int chunk, int n_cols, const u32x4& v) {
+  const int col0 = chunk * Chunk<Tag>::N;
+  if constexpr (Tag::bytes == 4) {
+    unsigned* e = reinterpret_cast<unsigned*>(part) + col0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) if (col0 + d < n_cols) e[d] = v[d];
+  } else {
+    unsigned short* e = reinterpret_cast<unsigned short*>(part) + col0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      if (col0 + 2 * d < n_cols) e[2 * d] = (unsigned short)(v[d] & 0xffffu);
+      if (col0 + 2 * d + 1 < n_cols) e[2 * d + 1] = (unsigned short)(v[d] >> 16);
+    }
+  }
+}
 
 // zero-fill one gradient row (masked / padded token positions)
 template <class Tag, int NT>

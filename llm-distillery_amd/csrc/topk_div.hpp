@@ -456,6 +456,19 @@ __device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, f
   sm = block_sum<NT>(sm, red);
 }
 
+// Chunk ch of a row that may lie off the 16-byte grid and may end inside its last chunk (ANY rows of
+// the register kernels; `row` points at the row's first column, one part per row).
+template <class Tag>
+__device__ __forceinline__ void store_chunk_any(char* row, int64_t ch, int64_t V, const u32x4& v) {
+  if ((ch + 1) * Chunk<Tag>::N <= V) store16_unaligned(row + ch * 16, v);
+  else store_chunk_elementwise<Tag>(row, (int)ch, (int)V, v);
+}
+template <class Tag, int NT, bool ANY>
+__device__ __forceinline__ void zero_part(char* gpart, int64_t nch, int64_t V) {
+  if constexpr (!ANY) zero_row<Tag, NT>(gpart, nch);
+  else for (int64_t ch = threadIdx.x; ch < nch; ch += NT) store_chunk_any<Tag>(gpart, ch, V, u32x4{0u, 0u, 0u, 0u});
+}
+
 // ---------------------------------------------------------------------------------------
 // Forward KL, (part of) a row resident in registers: NT threads x NCH 16-byte chunks per thread.
 // SPLIT: P = p.parts workgroups per row.  Consecutive workgroup ids are dealt round-robin to the 8
@@ -468,20 +481,26 @@ __device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, f
 // RETRY: second launch over the parts that gave up waiting in the first (see split_retry_list):
 // every record of the row is published by then, so nothing is waited for.
 // MULTI: the row's teachers arrive prepared in buckets (TopkParams::bk), J * NT = cap0 entries in registers.
-template <class Tag, int NT, int NCH, bool SPLIT, int J, bool RETRY, bool MULTI>
+// ANY: rows may start anywhere (element-aligned) and V need not be a whole number of chunks: whole chunks
+// move by unaligned 16-byte accesses, the last, partly filled chunk of a row element by element with
+// -inf in the columns it lacks (they add nothing to any statistic and are not stored).
+template <class Tag, int NT, int NCH, bool SPLIT, int J, bool RETRY, bool MULTI, bool ANY = false>
 __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds& s, int64_t r, int h) {
   static_assert(!MULTI || J > 0, "the head of a bucket travels in registers");
+  static_assert(!ANY || (!SPLIT && !MULTI), "rows off the 16-byte grid: one workgroup per row, one stored teacher");
   using C = Chunk<Tag>;
   const int tid = threadIdx.x;
   const int P = SPLIT ? p.parts : 1;
   const int64_t c0 = (int64_t)h * NT * NCH;                       // first chunk of this part
-  const int64_t nch = min((int64_t)NT * NCH, p.V / C::N - c0);    // chunks of this part
-  const int lo = (int)(c0 * C::N), hi = lo + (int)(nch * C::N);   // its column range
+  const int64_t nch_row = ANY ? (p.V + C::N - 1) / C::N : p.V / C::N;
+  const int64_t nch = min((int64_t)NT * NCH, nch_row - c0);       // chunks of this part
+  const int lo = (int)(c0 * C::N);                                // its column range
+  const int hi = ANY ? (int)min(p.V, (int64_t)lo + nch * C::N) : lo + (int)(nch * C::N);
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
   char* gpart = grow ? grow + c0 * 16 : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   if (trow < 0) {
-    if (gpart) zero_row<Tag, NT>(gpart, nch);
+    if (gpart) zero_part<Tag, NT, ANY>(gpart, nch, p.V);
     if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
@@ -499,7 +518,9 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
     const int64_t c = ChunkMap<NT, NCH>::chunk(i, tid);
     // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
     // finds its lines in L2 instead of fetching them a second time (0.47 GB less per 32768 rows of K = 200)
-    reg[i] = c < nch ? *reinterpret_cast<const u32x4*>(rpart + c * 16) : C::neg_inf();
+    if constexpr (!ANY) reg[i] = c < nch ? *reinterpret_cast<const u32x4*>(rpart + c * 16) : C::neg_inf();
+    else reg[i] = c >= nch ? C::neg_inf() : (c + 1) * C::N <= p.V ? load16_unaligned(rpart + c * 16)
+                                                                  : load_chunk_elementwise<Tag>(rpart, (int)c, (int)p.V);
   }
 
   // teacher side while the row is in flight
@@ -517,7 +538,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
     tlse = stage_teacher<Tag, NT>(p, s, trow, row, lo, hi);
   }
   if (tlse == -INFINITY) {            // no usable teacher entry: the row contributes nothing
-    if (gpart) zero_row<Tag, NT>(gpart, nch);
+    if (gpart) zero_part<Tag, NT, ANY>(gpart, nch, p.V);
     if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
@@ -618,7 +639,8 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
         if (mine & (1u << i))
           if (correction_apply<Tag, NT, NCH>(s.head, s.next, s.idx, lo, i, f, mass, value)) repeats |= 1u << i;
-        store16_stream(gpart + ch * 16, C::pack(f));
+        if constexpr (!ANY) store16_stream(gpart + ch * 16, C::pack(f));
+        else store_chunk_any<Tag>(gpart, ch, p.V, C::pack(f));
       }
     }
     if (may_repeat && repeats)
@@ -638,7 +660,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   }
 }
 
-template <class Tag, int NT, int NCH, bool SPLIT, int J, bool MULTI = false>
+template <class Tag, int NT, int NCH, bool SPLIT, int J, bool MULTI = false, bool ANY = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void fkl_topk_reg_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -648,7 +670,7 @@ void fkl_topk_reg_kernel(const TopkParams p) {
   const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : xcd_banded_row(blockIdx.x);
   const int h = SPLIT ? (int)(t_in >> 3) : 0;
   if (r >= p.n_rows) return;
-  fkl_topk_part<Tag, NT, NCH, SPLIT, J, false, MULTI>(p, s, r, h);
+  fkl_topk_part<Tag, NT, NCH, SPLIT, J, false, MULTI, ANY>(p, s, r, h);
 }
 
 // One listed part, as a real call: the loop around it then costs the body no registers.
@@ -892,6 +914,17 @@ static void launch_reg_j(const TopkParams& p, unsigned grid, hipStream_t st) {
 #undef DL_REG_KERNEL
 }
 
+// one workgroup per row, rows of any alignment and length (one stored teacher)
+template <class Tag, int NT, int NCH>
+static int launch_reg_any(const TopkParams& p, hipStream_t st) {
+  constexpr bool MULTI = false;
+  const unsigned grid = xcd_banded_grid(p.n_rows);
+#define DL_REG_ANY_KERNEL(J) fkl_topk_reg_kernel<Tag, NT, NCH, false, J, false, true>
+  DL_LAUNCH_BY_SLOTS(DL_REG_ANY_KERNEL, grid)
+#undef DL_REG_ANY_KERNEL
+  return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}
+
 template <class Tag, int NT, int NCH, bool MULTI>
 static void launch_retry_j(const TopkParams& p, unsigned grid, hipStream_t st) {
 #define DL_RETRY_KERNEL(J) fkl_topk_retry_kernel<Tag, NT, NCH, J, MULTI>
@@ -991,10 +1024,34 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
     default: break;
   }
   if (MULTI) return aligned ? DL_ERR_LIMIT : DL_ERR_ALIGN;
-  // rows off the 16-byte grid: their chunks by vector accesses if logits and gradient rows share their
-  // address modulo 16 (the same pitch from 16-byte aligned bases, or the gradient written over the logits)
+  // rows off the 16-byte grid: the streaming kernel moves their chunks by aligned vector accesses if logits
+  // and gradient rows share their address modulo 16 (the same pitch from 16-byte aligned bases, or the
+  // gradient written over the logits)
   const bool same_phase = !p.grad || (reinterpret_cast<uintptr_t>(p.logits) % 16 == reinterpret_cast<uintptr_t>(p.grad) % 16 &&
                                       ((p.row_stride - p.grad_stride) * Tag::bytes) % 16 == 0);
+  if constexpr (!MULTI) {
+    if (!aligned) {
+      // ... or, as far as one workgroup holds a row, the register kernels with unaligned accesses.  Measured
+      // (16384 x 32100 bf16: 0.47 ms against 0.75 ms streaming; 16384 x 50257: 1.27 against 0.92): up to
+      // 256 x 16 chunks they win; the 512 x 16 shape spills under the extra addressing and only beats the
+      // element-wise kernel, which rows on different phases would otherwise take.
+      const FklShape any = fkl_shape((p.V + Tag::epc - 1) / Tag::epc, Tag::bytes, 0, false);
+      if (any.parts == 1) switch (any.NT * 100 + any.NCH) {
+        case 256 * 100 + 4: return launch_reg_any<Tag, 256, 4>(p, st);
+        case 256 * 100 + 8: return launch_reg_any<Tag, 256, 8>(p, st);
+        case 512 * 100 + 8:
+          if constexpr (Tag::bytes == 4) return launch_reg_any<Tag, 512, 8>(p, st);
+          break;
+        case 256 * 100 + 16:
+          if constexpr (Tag::bytes != 4) return launch_reg_any<Tag, 256, 16>(p, st);
+          break;
+        case 512 * 100 + 16:
+          if (!same_phase) return launch_reg_any<Tag, 512, 16>(p, st);
+          break;
+        default: break;
+      }
+    }
+  }
   if (aligned) {
     hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, 1>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
                        TopkLds::bytes(p.K), st, p);

@@ -272,28 +272,6 @@ __device__ __forceinline__ int64_t producer_row(const ProducerParams& p, int64_t
   return (r >= 0 && r < p.n_rows) ? r : -1;
 }
 
-// One 16-byte chunk of a row that keeps no alignment promise (odd vocabulary size, a cropped view
-// with an odd pitch): assembled from element-sized loads, columns at or beyond n_cols read as -inf.
-template <class Tag>
-__device__ __forceinline__ u32x4 load_chunk_elementwise(const char* part, int chunk, int n_cols) {
-  u32x4 v = Chunk<Tag>::neg_inf();
-  const int col0 = chunk * Chunk<Tag>::N;
-  if constexpr (Tag::bytes == 4) {
-    const unsigned* e = reinterpret_cast<const unsigned*>(part) + col0;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) if (col0 + d < n_cols) v[d] = e[d];
-  } else {
-    const unsigned short* e = reinterpret_cast<const unsigned short*>(part) + col0;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const unsigned lo = col0 + 2 * d < n_cols ? (unsigned)e[2 * d] : (v[d] & 0xffffu);
-      const unsigned hi = col0 + 2 * d + 1 < n_cols ? (unsigned)e[2 * d + 1] : (v[d] >> 16);
-      v[d] = lo | (hi << 16);
-    }
-  }
-  return v;
-}
-
 // G = chunk groups per thread whose maxima feed the threshold search: 256 * G groups per part must
 // be a few times K for the candidate set to stay close to K (4 for K <= 256, else 16).
 // ALIGNED: rows start on 16-byte boundaries and hold a whole number of chunks (16-byte loads);
@@ -343,10 +321,12 @@ void topk_part_kernel(const ProducerParams p) {
     if constexpr (ALIGNED) {
       reg[i] = c < nch ? load16_stream(rpart + (int64_t)c * 16) : C::neg_inf();
     } else {
-      // rows that start on the 16-byte grid but end off it (a crop of padded rows): only the last chunk
-      // has to be put together element by element
-      const bool whole = on_grid && (c + 1) * C::N <= n_elems;
-      reg[i] = c >= nch ? C::neg_inf() : whole ? load16_stream(rpart + (int64_t)c * 16) : load_chunk_elementwise<Tag>(rpart, c, n_elems);
+      // only a last chunk that the row does not fill is put together element by element; the others
+      // come by 16-byte loads, from rows off the 16-byte grid by unaligned ones (which the device takes)
+      const bool whole = (c + 1) * C::N <= n_elems;
+      reg[i] = c >= nch ? C::neg_inf()
+               : !whole ? load_chunk_elementwise<Tag>(rpart, c, n_elems)
+               : on_grid ? load16_stream(rpart + (int64_t)c * 16) : load16_unaligned(rpart + (int64_t)c * 16);
     }
   }
   if (tid == 0) s_n = 0;

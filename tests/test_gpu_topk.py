@@ -98,15 +98,19 @@ def test_streaming_path_odd_vocab_and_int64_fp32_teacher(D, V):
                                                   (torch.float32, 1003, 1003, 0),
                                                   (torch.bfloat16, 5001, 5120, 3),          # a column slice of aligned rows: one phase for all rows
                                                   (torch.float16, 7, 7, 0),                 # rows shorter than a chunk
-                                                  (torch.float32, 4099, 4104, 2)])
+                                                  (torch.float32, 4099, 4104, 2),
+                                                  (torch.bfloat16, 50257, 50257, 0),        # wider than 256 x 16 chunks: streaming, or 512 x 16 unaligned
+                                                  (torch.float32, 10001, 10001, 0)])        # 512 threads x 8 chunks of fp32
 @pytest.mark.parametrize("grad_mode", ["fresh", "in_place", "other_phase"])
 @pytest.mark.parametrize("kind", ["fkl", "rkl"])
 def test_rows_off_the_16_byte_grid(D, kind, dtype, V, pitch, offset, grad_mode):
-    """Rows that do not start on 16-byte boundaries or do not end on one: their 16-byte chunks go through
-    vector accesses when logits and gradient rows share their address modulo 16 (a fresh gradient of the
-    same pitch, or the gradient written over the logits), the few elements on either side one by one;
-    a gradient buffer on another phase takes the element-wise kernel (reverse KL, which only gathers from
-    the logits, goes by the gradient rows alone).  All three against the oracle."""
+    """Rows that do not start on 16-byte boundaries or do not end on one.  Forward KL: rows of up to
+    256 x 16 chunks stay in the register kernels (unaligned 16-byte accesses, the last, partly filled chunk
+    element by element); wider ones stream, their 16-byte chunks through aligned vector accesses when
+    logits and gradient rows share their address modulo 16 (a fresh gradient of the same pitch, or the
+    gradient written over the logits), else through the unaligned register kernel as far as that holds a
+    row.  Reverse KL, which only gathers from the logits, goes by the gradient rows alone.  All against
+    the oracle."""
     R, K = 7, min(24, V)
     logits, tv, ti = _case(R, V, K, dtype, 61, std=3.0)
     valid = torch.ones(R, dtype=torch.bool)
@@ -137,7 +141,9 @@ def test_rows_off_the_16_byte_grid(D, kind, dtype, V, pitch, offset, grad_mode):
     np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
     assert rl[2].item() == 0 and torch.count_nonzero(grad[2]) == 0
     err = (grad.cpu().double() - grad64).abs()
-    assert (err <= O.storage_tolerance(grad64, dtype, TOL[dtype])).all(), f"worst {(err / O.storage_tolerance(grad64, dtype, TOL[dtype])).max():.2f}"
+    # reverse KL: r_k ((log r_k - log q_k) - RKL), two terms of like size that cancel: twice the relative tolerance
+    bound = O.storage_tolerance(grad64, dtype, TOL[dtype] * (2 if kind == "rkl" else 1))
+    assert (err <= bound).all(), f"worst {(err / bound).max():.2f}"
     if pitch != V and grad_mode != "in_place":      # nothing outside the slice was touched
         assert torch.count_nonzero(full[:, :offset]) == 0 and torch.count_nonzero(full[:, offset + V:]) == 0
 
