@@ -12,21 +12,33 @@ struct DenseParams {
   float* row_loss; void* grad; int64_t grad_stride;
 };
 
-// Both rows in registers: NU units of 8 columns per thread.
-template <class TagS, class TagT, int NT, int NU>
+// Both rows in registers: NU units of 8 columns per thread.  ANY: rows of V columns that may start
+// anywhere and end inside a unit (unaligned 16-byte accesses; columns beyond the row read as -inf, which
+// adds nothing to any statistic, and are not stored).
+template <class TagS, class TagT, int NT, int NU, bool ANY = false>
 struct RegRows {
   static constexpr bool ONLINE = false;      // sweeps cost no memory traffic: maxima first, then sums
   Unit<TagS> s[NU];
   Unit<TagT> t[NU];
   int64_t nunits;
-  __device__ __forceinline__ void load(const char* srow, const char* trow, int64_t nu) {
+  int64_t V;
+  __device__ __forceinline__ void load(const char* srow, const char* trow, int64_t nu, int64_t n_cols = 0) {
     nunits = nu;
+    V = n_cols;
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int64_t u = (int64_t)i * NT + threadIdx.x;
-      if (u < nunits) { s[i].load(srow, u); t[i].load(trow, u); }
-      else { s[i].fill_neg_inf(); t[i].fill_neg_inf(); }
+      if (u < nunits) {
+        if constexpr (ANY) { s[i].load_any(srow, u, V); t[i].load_any(trow, u, V); }
+        else { s[i].load(srow, u); t[i].load(trow, u); }
+      } else {
+        s[i].fill_neg_inf(); t[i].fill_neg_inf();
+      }
     }
+  }
+  __device__ __forceinline__ void store(char* grow, int64_t u, const float* g) const {
+    if constexpr (ANY) Unit<TagS>::store_any(grow, u, V, g);
+    else Unit<TagS>::store(grow, u, g);
   }
   template <class F>
   __device__ __forceinline__ void sweep(F f) {
@@ -74,7 +86,7 @@ struct RegRows {
   }
 };
 
-template <int KIND, class TagS, class TagT, int NT, int NU>
+template <int KIND, class TagS, class TagT, int NT, int NU, bool ANY = false>
 __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
   __shared__ float red[64];
   const int64_t r = xcd_banded_row(blockIdx.x);
@@ -82,14 +94,22 @@ __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
   const int tid = threadIdx.x;
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  const int64_t nunits = ANY ? (p.V + 7) / 8 : p.V / 8;
   if (trow < 0) {
-    if (grow) zero_row<TagS, NT>(grow, p.V / TagS::epc);
+    if (grow) {
+      if constexpr (!ANY) {
+        zero_row<TagS, NT>(grow, p.V / TagS::epc);
+      } else {
+        const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int64_t u = tid; u < nunits; u += NT) Unit<TagS>::store_any(grow, u, p.V, z);
+      }
+    }
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
-  RegRows<TagS, TagT, NT, NU> rows;
+  RegRows<TagS, TagT, NT, NU, ANY> rows;
   rows.load(reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes,
-            reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * TagT::bytes, p.V / 8);
+            reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * TagT::bytes, nunits, p.V);
   const DenseStats st = dense_stats<KIND, NT>(rows, p.inv_T_s, p.inv_T_t, red);
   if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
   if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
@@ -104,6 +124,7 @@ struct StreamRows {
   const char* srow;
   const char* trow;
   int64_t nunits;
+  __device__ __forceinline__ void store(char* grow, int64_t u, const float* g) const { Unit<TagS>::store(grow, u, g); }
   template <class Tag>
   static __device__ __forceinline__ void fetch(Unit<Tag>& x, const char* row, int64_t u) {
 #pragma unroll
@@ -171,6 +192,7 @@ struct StudentRegRows {
   u32x4* lds;
   const char* trow;
   int64_t nunits;
+  __device__ __forceinline__ void store(char* grow, int64_t u, const float* g) const { Unit<TagS>::store(grow, u, g); }
   __device__ __forceinline__ void load(const char* srow, const char* trow_, int64_t nu, u32x4* lds_) {
     trow = trow_;
     nunits = nu;
@@ -331,6 +353,31 @@ static bool launch_dense_kind(const DenseParams& p, hipStream_t st) {
   return true;
 }
 
+// Rows off the 16-byte grid or not a whole number of units long, student and teacher of one dtype: the
+// register kernel with unaligned accesses, as far as a workgroup holds the pair of rows.
+template <int KIND, class Tag, int NU>
+static bool launch_dense_any_kind(const DenseParams& p, hipStream_t st) {
+  const int64_t units = (p.V + 7) / 8;
+  const dim3 grid(xcd_banded_grid(p.n_rows));
+  if (units <= 256 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, Tag, Tag, 256, NU, true>), grid, dim3(256), 0, st, p);
+  else if (units <= 512 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, Tag, Tag, 512, NU, true>), grid, dim3(512), 0, st, p);
+  else if (units <= 1024 * NU) hipLaunchKernelGGL((dense_reg_kernel<KIND, Tag, Tag, 1024, NU, true>), grid, dim3(1024), 0, st, p);
+  else return false;
+  return true;
+}
+template <class Tag, int NU>
+static bool launch_dense_any(const DenseParams& p, hipStream_t st) {
+  if (p.kind == DL_FKL) return launch_dense_any_kind<DL_FKL, Tag, NU>(p, st);
+  if (p.kind == DL_RKL) return launch_dense_any_kind<DL_RKL, Tag, NU>(p, st);
+  return launch_dense_any_kind<DL_JSD, Tag, NU>(p, st);
+}
+static bool launch_dense_any_pair(const DenseParams& p, hipStream_t st) {
+  if (p.s_dtype == F32 && p.t_dtype == F32) return launch_dense_any<TagF32, 4>(p, st);
+  if (p.s_dtype == BF16 && p.t_dtype == BF16) return launch_dense_any<TagBF16, 8>(p, st);
+  if (p.s_dtype == F16 && p.t_dtype == F16) return launch_dense_any<TagF16, 8>(p, st);
+  return false;
+}
+
 template <class TagS, class TagT, int NU>
 static bool launch_dense_reg(const DenseParams& p, hipStream_t st) {
   if (p.kind == DL_FKL) return launch_dense_kind<DL_FKL, TagS, TagT, NU>(p, st);
@@ -372,7 +419,10 @@ extern "C" int dl_div_dense(int kind, const void* logits, int logits_dtype, int6
   DenseParams p{kind, logits, logits_dtype, row_stride, n_rows, V, row_map, t_logits, t_dtype, t_stride,
                 n_teacher_rows, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (!(vec && launch_dense_pair(p, st)))
+  const bool elem = reinterpret_cast<uintptr_t>(logits) % sb == 0 && reinterpret_cast<uintptr_t>(t_logits) % tb == 0 &&
+                    (!grad || reinterpret_cast<uintptr_t>(grad) % sb == 0);
+  if (!elem) return DL_ERR_ALIGN;
+  if (!(vec ? launch_dense_pair(p, st) : launch_dense_any_pair(p, st)))
     hipLaunchKernelGGL((dense_stream_kernel<1024>), dim3((unsigned)n_rows), dim3(1024), 0, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }

@@ -19,9 +19,16 @@ namespace dl {
 template <class Tag> struct Unit {
   static constexpr int NC = Tag::bytes == 4 ? 2 : 1;
   u32x4 c[NC];
+  // A unit of a 4-byte row is two chunks side by side: a wave's load (or store) instruction then touches
+  // every other 16 bytes, half of each 64-byte line, and the instruction for the other chunk the other
+  // half.  With streaming accesses the halves travel separately (8192 x 32000 fp32 forward KL: 52 % of the
+  // HBM peak); through the cache they meet there (64 %).  Units of one chunk keep the streaming hints.
   __device__ __forceinline__ void load(const char* row, int64_t u) {
 #pragma unroll
-    for (int k = 0; k < NC; ++k) c[k] = load16_stream(row + (u * NC + k) * 16);
+    for (int k = 0; k < NC; ++k) {
+      if constexpr (NC == 1) c[k] = load16_stream(row + (u * NC + k) * 16);
+      else c[k] = *reinterpret_cast<const u32x4*>(row + (u * NC + k) * 16);
+    }
   }
   __device__ __forceinline__ void fill_neg_inf() {
 #pragma unroll
@@ -33,7 +40,33 @@ template <class Tag> struct Unit {
   }
   __device__ static __forceinline__ void store(char* row, int64_t u, const float* f) {
 #pragma unroll
-    for (int k = 0; k < NC; ++k) store16_stream(row + (u * NC + k) * 16, Chunk<Tag>::pack(f + k * Chunk<Tag>::N));
+    for (int k = 0; k < NC; ++k) {
+      if constexpr (NC == 1) store16_stream(row + (u * NC + k) * 16, Chunk<Tag>::pack(f + k * Chunk<Tag>::N));
+      else *reinterpret_cast<u32x4*>(row + (u * NC + k) * 16) = Chunk<Tag>::pack(f + k * Chunk<Tag>::N);
+    }
+  }
+  // The same for rows of V columns that may start anywhere (element-aligned) and end inside a chunk:
+  // whole chunks by unaligned 16-byte accesses, a partly filled one element by element (-inf / not
+  // stored beyond the row), nothing for chunks wholly beyond it.
+  __device__ __forceinline__ void load_any(const char* row, int64_t u, int64_t V) {
+    constexpr int N = Chunk<Tag>::N;
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+      const int64_t ch = u * NC + k;
+      c[k] = (ch + 1) * N <= V ? load16_unaligned(row + ch * 16)
+             : ch * N < V      ? load_chunk_elementwise<Tag>(row, (int)ch, (int)V)
+                               : Chunk<Tag>::neg_inf();
+    }
+  }
+  __device__ static __forceinline__ void store_any(char* row, int64_t u, int64_t V, const float* f) {
+    constexpr int N = Chunk<Tag>::N;
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+      const int64_t ch = u * NC + k;
+      const u32x4 v = Chunk<Tag>::pack(f + k * N);
+      if ((ch + 1) * N <= V) store16_unaligned(row + ch * 16, v);
+      else if (ch * N < V) store_chunk_elementwise<Tag>(row, (int)ch, (int)V, v);
+    }
   }
 };
 
@@ -199,7 +232,7 @@ __device__ __forceinline__ void dense_grad_sweep(Rows& rows, const DenseStats& s
     float g[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) g[e] = dense_grad(KIND, fmaf(s[e], a_s, -ls), fmaf(t[e], a_t, -lt), aux) * c;
-    Unit<TagS>::store(grow, u, g);
+    rows.store(grow, u, g);
   });
 }
 

@@ -92,6 +92,45 @@ def test_dense_16bit_rows_with_one_towering_logit(D, kind, dtype):
 
 
 @pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+@pytest.mark.parametrize("dtype,V,pitch,offset", [(torch.bfloat16, 5001, 5001, 0),      # contiguous odd rows: every row starts elsewhere on the 16-byte grid
+                                                  (torch.float32, 1003, 1003, 0),
+                                                  (torch.float16, 7, 7, 0),               # rows shorter than a chunk
+                                                  (torch.bfloat16, 4099, 4104, 3),        # a column slice of aligned rows
+                                                  (torch.float32, 20001, 20001, 0)])      # 1024 threads
+@pytest.mark.parametrize("in_place", [False, True])
+def test_dense_rows_off_the_16_byte_grid(D, kind, dtype, V, pitch, offset, in_place):
+    """Student and teacher rows of one dtype that do not start on 16-byte boundaries or do not end on one
+    stay in the register kernel (unaligned 16-byte accesses, the last, partly filled chunk element by
+    element), with masked rows and the gradient written over the logits."""
+    R = 6
+    s, t = _pair(R, V, dtype, 13)
+    valid = torch.ones(R, dtype=torch.bool)
+    valid[1] = False
+    if kind == "rkl":
+        t[:, ::5] = -float("inf")                     # a teacher without mass on a fifth of the columns, the last one among them or not
+    loss64, rows64, grad64 = O.mean_loss_and_grad(kind, s, 1.3, t_logits=t[valid], valid=valid, dtype=torch.float64)
+    rm = torch.full((R,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(R - 1, dtype=torch.int32)
+
+    def on_gpu(x):
+        if pitch == V:
+            return x.to(DEV)
+        wide = torch.zeros(x.shape[0], pitch + 8, dtype=dtype, device=DEV)
+        wide[:, offset:offset + V] = x.to(DEV)
+        return wide[:, offset:offset + V]
+
+    xs, xt = on_gpu(s), on_gpu(t[valid])
+    rl, grad = D.div_dense(kind, xs, xt, row_map=rm.to(DEV), T=1.3, grad_scale=1.0 / (R - 1), grad_out=xs if in_place else None)
+    np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    assert rl[1].item() == 0 and torch.count_nonzero(grad[1]) == 0
+    err = (grad.cpu().double() - grad64).abs()
+    sel = torch.nonzero(valid).squeeze(-1)
+    bound = O.storage_tolerance(grad64, dtype, RTOL[dtype])
+    bound[sel] = O.dense_gradient_tolerance(grad64[sel], s[sel], t[valid], rows64, 1.3, 1.3, 1.0 / (R - 1), dtype, RTOL[dtype])
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
 def test_dense_vocab_32000_bf16_temperature_ragged_mask(D, kind):
     s, t = _pair(48, 32000, torch.bfloat16, 2, noise=1.5)
     valid = torch.ones(48, dtype=torch.bool)
