@@ -153,6 +153,12 @@ int dl_div_topk_static(int kind,
  * 0.5 KL(P||M) + 0.5 KL(Q||M), natural log.
  * t_logits [n_teacher_rows, V] (stride t_stride): teacher logits or log-probs (any per-row constant
  * is irrelevant), scaled by inv_T_teacher.  Other arguments as for dl_div_topk.
+ * Rows on the 16-byte grid (student, teacher and gradient; V a multiple of 8) are read once as far as
+ * a workgroup's registers hold the pair (65536 columns of 16-bit rows, 32768 with an fp32 row) and
+ * streamed in 16-byte chunks beyond that; rows off the grid take the same register kernels through
+ * unaligned 16-byte accesses when student and teacher share a dtype and the pair fits, and a
+ * kernel that streams them element by element otherwise.
+ * Pointers and strides must be whole elements (else DL_ERR_ALIGN).
  */
 int dl_div_dense(int kind,
                  const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
