@@ -53,6 +53,25 @@ struct RegRows {
       }
     }
   }
+  // The same, and what f leaves in its arguments goes back into the registers (fp32 rows: bit moves).
+  // The branch is per wave, not per lane (lanes beyond the row hold -inf, which f must take): a value
+  // rewritten under a per-lane branch would get a second register beside the one that the idle lanes keep.
+  static constexpr bool EXACT_STASH = TagS::bytes == 4 && TagT::bytes == 4;
+  template <class F>
+  __device__ __forceinline__ void sweep_rewrite(F f) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * NT + threadIdx.x;
+      if (__builtin_amdgcn_readfirstlane((int)((u & ~(int64_t)63) < nunits))) {
+        float a[8], b[8];
+        s[i].unpack(a);
+        t[i].unpack(b);
+        f(u, a, b);
+        s[i].repack(a);
+        t[i].repack(b);
+      }
+    }
+  }
   // Maxima of both rows from the raw bit patterns, for two 16-bit rows: non-negative 16-bit floats
   // order like their patterns read as signed integers and every negative one reads as a negative
   // integer, so the packed integer maximum is the row's maximum whenever that is not negative (half
@@ -110,9 +129,17 @@ __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
   RegRows<TagS, TagT, NT, NU, ANY> rows;
   rows.load(reinterpret_cast<const char*>(p.logits) + r * p.row_stride * TagS::bytes,
             reinterpret_cast<const char*>(p.t_logits) + trow * p.t_stride * TagT::bytes, nunits, p.V);
-  const DenseStats st = dense_stats<KIND, NT>(rows, p.inv_T_s, p.inv_T_t, red);
-  if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
-  if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
+  if constexpr (KIND == DL_JSD && RegRows<TagS, TagT, NT, NU, ANY>::EXACT_STASH) {
+    // The divergence sweep leaves the gradient's ingredients in the rows' registers (at no cost for fp32
+    // rows, so also when no gradient is asked for: a second copy of the sweeps for that case costs registers).
+    const DenseStats st = dense_stats<KIND, NT, true>(rows, p.inv_T_s, p.inv_T_t, red);
+    if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
+    if (grow) dense_jsd_grad_from_stash<TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
+  } else {
+    const DenseStats st = dense_stats<KIND, NT>(rows, p.inv_T_s, p.inv_T_t, red);
+    if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
+    if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
+  }
 }
 
 // Rows too wide for the registers, 16-byte aligned: the same sweeps, every one of them over global

@@ -38,6 +38,10 @@ template <class Tag> struct Unit {
 #pragma unroll
     for (int k = 0; k < NC; ++k) { forget(c[k]); Chunk<Tag>::unpack(c[k], f + k * Chunk<Tag>::N); }
   }
+  __device__ __forceinline__ void repack(const float* f) {
+#pragma unroll
+    for (int k = 0; k < NC; ++k) c[k] = Chunk<Tag>::pack(f + k * Chunk<Tag>::N);
+  }
   __device__ static __forceinline__ void store(char* row, int64_t u, const float* f) {
 #pragma unroll
     for (int k = 0; k < NC; ++k) {
@@ -89,14 +93,19 @@ __device__ __forceinline__ void rkl_term(float lp, float lq, float& acc) {
   acc += (lq > -INFINITY && r > 0.f) ? r * (lp - lq) : 0.f;
 }
 // Three transcendentals per column: the mixture's logarithm is taken of the probabilities themselves.
-// Columns where a probability underflows contribute nothing for it: the logarithms are held at a
-// finite floor, so their differences are finite and 0 * difference is 0 without a select.
+// Columns where a probability underflows contribute nothing for it: log2 p - log2 m is at most 1
+// (m >= p / 2) and is held inside [LOG_FLOOR, 1], so that 0 * difference is 0 without a select.  One
+// median instruction does it for every case: -inf (p = 0 < m) -> the floor, +inf (m underflows, log2 p
+// finite) -> 1, and the NaN of -inf - -inf -> the floor (the median of a NaN is the smaller bound).
 constexpr float LOG_FLOOR = -1e30f;
+__device__ __forceinline__ float log_ratio_to_mixture(float lp, float lm) {
+  return __builtin_amdgcn_fmed3f(lp - lm, LOG_FLOOR, 1.f);
+}
 __device__ __forceinline__ void jsd_term(float lp, float lq, float& kl_pm, float& kl_qm) {
   const float pr = fast_exp2(lp), q = fast_exp2(lq);
-  const float lm = fmaxf(fast_log2(0.5f * pr + 0.5f * q), LOG_FLOOR);
-  kl_pm = fmaf(pr, fmaxf(lp, LOG_FLOOR) - lm, kl_pm);
-  kl_qm = fmaf(q, fmaxf(lq, LOG_FLOOR) - lm, kl_qm);
+  const float lm = fast_log2(0.5f * pr + 0.5f * q);
+  kl_pm = fmaf(pr, log_ratio_to_mixture(lp, lm), kl_pm);
+  kl_qm = fmaf(q, log_ratio_to_mixture(lq, lm), kl_qm);
 }
 
 // Gradient of one column (before the common factor c = inv_T * scale).
@@ -106,6 +115,18 @@ __device__ __forceinline__ float dense_grad(int kind, float lp, float lq, float 
   const float pr = fast_exp2(lp);
   if (!(pr > 0.f)) return 0.f;
   return 0.5f * pr * ((lp - fast_log2(0.5f * pr + 0.5f * fast_exp2(lq))) * LN2 - aux);
+}
+
+// The same with the kind a compile-time constant and the row's constants folded:
+//   FKL  c (p - q)                                             kb, k0 unused
+//   RKL  r (kb (lp - lq) + k0)            kb = c ln 2,         k0 = -c RKL
+//   JSD  p (kb (lp - lm) + k0)            kb = c ln 2 / 2,     k0 = -c KL(P || M) / 2
+template <int KIND>
+__device__ __forceinline__ float dense_grad_column(float lp, float lq, float c, float kb, float k0) {
+  if (KIND == DL_FKL) return (fast_exp2(lp) - fast_exp2(lq)) * c;
+  if (KIND == DL_RKL) return lq > -INFINITY ? fast_exp2(lp) * fmaf(lp - lq, kb, k0) : 0.f;
+  const float pr = fast_exp2(lp);
+  return pr * fmaf(log_ratio_to_mixture(lp, fast_log2(0.5f * pr + 0.5f * fast_exp2(lq))), kb, k0);
 }
 
 // The sweeps over a row pair held in registers.  `Rows` provides
@@ -119,7 +140,15 @@ __device__ __forceinline__ float dense_grad(int kind, float lp, float lq, float 
 //   RKL = sum r (lp - lq) = (1/S) sum es ((s a_s - bs) - (t a_t - bt)) - log2 S + log2 T      (r = es / S, support only)
 // so the divergence sum rides along with the sums of exponentials.  JSD needs the normalised
 // probabilities inside a logarithm and keeps its own sweep.
-template <int KIND, int NT, class Rows>
+//
+// STASH (JSD on rows of fp32 pairs held in registers): the divergence sweep leaves p and
+// log2 p - log2 m in the registers of the logits, exactly, and the gradient
+//   g = c p / 2 ((log2 p - log2 m) ln 2 - KL(P || M))
+// takes two instructions per column (dense_jsd_grad_from_stash) instead of recomputing three
+// transcendentals (8192 x 32000: 0.70 -> 0.67 ms).  The same for forward and reverse KL (their
+// exponentials kept) shortened the arithmetic by a third and the kernel not at all: with fp32 rows
+// those two are not bound by the vector ALU.
+template <int KIND, int NT, bool STASH = false, class Rows>
 __device__ __forceinline__ DenseStats dense_stats(Rows& rows, float inv_T_s, float inv_T_t, float* red) {
   DenseStats st;
   st.a_s = inv_T_s * LOG2E;
@@ -215,10 +244,26 @@ __device__ __forceinline__ DenseStats dense_stats(Rows& rows, float inv_T_s, flo
     return st;
   }
   float x = 0.f, y = 0.f;
-  rows.sweep([&](int64_t, const float* s, const float* t) {
+  if constexpr (STASH) {
+    rows.sweep_rewrite([&](int64_t, float* s, float* t) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) jsd_term(fmaf(s[e], a_s, -st.ls), fmaf(t[e], a_t, -st.lt), x, y);
-  });
+      for (int e = 0; e < 8; ++e) {
+        const float lp = fmaf(s[e], a_s, -st.ls), lq = fmaf(t[e], a_t, -st.lt);
+        const float pr = fast_exp2(lp), q = fast_exp2(lq);
+        const float lm = fast_log2(0.5f * pr + 0.5f * q);
+        const float d = log_ratio_to_mixture(lp, lm);       // finite: pr = 0 then gives a gradient of 0
+        x = fmaf(pr, d, x);
+        y = fmaf(q, log_ratio_to_mixture(lq, lm), y);
+        s[e] = pr;
+        t[e] = d;
+      }
+    });
+  } else {
+    rows.sweep([&](int64_t, const float* s, const float* t) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) jsd_term(fmaf(s[e], a_s, -st.ls), fmaf(t[e], a_t, -st.lt), x, y);
+    });
+  }
   block_sum2<NT>(x, y, red);
   st.loss = 0.5f * LN2 * (x + y);
   st.aux = x * LN2;
@@ -227,11 +272,24 @@ __device__ __forceinline__ DenseStats dense_stats(Rows& rows, float inv_T_s, flo
 
 template <int KIND, class TagS, class Rows>
 __device__ __forceinline__ void dense_grad_sweep(Rows& rows, const DenseStats& st, float c, char* grow) {
-  const float a_s = st.a_s, a_t = st.a_t, ls = st.ls, lt = st.lt, aux = st.aux;
+  const float a_s = st.a_s, a_t = st.a_t, ls = st.ls, lt = st.lt;
+  const float kb = (KIND == DL_JSD ? 0.5f : 1.f) * c * LN2, k0 = (KIND == DL_JSD ? -0.5f : -1.f) * c * st.aux;
   rows.sweep([&](int64_t u, const float* s, const float* t) {
     float g[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) g[e] = dense_grad(KIND, fmaf(s[e], a_s, -ls), fmaf(t[e], a_t, -lt), aux) * c;
+    for (int e = 0; e < 8; ++e) g[e] = dense_grad_column<KIND>(fmaf(s[e], a_s, -ls), fmaf(t[e], a_t, -lt), c, kb, k0);
+    rows.store(grow, u, g);
+  });
+}
+
+// The JSD gradient from what dense_stats<DL_JSD, NT, true> left in the registers.
+template <class TagS, class Rows>
+__device__ __forceinline__ void dense_jsd_grad_from_stash(Rows& rows, const DenseStats& st, float c, char* grow) {
+  const float kb = 0.5f * c * LN2, k0 = -0.5f * c * st.aux;
+  rows.sweep([&](int64_t u, const float* pr, const float* d) {
+    float g[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] = pr[e] * fmaf(d[e], kb, k0);
     rows.store(grow, u, g);
   });
 }
