@@ -206,6 +206,39 @@ def test_jsd_bounded_by_ln2_on_disjoint_supports(D):
     np.testing.assert_allclose(rl.cpu().numpy(), np.log(2.0), rtol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_jsd_with_student_logits_of_minus_infinity(D, dtype):
+    """Masked vocabulary entries (-inf) in the student row, some of them where the teacher has no mass
+    either: the loss stays finite and equals the oracle's, the gradient is exactly 0 on the masked columns
+    and matches central differences of the oracle's float64 loss elsewhere (autograd through the oracle
+    yields NaN for such rows: 0 * inf in the branch that `where` drops)."""
+    R, V = 3, 2048
+    s, t = _pair(R, V, dtype, 21)
+    s, t = s.float(), t.float()
+    s[:, 40:90] = -float("inf")
+    t[:, 70:130] = -float("inf")
+    s[1, ::7] = -float("inf")
+    s, t = s.to(dtype), t.to(dtype)
+    rl, grad = D.div_dense("jsd", s.to(DEV), t.to(DEV), T=1.5, teacher_T=1.0)
+    rows64 = O.jsd_dense_rows(s.double() / 1.5, t.double())
+    np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=2e-5)
+    g = grad.cpu().double()
+    assert torch.isfinite(g).all() and torch.count_nonzero(g[torch.isinf(s.float())]) == 0
+    gen = torch.Generator().manual_seed(5)
+    eps = 1e-5
+    for _ in range(24):
+        r = int(torch.randint(0, R, (1,), generator=gen))
+        j = int(torch.randint(0, V, (1,), generator=gen))
+        if torch.isinf(s[r, j].float()):
+            continue
+        hi, lo = s[r].double().clone(), s[r].double().clone()
+        hi[j] += eps
+        lo[j] -= eps
+        fd = (O.jsd_dense_rows(hi[None] / 1.5, t[r:r + 1].double()) - O.jsd_dense_rows(lo[None] / 1.5, t[r:r + 1].double())).item() / (2 * eps)
+        tol = (1e-4 if dtype == torch.float32 else 2e-3 + 2.0 ** -8) * abs(fd) + 2e-9
+        assert abs(g[r, j].item() - fd) <= tol, (r, j, g[r, j].item(), fd)
+
+
 def test_synthetic_configs_1_and_2_at_reduced_rows(D):
     from llm_distillery_amd import synthetic as S
     c = S.config1(DEV, B=1, S=64)
