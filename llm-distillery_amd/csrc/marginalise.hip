@@ -366,7 +366,9 @@ struct StudentRow {
 // registers only.  Pass B: xt (written over the marginal; a log-domain value, exact whatever the
 // bias), the three sums.  If T or S then lies outside [2^-64, 2^64] -- the row carries no or hardly any
 // mass, an unnormalised teacher, or a student whose mass sits far off the support -- the maxima are
-// taken after all, from the stored xt, and the sums are redone on them.  Pass C: gradient.
+// taken after all, from the stored xt, and the sums are redone on them.  Pass C: gradient.  When a
+// gradient follows, pass B leaves 2^xs in the registers of the logits and xs - xt in the marginal's
+// slots (rkl_sums_stash), and pass C is a multiply-add and a multiply per column.
 // What stands for log2(0) in the stored xt and for a student logit of -inf: finite, so that differences
 // of two such values are finite (0 * finite = 0 needs no select), and far below anything a sum notices.
 constexpr float XT_OFF = -1e30f;
@@ -374,8 +376,7 @@ constexpr float XT_OFF = -1e30f;
 // entries above 2^103 would overflow (probabilities are at most 1).
 constexpr float MARG_LOG_SCALE = 0x1p24f, MARG_LOG_SHIFT = 24.f;
 
-// WITH_T: T is summed here; else the caller sums it in the gradient pass (see rkl_against_marginal).
-template <class TagS, int NU, bool UNIT_T, bool WITH_T>
+template <class TagS, int NU, bool UNIT_T>
 __device__ __forceinline__ void rkl_sums_optimistic(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float a_s, float bs,
                                                     float inv_T_t, float& ss, float& stt, float& w) {
   const int tid = threadIdx.x;
@@ -394,7 +395,7 @@ __device__ __forceinline__ void rkl_sums_optimistic(Unit<TagS> (&s)[NU], int64_t
         const float xt = fmaxf(UNIT_T ? l2 - MARG_LOG_SHIFT : fmaf(l2, inv_T_t, -MARG_LOG_SHIFT * inv_T_t), XT_OFF);
         const float xs = fmaxf(fmaf(sv[e], a_s, -bs), XT_OFF);
         const float eon = m[e] > 0.f ? fast_exp2(xs) : 0.f;
-        if (WITH_T) stt += UNIT_T ? m[e] : fast_exp2(xt);      // 2^xt; 0 off the support
+        stt += UNIT_T ? m[e] : fast_exp2(xt);      // 2^xt; 0 off the support
         ss += eon;
         w = fmaf(eon, xs - xt, w);                 // the difference is finite: no 0 * inf
         m[e] = xt;
@@ -405,10 +406,80 @@ __device__ __forceinline__ void rkl_sums_optimistic(Unit<TagS> (&s)[NU], int64_t
   }
 }
 
-// Pass C.  WITH_T: T = sum 2^xt is taken along (into stt, this thread's share).
-template <class TagS, int NU, bool WITH_T>
+// The same pass when a gradient follows: it leaves what the gradient is made of, so that the
+// gradient pass needs no transcendental and a third of the instructions.  With B = the stash bias of
+// the row's type (Chunk<TagS>::stash_bias: 2^xs in fp16 keeps 11 bits down to 2^-29 of the row's
+// largest entry; fp32 rows keep all of it) and both biases lifted by B,
+//   registers of the logits <- 2^(xs + B)   (0 off the support)
+//   marginal's slot         <- xs - xt      (of a column whose 2^xs underflows anyway, xs <= -256: 0 - xt,
+//                                            so that xt can be had back exactly enough from any slot)
+// ss, stt (unless UNIT_T) and w come out multiplied by 2^B.
+constexpr float XS_DEAD = -256.f;
+template <class TagS, int NU, bool UNIT_T>
+__device__ __forceinline__ void rkl_sums_stash(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float a_s, float bs2,
+                                               float inv_T_t, float& ss, float& stt, float& w) {
+  constexpr float B = Chunk<TagS>::stash_bias;
+  const int tid = threadIdx.x;
+  const float ct = UNIT_T ? B - MARG_LOG_SHIFT : B - MARG_LOG_SHIFT * inv_T_t;
+#pragma unroll
+  for (int i = 0; i < NU; ++i) {
+    const int64_t u = (int64_t)i * MARG_NT + tid;
+    if (u < nunits) {
+      float sv[8], m[8];
+      s[i].unpack(sv);
+      const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
+      m[0] = m0.x; m[1] = m0.y; m[2] = m0.z; m[3] = m0.w; m[4] = m1.x; m[5] = m1.y; m[6] = m1.z; m[7] = m1.w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float l2 = fast_log2(m[e] * MARG_LOG_SCALE);
+        const float xt = fmaxf(UNIT_T ? l2 + ct : fmaf(l2, inv_T_t, ct), XT_OFF);
+        const float xs = fmaf(sv[e], a_s, -bs2);                   // -inf for a logit of -inf
+        // 2^xs on the support, 0 off it, without a select: xt is XT_OFF exactly off the support, where
+        // xt * 2^-90 = -800 sinks the exponent, and so small on it that the sum rounds back to xs
+        const float eon = fast_exp2(fmaf(xt, 0x1p-90f, xs));
+        const float d = (xs > XS_DEAD ? xs : 0.f) - xt;            // finite
+        stt += UNIT_T ? m[e] : fast_exp2(xt);
+        ss += eon;
+        w = fmaf(eon, d, w);
+        m[e] = d;
+        sv[e] = eon;
+      }
+      *reinterpret_cast<float4*>(marg + u * 8) = float4{m[0], m[1], m[2], m[3]};        // own columns only: no barrier needed
+      *reinterpret_cast<float4*>(marg + u * 8 + 4) = float4{m[4], m[5], m[6], m[7]};
+#pragma unroll
+      for (int k = 0; k < Unit<TagS>::NC; ++k) s[i].c[k] = Chunk<TagS>::stash(sv + k * Chunk<TagS>::N);
+    }
+  }
+}
+
+// The gradient from what rkl_sums_stash left: 2^(xs + B) * (k1 (xs - xt) - k1 wbar), k1 over the sum
+// that carries the same 2^B.  The factor is held finite (a column off the support stores 1e30 for its
+// difference), so that 0 * factor is 0.
+template <class TagS, int NU>
+__device__ __forceinline__ void rkl_gradient_from_stash(Unit<TagS> (&s)[NU], int64_t nunits, const float* marg, float k1,
+                                                        float wbar, char* grow) {
+  const int tid = threadIdx.x;
+  const float k0 = -k1 * wbar;
+#pragma unroll
+  for (int i = 0; i < NU; ++i) {
+    const int64_t u = (int64_t)i * MARG_NT + tid;
+    if (u < nunits) {
+      float es[8], d[8], g[8];
+#pragma unroll
+      for (int k = 0; k < Unit<TagS>::NC; ++k) Chunk<TagS>::unstash(s[i].c[k], es + k * Chunk<TagS>::N);
+      const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
+      d[0] = m0.x; d[1] = m0.y; d[2] = m0.z; d[3] = m0.w; d[4] = m1.x; d[5] = m1.y; d[6] = m1.z; d[7] = m1.w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] = es[e] * __builtin_amdgcn_fmed3f(fmaf(d[e], k1, k0), -3e38f, 3e38f);
+      Unit<TagS>::store(grow, u, g);
+    }
+  }
+}
+
+// Pass C on the stored xt (rows whose sums were redone on their maxima).
+template <class TagS, int NU>
 __device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t nunits, const float* marg, float a_s, float bs,
-                                                  float k1, float wbar, char* grow, float& stt) {
+                                                  float k1, float wbar, char* grow) {
   const int tid = threadIdx.x;
 #pragma unroll
   for (int i = 0; i < NU; ++i) {
@@ -422,19 +493,19 @@ __device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t n
       for (int e = 0; e < 8; ++e) {
         const float xs = fmaf(sv[e], a_s, -bs);
         g[e] = xt[e] > 0.5f * XT_OFF ? fast_exp2(xs) * k1 * ((xs - xt[e]) - wbar) : 0.f;
-        if (WITH_T) stt += fast_exp2(xt[e]);
       }
       Unit<TagS>::store(grow, u, g);
     }
   }
 }
 
-// The sums' pass is bound by its three transcendentals per column (2^xs, log2 m, 2^xt), the gradient
-// pass, with one, by its other instructions: when a gradient is asked for and T_t != 1, 2^xt moves to
-// the gradient pass -- T enters the loss only, not the gradient -- and the row's loss is written last.
+// With a gradient asked for, the sums' pass leaves its ingredients behind (rkl_sums_stash).  If the sums
+// then turn out to be out of range, the row is put back -- logits read again (nothing of the row has
+// been written yet, also when the gradient goes over the logits), xt from the stored differences --
+// and takes the passes on its maxima like a row without a gradient.
 template <class TagS, int NU>
 __device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float* red,
-                                                     const MargParams& p, int64_t r, char* grow) {
+                                                     const MargParams& p, int64_t r, char* grow, const char* srow) {
   const int tid = threadIdx.x;
   const float a_s = p.inv_T_s * LOG2E;
   const auto stored_of = [&](int64_t u, float (&m)[8]) {
@@ -442,28 +513,89 @@ __device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_
     m[0] = m0.x; m[1] = m0.y; m[2] = m0.z; m[3] = m0.w; m[4] = m1.x; m[5] = m1.y; m[6] = m1.z; m[7] = m1.w;
   };
   const auto in_range = [](float v) { return v > 0x1p-64f && v < 0x1p64f; };
+  const bool unit_T = p.inv_T_t == 1.f;
+  // The row's largest logit (units beyond the row hold -inf).  16-bit rows: non-negative values order like
+  // their bit patterns read as signed integers and every negative one reads as a negative integer, so the
+  // packed integer maximum of the raw pairs is the maximum whenever that is not negative -- half an
+  // instruction per column instead of two.
   float ms = -INFINITY;
+  bool have_ms = false;
+  if constexpr (TagS::bytes == 2) {
+    typedef short i16x2 __attribute__((ext_vector_type(2)));
+    i16x2 pm = {(short)-32768, (short)-32768};
 #pragma unroll
-  for (int i = 0; i < NU; ++i) {      // units beyond the row hold -inf
-    float sv[8];
-    s[i].unpack(sv);
+    for (int i = 0; i < NU; ++i) {
+      forget(s[i].c[0]);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) ms = fmaxf(ms, sv[e]);
+      for (int d = 0; d < 4; ++d) {
+        const unsigned w16 = s[i].c[0][d];      // by value: a bit cast straight from a vector element reads element 0
+        pm = __builtin_elementwise_max(pm, __builtin_bit_cast(i16x2, w16));
+      }
+    }
+    const float top = block_max<MARG_NT>((float)max((int)pm.x, (int)pm.y), red);      // exact, order-preserving
+    if (top >= 0.f) {                                                                 // the same for every thread
+      const unsigned bits = (unsigned)(int)top;
+      ms = TagS::id == BF16 ? __uint_as_float(bits << 16) : (float)__builtin_bit_cast(_Float16, (unsigned short)bits);
+      have_ms = true;
+    }
   }
-  ms = block_max<MARG_NT>(ms, red);
+  if (!have_ms) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      float sv[8];
+      s[i].unpack(sv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ms = fmaxf(ms, sv[e]);
+    }
+    ms = block_max<MARG_NT>(ms, red);
+  }
   float bs = ms > -INFINITY ? ms * a_s : 0.f;
   float ss = 0.f, stt = 0.f, w = 0.f;
-  bool t_known = true;
-  if (p.inv_T_t == 1.f) {
-    rkl_sums_optimistic<TagS, NU, true, true>(s, nunits, marg, a_s, bs, 1.f, ss, stt, w);
-  } else if (!grow) {
-    rkl_sums_optimistic<TagS, NU, false, true>(s, nunits, marg, a_s, bs, p.inv_T_t, ss, stt, w);
+  bool redo;
+  // fp32 rows always: for them the stash is free, and a second form of the pass beside it costs registers
+  if (TagS::bytes == 4 || grow) {
+    constexpr float B = Chunk<TagS>::stash_bias;
+    const float bs2 = bs - B;
+    if (unit_T) rkl_sums_stash<TagS, NU, true>(s, nunits, marg, a_s, bs2, 1.f, ss, stt, w);
+    else rkl_sums_stash<TagS, NU, false>(s, nunits, marg, a_s, bs2, p.inv_T_t, ss, stt, w);
+    block_sum3<MARG_NT>(ss, stt, w, red);
+    const float unscale = __uint_as_float((unsigned)(127 - (int)B) << 23);      // 2^-B
+    const float ss1 = ss * unscale, stt1 = unit_T ? stt : stt * unscale;
+    // 16-bit rows: the stash keeps 2^xs down to 2^-29 of the row's largest entry, on the support or off it.
+    // If the support holds less than 1/64 of that entry's weight (the student's mass sits off the support),
+    // entries that matter would fall below: such a row is redone on the support's maximum as well.
+    const bool stash_ok = TagS::bytes == 4 || ss1 >= 0x1p-6f;
+    if (stash_ok && in_range(ss1) && in_range(stt1)) {      // the same for every thread
+      const float wbar = w / ss;
+      if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - fast_log2(ss1) + fast_log2(stt1)) * LN2;
+      if (grow) rkl_gradient_from_stash<TagS, NU>(s, nunits, marg, p.inv_T_s * p.grad_scale * LN2 / ss, wbar, grow);
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + tid;
+      if (u < nunits) {
+        s[i].load(srow, u);
+        float sv[8], d[8];
+        s[i].unpack(sv);
+        stored_of(u, d);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xs = fmaf(sv[e], a_s, -bs2);
+          d[e] = fmaxf(((xs > XS_DEAD ? xs : 0.f) - d[e]) - B, XT_OFF);
+        }
+        *reinterpret_cast<float4*>(marg + u * 8) = float4{d[0], d[1], d[2], d[3]};
+        *reinterpret_cast<float4*>(marg + u * 8 + 4) = float4{d[4], d[5], d[6], d[7]};
+      }
+    }
+    redo = true;
   } else {
-    rkl_sums_optimistic<TagS, NU, false, false>(s, nunits, marg, a_s, bs, p.inv_T_t, ss, stt, w);
-    t_known = false;
+    if (unit_T) rkl_sums_optimistic<TagS, NU, true>(s, nunits, marg, a_s, bs, 1.f, ss, stt, w);
+    else rkl_sums_optimistic<TagS, NU, false>(s, nunits, marg, a_s, bs, p.inv_T_t, ss, stt, w);
+    block_sum3<MARG_NT>(ss, stt, w, red);
+    redo = !(in_range(ss) && in_range(stt));      // the same for every thread
   }
-  block_sum3<MARG_NT>(ss, stt, w, red);
-  if (!(in_range(ss) && (!t_known || in_range(stt)))) {      // the same for every thread
+  if (redo) {
     float tmax = -INFINITY;
     ms = -INFINITY;
 #pragma unroll
@@ -510,51 +642,10 @@ __device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_
       }
     }
     block_sum3<MARG_NT>(ss, stt, w, red);
-    t_known = true;
   }
-  const float wbar = w / ss, l2s = fast_log2(ss);
-  if (t_known) {
-    if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - l2s + fast_log2(stt)) * LN2;
-    if (!grow) return;
-  }
-  const float k1 = p.inv_T_s * p.grad_scale * LN2 / ss;
-  if (t_known) {
-    rkl_gradient_pass<TagS, NU, false>(s, nunits, marg, a_s, bs, k1, wbar, grow, stt);
-    return;
-  }
-  stt = 0.f;
-  rkl_gradient_pass<TagS, NU, true>(s, nunits, marg, a_s, bs, k1, wbar, grow, stt);
-  if (!p.row_loss) return;
-  stt = block_sum<MARG_NT>(stt, red);
-  float l2t = fast_log2(stt);
-  if (!in_range(stt)) {      // hardly any teacher mass, or an unnormalised teacher: T on the largest entry after all
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < NU; ++i) {
-      const int64_t u = (int64_t)i * MARG_NT + tid;
-      if (u < nunits) {
-        float xt[8];
-        stored_of(u, xt);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) tmax = fmaxf(tmax, xt[e]);
-      }
-    }
-    tmax = block_max<MARG_NT>(tmax, red);
-    stt = 0.f;
-#pragma unroll
-    for (int i = 0; i < NU; ++i) {
-      const int64_t u = (int64_t)i * MARG_NT + tid;
-      if (u < nunits) {
-        float xt[8];
-        stored_of(u, xt);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) stt += fast_exp2(xt[e] - tmax);
-      }
-    }
-    stt = block_sum<MARG_NT>(stt, red);
-    l2t = tmax + fast_log2(stt);
-  }
-  if (tid == 0) p.row_loss[r] = (wbar - l2s + l2t) * LN2;
+  const float wbar = w / ss;
+  if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - fast_log2(ss) + fast_log2(stt)) * LN2;
+  if (grow) rkl_gradient_pass<TagS, NU>(s, nunits, marg, a_s, bs, p.inv_T_s * p.grad_scale * LN2 / ss, wbar, grow);
 }
 
 template <class TagS, int NU, bool VEC>
@@ -584,7 +675,7 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
     rows.load(srow, p.Vs / 8);                   // in flight during the scatter
     accumulate_marginal<VEC>(p, prow, acc, 0, (int)p.Vs);
   }
-  rkl_against_marginal<TagS, NU>(rows.s, rows.nunits, marg, red, p, r, grow);
+  rkl_against_marginal<TagS, NU>(rows.s, rows.nunits, marg, red, p, r, grow, srow);
 }
 
 static bool ok16(const void* ptr, int64_t stride, int eb) {

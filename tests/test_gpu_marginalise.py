@@ -198,6 +198,70 @@ def test_fused_reverse_kl_on_rows_whose_sums_leave_the_range(D, T, planned):
     np.testing.assert_allclose(rl_only.cpu().numpy(), rl.numpy(), rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("lift", [3.0, 6.0, 12.0, 30.0])
+def test_fused_reverse_kl_16bit_student_with_its_largest_logits_off_the_support(D, dtype, lift):
+    """The student's largest logits sit on columns without teacher mass, `lift` above the rest: reverse KL
+    renormalises the student over the support, so the columns that carry the gradient lie far below the
+    row's maximum (what the kernel keeps of 2^logit between its passes must still resolve them)."""
+    R, Vs, Vt = 5, 4096, 12000
+    t2s, probs = _case(R, Vs, Vt, 7, 16, drop=0.01)
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(R, Vs, generator=g) * 2
+    marg0 = torch.tensor(O.marginalise_map(probs.double().numpy(), t2s, Vs))
+    on = torch.nonzero(marg0[0] > 0).squeeze(-1)
+    off_cols = on[:6]                                # taken off the support of every row
+    probs = probs.clone()
+    probs[:, torch.isin(torch.tensor(t2s), off_cols)] = 0.0
+    logits[:, off_cols] += lift
+    logits = logits.to(dtype)
+    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), torch.tensor(t2s, device=DEV), T=0.7,
+                                              teacher_T=1.0, grad_scale=1.0 / R)
+    marg = torch.tensor(O.marginalise_map(probs.double().numpy(), t2s, Vs))
+    assert (marg[:, off_cols] == 0).all()
+    with np.errstate(divide="ignore"):
+        t_logits = O.marginal_to_teacher_logits(marg)
+    _, rows64, grad64 = O.mean_loss_and_grad("rkl", logits, 0.7, t_logits=t_logits, t_T=1.0, dtype=torch.float64)
+    np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    err = (grad.cpu().double() - grad64).abs()
+    bound = O.storage_tolerance(grad64, dtype, 2e-3)
+    bound += 4e-6 * torch.softmax(logits.double() / 0.7, -1) * (1 + rows64.unsqueeze(-1)) * 20 / (0.7 * R)
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+    assert torch.count_nonzero(grad.cpu()[:, off_cols]) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_reverse_kl_16bit_rows_whose_maximum_is_negative_zero_or_towering(D, dtype):
+    """16-bit student rows take a non-negative maximum from the raw bit patterns, else from the values: rows
+    of negative logits only, maxima of exactly +0 and -0, and one logit far above the rest at every position
+    inside a 16-byte chunk in turn (a maximum that missed it would let the sums overflow)."""
+    R, Vs, Vt = 12, 4096, 12000
+    t2s, probs = _case(R, Vs, Vt, 9, 16, drop=0.01)
+    g = torch.Generator().manual_seed(4)
+    logits = torch.randn(R, Vs, generator=g) * 2
+    logits[0] = -logits[0].abs() - 0.5
+    logits[1] = -logits[1].abs() - 1.0
+    logits[1, 77] = 0.0
+    logits[2] = -logits[2].abs() - 1.0
+    logits[2, 1234] = -0.0
+    marg0 = torch.tensor(O.marginalise_map(probs.double().numpy(), t2s, Vs))
+    for r in range(4, 12):
+        on = torch.nonzero(marg0[r] > 0).squeeze(-1)
+        col = int(on[(on % 8) == (r - 4)][5])          # a column of the support at position r - 4 of its chunk
+        logits[r, col] = 120.0
+    logits = logits.to(dtype)
+    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), torch.tensor(t2s, device=DEV), T=1.0,
+                                              grad_scale=1.0 / R)
+    with np.errstate(divide="ignore"):
+        t_logits = O.marginal_to_teacher_logits(marg0)
+    _, rows64, grad64 = O.mean_loss_and_grad("rkl", logits, 1.0, t_logits=t_logits, dtype=torch.float64)
+    np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    err = (grad.cpu().double() - grad64).abs()
+    bound = O.storage_tolerance(grad64, dtype, 2e-3)
+    bound += 4e-6 * torch.softmax(logits.double(), -1) * (1 + rows64.unsqueeze(-1)) * 20 / R
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+
+
 def test_fused_path_limits_are_reported(D):
     with pytest.raises(RuntimeError, match="exceeds"):
         D.vocab_utils.rkl_marginalised(torch.zeros(2, 40000, device=DEV), torch.zeros(2, 64, device=DEV),
