@@ -262,6 +262,37 @@ def test_fused_reverse_kl_16bit_rows_whose_maximum_is_negative_zero_or_towering(
     assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("planned", [False, True])
+def test_fused_reverse_kl_gradient_may_overwrite_the_logits(D, dtype, planned):
+    """The gradient written over the logits, also for rows that are put back and redone (their logits are
+    read a second time before anything of the row is written): the same bits as into a buffer of its own."""
+    R, Vs, Vt = 6, 4096, 12000
+    t2s, probs = _case(R, Vs, Vt, 7, 16, drop=0.01)
+    g = torch.Generator().manual_seed(6)
+    logits = torch.randn(R, Vs, generator=g) * 2
+    marg0 = torch.tensor(O.marginalise_map(probs.double().numpy(), t2s, Vs))
+    off_cols = torch.nonzero(marg0[0] > 0).squeeze(-1)[:4]
+    probs = probs.clone()
+    probs[:, torch.isin(torch.tensor(t2s), off_cols)] = 0.0
+    logits[1::2, off_cols] += 40.0                   # every other row has its mass off the support
+    probs[4] *= 1e-30                                # and one hardly any teacher mass
+    x = logits.to(dtype).to(DEV)
+    tmap = D.vocab_utils.MarginalPlan(t2s, Vs, DEV) if planned else torch.tensor(t2s, device=DEV)
+    rl, grad = D.vocab_utils.rkl_marginalised(x, probs.to(DEV), tmap, T=1.3, grad_scale=0.5)
+    y = x.clone()
+    rl2, g2 = D.vocab_utils.rkl_marginalised(y, probs.to(DEV), tmap, T=1.3, grad_scale=0.5, grad_out=y)
+    assert g2.data_ptr() == y.data_ptr()
+    if planned:                                      # fixed summation order: the same bits
+        assert torch.equal(rl, rl2) and torch.equal(grad, y)
+    else:                                            # LDS atomics: the marginal's sums come in any order
+        np.testing.assert_allclose(rl2.cpu().numpy(), rl.cpu().numpy(), rtol=1e-5)
+        tol = 1e-4 if dtype == torch.float32 else 2.0 ** -7
+        diff = (grad.float() - y.float()).abs()
+        assert (diff <= tol * grad.float().abs() + 1e-6 * grad.float().abs().max()).all()
+    assert torch.isfinite(rl).all() and torch.isfinite(grad.float()).all() and grad.float().abs().max() > 0
+
+
 def test_fused_path_limits_are_reported(D):
     with pytest.raises(RuntimeError, match="exceeds"):
         D.vocab_utils.rkl_marginalised(torch.zeros(2, 40000, device=DEV), torch.zeros(2, 64, device=DEV),
