@@ -231,15 +231,147 @@ def mean_loss_and_grad(kind: str, logits: torch.Tensor, T: float, *,
     return loss.detach(), rows.detach(), leaf.grad.detach()
 
 
-def storage_tolerance(ref: torch.Tensor, storage_dtype, rtol: float) -> torch.Tensor:
+F32_HALF_ULP = 2.0 ** -24
+
+
+def storage_tolerance(ref: torch.Tensor, storage_dtype, rtol: float, terms: torch.Tensor | None = None) -> torch.Tensor:
     """Element-wise bound for comparing a gradient stored in `storage_dtype` with an
-    unrounded reference: `rtol` on the value plus the half-ulp the round-to-nearest
-    store may add (bf16 2^-8, fp16 2^-11 relative; fp16 also its subnormal spacing),
-    plus fp32 epsilon on the scale of the largest entry (entries that should be exactly
-    zero come out of the float64 autograd as ~1e-20 cancellation residue)."""
+    unrounded float64 reference: `rtol` on the entry's own value plus the half-ulp the
+    round-to-nearest store may add (bf16 2^-8, fp16 2^-11 relative; fp16 also its subnormal
+    spacing), plus `terms`: an absolute, per-entry bound on what fp32 evaluation loses where
+    the entry is a difference of larger quantities (built by the helpers below from the
+    entry's own operands).  Nothing in the bound depends on other entries' size: an entry
+    that is 1e-6 of the tensor's largest is still held to `rtol` of itself."""
     half_ulp = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[storage_dtype]
     floor = {torch.float32: 1e-30, torch.bfloat16: 1e-30, torch.float16: 2.0 ** -25}[storage_dtype]
-    return ref.abs() * (rtol + half_ulp) + floor + 1.2e-7 * ref.abs().max()
+    bound = ref.abs() * (rtol + half_ulp) + floor
+    return bound if terms is None else bound + terms
+
+
+def softmax_rounding(z: torch.Tensor) -> torch.Tensor:
+    """Relative error that fp32 evaluation leaves on the entries of softmax(z), `z` [n, V] the scaled
+    logits in float64.  The exponent z_j - max is a difference of fp32 numbers of size |z_j| and |max|,
+    each rounded to half an ulp, and an absolute error of the exponent is a relative error of the
+    exponential; the exponential, the row sum, its reciprocal and the product add about eight more
+    half-ulps.  (The reference's own fp32 log-softmax carries the same.)"""
+    zmax = z.max(-1, keepdim=True).values
+    mag = torch.nan_to_num(z.abs(), posinf=0.0) + zmax.abs()
+    return F32_HALF_ULP * (8.0 + mag)
+
+
+def _support_sum(idx: torch.Tensor, vals: torch.Tensor, V: int) -> torch.Tensor:
+    """[n, V] with vals[i, k] summed at column idx[i, k]; ids outside [0, V) are ignored."""
+    ok = (idx >= 0) & (idx < V)
+    out = torch.zeros(idx.shape[0], V, dtype=vals.dtype)
+    out.scatter_add_(1, torch.where(ok, idx, torch.zeros_like(idx)).long(), torch.where(ok, vals, torch.zeros_like(vals)))
+    return out
+
+
+def sparse_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, T: float, idx: torch.Tensor, storage_dtype,
+                              rtol: float, support_scale: float = 0.0, row_coef=None) -> torch.Tensor:
+    """Element-wise bound for a gradient of the form g_ij = a_i softmax(z_i)_j + c_ij with c_i zero off the
+    K ids of row i (forward KL on a sparse teacher: a_i = scale / T, c_ik = -q_ik scale / T; the alpha-weighted
+    composite: a_i, c_ik its row coefficients).  `grad64`, `logits` [n, V] (rows already selected),
+    `idx` [n, K] (ids outside [0, V) ignored), `T` the student temperature.
+
+    a_i is `row_coef` where the caller knows it (a number or [n, 1]), else read off the float64 gradient on the
+    columns outside the support; c_ij = g_ij - a_i p_ij on the support.
+    The bound is `storage_tolerance` of the entry itself plus, per entry,
+      |a_i| p_ij softmax_rounding(z)_ij          the dense term as fp32 computes it,
+      |c_ij| 2^-24 (8 + 32)                      the sparse term: a teacher mass exp(t - lse_K) from stored
+                                                 log-probs of magnitude up to 32, rounded like the softmax,
+      |a_i| 2^-40 max_j p_ij  (16-bit rows)      the kernel keeps 2^(z_j - max) of a 16-bit row between its sum
+                                                 and gradient sweeps as fp16 scaled by 2^15: 11 bits (inside
+                                                 `rtol`) down to 2^-29 of the row's largest probability, below
+                                                 that fp16's subnormal spacing, 2^-39 of the largest,
+    so off the support an entry is held to `rtol` (+ half an ulp of the store) of itself, and on the support to
+    that plus fp32 rounding of its two cancelling terms.  `support_scale` > 0 adds, on the support only,
+    that fraction of the row's largest coefficient max(|a_i|, max_k |c_ik|): for gradients whose sparse term is
+    itself a sum of cancelling pieces the float64 gradient does not show (the composite's reverse-KL and
+    cross-entropy parts)."""
+    z = logits.double() / T
+    p = torch.softmax(z, -1)
+    n, V = p.shape
+    on = _support_sum(idx.long(), torch.ones(idx.shape, dtype=torch.float64), V) > 0
+    off_mass = torch.where(on, torch.zeros_like(p), p).sum(-1, keepdim=True)
+    off_grad = torch.where(on, torch.zeros_like(p), grad64).sum(-1, keepdim=True)
+    if row_coef is not None:
+        a = torch.as_tensor(row_coef, dtype=torch.float64) * torch.ones(n, 1, dtype=torch.float64)
+    else:
+        # rows whose whole vocabulary is support have nothing to read a_i from and take their largest entry as the scale
+        a = torch.where(off_mass > 1e-12, off_grad / off_mass.clamp_min(1e-300), grad64.abs().max(-1, keepdim=True).values)
+    c = torch.where(on, grad64 - a * p, torch.zeros_like(p))
+    terms = a.abs() * p * softmax_rounding(z) + c.abs() * (F32_HALF_ULP * 40.0)
+    if storage_dtype != torch.float32:
+        terms = terms + a.abs() * p.max(-1, keepdim=True).values * 2.0 ** -40
+    if support_scale:
+        row_scale = torch.maximum(a.abs(), c.abs().max(-1, keepdim=True).values)
+        terms = terms + on * (support_scale * row_scale)
+    return storage_tolerance(grad64, storage_dtype, rtol, terms)
+
+
+def rkl_topk_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, t_vals: torch.Tensor, t_idx: torch.Tensor,
+                                T: float, t_T: float, scale: float, storage_dtype, rtol: float) -> torch.Tensor:
+    """Element-wise bound for the reverse-KL gradient on a sparse teacher,
+    g_ij = sum_{k: idx_ik = j} r_k ((s'_k - t_k) - rkl_i) scale / T (utils/finetuning_utils.py:105): zero off the
+    support (exactly in the kernel, to float64 rounding in the reference); on it `storage_tolerance` plus fp32 rounding of the pieces the bracket is a difference of:
+    r_k to `softmax_rounding`, s'_k and t_k (log-softmaxes over K) to half-ulps of their operands, rkl_i to the
+    r-weighted sum of those."""
+    n, V = logits.shape
+    idx = t_idx.long()
+    ok = (idx >= 0) & (idx < V)
+    z = torch.gather(logits.double() / T, 1, torch.where(ok, idx, torch.zeros_like(idx)))
+    z = z.masked_fill(~ok, NEG_INF)
+    t_in = (t_vals.double() / t_T).masked_fill(~ok, NEG_INF)
+    live = ok & ~torch.isneginf(t_in)
+    z = z.masked_fill(~live, NEG_INF)
+    s = F.log_softmax(z, -1)
+    t = F.log_softmax(t_in, -1)
+    r = torch.exp(s)
+    diff = torch.where(live, s - t, torch.zeros_like(s))
+    rkl = (r * diff).sum(-1, keepdim=True)
+    e_r = torch.where(live, softmax_rounding(z), torch.zeros_like(z))
+    tmax = t_in.max(-1, keepdim=True).values
+    d_diff = e_r + F32_HALF_ULP * (8.0 + torch.nan_to_num(t_in.abs(), posinf=0.0) + tmax.abs())
+    d_rkl = (r * (d_diff + e_r * diff.abs())).sum(-1, keepdim=True)
+    per_entry = r * (e_r * (diff.abs() + rkl.abs()) + d_diff + d_rkl) * (abs(scale) / T)
+    terms = _support_sum(idx, torch.where(live, per_entry, torch.zeros_like(per_entry)), V)
+    # the float64 reference itself: its backward through the full-vocabulary log-softmax leaves
+    # softmax_j * (sum_k g_k), a sum that is zero only up to float64 rounding, on every column
+    pieces = (r * (diff.abs() + rkl.abs())).sum(-1, keepdim=True) * (abs(scale) / T)
+    terms = terms + torch.softmax(logits.double() / T, -1) * pieces * 2.0 ** -46
+    return storage_tolerance(grad64, storage_dtype, rtol, terms)
+
+
+def topk_gradient_tolerance(kind: str, grad64: torch.Tensor, logits: torch.Tensor, t_vals: torch.Tensor, t_idx: torch.Tensor,
+                            T: float, t_T: float | None, scale: float, storage_dtype, rtol: float,
+                            valid: torch.Tensor | None = None) -> torch.Tensor:
+    """The bound of `sparse_gradient_tolerance` (forward KL) or `rkl_topk_gradient_tolerance` (reverse KL) for
+    the arguments of `mean_loss_and_grad`: `grad64`, `logits` [R, V]; teacher rows for the valid rows only; rows
+    with `valid == False` must be exactly zero."""
+    bound = storage_tolerance(grad64, storage_dtype, rtol)
+    sel = torch.arange(logits.shape[0]) if valid is None else torch.nonzero(valid).squeeze(-1)
+    if kind == "fkl":
+        bound[sel] = sparse_gradient_tolerance(grad64[sel], logits[sel], T, t_idx, storage_dtype, rtol, row_coef=scale / T)
+    else:
+        bound[sel] = rkl_topk_gradient_tolerance(grad64[sel], logits[sel], t_vals, t_idx, T, T if t_T is None else t_T,
+                                                 scale, storage_dtype, rtol)
+    return bound
+
+
+def marginal_rkl_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, rows64: torch.Tensor, T: float, scale: float,
+                                    storage_dtype, rtol: float) -> torch.Tensor:
+    """Element-wise bound for the reverse-KL gradient against a marginalised dense teacher,
+    g_ij = r_j (log r_j / q_j - rkl_i) scale / T on the marginal's support (rows already selected).
+    `storage_tolerance` plus 4e-6 of the entry's own cancelling terms, taken as p_j (1 + rkl_i) 20 scale / T
+    (log ratios of up to 20 nats); for 16-bit rows also what the kernel's fp16 copy of 2^(z_j - max), scaled by
+    2^15, loses below 2^-29 of the row's largest logit's weight: 2^-40 exp(max - z_j) of the entry."""
+    z = logits.double() / T
+    terms = 4e-6 * torch.softmax(z, -1) * (1 + rows64.unsqueeze(-1)) * 20 * abs(scale) / T
+    if storage_dtype != torch.float32:
+        gap = torch.nan_to_num(z.max(-1, keepdim=True).values - z, posinf=0.0)
+        terms = terms + grad64.abs() * 2.0 ** -40 * torch.exp(gap.clamp_max(600.0))
+    return storage_tolerance(grad64, storage_dtype, rtol, terms)
 
 
 def dense_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, t_logits: torch.Tensor, rows64: torch.Tensor,

@@ -48,7 +48,10 @@ def test_config3_full(D):
     np.testing.assert_allclose(rl[sel.to(DEV)].cpu().double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
     g = grad[sel.to(DEV)].cpu().double() * rows
     ref = grad64 * 48
-    assert ((g - ref).abs() <= O.storage_tolerance(ref, torch.bfloat16, 2e-3)).all()
+    # every sampled entry against float64: 2e-3 of its own value + the bf16 store's half ulp + fp32 rounding of
+    # its own terms + (rows kept as fp16 between the sweeps) 2^-40 of the row's largest probability
+    bound = O.sparse_gradient_tolerance(ref, sub, 1.0, c["t_idx"][sel.to(DEV)].cpu().long(), torch.bfloat16, 2e-3)
+    assert ((g - ref).abs() <= bound).all(), f"worst ratio {((g - ref).abs() / bound).max():.2f}"
     # linearity in the upstream scale (checked on a slice to bound memory)
     _, g_half = D.div_topk("fkl", c["logits"][:2048], c["t_val"][:2048], c["t_idx"][:2048], grad_scale=0.5 / rows)
     assert torch.equal(g_half.float() * 2, grad[:2048].float())
@@ -81,7 +84,8 @@ def test_config4_full(D):
     ref.sum().backward()
     np.testing.assert_allclose(rl[sd].cpu().double().numpy(), ref.detach().numpy(), rtol=3e-5, atol=3e-6)
     g = grad[sd].cpu().double() * rows
-    assert ((g - z.grad).abs() <= O.storage_tolerance(z.grad, torch.bfloat16, 2e-3)).all()
+    bound = O.sparse_gradient_tolerance(z.grad, c["logits"][sd].cpu(), 1.0, torch.as_tensor(oi).long(), torch.bfloat16, 2e-3)
+    assert ((g - z.grad).abs() <= bound).all(), f"worst ratio {((g - z.grad).abs() / bound).max():.2f}"
     # the bucketed form (no sort; the loss kernel's workgroups read their own share of the entries) on the same input
     rl1, grad1 = D.fkl_multi_teacher(c["logits"], c["t_vals"], c["t_idxs"], c["weights"], c["id_map"], grad_scale=1.0 / rows,
                                      fused=True)
@@ -89,7 +93,7 @@ def test_config4_full(D):
     np.testing.assert_allclose(rl1[sd].cpu().double().numpy(), ref.detach().numpy(), rtol=3e-5, atol=3e-6)
     np.testing.assert_allclose(rl1.cpu().numpy(), rl.cpu().numpy(), rtol=3e-5, atol=3e-6)
     g1 = grad1[sd].cpu().double() * rows
-    assert ((g1 - z.grad).abs() <= O.storage_tolerance(z.grad, torch.bfloat16, 2e-3)).all()
+    assert ((g1 - z.grad).abs() <= bound).all(), f"worst ratio {((g1 - z.grad).abs() / bound).max():.2f}"
     rl2, grad2 = D.fkl_multi_teacher(c["logits"], c["t_vals"], c["t_idxs"], c["weights"], c["id_map"], grad_scale=1.0 / rows,
                                      fused=True)
     assert torch.equal(rl1, rl2) and torch.equal(grad1, grad2)              # bit-reproducible
@@ -145,6 +149,5 @@ def test_config5_full(D):
     g = grad[sd].cpu().double() * rows
     ref = grad64 * 16
     # reverse-KL entries are r_j (log r_j/q_j - rkl) / T: the bound of the reduced-size test, per element
-    bound = O.storage_tolerance(ref, torch.bfloat16, 2e-3) + \
-        4e-6 * torch.softmax(c["logits"][sd].cpu().double() / c["T"], -1) * (1 + rows64.unsqueeze(-1)) * 20 / c["T"]
+    bound = O.marginal_rkl_gradient_tolerance(ref, c["logits"][sd].cpu(), rows64, c["T"], 1.0, torch.bfloat16, 2e-3)
     assert ((g - ref).abs() <= bound).all(), f"worst ratio {((g - ref).abs() / bound).max():.2f}"
