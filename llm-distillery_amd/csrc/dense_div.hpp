@@ -109,12 +109,18 @@ __device__ __forceinline__ void jsd_term(float lp, float lq, float& kl_pm, float
 }
 
 // Gradient of one column (before the common factor c = inv_T * scale).
+// A student column of -inf (a masked vocabulary entry) where the teacher has mass carries no student mass:
+// its log ratio is held finite so that 0 * ratio is 0, as in the loss sweeps.  The mixture's logarithm goes
+// through log_ratio_to_mixture here as everywhere: a student mass so small that half of it is a denormal,
+// on a column without teacher mass, gives log2 m = -inf (the hardware logarithm takes denormals for zero).
+__device__ __forceinline__ float rkl_log_ratio(float lp, float lq) {
+  return __builtin_amdgcn_fmed3f(lp - lq, LOG_FLOOR, -LOG_FLOOR);
+}
 __device__ __forceinline__ float dense_grad(int kind, float lp, float lq, float aux) {
   if (kind == DL_FKL) return fast_exp2(lp) - fast_exp2(lq);
-  if (kind == DL_RKL) return lq > -INFINITY ? fast_exp2(lp) * ((lp - lq) * LN2 - aux) : 0.f;
+  if (kind == DL_RKL) return lq > -INFINITY ? fast_exp2(lp) * (rkl_log_ratio(lp, lq) * LN2 - aux) : 0.f;
   const float pr = fast_exp2(lp);
-  if (!(pr > 0.f)) return 0.f;
-  return 0.5f * pr * ((lp - fast_log2(0.5f * pr + 0.5f * fast_exp2(lq))) * LN2 - aux);
+  return 0.5f * pr * (log_ratio_to_mixture(lp, fast_log2(0.5f * pr + 0.5f * fast_exp2(lq))) * LN2 - aux);
 }
 
 // The same with the kind a compile-time constant and the row's constants folded:
@@ -124,7 +130,7 @@ __device__ __forceinline__ float dense_grad(int kind, float lp, float lq, float 
 template <int KIND>
 __device__ __forceinline__ float dense_grad_column(float lp, float lq, float c, float kb, float k0) {
   if (KIND == DL_FKL) return (fast_exp2(lp) - fast_exp2(lq)) * c;
-  if (KIND == DL_RKL) return lq > -INFINITY ? fast_exp2(lp) * fmaf(lp - lq, kb, k0) : 0.f;
+  if (KIND == DL_RKL) return lq > -INFINITY ? fast_exp2(lp) * fmaf(rkl_log_ratio(lp, lq), kb, k0) : 0.f;
   const float pr = fast_exp2(lp);
   return pr * fmaf(log_ratio_to_mixture(lp, fast_log2(0.5f * pr + 0.5f * fast_exp2(lq))), kb, k0);
 }

@@ -491,7 +491,7 @@ __device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t n
       xt[0] = m0.x; xt[1] = m0.y; xt[2] = m0.z; xt[3] = m0.w; xt[4] = m1.x; xt[5] = m1.y; xt[6] = m1.z; xt[7] = m1.w;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float xs = fmaf(sv[e], a_s, -bs);
+        const float xs = fmaxf(fmaf(sv[e], a_s, -bs), XT_OFF);     // finite for a logit of -inf: 0 * difference is 0
         g[e] = xt[e] > 0.5f * XT_OFF ? fast_exp2(xs) * k1 * ((xs - xt[e]) - wbar) : 0.f;
       }
       Unit<TagS>::store(grow, u, g);

@@ -456,17 +456,40 @@ __device__ __forceinline__ void row_stats_streamed(const char* row, int64_t V, f
   sm = block_sum<NT>(sm, red);
 }
 
-// Chunk ch of a row that may lie off the 16-byte grid and may end inside its last chunk (ANY rows of
-// the register kernels; `row` points at the row's first column, one part per row).
-template <class Tag>
-__device__ __forceinline__ void store_chunk_any(char* row, int64_t ch, int64_t V, const u32x4& v) {
-  if ((ch + 1) * Chunk<Tag>::N <= V) store16_unaligned(row + ch * 16, v);
-  else store_chunk_elementwise<Tag>(row, (int)ch, (int)V, v);
+// How the rows of a register kernel lie in memory (template parameter RAG):
+//   ROWS_WHOLE  on the 16-byte grid (base and pitch), a whole number of chunks long
+//   ROWS_ANY    anywhere (element-aligned), any length: whole chunks move by unaligned 16-byte accesses
+//   ROWS_TAIL   on the 16-byte grid, but V is not a whole number of chunks (a crop of a padded vocabulary,
+//               logits[:, :, :crop]): every chunk but the row's last moves like a ROWS_WHOLE one
+// In the last two the row's last, partly filled chunk moves element by element, with -inf in the columns
+// it lacks (they add nothing to any statistic and are not stored).
+constexpr int ROWS_WHOLE = 0, ROWS_ANY = 1, ROWS_TAIL = 2;
+
+// Chunk c of a part that starts at `part`; `ncols` = columns from the part's first to the row's end.
+template <class Tag, int RAG>
+__device__ __forceinline__ u32x4 load_part_chunk(const char* part, int64_t c, int64_t ncols) {
+  // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
+  // finds its lines in L2 instead of fetching them a second time (0.47 GB less per 32768 rows of K = 200)
+  if constexpr (RAG == ROWS_WHOLE) return *reinterpret_cast<const u32x4*>(part + c * 16);
+  else if ((c + 1) * Chunk<Tag>::N <= ncols) {
+    if constexpr (RAG == ROWS_ANY) return load16_unaligned(part + c * 16);
+    else return *reinterpret_cast<const u32x4*>(part + c * 16);
+  }
+  else return load_chunk_elementwise<Tag>(part, (int)c, (int)ncols);
 }
-template <class Tag, int NT, bool ANY>
-__device__ __forceinline__ void zero_part(char* gpart, int64_t nch, int64_t V) {
-  if constexpr (!ANY) zero_row<Tag, NT>(gpart, nch);
-  else for (int64_t ch = threadIdx.x; ch < nch; ch += NT) store_chunk_any<Tag>(gpart, ch, V, u32x4{0u, 0u, 0u, 0u});
+template <class Tag, int RAG>
+__device__ __forceinline__ void store_part_chunk(char* part, int64_t c, int64_t ncols, const u32x4& v) {
+  if constexpr (RAG == ROWS_WHOLE) store16_stream(part + c * 16, v);
+  else if ((c + 1) * Chunk<Tag>::N <= ncols) {
+    if constexpr (RAG == ROWS_ANY) store16_unaligned(part + c * 16, v);
+    else store16_stream(part + c * 16, v);
+  }
+  else store_chunk_elementwise<Tag>(part, (int)c, (int)ncols, v);
+}
+template <class Tag, int NT, int RAG>
+__device__ __forceinline__ void zero_part(char* gpart, int64_t nch, int64_t ncols) {
+  if constexpr (RAG == ROWS_WHOLE) zero_row<Tag, NT>(gpart, nch);
+  else for (int64_t ch = threadIdx.x; ch < nch; ch += NT) store_part_chunk<Tag, RAG>(gpart, ch, ncols, u32x4{0u, 0u, 0u, 0u});
 }
 
 // ---------------------------------------------------------------------------------------
@@ -481,26 +504,25 @@ __device__ __forceinline__ void zero_part(char* gpart, int64_t nch, int64_t V) {
 // RETRY: second launch over the parts that gave up waiting in the first (see split_retry_list):
 // every record of the row is published by then, so nothing is waited for.
 // MULTI: the row's teachers arrive prepared in buckets (TopkParams::bk), J * NT = cap0 entries in registers.
-// ANY: rows may start anywhere (element-aligned) and V need not be a whole number of chunks: whole chunks
-// move by unaligned 16-byte accesses, the last, partly filled chunk of a row element by element with
-// -inf in the columns it lacks (they add nothing to any statistic and are not stored).
-template <class Tag, int NT, int NCH, bool SPLIT, int J, bool RETRY, bool MULTI, bool ANY = false>
+// RAG: how the rows lie in memory (ROWS_WHOLE / ROWS_ANY / ROWS_TAIL above).
+template <class Tag, int NT, int NCH, bool SPLIT, int J, bool RETRY, bool MULTI, int RAG = ROWS_WHOLE>
 __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds& s, int64_t r, int h) {
   static_assert(!MULTI || J > 0, "the head of a bucket travels in registers");
-  static_assert(!ANY || (!SPLIT && !MULTI), "rows off the 16-byte grid: one workgroup per row, one stored teacher");
+  static_assert(RAG != ROWS_ANY || (!SPLIT && !MULTI), "rows off the 16-byte grid: one workgroup per row, one stored teacher");
   using C = Chunk<Tag>;
   const int tid = threadIdx.x;
   const int P = SPLIT ? p.parts : 1;
   const int64_t c0 = (int64_t)h * NT * NCH;                       // first chunk of this part
-  const int64_t nch_row = ANY ? (p.V + C::N - 1) / C::N : p.V / C::N;
+  const int64_t nch_row = RAG != ROWS_WHOLE ? (p.V + C::N - 1) / C::N : p.V / C::N;
   const int64_t nch = min((int64_t)NT * NCH, nch_row - c0);       // chunks of this part
   const int lo = (int)(c0 * C::N);                                // its column range
-  const int hi = ANY ? (int)min(p.V, (int64_t)lo + nch * C::N) : lo + (int)(nch * C::N);
+  const int hi = RAG != ROWS_WHOLE ? (int)min(p.V, (int64_t)lo + nch * C::N) : lo + (int)(nch * C::N);
+  const int64_t ncols = p.V - lo;                                 // columns from the part's first to the row's end
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * Tag::bytes : nullptr;
   char* gpart = grow ? grow + c0 * 16 : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   if (trow < 0) {
-    if (gpart) zero_part<Tag, NT, ANY>(gpart, nch, p.V);
+    if (gpart) zero_part<Tag, NT, RAG>(gpart, nch, ncols);
     if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
@@ -516,11 +538,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int64_t c = ChunkMap<NT, NCH>::chunk(i, tid);
-    // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
-    // finds its lines in L2 instead of fetching them a second time (0.47 GB less per 32768 rows of K = 200)
-    if constexpr (!ANY) reg[i] = c < nch ? *reinterpret_cast<const u32x4*>(rpart + c * 16) : C::neg_inf();
-    else reg[i] = c >= nch ? C::neg_inf() : (c + 1) * C::N <= p.V ? load16_unaligned(rpart + c * 16)
-                                                                  : load_chunk_elementwise<Tag>(rpart, (int)c, (int)p.V);
+    reg[i] = c < nch ? load_part_chunk<Tag, RAG>(rpart, c, ncols) : C::neg_inf();
   }
 
   // teacher side while the row is in flight
@@ -538,7 +556,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
     tlse = stage_teacher<Tag, NT>(p, s, trow, row, lo, hi);
   }
   if (tlse == -INFINITY) {            // no usable teacher entry: the row contributes nothing
-    if (gpart) zero_part<Tag, NT, ANY>(gpart, nch, p.V);
+    if (gpart) zero_part<Tag, NT, RAG>(gpart, nch, ncols);
     if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
@@ -639,8 +657,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
         if (mine & (1u << i))
           if (correction_apply<Tag, NT, NCH>(s.head, s.next, s.idx, lo, i, f, mass, value)) repeats |= 1u << i;
-        if constexpr (!ANY) store16_stream(gpart + ch * 16, C::pack(f));
-        else store_chunk_any<Tag>(gpart, ch, p.V, C::pack(f));
+        store_part_chunk<Tag, RAG>(gpart, ch, ncols, C::pack(f));
       }
     }
     if (may_repeat && repeats)
@@ -660,7 +677,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   }
 }
 
-template <class Tag, int NT, int NCH, bool SPLIT, int J, bool MULTI = false, bool ANY = false>
+template <class Tag, int NT, int NCH, bool SPLIT, int J, bool MULTI = false, int RAG = ROWS_WHOLE>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void fkl_topk_reg_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -670,18 +687,18 @@ void fkl_topk_reg_kernel(const TopkParams p) {
   const int64_t r = SPLIT ? (int64_t)grp * 8 + (t_in & 7u) : xcd_banded_row(blockIdx.x);
   const int h = SPLIT ? (int)(t_in >> 3) : 0;
   if (r >= p.n_rows) return;
-  fkl_topk_part<Tag, NT, NCH, SPLIT, J, false, MULTI, ANY>(p, s, r, h);
+  fkl_topk_part<Tag, NT, NCH, SPLIT, J, false, MULTI, RAG>(p, s, r, h);
 }
 
 // One listed part, as a real call: the loop around it then costs the body no registers.
-template <class Tag, int NT, int NCH, int J, bool MULTI>
+template <class Tag, int NT, int NCH, int J, bool MULTI, int RAG>
 __device__ __attribute__((noinline)) void fkl_topk_part_again(const TopkParams& p, const TopkLds& s, unsigned at) {
-  fkl_topk_part<Tag, NT, NCH, true, J, true, MULTI>(p, s, (int64_t)(at / (unsigned)p.parts), (int)(at % (unsigned)p.parts));
+  fkl_topk_part<Tag, NT, NCH, true, J, true, MULTI, RAG>(p, s, (int64_t)(at / (unsigned)p.parts), (int)(at % (unsigned)p.parts));
 }
 
 // The parts on the retry list, a fixed grid striding over it (normally the list is empty and
 // every workgroup leaves after one load).
-template <class Tag, int NT, int NCH, int J, bool MULTI = false>
+template <class Tag, int NT, int NCH, int J, bool MULTI = false, int RAG = ROWS_WHOLE>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void fkl_topk_retry_kernel(const TopkParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -690,7 +707,7 @@ void fkl_topk_retry_kernel(const TopkParams p) {
   const unsigned n = *list.count;
 #pragma unroll 1
   for (unsigned e = blockIdx.x; e < n; e += gridDim.x) {
-    fkl_topk_part_again<Tag, NT, NCH, J, MULTI>(p, s, list.entries[e]);
+    fkl_topk_part_again<Tag, NT, NCH, J, MULTI, RAG>(p, s, list.entries[e]);
     __syncthreads();      // LDS is reused by the next entry
   }
 }
@@ -907,9 +924,9 @@ static int entry_slots(const TopkParams& p) {
     }                                                                                                           \
   }
 
-template <class Tag, int NT, int NCH, bool SPLIT, bool MULTI>
+template <class Tag, int NT, int NCH, bool SPLIT, bool MULTI, int RAG>
 static void launch_reg_j(const TopkParams& p, unsigned grid, hipStream_t st) {
-#define DL_REG_KERNEL(J) fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, J, MULTI>
+#define DL_REG_KERNEL(J) fkl_topk_reg_kernel<Tag, NT, NCH, SPLIT, J, MULTI, RAG>
   DL_LAUNCH_BY_SLOTS(DL_REG_KERNEL, grid)
 #undef DL_REG_KERNEL
 }
@@ -919,15 +936,15 @@ template <class Tag, int NT, int NCH>
 static int launch_reg_any(const TopkParams& p, hipStream_t st) {
   constexpr bool MULTI = false;
   const unsigned grid = xcd_banded_grid(p.n_rows);
-#define DL_REG_ANY_KERNEL(J) fkl_topk_reg_kernel<Tag, NT, NCH, false, J, false, true>
+#define DL_REG_ANY_KERNEL(J) fkl_topk_reg_kernel<Tag, NT, NCH, false, J, false, ROWS_ANY>
   DL_LAUNCH_BY_SLOTS(DL_REG_ANY_KERNEL, grid)
 #undef DL_REG_ANY_KERNEL
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
-template <class Tag, int NT, int NCH, bool MULTI>
+template <class Tag, int NT, int NCH, bool MULTI, int RAG>
 static void launch_retry_j(const TopkParams& p, unsigned grid, hipStream_t st) {
-#define DL_RETRY_KERNEL(J) fkl_topk_retry_kernel<Tag, NT, NCH, J, MULTI>
+#define DL_RETRY_KERNEL(J) fkl_topk_retry_kernel<Tag, NT, NCH, J, MULTI, RAG>
   DL_LAUNCH_BY_SLOTS(DL_RETRY_KERNEL, grid)
 #undef DL_RETRY_KERNEL
 }
@@ -935,9 +952,9 @@ static void launch_retry_j(const TopkParams& p, unsigned grid, hipStream_t st) {
 
 static int launch_status() { return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH; }
 
-template <class Tag, int NT, int NCH, bool MULTI>
+template <class Tag, int NT, int NCH, bool MULTI, int RAG>
 static int launch_reg(const TopkParams& p, hipStream_t st) {
-  launch_reg_j<Tag, NT, NCH, false, MULTI>(p, xcd_banded_grid(p.n_rows), st);
+  launch_reg_j<Tag, NT, NCH, false, MULTI, RAG>(p, xcd_banded_grid(p.n_rows), st);
   return launch_status();
 }
 
@@ -946,15 +963,15 @@ static int launch_reg(const TopkParams& p, hipStream_t st) {
 static int64_t split_clear_words(int64_t n_rows, int parts) { return n_rows * parts + 1; }
 
 // `cleared`: an earlier launch on the same stream has already zeroed those words
-template <class Tag, int NT, int NCH, bool MULTI>
+template <class Tag, int NT, int NCH, bool MULTI, int RAG>
 static int launch_split(TopkParams p, int parts, hipStream_t st, bool cleared) {
   p.parts = parts;
   const int64_t n16 = split_clear_words(p.n_rows, parts);
   if (!cleared)
     hipLaunchKernelGGL(clear_workspace_kernel<256>, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
                        reinterpret_cast<u32x4*>(p.workspace), n16);
-  launch_reg_j<Tag, NT, NCH, true, MULTI>(p, (unsigned)((p.n_rows + 7) / 8 * 8 * parts), st);
-  launch_retry_j<Tag, NT, NCH, MULTI>(p, (unsigned)std::min<int64_t>(p.n_rows * parts, 256), st);
+  launch_reg_j<Tag, NT, NCH, true, MULTI, RAG>(p, (unsigned)((p.n_rows + 7) / 8 * 8 * parts), st);
+  launch_retry_j<Tag, NT, NCH, MULTI, RAG>(p, (unsigned)std::min<int64_t>(p.n_rows * parts, 256), st);
   return launch_status();
 }
 
@@ -995,9 +1012,12 @@ static FklShape fkl_shape(int64_t nch, int bytes, int forced_parts, bool split_o
 }
 
 // MULTI has no streaming form: the caller checks fkl_shape first.
-template <class Tag, bool MULTI>
+// RAG = ROWS_WHOLE: `aligned` tells whether the rows are whole chunks on the 16-byte grid (else: the unaligned
+// register kernels or the streaming kernel).  RAG = ROWS_TAIL: rows on the grid that end inside a chunk
+// (`aligned` is true); the same shapes as whole rows of ceil(V / chunk) chunks.
+template <class Tag, bool MULTI, int RAG = ROWS_WHOLE>
 static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipStream_t st, bool ws_cleared = false) {
-  const int64_t nch = p.V / Tag::epc;
+  const int64_t nch = RAG == ROWS_TAIL ? (p.V + Tag::epc - 1) / Tag::epc : p.V / Tag::epc;
   const int forced = (p.flags >> DL_TOPK_PARTS_SHIFT) & 15;
   const bool fine = !MULTI && (p.flags & DL_TOPK_FINE_PARTS) != 0 &&
                     ws_bytes >= RetryList::bytes(p.n_rows, split_parts(nch, forced, true));
@@ -1008,19 +1028,19 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
   switch (sh.NT * 100 + sh.NCH) {
     case 256 * 100 + 4:
       if constexpr (!MULTI)
-        if (sh.parts > 1) return launch_split<Tag, 256, 4, MULTI>(p, sh.parts, st, ws_cleared);
-      return launch_reg<Tag, 256, 4, MULTI>(p, st);
-    case 256 * 100 + 8: return launch_reg<Tag, 256, 8, MULTI>(p, st);
+        if (sh.parts > 1) return launch_split<Tag, 256, 4, MULTI, RAG>(p, sh.parts, st, ws_cleared);
+      return launch_reg<Tag, 256, 4, MULTI, RAG>(p, st);
+    case 256 * 100 + 8: return launch_reg<Tag, 256, 8, MULTI, RAG>(p, st);
     case 512 * 100 + 8:
-      if constexpr (Tag::bytes == 4) return launch_reg<Tag, 512, 8, MULTI>(p, st);
+      if constexpr (Tag::bytes == 4) return launch_reg<Tag, 512, 8, MULTI, RAG>(p, st);
       break;
     case 256 * 100 + 16:
-      if (sh.parts > 1) return launch_split<Tag, 256, 16, MULTI>(p, sh.parts, st, ws_cleared);
-      if constexpr (Tag::bytes != 4) return launch_reg<Tag, 256, 16, MULTI>(p, st);
+      if (sh.parts > 1) return launch_split<Tag, 256, 16, MULTI, RAG>(p, sh.parts, st, ws_cleared);
+      if constexpr (Tag::bytes != 4) return launch_reg<Tag, 256, 16, MULTI, RAG>(p, st);
       break;
     case 512 * 100 + 16:
-      return sh.parts > 1 ? launch_split<Tag, 512, 16, MULTI>(p, sh.parts, st, ws_cleared) : launch_reg<Tag, 512, 16, MULTI>(p, st);
-    case 1024 * 100 + 16: return launch_reg<Tag, 1024, 16, MULTI>(p, st);
+      return sh.parts > 1 ? launch_split<Tag, 512, 16, MULTI, RAG>(p, sh.parts, st, ws_cleared) : launch_reg<Tag, 512, 16, MULTI, RAG>(p, st);
+    case 1024 * 100 + 16: return launch_reg<Tag, 1024, 16, MULTI, RAG>(p, st);
     default: break;
   }
   if (MULTI) return aligned ? DL_ERR_LIMIT : DL_ERR_ALIGN;
@@ -1052,7 +1072,7 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
       }
     }
   }
-  if (aligned) {
+  if (aligned && RAG == ROWS_WHOLE) {
     hipLaunchKernelGGL((fkl_topk_stream_kernel<Tag, 1024, 1>), dim3(xcd_banded_grid(p.n_rows)), dim3(1024),
                        TopkLds::bytes(p.K), st, p);
   } else if (same_phase) {

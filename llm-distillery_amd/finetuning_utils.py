@@ -116,7 +116,7 @@ def _fused_dicts(x: Tensor, row_map, inv_T: float, crop: int, counts, t_vals, t_
     for c in range(C):
         row = nine[c]
         d = LossDict(zip(LOSS_KEYS, row.unbind(0)))
-        d["train_loss"] = train[c]          # the one value with a graph; "custom loss" is the same number without
+        d["train_loss"] = d["custom loss"] = train[c]      # one tensor under both keys, with its graph, as in the reference
         d.packed, d.keys_packed = row, LOSS_KEYS
         out.append(d)
     return out

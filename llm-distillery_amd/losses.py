@@ -32,10 +32,9 @@ class Losses:
         self.logger = logger
         self.num_steps_accumulated = 0
 
-    @property
-    def loss_dict(self) -> dict[str, torch.Tensor]:
-        """The accumulated values by key.  While only packed dicts have been added this is a fresh dict
-        of views into the running sum: read it, do not write into it."""
+    def _view(self) -> dict[str, torch.Tensor]:
+        """The accumulated values by key, for reading: while only packed dicts have been added, a fresh
+        dict of views into the running sum."""
         if self._packed is None:
             return self._dict
         d = {}
@@ -44,13 +43,21 @@ class Losses:
         d.update(zip(self._packed_keys[1:], self._packed.unbind(0)[1:]))
         return d
 
+    @property
+    def loss_dict(self) -> dict[str, torch.Tensor]:
+        """The accumulated values by key: a plain dict that the caller may write into, as the
+        reference's attribute is (classes/losses.py:22).  Touching it ends the packed accumulation (the
+        running sum is spread out into the dict once; later additions go key by key)."""
+        self._unpack()
+        return self._dict
+
     @loss_dict.setter
     def loss_dict(self, value: dict[str, torch.Tensor]) -> None:
         self._dict, self._packed, self._train = value, None, None
 
     def _unpack(self) -> None:
         if self._packed is not None:
-            self.loss_dict = self.loss_dict
+            self.loss_dict = self._view()
 
     def add_losses(self, new_losses: dict[str, torch.Tensor]) -> None:
         """Every key except `train_loss` is cut from the autograd graph; the first dict is adopted,
@@ -128,7 +135,7 @@ class Losses:
         if self.logger is None:
             return
         prefix = "Val Loss" if self.validation else "Loss"
-        for key, value in self.loss_dict.items():
+        for key, value in self._view().items():
             if key == "train_loss":
                 continue
             shown = value / self.num_steps_accumulated if average else value
@@ -138,6 +145,8 @@ class Losses:
         """`train_loss / divisor` backward, then the key is dropped: the sum over the batch's
         conversations divided by the gradient-accumulation count, not a batch mean."""
         if self._packed is not None:
+            if self._train is None:
+                raise KeyError("train_loss")                  # a second backward: the key is gone, as in the reference
             loss, self._train = self._train / divisor, None
         else:
             loss = self._dict.pop("train_loss") / divisor
@@ -145,7 +154,7 @@ class Losses:
 
     def _scaled(self, fn) -> "Losses":
         out = Losses(self.logger, self.validation)
-        out.loss_dict = {k: fn(v) for k, v in self.loss_dict.items()}
+        out.loss_dict = {k: fn(v) for k, v in self._view().items()}
         out.num_steps_accumulated = self.num_steps_accumulated
         return out
 
@@ -156,7 +165,7 @@ class Losses:
 
     def __itruediv__(self, other):
         if isinstance(other, (int, float, torch.Tensor)):
-            self.loss_dict = {k: v / other for k, v in self.loss_dict.items()}
+            self.loss_dict = {k: v / other for k, v in self._view().items()}
             return self
         return NotImplemented
 
@@ -167,10 +176,10 @@ class Losses:
 
     def __imul__(self, other):
         if isinstance(other, (int, float, torch.Tensor)):
-            self.loss_dict = {k: v * other for k, v in self.loss_dict.items()}
+            self.loss_dict = {k: v * other for k, v in self._view().items()}
             return self
         return NotImplemented
 
     def __str__(self) -> str:
         head = " Validation Losses:\n" if self.validation else " Training Losses:\n"
-        return head + "".join(f"{k}: {v.item():.4f}\n" for k, v in self.loss_dict.items())
+        return head + "".join(f"{k}: {v.item():.4f}\n" for k, v in self._view().items())

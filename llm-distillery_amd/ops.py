@@ -232,8 +232,9 @@ def _rowstats_raw(x: torch.Tensor, t_idx: torch.Tensor, row_map, inv_T: float):
     if row_map is None and N < R:
         raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
     _, rm_ptr = _opt_i32(row_map, R, "row_map", x.device)
-    # every teacher row is written by the kernel unless a row map leaves some out: no zero fill then
-    make = torch.empty if row_map is None else torch.zeros
+    # every teacher row is written by the kernel unless a row map leaves some out, or there are more
+    # teacher rows than logits rows (rows R .. N-1 are then nobody's): no zero fill in that case only
+    make = torch.empty if row_map is None and N == R else torch.zeros
     lse = make(N, dtype=torch.float32, device=x.device)
     zk = make((N, K), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
@@ -353,8 +354,8 @@ class _CompositeLoss(torch.autograd.Function):
         lib = _lib.load()
         offs, on_host, C = _offsets_arg(offsets)
         need_grad = ctx.needs_input_grad[0]          # False under torch.no_grad() (the validation loop) and for detached logits
-        # every teacher row is written by phase 1 unless a row map leaves some out
-        make = torch.empty if row_map is None else torch.zeros
+        # every teacher row is written by phase 1 unless a row map leaves some out or teacher rows outnumber the logits rows
+        make = torch.empty if row_map is None and N == R else torch.zeros
         lse = make(N, dtype=torch.float32, device=dev)
         zk = make((N, K), dtype=torch.float32, device=dev)
         rec = torch.empty((N, 8), dtype=torch.float32, device=dev)

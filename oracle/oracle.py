@@ -171,6 +171,7 @@ def rev_kl_dense_rows(z: torch.Tensor, t_logits: torch.Tensor) -> torch.Tensor:
     t = F.log_softmax(t_logits, dim=-1)
     sup = ~torch.isneginf(t)
     s_sup = F.log_softmax(z.masked_fill(~sup, NEG_INF), dim=-1)
+    sup = sup & ~torch.isneginf(s_sup)       # a masked student entry (-inf) carries no student mass: 0 log 0 = 0
     # off the support both operands are replaced by finite stand-ins before the product, so that
     # autograd does not turn 0 * inf into NaN gradients
     s_safe = torch.where(sup, s_sup, torch.zeros_like(s_sup))
@@ -343,6 +344,24 @@ def rkl_topk_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, t_va
     return storage_tolerance(grad64, storage_dtype, rtol, terms)
 
 
+def composite_gradient_tolerance(gref: torch.Tensor, logits: torch.Tensor, T: float, storage_dtype, rtol: float, rows,
+                                 idx: torch.Tensor, crop: int | None = None) -> torch.Tensor:
+    """Entry-by-entry bound for the gradient of the alpha-weighted composite (utils/finetuning_utils.py:107-110) over
+    one sequence of logits: `gref`, `logits` [S, Vm]; `rows` the content rows (None: all), `idx` [N, K] their teacher
+    ids, `crop` the vocabulary in use.  Every entry is a_i softmax_j + (K sparse corrections): `rtol` of the entry
+    itself, the store's half ulp, fp32 rounding of the entry's two parts, and on the K support columns 4e-6 of the
+    row's largest coefficient (the correction there is a sum of forward-KL, reverse-KL and cross-entropy pieces that
+    cancel).  Rows outside `rows`, rows beyond the teacher's and columns beyond `crop` must be exactly zero."""
+    bound = storage_tolerance(gref, storage_dtype, rtol)
+    rows = torch.arange(gref.shape[0]) if rows is None else rows
+    n = min(len(rows), len(idx))
+    crop = gref.shape[1] if crop is None else crop
+    r = rows[:n].long()
+    bound[r, :crop] = sparse_gradient_tolerance(gref[r, :crop].double(), logits[r, :crop], T, idx[:n].long(), storage_dtype,
+                                                rtol, support_scale=4e-6)
+    return bound
+
+
 def topk_gradient_tolerance(kind: str, grad64: torch.Tensor, logits: torch.Tensor, t_vals: torch.Tensor, t_idx: torch.Tensor,
                             T: float, t_T: float | None, scale: float, storage_dtype, rtol: float,
                             valid: torch.Tensor | None = None) -> torch.Tensor:
@@ -359,33 +378,43 @@ def topk_gradient_tolerance(kind: str, grad64: torch.Tensor, logits: torch.Tenso
     return bound
 
 
-def marginal_rkl_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, rows64: torch.Tensor, T: float, scale: float,
-                                    storage_dtype, rtol: float) -> torch.Tensor:
-    """Element-wise bound for the reverse-KL gradient against a marginalised dense teacher,
-    g_ij = r_j (log r_j / q_j - rkl_i) scale / T on the marginal's support (rows already selected).
-    `storage_tolerance` plus 4e-6 of the entry's own cancelling terms, taken as p_j (1 + rkl_i) 20 scale / T
-    (log ratios of up to 20 nats); for 16-bit rows also what the kernel's fp16 copy of 2^(z_j - max), scaled by
-    2^15, loses below 2^-29 of the row's largest logit's weight: 2^-40 exp(max - z_j) of the entry."""
-    z = logits.double() / T
-    terms = 4e-6 * torch.softmax(z, -1) * (1 + rows64.unsqueeze(-1)) * 20 * abs(scale) / T
-    if storage_dtype != torch.float32:
-        gap = torch.nan_to_num(z.max(-1, keepdim=True).values - z, posinf=0.0)
+def dense_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, t_logits: torch.Tensor, rows64: torch.Tensor,
+                             T: float, t_T: float, scale: float, storage_dtype, rtol: float, stash: bool = False,
+                             kind: str = "fkl") -> torch.Tensor:
+    """Element-wise bound for the gradient of a dense-teacher divergence, rows already selected
+    (`logits`, `t_logits`, `grad64` [n, V]; `rows64` [n] the per-row losses; `scale` the factor the
+    gradient carries, e.g. 1 / n_valid).  `storage_tolerance` of the entry itself plus fp32 rounding of the
+    terms the entry is a difference of, (p_j + q_j)(1 + |log p_j / q_j| + loss_i) scale / T: 4e-6 of them (the
+    logarithms, the row sums and the loss each carry a few half-ulps, and where the terms cancel the result
+    keeps that much of the TERMS -- the reference's fp32 evaluation as well) plus `softmax_rounding` of the two
+    rows (logits of large magnitude lose absolute precision in the exponent).  `kind` "rkl": p is the student
+    renormalised over the teacher's support.  `stash`: the fused
+    marginal kernel keeps 2^(z_j - max) of a 16-bit student row between its passes as fp16 scaled by 2^15, which
+    below 2^-29 of the row's largest logit's weight resolves 2^-40 exp(max - z_j) of the entry."""
+    zs, zt = logits.double() / T, t_logits.double() / t_T
+    lq = torch.log_softmax(zt, -1)
+    zs_all = zs
+    if kind == "rkl":      # the student renormalised over the teacher's support, as `rev_kl_dense_rows` takes it
+        zs = zs.masked_fill(torch.isneginf(lq), NEG_INF)
+    lp = torch.log_softmax(zs, -1)
+    ratio = torch.nan_to_num((lp - lq).abs(), nan=0.0, posinf=0.0)
+    terms = (lp.exp() + lq.exp()) * (1 + ratio + rows64.unsqueeze(-1)) * (abs(scale) / T)
+    terms = terms * (4e-6 + softmax_rounding(zs) + softmax_rounding(zt))
+    if stash:
+        # the teacher row is the logarithm of a marginal that the kernel sums in fp32 (a few dozen terms per
+        # student id) and takes through the hardware logarithm (an ulp of |log2 m|), divided by T_t
+        eps_t = F32_HALF_ULP * (4.0 * torch.nan_to_num(zt.abs(), posinf=0.0) + 64.0 / t_T)
+        terms = terms + (lp.exp() + lq.exp()) * eps_t * (abs(scale) / T)
+    if stash and storage_dtype != torch.float32:
+        gap = torch.nan_to_num(zs_all.max(-1, keepdim=True).values - zs_all, posinf=0.0)     # from the row's largest logit, on the support or off it
         terms = terms + grad64.abs() * 2.0 ** -40 * torch.exp(gap.clamp_max(600.0))
     return storage_tolerance(grad64, storage_dtype, rtol, terms)
 
 
-def dense_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, t_logits: torch.Tensor, rows64: torch.Tensor,
-                             T: float, t_T: float, scale: float, storage_dtype, rtol: float) -> torch.Tensor:
-    """Element-wise bound for the gradient of a dense-teacher divergence, rows already selected
-    (`logits`, `t_logits`, `grad64` [n, V]; `rows64` [n] the per-row losses; `scale` the factor the
-    gradient carries, e.g. 1 / n_valid).  `storage_tolerance` plus 4e-6 of the terms a gradient entry
-    is a difference of, (p + q)(1 + |log p/q| + loss) * scale / T: where they cancel, fp32 evaluation
-    (the reference's as well) keeps ~1e-6 of the TERMS, not of the result."""
-    lp = torch.log_softmax(logits.double() / T, -1)
-    lq = torch.log_softmax(t_logits.double() / t_T, -1)
-    ratio = torch.nan_to_num((lp - lq).abs(), nan=0.0, posinf=0.0)
-    terms = (lp.exp() + lq.exp()) * (1 + ratio + rows64.unsqueeze(-1)) * (scale / T)
-    return storage_tolerance(grad64, storage_dtype, rtol) + 4e-6 * terms
+def marginal_rkl_gradient_tolerance(grad64: torch.Tensor, logits: torch.Tensor, t_logits: torch.Tensor, rows64: torch.Tensor,
+                                    T: float, t_T: float, scale: float, storage_dtype, rtol: float) -> torch.Tensor:
+    """`dense_gradient_tolerance` for the fused marginal + reverse-KL kernel (which stashes, see there)."""
+    return dense_gradient_tolerance(grad64, logits, t_logits, rows64, T, t_T, scale, storage_dtype, rtol, stash=True, kind="rkl")
 
 
 # ---------------------------------------------------------------------------
@@ -575,7 +604,8 @@ def merge_remap_rows(vals: Sequence[np.ndarray], idxs: Sequence[np.ndarray],
         if ids.size:
             with np.errstate(divide="ignore"):                    # an id all of whose entries carry zero mass: log 0 = -inf
                 lg = np.log(mass.astype(np.float64)) / T
-            lg = lg - (lg.max() + math.log(np.exp(lg - lg.max()).sum()))
+            if np.isfinite(lg.max()):                             # all mass zero (a teacher of weight 0 alone): stays -inf
+                lg = lg - (lg.max() + math.log(np.exp(lg - lg.max()).sum()))
         else:
             lg = np.zeros(0, dtype=np.float64)
         out.append((ids, mass, lg))

@@ -19,21 +19,7 @@ def D():
     return d
 
 
-def _bound(gref, logits, T, dtype, rtol, rows, idx, crop=None):
-    """Entry-by-entry bound for the composite's gradient over one sequence of logits: `gref`, `logits` [S, Vm];
-    `rows` the content rows (None: all), `idx` [N, K] their teacher ids, `crop` the vocabulary in use.  Every
-    entry is a_i softmax_j + (K sparse corrections): `rtol` of the entry itself, the store's half ulp, fp32
-    rounding of the entry's two parts, and on the K support columns 4e-6 of the row's largest coefficient (the
-    correction there is a sum of forward-KL, reverse-KL and cross-entropy pieces that cancel).  Rows outside
-    `rows`, rows beyond the teacher's and columns beyond `crop` must be exactly zero."""
-    bound = O.storage_tolerance(gref, dtype, rtol)
-    rows = torch.arange(gref.shape[0]) if rows is None else rows
-    n = min(len(rows), len(idx))
-    crop = gref.shape[1] if crop is None else crop
-    r = rows[:n].long()
-    bound[r, :crop] = O.sparse_gradient_tolerance(gref[r, :crop].double(), logits[r, :crop], T, idx[:n].long(), dtype, rtol,
-                                                  support_scale=4e-6)
-    return bound
+_bound = O.composite_gradient_tolerance
 
 
 def _golden(golden_dir, case):
@@ -191,6 +177,20 @@ def test_rowstats_raw_outputs_and_losses_accumulator_on_gpu(D):
     L.backward(divisor=2)
     assert all(s.grad is not None and torch.isfinite(s.grad).all() for s in leafs)
     assert total > 0 and L.num_steps_accumulated == 2
+
+
+def test_rowstats_with_more_teacher_rows_than_logits_rows(D):
+    """utils/finetuning_utils.py:87: only min(#student, #teacher) rows count.  Teacher rows beyond the logits'
+    are nobody's: their statistics come back as zeros, not as whatever the allocation held."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(5, 4096, generator=g).to(DEV)
+    idx = torch.randint(0, 4096, (9, 12), generator=g, dtype=torch.int32).to(DEV)
+    junk = torch.full((9, 12), float("nan"), device=DEV)          # make the allocator's next block dirty
+    del junk
+    lse, zk = D.rowstats_topk(x, idx, None, 1.0)
+    assert lse.shape == (9,) and zk.shape == (9, 12)
+    assert torch.count_nonzero(lse[5:]) == 0 and torch.count_nonzero(zk[5:]) == 0
+    np.testing.assert_allclose(lse[:5].cpu().numpy(), torch.logsumexp(x.cpu().double(), -1).numpy(), rtol=1e-6)
 
 
 @pytest.mark.parametrize("dtype,V,pitch,offset", [(torch.bfloat16, 32003, 32003, 0), (torch.float32, 1003, 1003, 0),

@@ -152,7 +152,7 @@ def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T, planne
     rtol = 1e-4 if dtype == torch.float32 else 2e-3
     bound = O.storage_tolerance(grad64, dtype, rtol)
     sel = torch.nonzero(valid).squeeze(-1)
-    bound[sel] = O.marginal_rkl_gradient_tolerance(grad64[sel], logits[sel], rows64, T, 1.0 / R, dtype, rtol)
+    bound[sel] = O.marginal_rkl_gradient_tolerance(grad64[sel], logits[sel], t_logits, rows64, T, T, 1.0 / R, dtype, rtol)
     assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
     # the gradient is confined to the marginal's support
     assert torch.count_nonzero(grad.cpu()[valid][:, (marg.sum(0) == 0)]) == 0
@@ -224,7 +224,7 @@ def test_fused_reverse_kl_16bit_student_with_its_largest_logits_off_the_support(
     _, rows64, grad64 = O.mean_loss_and_grad("rkl", logits, 0.7, t_logits=t_logits, t_T=1.0, dtype=torch.float64)
     np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
     err = (grad.cpu().double() - grad64).abs()
-    bound = O.marginal_rkl_gradient_tolerance(grad64, logits, rows64, 0.7, 1.0 / R, dtype, 2e-3)
+    bound = O.marginal_rkl_gradient_tolerance(grad64, logits, t_logits, rows64, 0.7, 1.0, 1.0 / R, dtype, 2e-3)
     assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
     assert torch.count_nonzero(grad.cpu()[:, off_cols]) == 0
 
@@ -256,7 +256,7 @@ def test_fused_reverse_kl_16bit_rows_whose_maximum_is_negative_zero_or_towering(
     _, rows64, grad64 = O.mean_loss_and_grad("rkl", logits, 1.0, t_logits=t_logits, dtype=torch.float64)
     np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
     err = (grad.cpu().double() - grad64).abs()
-    bound = O.marginal_rkl_gradient_tolerance(grad64, logits, rows64, 1.0, 1.0 / R, dtype, 2e-3)
+    bound = O.marginal_rkl_gradient_tolerance(grad64, logits, t_logits, rows64, 1.0, 1.0, 1.0 / R, dtype, 2e-3)
     assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
 
 

@@ -124,6 +124,42 @@ def test_losses_packed_dicts_accumulate_like_plain_ones():
     assert half.loss_dict["kl_div"].item() == 9.0
 
 
+def test_losses_loss_dict_is_a_plain_writable_dict_also_after_packed_additions():
+    """classes/losses.py:22 keeps a plain dict attribute that callers may write into, delete from or scale in
+    place; the packed accumulation must not turn such writes into no-ops, and a second backward finds the key
+    gone (KeyError) as in the reference (classes/losses.py:77-79)."""
+    from llm_distillery_amd.losses import LossDict
+    keys = D.LOSS_KEYS
+    leaf = torch.tensor(1.0, requires_grad=True)
+
+    def make(i):
+        row = torch.arange(9, dtype=torch.float32) * (i + 1)
+        d = LossDict(zip(keys, row.unbind(0)))
+        d["train_loss"] = leaf * (i + 1)
+        d.packed, d.keys_packed = row, keys
+        return d
+
+    L = D.Losses(_Log())
+    L.add_losses(make(0))
+    L.add_losses(make(1))
+    L.loss_dict["kl_div"] = torch.tensor(100.0)
+    L.loss_dict["CE loss"] /= 2
+    del L.loss_dict["CE diff"]
+    assert L.loss_dict["kl_div"].item() == 100.0 and L.loss_dict["CE loss"].item() == 2 * 3 / 2 and "CE diff" not in L.loss_dict
+    L.add_losses(make(2))                                     # a packed dict after the write: added key by key
+    assert L.loss_dict["kl_div"].item() == 100.0 + 3 * 3 and L.loss_dict["CE diff"].item() == 8 * 3
+    assert L.loss_dict["train_loss"].item() == 6.0 and L.num_steps_accumulated == 3
+    L.backward(divisor=3)
+    assert leaf.grad.item() == pytest.approx(2.0)
+    with pytest.raises(KeyError):
+        L.backward()
+    P = D.Losses(None)                                        # never touched from outside: still packed at the second backward
+    P.add_losses(make(0))
+    P.backward()
+    with pytest.raises(KeyError):
+        P.backward()
+
+
 def test_library_exports_every_symbol_the_header_declares():
     header = open(os.path.join(ROOT, "include", "distill_hip.h")).read()
     declared = set(re.findall(r"\b(dl_[a-z0-9_]+)\s*\(", header))

@@ -38,8 +38,8 @@ def _masked_map(R, masked):
                                            (152064, torch.float16, {}), (40000, torch.float32, {"no_wait": True}),
                                            (32000, torch.bfloat16, {})])
 def test_static_scratch_entry_point_matches_the_workspace_one(D, V, dtype, hooks):
-    """Rows cut into 4 parts (128256 bf16, 40000 fp32) and into 5 (152064 fp16) meet through the
-    scratch; 32000-wide rows need none.  With `no_wait` every part also goes through the list of
+    """Rows cut into 4 parts (128256 bf16), 3 (40000 fp32: 10000 chunks in parts of 4096) and 5 (152064 fp16)
+    meet through the scratch; 32000-wide rows need none.  With `no_wait` every part also goes through the list of
     deferred parts that lives in the same array."""
     K = 200
     big = _case(72, V, K, dtype, 5)
@@ -60,6 +60,30 @@ def test_static_scratch_entry_point_matches_the_workspace_one(D, V, dtype, hooks
     want_rl, want_g = D.div_topk("rkl", x, tv, ti, T=0.9)
     rl, g = torch.empty(x.shape[0], device=DEV), torch.empty_like(x)
     D.div_topk_static("rkl", x, tv, ti, rl, g, T=0.9)
+    assert torch.equal(rl, want_rl) and torch.equal(g, want_g)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("no_wait", [False, True])
+def test_static_scratch_close_to_its_limit(D, no_wait):
+    """52000 rows of 128256 bf16 columns need 4.16 MB of the 4 MiB array (records of 4 parts, a counter and a
+    list slot per part): offsets and the clear at a realistic size, with and without the list of deferred parts,
+    bit for bit against the workspace entry point; then a small call, which must not see what the large one left."""
+    from llm_distillery_amd import synthetic as S
+    lib = D._lib.load()
+    rows, V = 52000, 128256
+    assert 0.95 * D._lib.DL_STATIC_SCRATCH_BYTES < lib.dl_div_topk_workspace_bytes(0, D._lib.DL_BF16, rows, V) <= D._lib.DL_STATIC_SCRATCH_BYTES
+    c = S.config3(DEV, rows=rows, V=V, K=64)
+    want_rl, want_g = D.div_topk("fkl", c["logits"], c["t_val"], c["t_idx"], grad_scale=1.0 / rows, no_wait=no_wait)
+    rl = torch.full((rows,), float("nan"), device=DEV)
+    g = torch.empty_like(c["logits"])
+    D.div_topk_static("fkl", c["logits"], c["t_val"], c["t_idx"], rl, g, grad_scale=1.0 / rows, no_wait=no_wait)
+    assert torch.equal(rl, want_rl) and torch.equal(g, want_g)
+    del g, want_g
+    x, tv, ti = _case(9, V, 64, torch.bfloat16, 12)
+    want_rl, want_g = D.div_topk("fkl", x, tv, ti, no_wait=no_wait)
+    rl, g = torch.empty(9, device=DEV), torch.empty_like(x)
+    D.div_topk_static("fkl", x, tv, ti, rl, g, no_wait=no_wait)
     assert torch.equal(rl, want_rl) and torch.equal(g, want_g)
 
 
