@@ -32,13 +32,32 @@ INPLACE = False        # --inplace: the gradient is written over the logits (C3 
 PARTS = 0              # --parts: column parts per row of the C3 loss kernel (0 = the library's choice)
 
 
+VOCAB = 0              # --vocab / --pitch: C3 on logits[:, :vocab] of rows `pitch` columns wide (a crop of a padded vocabulary)
+PITCH = 0
+
+
 def _wl_c3(D, S, dev, rows):
     import torch
     rows = rows or 8 * 4096
-    V, K = 128256, 200
-    c = S.config3(dev, rows=rows, seed=3)
-    grad = c["logits"] if INPLACE else torch.empty_like(c["logits"])
+    V, K = VOCAB or 128256, 200
+    c = S.config3(dev, rows=rows, seed=3, V=V)
+    if PITCH and PITCH != V:
+        wide = torch.zeros((rows, PITCH), dtype=c["logits"].dtype, device=dev)
+        wide[:, :V] = c["logits"]
+        c["logits"] = wide[:, :V]
+    if INPLACE:
+        grad = c["logits"]
+    elif PITCH and PITCH != V:
+        grad = torch.empty((rows, PITCH), dtype=c["logits"].dtype, device=dev)[:, :V]
+    else:
+        grad = torch.empty_like(c["logits"])
     scale = 1.0 / rows
+    if VOCAB or PITCH:
+        def main_crop():
+            return D.div_topk("fkl", c["logits"], c["t_val"], c["t_idx"], T=1.0, grad_scale=scale, grad_out=grad, parts=PARTS)[0]
+        return (lambda: D.reduce_sum(main_crop(), scale), main_crop, rows * (V * 2 + V * 2 + K * 6), rows,
+                f"forward-KL fwd+bwd, top-K={K} fp16/int32 teacher, {rows} tokens x {V} vocab bf16 logits in rows of "
+                f"{PITCH or V} columns, T=1, bf16 gradient", "fkl_topk_reg_kernel<bf16,...>", c, grad)
 
     def main():
         return D.div_topk("fkl", c["logits"], c["t_val"], c["t_idx"], T=1.0, grad_scale=scale, grad_out=grad, parts=PARTS)[0]
@@ -389,12 +408,17 @@ def main():
     ap.add_argument("--lds-kb", type=int, default=0, help="copyshape: LDS held per workgroup (bounds workgroups per CU at 160 / n)")
     ap.add_argument("--parts", type=int, default=0, choices=(0, 1, 2, 4, 16),
                     help="c3 only: column parts per row of the loss kernel (0 = the library's choice)")
+    ap.add_argument("--vocab", type=int, default=0, help="c3: vocabulary size (default 128256)")
+    ap.add_argument("--pitch", type=int, default=0, help="c3: columns per stored row, >= --vocab: the logits are the crop "
+                    "[:, :vocab] of such rows")
     ap.add_argument("--inplace", action="store_true",
                     help="c3 only: write the gradient over the logits (same DRAM pages: about 4 %% faster).  After the "
                          "first step the buffer holds gradients, not logits, so the printed loss means nothing; the "
                          "traffic and the arithmetic per step are unchanged.  Not the default for that reason")
     args = ap.parse_args()
     global INPLACE, PARTS
+    global VOCAB, PITCH
+    VOCAB, PITCH = (args.vocab, args.pitch) if args.workload == "c3" else (0, 0)
     PARTS = args.parts if args.workload == "c3" else 0
     INPLACE = bool(args.inplace and args.workload == "c3")
     COPY_SHAPE.update(threads=args.threads, chunks=args.chunks, one_xcd=not args.row_major, wave_major=not args.striped,

@@ -93,11 +93,18 @@ const char* dl_status_string(int status);
  *            change neither results nor requirements.  The library keeps no state between calls.
  * K <= DL_MAX_TOPK.
  * Alignment: any V and any element-aligned pointers and row strides are taken (else DL_ERR_ALIGN).  Rows
- * on the 16-byte grid (16-byte aligned pointers; row strides and V whole numbers of 16-byte chunks)
- * take the aligned register kernels.  Other rows (an odd vocabulary, a column slice) are still moved
- * 16 bytes at a time: forward-KL rows of up to 4096 16-byte chunks by unaligned accesses in the register
- * kernels; wider ones, and dl_rowstats_topk / dl_rowcoef_grad_topk, by the aligned chunks inside each
- * row, provided that logits and gradient rows share their address modulo 16 (the same stride from
+ * on the 16-byte grid (16-byte aligned pointers, logits and gradient; row strides whole numbers of 16-byte
+ * chunks) take the aligned register kernels whatever V is: a row that ends inside a chunk -- the crop
+ * logits[:, :, :V] of a vocabulary padded to a multiple of 8 (4 for fp32) columns,
+ * classes/student/model.py:408 -- moves like a whole one, one workgroup per row or cut into column parts,
+ * and only its last chunk is stored element by element; nothing beyond column V is written.  The kernels
+ * READ that chunk's 16 bytes whole: they begin inside the row and, aligned as they are, end inside the
+ * row's stride or at least inside the memory page of the row's last column, so the read cannot fault; what
+ * it brings in from beyond column V is discarded.  The same holds for dl_rowcoef_grad_topk and
+ * dl_fkl_multi_teacher.  Other rows (an odd row stride, a column slice that starts off the grid) are still
+ * moved 16 bytes at a time: forward-KL rows of up to 4096 16-byte chunks by unaligned accesses in the
+ * register kernels; wider ones, and dl_rowstats_topk / dl_rowcoef_grad_topk, by the aligned chunks inside
+ * each row, provided that logits and gradient rows share their address modulo 16 (the same stride from
  * 16-byte aligned bases, or the gradient written over the logits; reverse KL: any gradient row), and
  * element by element otherwise.
  * grad may be the logits buffer itself (same pointer and stride): every kernel holds, or has
@@ -297,8 +304,9 @@ int dl_merge_remap_topk(int n_teachers, const void* const* t_vals, const void* c
  * DL_TOPK_PARTS as for dl_div_topk.  workspace: at least dl_fkl_multi_teacher_workspace_bytes(...)
  * bytes (same flags), 256-byte aligned, contents irrelevant on entry and on return; two launches
  * that may overlap in time need different workspaces.
- * Limits: n_teachers <= DL_MAX_TEACHERS, n_teachers * K <= DL_MAX_TOPK; rows 16-byte aligned with
- * V % 8 == 0 (4 for fp32), else DL_ERR_ALIGN; V <= 262144 two-byte / 131072 four-byte columns, else
+ * Limits: n_teachers <= DL_MAX_TEACHERS, n_teachers * K <= DL_MAX_TOPK; logits and gradient rows on the
+ * 16-byte grid (aligned pointers, strides whole numbers of chunks; V itself may end inside a chunk, see
+ * dl_div_topk), else DL_ERR_ALIGN; V <= 262144 two-byte / 131072 four-byte columns, else
  * DL_ERR_LIMIT (dl_fkl_multi_teacher_workspace_bytes then returns 0).  In those cases nothing was
  * launched: call dl_merge_remap_topk + dl_div_topk.
  */

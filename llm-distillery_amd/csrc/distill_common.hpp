@@ -512,6 +512,22 @@ __device__ __forceinline__ u32x4 load_chunk_elementwise(const char* part, int ch
   return v;
 }
 // The counterpart for stores: the elements of chunk `chunk` that lie before column n_cols.
+// The chunk with -inf in place of its elements n .. N-1 (the columns behind a row's end).
+template <class Tag>
+__device__ __forceinline__ u32x4 chunk_keep_first(u32x4 v, int n) {
+  const u32x4 ninf = Chunk<Tag>::neg_inf();
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    if constexpr (Tag::bytes == 4) {
+      v[d] = d < n ? v[d] : ninf[d];
+    } else {
+      const unsigned keep = (2 * d < n ? 0xffffu : 0u) | (2 * d + 1 < n ? 0xffff0000u : 0u);
+      v[d] = (v[d] & keep) | (ninf[d] & ~keep);
+    }
+  }
+  return v;
+}
+
 template <class Tag>
 __device__ __forceinline__ void store_chunk_elementwise(char* part, int chunk, int n_cols, const u32x4& v) {
   const int col0 = chunk * Chunk<Tag>::N;

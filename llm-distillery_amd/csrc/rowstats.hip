@@ -100,6 +100,10 @@ __device__ __forceinline__ float coef_on_id(const int* s_idx, const float* s_c, 
 // MODE as for phase 1.  MODE 2 needs the gradient row to sit on the 16-byte grid exactly as the logits row does
 // (same address modulo 16): the kernel then works on the rows' bodies, with the teacher ids counted
 // from the body's first column, and part 0 adds the few columns before and behind the body one by one.
+// MODE 3: logits and gradient rows on the 16-byte grid that end inside a chunk (logits[:, :, :crop] of padded
+// rows): the ragged chunk is loaded and converted like the others -- its 16 bytes start inside the row and,
+// aligned as they are, end inside the row's pitch or at least inside the page of the row's last column; what
+// lies behind the row is computed on and dropped -- and stored element by element.
 template <class Tag, int NT, int NCH, int MODE>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 void rowcoef_grad_kernel(const StatsParams p, int parts) {
@@ -132,8 +136,14 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
   char* grow = grow_all + (int64_t)shift * Tag::bytes;
   const char* row = row_all + (int64_t)shift * Tag::bytes;
   const int64_t lo = min(V, h * per_part), hi = min(V, lo + per_part);
+  // chunk `ch` of the row: whole, or (MODE 3) the ragged one at the row's end
+  const auto put = [&](int64_t ch, const u32x4& v) {
+    if (MODE != 3 || (ch + 1) * C::N <= V) store16_stream(grow + ch * 16, v);
+    else store_chunk_elementwise<Tag>(grow, (int)ch, (int)V, v);
+  };
   if (trow < 0) {
-    if (VEC) zero_row<Tag, NT>(grow + lo * Tag::bytes, (hi - lo) / C::N);
+    if (MODE == 3) for (int64_t ch = lo / C::N + tid; ch * C::N < hi; ch += NT) put(ch, u32x4{0u, 0u, 0u, 0u});
+    else if (VEC) zero_row<Tag, NT>(grow + lo * Tag::bytes, (hi - lo) / C::N);
     else for (int64_t j = lo + tid; j < hi; j += NT) store_from_float(grow, Tag::id, j, 0.f);
     if (MODE == 2 && h == 0 && tid < sp.leftovers()) store_from_float(grow_all, Tag::id, sp.column(tid), 0.f);
     return;
@@ -169,7 +179,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     }
   };
   if (VEC) {
-    const int64_t c_lo = lo / C::N, c_hi = hi / C::N;
+    const int64_t c_lo = lo / C::N, c_hi = (hi + (MODE == 3 ? C::N - 1 : 0)) / C::N;
     u32x4 v[NCH];
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -203,7 +213,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
         for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * w;
         if (mine & (1u << i))
           if (correction_apply<Tag, NT>(s_head, s_next, s_idx, (int)lo, i, f, coef, value)) repeats |= 1u << i;
-        store16_stream(grow + ch * 16, C::pack(f));
+        put(ch, C::pack(f));
       }
     }
     if (repeats)
@@ -261,6 +271,7 @@ static hipError_t launch_coef(const StatsParams& p, int mode, hipStream_t st) {
   const dim3 grid((unsigned)((p.n_rows + 7) / 8 * 8 * parts));
   if (mode == 1) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 1>), grid, dim3(NT), lds, st, p, parts);
   else if (mode == 2) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 2>), grid, dim3(NT), lds, st, p, parts);
+  else if (mode == 3) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 3>), grid, dim3(NT), lds, st, p, parts);
   else hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 0>), grid, dim3(NT), lds, st, p, parts);
   return hipGetLastError();
 }
@@ -308,8 +319,8 @@ extern "C" int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_
   if (n_rows == 0) return DL_OK;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
   if (reinterpret_cast<uintptr_t>(logits) % eb != 0 || reinterpret_cast<uintptr_t>(grad) % eb != 0) return DL_ERR_ALIGN;
-  const int vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb) && aligned16(grad, grad_stride, eb) ? 1
-                  : same_phase16(logits, row_stride, grad, grad_stride, eb) ? 2 : 0;
+  const bool on_grid = aligned16(logits, row_stride, eb) && aligned16(grad, grad_stride, eb);
+  const int vec = on_grid ? (V % (16 / eb) == 0 ? 1 : 3) : same_phase16(logits, row_stride, grad, grad_stride, eb) ? 2 : 0;
   StatsParams p{logits, row_stride, n_rows, V, row_map, t_idx, t_idx_itype, K, n_teacher_rows, inv_T,
                 const_cast<float*>(lse), nullptr, coef_lse, coef_zk, grad, grad_stride};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);

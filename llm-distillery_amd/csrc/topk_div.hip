@@ -5,7 +5,8 @@
 
 extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64_t n_rows, int64_t V) {
   if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
-  const int64_t nch = V / (logits_dtype == DL_F32 ? 4 : 8);
+  const int epc = logits_dtype == DL_F32 ? 4 : 8;
+  const int64_t nch = (V + epc - 1) / epc;      // a row that ends inside a chunk holds that chunk too
   if (nch <= 512 * 16 || nch > (int64_t)dl::MAX_COARSE_PARTS * 256 * 16) return 0;
   return dl::RetryList::bytes(n_rows, nch <= 1024 * 16 ? 4 : dl::MAX_COARSE_PARTS);
 }
@@ -29,14 +30,15 @@ static int div_topk_checked(int kind, const void* logits, int logits_dtype, int6
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
   const int epc = 16 / eb;
   if (reinterpret_cast<uintptr_t>(logits) % eb != 0 || (grad && reinterpret_cast<uintptr_t>(grad) % eb != 0)) return DL_ERR_ALIGN;
-  const bool aligned = (V % epc == 0) && (reinterpret_cast<uintptr_t>(logits) % 16 == 0) &&
-                       ((row_stride * eb) % 16 == 0) &&
+  const bool on_grid = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && ((row_stride * eb) % 16 == 0) &&
                        (!grad || (reinterpret_cast<uintptr_t>(grad) % 16 == 0 && (grad_stride * eb) % 16 == 0));
+  const bool aligned = on_grid && V % epc == 0;
   TopkParams p{logits, row_stride, n_rows, V, row_map, t_val, t_val_dtype, t_idx, t_idx_itype, K, n_teacher_rows,
                t_cnt, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride,
                (reinterpret_cast<uintptr_t>(workspace) % 16 == 0) ? workspace : nullptr, 1,
                (flags & DL_TOPK_NO_WAIT) ? 0 : SPIN_LIMIT, flags};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (kind == DL_FKL && on_grid && !aligned) return launch_fkl_tail(logits_dtype, p, workspace_bytes, st);
   if (kind == DL_FKL)
     return logits_dtype == DL_F32 ? launch_fkl<TagF32, false>(p, aligned, workspace_bytes, st)
            : logits_dtype == DL_BF16 ? launch_fkl<TagBF16, false>(p, aligned, workspace_bytes, st)

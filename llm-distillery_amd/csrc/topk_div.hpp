@@ -123,6 +123,7 @@ struct TopkLds {
   int* next;         // Kp  next entry owned by the same thread, or -1
   int* head;         // CORRECTION_HEADS list heads: first entry of a chunk's list, or -1
   unsigned* own;     // one per thread: bit i set = chunk i of the thread holds an entry
+  u32x4* tail;       // ROWS_TAIL: the logits of the row's ragged chunk, kept for the gradient by the one thread that holds it
   int Kp;
   __device__ TopkLds(unsigned char* base, int K, int owners = 0) {
     Kp = (K + 15) & ~15;
@@ -136,10 +137,11 @@ struct TopkLds {
     next = reinterpret_cast<int*>(val + Kp);
     head = next + Kp;
     own = reinterpret_cast<unsigned*>(head + (owners ? CORRECTION_HEADS : 0));
+    tail = reinterpret_cast<u32x4*>(own + owners);
   }
   __host__ __device__ static size_t bytes(int K, int owners = 0) {
     const size_t Kp = (size_t)((K + 15) & ~15);
-    return 512 + Kp * 16 + (owners ? Kp * 8 + (size_t)CORRECTION_HEADS * 4 + (size_t)owners * 4 : 0);
+    return 512 + Kp * 16 + (owners ? Kp * 8 + (size_t)CORRECTION_HEADS * 4 + (size_t)owners * 4 + 16 : 0);
   }
 };
 
@@ -534,11 +536,31 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   BucketHead hd{};
   if constexpr (MULTI) bucket_issue<NT, J>(p, trow, h, P, te, hd);
   else if constexpr (J > 0) teacher_issue<NT, J>(p, trow, te);
+  // ROWS_TAIL: the part that holds the row's ragged chunk (part-relative number tail_c, else -1) loads it like the
+  // others -- the 16 bytes start inside the row and, aligned as they are, end inside the row's pitch or at least
+  // inside the page the row's last column lies in -- and the one thread that holds it puts -inf in the columns
+  // beyond the row.  Which of a thread's registers that is, is the same for every thread (a scalar): the
+  // unrolled sweeps pay a scalar compare per chunk for it, no vector work and no registers.
+  const int64_t tail_c = (RAG == ROWS_TAIL && ncols < nch * C::N) ? nch - 1 : -1;
+  const int tail_reg = tail_c >= 0 ? ChunkMap<NT, NCH>::reg((int)tail_c) : -1;
+  const bool tail_mine = tail_c >= 0 && ChunkMap<NT, NCH>::owner((int)tail_c) == tid;
+  const int64_t nfull = tail_c >= 0 ? nch - 1 : nch;              // chunks of this part that are stored whole
   u32x4 reg[NCH];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int64_t c = ChunkMap<NT, NCH>::chunk(i, tid);
-    reg[i] = c < nch ? load_part_chunk<Tag, RAG>(rpart, c, ncols) : C::neg_inf();
+    if constexpr (RAG == ROWS_TAIL) reg[i] = c < nch ? load_part_chunk<Tag, ROWS_WHOLE>(rpart, c, ncols) : C::neg_inf();
+    else reg[i] = c < nch ? load_part_chunk<Tag, RAG>(rpart, c, ncols) : C::neg_inf();
+  }
+  u32x4 tail_raw = C::neg_inf();
+  if constexpr (RAG == ROWS_TAIL) {
+    if (tail_c >= 0) {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+        if (i == tail_reg && tail_mine) reg[i] = chunk_keep_first<Tag>(reg[i], (int)(ncols - tail_c * C::N));
+    }
+    // a second copy of the ragged chunk for the gradient sweep (same line: no traffic), parked in LDS below
+    if (tail_mine) tail_raw = load_part_chunk<Tag, ROWS_WHOLE>(rpart, tail_c, ncols);
   }
 
   // teacher side while the row is in flight
@@ -562,6 +584,9 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
   }
   if constexpr (!MULTI) fkl_partials<NT>(p, s, lo, hi, B, Q);
 
+  if constexpr (RAG == ROWS_TAIL) {
+    if (tail_mine) *s.tail = chunk_keep_first<Tag>(tail_raw, (int)(ncols - tail_c * C::N));      // read back by this thread only
+  }
   const float a = p.inv_T_s * LOG2E;
   float mx = -INFINITY;
 #pragma unroll
@@ -649,7 +674,7 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = ChunkMap<NT, NCH>::chunk(i, tid);
-      if (ch < nch) {
+      if (ch < nfull) {
         float f[C::N];
         forget(reg[i]);
         C::unstash(reg[i], f);
@@ -657,7 +682,23 @@ __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds
         for (int e = 0; e < C::N; ++e) f[e] *= kc;
         if (mine & (1u << i))
           if (correction_apply<Tag, NT, NCH>(s.head, s.next, s.idx, lo, i, f, mass, value)) repeats |= 1u << i;
-        store_part_chunk<Tag, RAG>(gpart, ch, ncols, C::pack(f));
+        if constexpr (RAG == ROWS_TAIL) store16_stream(gpart + ch * 16, C::pack(f));
+        else store_part_chunk<Tag, RAG>(gpart, ch, ncols, C::pack(f));
+      }
+    }
+    if constexpr (RAG == ROWS_TAIL) {
+      // The ragged chunk, by the one thread that holds it, from the copy of its logits in LDS, stored element by
+      // element.  The sweep above covers the whole chunks
+      // only and is the sweep of whole rows, instruction for instruction: a second bound inside it, or
+      // registers that must outlive it, make the 512 x 16 shape spill.
+      if (tail_mine) {
+        float f[C::N];
+        C::unpack(*s.tail, f);
+#pragma unroll
+        for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * c;
+        if (mine & (1u << tail_reg))
+          if (correction_apply<Tag, NT, NCH>(s.head, s.next, s.idx, lo, tail_reg, f, mass, value)) repeats |= 1u << tail_reg;
+        store_chunk_elementwise<Tag>(gpart, (int)tail_c, (int)ncols, C::pack(f));
       }
     }
     if (may_repeat && repeats)
@@ -1049,7 +1090,7 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
   // gradient written over the logits)
   const bool same_phase = !p.grad || (reinterpret_cast<uintptr_t>(p.logits) % 16 == reinterpret_cast<uintptr_t>(p.grad) % 16 &&
                                       ((p.row_stride - p.grad_stride) * Tag::bytes) % 16 == 0);
-  if constexpr (!MULTI) {
+  if constexpr (!MULTI && RAG == ROWS_WHOLE) {
     if (!aligned) {
       // ... or, as far as one workgroup holds a row, the register kernels with unaligned accesses.  Measured
       // (16384 x 32100 bf16: 0.47 ms against 0.75 ms streaming; 16384 x 50257: 1.27 against 0.92): up to
@@ -1084,6 +1125,11 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
   }
   return launch_status();
 }
+
+// The ROWS_TAIL instantiations of launch_fkl live in translation units of their own (topk_div_tail.hip,
+// topk_multi_tail.hip), so that they compile beside the others.
+int launch_fkl_tail(int logits_dtype, const TopkParams& p, int64_t ws_bytes, hipStream_t st);
+int launch_fkl_tail_multi(int logits_dtype, const TopkParams& p, int64_t ws_bytes, hipStream_t st, bool ws_cleared);
 
 template <class Tag>
 static hipError_t launch_rkl(const TopkParams& p, bool aligned, hipStream_t st) {

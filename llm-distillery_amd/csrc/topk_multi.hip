@@ -225,7 +225,7 @@ struct MultiPlan { FklShape shape; int cap0; int64_t exchange_bytes, first_bytes
 
 static bool multi_plan(int logits_dtype, int64_t n_rows, int64_t V, int E, int64_t n_trows, int flags, MultiPlan& out) {
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
-  const int64_t nch = V / (16 / eb);
+  const int64_t nch = (V + 16 / eb - 1) / (16 / eb);      // a row that ends inside a chunk holds that chunk too
   const FklShape sh = fkl_shape(nch, eb, (flags >> DL_TOPK_PARTS_SHIFT) & 15, true);
   if (sh.NT == 0) return false;
   out.shape = sh;
@@ -290,10 +290,10 @@ extern "C" int dl_fkl_multi_teacher(const void* logits, int logits_dtype, int64_
   if (n_rows == 0) return DL_OK;
   const int E = n_teachers * K;
   const int eb = logits_dtype == DL_F32 ? 4 : 2;
-  const bool aligned = (V % (16 / eb) == 0) && (reinterpret_cast<uintptr_t>(logits) % 16 == 0) &&
-                       ((row_stride * eb) % 16 == 0) &&
+  const bool on_grid = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && ((row_stride * eb) % 16 == 0) &&
                        (!grad || (reinterpret_cast<uintptr_t>(grad) % 16 == 0 && (grad_stride * eb) % 16 == 0));
-  if (!aligned) return DL_ERR_ALIGN;
+  if (!on_grid) return DL_ERR_ALIGN;
+  const bool whole = V % (16 / eb) == 0;      // else the rows end inside a chunk: the ROWS_TAIL kernels
   MultiPlan plan;
   if (!multi_plan(logits_dtype, n_rows, V, E, n_teacher_rows, flags, plan)) return DL_ERR_LIMIT;
   if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 256 != 0 ||
@@ -351,6 +351,7 @@ extern "C" int dl_fkl_multi_teacher(const void* logits, int logits_dtype, int64_
       else launch_prep<40, false>(q, st);
     }
   }
+  if (!whole) return launch_fkl_tail_multi(logits_dtype, p, plan.exchange_bytes, st, ws_cleared);
   return logits_dtype == DL_F32 ? launch_fkl<TagF32, true>(p, true, plan.exchange_bytes, st, ws_cleared)
          : logits_dtype == DL_BF16 ? launch_fkl<TagBF16, true>(p, true, plan.exchange_bytes, st, ws_cleared)
                                    : launch_fkl<TagF16, true>(p, true, plan.exchange_bytes, st, ws_cleared);

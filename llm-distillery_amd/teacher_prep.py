@@ -150,7 +150,7 @@ def _fkl_multi_fused(logits, vals, idxs, weights, id_map, row_map, T, grad_scale
     row_loss = torch.empty(R, dtype=torch.float32, device=dev)
     grad, g_ptr, g_stride = None, 0, V
     if want_grad:
-        grad = ops._grad_target(grad_out, R, V, x.dtype, dev)
+        grad = ops._grad_target(grad_out, R, V, x.dtype, dev, like=x)
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
     lib = _lib.load()
     n = len(vals)

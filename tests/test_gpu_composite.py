@@ -194,7 +194,10 @@ def test_rowstats_with_more_teacher_rows_than_logits_rows(D):
 
 
 @pytest.mark.parametrize("dtype,V,pitch,offset", [(torch.bfloat16, 32003, 32003, 0), (torch.float32, 1003, 1003, 0),
-                                                  (torch.bfloat16, 5001, 5120, 3), (torch.float16, 7, 7, 0)])
+                                                  (torch.bfloat16, 5001, 5120, 3), (torch.float16, 7, 7, 0),
+                                                  # crops of padded rows: on the 16-byte grid, the last chunk ragged
+                                                  (torch.bfloat16, 5001, 5120, 0), (torch.float32, 32003, 32064, 0),
+                                                  (torch.bfloat16, 50257, 50304, 0), (torch.float16, 16385, 16392, 0)])
 @pytest.mark.parametrize("grad_mode", ["fresh", "other_phase"])
 def test_two_phase_kernels_on_rows_off_the_16_byte_grid(D, dtype, V, pitch, offset, grad_mode):
     """Phase 1 and phase 2 on rows that do not start or end on 16-byte boundaries (vector accesses to the

@@ -186,6 +186,44 @@ def test_bucketed_multi_teacher_against_oracle(D, V, dtype, n, K, Vt, T):
     assert ((grad3.cpu().double() - grad64).abs() <= bound).all()
 
 
+@pytest.mark.parametrize("V,pitch,dtype", [(151665, 151936, torch.bfloat16), (50257, 50304, torch.float16), (32003, 32064, torch.float32)])
+def test_bucketed_multi_teacher_on_a_crop_of_padded_rows(D, V, pitch, dtype):
+    """Rows on the 16-byte grid that end inside a chunk (logits[:, :, :crop], classes/student/model.py:408) stay in the
+    bucketed form: entries in the ragged last chunk, masked rows, waiting or not."""
+    g = torch.Generator().manual_seed(V)
+    R, K, n, Vt = 9, 100, 3, V + 4000
+    logits = (torch.randn(R, V, generator=g) * 3).to(dtype)
+    valid = torch.ones(R, dtype=torch.bool)
+    valid[4] = False
+    nv = int(valid.sum())
+    vals, idxs = _teachers(nv, K, Vt, n, V + 1)
+    weights = [0.5, 0.3, 0.2]
+    id_map = torch.randint(0, V, (Vt,), generator=g, dtype=torch.int32)
+    id_map[torch.rand(Vt, generator=g) < 0.05] = -1
+    id_map[idxs[0][:, :3].long()] = V - 1                     # entries of every row in the last column
+    id_map[idxs[1][:, :2].long()] = V - 2
+    rm = torch.full((R,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(nv, dtype=torch.int32)
+    full = torch.full((R, pitch), 3.0, dtype=dtype, device=DEV)
+    x = full[:, :V]
+    x.copy_(logits.to(DEV))
+    args = (x, [v.to(DEV) for v in vals], [i.to(DEV) for i in idxs], weights, id_map.to(DEV))
+    rl, grad = D.fkl_multi_teacher(*args, row_map=rm.to(DEV), T=1.2, teacher_T=1.0, grad_scale=1.0 / nv, fused=True)
+    rows64, grad64, cnt, ids = _oracle_multi(logits, vals, idxs, weights, id_map, 1.2, valid)
+    np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+    assert torch.count_nonzero(rl.cpu()[~valid]) == 0 and torch.count_nonzero(grad.cpu()[~valid]) == 0
+    grad64 = grad64 / nv
+    rtol = 1e-4 if dtype == torch.float32 else 2e-3
+    bound = O.storage_tolerance(grad64, dtype, rtol)
+    vrows = torch.nonzero(valid).squeeze(-1)
+    bound[vrows] = O.sparse_gradient_tolerance(grad64[vrows], logits[vrows], 1.2, ids, dtype, rtol, row_coef=1.0 / (nv * 1.2))
+    err = (grad.cpu().double() - grad64).abs()
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+    assert (full[:, V:] == 3.0).all()
+    rl2, grad2 = D.fkl_multi_teacher(*args, row_map=rm.to(DEV), T=1.2, teacher_T=1.0, grad_scale=1.0 / nv, fused=True, no_wait=True)
+    assert torch.equal(rl, rl2) and torch.equal(grad, grad2)
+
+
 def test_bucketed_multi_teacher_edge_rows(D):
     """Rows whose entries are all dropped (loss 0, zero gradient), a teacher of weight 0, ids outside
     the teacher vocabulary, int64 ids with fp32 values, no map at all."""

@@ -147,6 +147,64 @@ def test_rows_off_the_16_byte_grid(D, kind, dtype, V, pitch, offset, grad_mode):
         assert torch.count_nonzero(full[:, :offset]) == 0 and torch.count_nonzero(full[:, offset + V:]) == 0
 
 
+@pytest.mark.parametrize("dtype,V,pitch", [(torch.bfloat16, 50257, 50304),      # GPT-2's vocabulary in its padded rows: 512 x 16, one workgroup per row
+                                           (torch.bfloat16, 151665, 151936),    # Qwen's: five column parts, the last one ragged
+                                           (torch.float32, 32003, 32064),       # 512 x 16 of four-byte chunks
+                                           (torch.float16, 4099, 4104),         # 256 x 4
+                                           (torch.bfloat16, 65537, 65544),      # one column more than two parts hold: the third part is one ragged chunk
+                                           (torch.float32, 70001, 70008),       # five parts of four-byte chunks
+                                           (torch.bfloat16, 262139, 262144)])   # eight parts in four workgroups of 512 threads
+@pytest.mark.parametrize("grad_mode", ["fresh", "in_place", "other_pitch", "other_phase"])
+def test_crop_of_a_padded_vocabulary(D, dtype, V, pitch, grad_mode):
+    """logits[:, :, :crop] of rows padded to a multiple of 16 bytes (classes/student/model.py:408): rows start on
+    the 16-byte grid and end inside a chunk.  The register kernels take them like whole rows, one workgroup per
+    row or cut into column parts, and move only the row's last chunk element by element; nothing beyond the crop
+    is written.  A gradient buffer off the grid (other_phase) falls back to the unaligned / streaming kernels.
+    With and without waiting for the partners: the oracle's numbers and the same bits."""
+    R, K = 11, 48
+    logits, tv, ti = _case(R, V, K, dtype, 71, std=3.0)
+    valid = torch.ones(R, dtype=torch.bool)
+    valid[[2, 10]] = False
+    nv = int(valid.sum())
+    rm = torch.full((R,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(nv, dtype=torch.int32)
+    tv, ti = tv[valid], ti[valid]
+    ti[:, 0] = 0                                                  # entries in the first and the last column
+    ti[:, 1] = V - 1
+    ti[:, 2] = V - 1                                              # a repeated id in the ragged chunk
+    ti[:, 3] = V - V % (8 if dtype != torch.float32 else 4)       # the ragged chunk's first column
+    tl = torch.log_softmax(logits[valid].float() * 1.1, -1)
+    tv = torch.gather(tl, 1, ti.long()).to(tv.dtype)
+    _, rows64, grad64 = O.mean_loss_and_grad("fkl", logits, 1.3, t_vals=tv, t_idx=ti, valid=valid, dtype=torch.float64)
+    bound = O.topk_gradient_tolerance("fkl", grad64, logits, tv, ti, 1.3, None, 1.0 / nv, dtype, TOL[dtype], valid)
+    results = []
+    for no_wait in (False, True):
+        full = torch.full((R, pitch), 7.0, dtype=dtype, device=DEV)
+        x = full[:, :V]
+        x.copy_(logits.to(DEV))
+        assert x.data_ptr() % 16 == 0 and (x.stride(0) * x.element_size()) % 16 == 0
+        if grad_mode == "fresh":
+            out = None
+        elif grad_mode == "in_place":
+            out = x
+        elif grad_mode == "other_pitch":
+            out = torch.full((R, pitch + 64), 5.0, dtype=dtype, device=DEV)[:, :V]
+        else:
+            out = torch.full((R, pitch + 1), 5.0, dtype=dtype, device=DEV)[:, 1:1 + V]
+        rl, grad = D.div_topk("fkl", x, tv.to(DEV), ti.to(DEV), row_map=rm.to(DEV), T=1.3, grad_scale=1.0 / nv, grad_out=out,
+                              no_wait=no_wait)
+        assert grad_mode == "fresh" or grad.data_ptr() == out.data_ptr()
+        np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=2e-5, atol=2e-6)
+        assert torch.count_nonzero(rl[~valid.to(DEV)]) == 0 and torch.count_nonzero(grad[~valid.to(DEV)]) == 0
+        err = (grad.cpu().double() - grad64).abs()
+        assert (err <= bound).all(), f"worst {(err / bound).max():.2f}"
+        assert (full[:, V:] == 7.0).all()                         # nothing beyond the crop was touched
+        if grad_mode == "other_pitch":
+            assert (out.as_strided((R, pitch + 64 - V), (pitch + 64, 1), out.storage_offset() + V) == 5.0).all()
+        results.append((rl.clone(), grad.clone()))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+
+
 def test_streaming_path_rows_larger_than_register_file(D):
     logits, tv, ti = _case(6, 152064, 200, torch.bfloat16, 6)
     _check(D, "fkl", logits, tv, ti, T=1.0)
