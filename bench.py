@@ -32,6 +32,7 @@ INPLACE = False        # --inplace: the gradient is written over the logits (C3 
 PARTS = 0              # --parts: column parts per row of the C3 loss kernel (0 = the library's choice)
 
 
+NO_SPLIT = False       # --no-split: dense rows are not cut into column parts (dl_div_dense without a workspace)
 VOCAB = 0              # --vocab / --pitch: C3 on logits[:, :vocab] of rows `pitch` columns wide (a crop of a padded vocabulary)
 PITCH = 0
 
@@ -131,7 +132,7 @@ def _wl_dense(kind_name):
 
         def main():
             return D.div_dense(c["kind"], c["logits"], c["t_logits"], row_map=c["row_map"], T=c["T"], grad_scale=scale,
-                               grad_out=grad)[0]
+                               grad_out=grad, split=not NO_SPLIT)[0]
 
         return (lambda: D.reduce_sum(main(), scale), main, nv * V * 2 * eb + R * V * eb, R,
                 f"{desc}; {R} tokens ({nv} valid) x {V} vocab", f"dense_reg_kernel ({c['kind']})", c, grad)
@@ -411,13 +412,15 @@ def main():
     ap.add_argument("--vocab", type=int, default=0, help="c3: vocabulary size (default 128256)")
     ap.add_argument("--pitch", type=int, default=0, help="c3: columns per stored row, >= --vocab: the logits are the crop "
                     "[:, :vocab] of such rows")
+    ap.add_argument("--no-split", action="store_true", help="c1 / dense: one workgroup per row pair (no workspace)")
     ap.add_argument("--inplace", action="store_true",
                     help="c3 only: write the gradient over the logits (same DRAM pages: about 4 %% faster).  After the "
                          "first step the buffer holds gradients, not logits, so the printed loss means nothing; the "
                          "traffic and the arithmetic per step are unchanged.  Not the default for that reason")
     args = ap.parse_args()
     global INPLACE, PARTS
-    global VOCAB, PITCH
+    global VOCAB, PITCH, NO_SPLIT
+    NO_SPLIT = args.no_split
     VOCAB, PITCH = (args.vocab, args.pitch) if args.workload == "c3" else (0, 0)
     PARTS = args.parts if args.workload == "c3" else 0
     INPLACE = bool(args.inplace and args.workload == "c3")

@@ -175,6 +175,32 @@ int dl_div_dense(int kind,
                  float* row_loss, void* grad, int64_t grad_stride, void* stream);
 
 /*
+ * dl_div_dense with a workspace: forward and reverse KL on rows that one 256-thread workgroup's registers do
+ * not hold (more than 16384 columns of two 16-bit rows, 8192 with an fp32 row; up to 8 times that) are then
+ * cut into column parts of that size, one workgroup each, which exchange their maxima and sums through the
+ * workspace -- the split of dl_div_topk applied to the dense pair (same reference lines as dl_div_dense).
+ * Four parts of different rows share a compute unit and hide each other's load, arithmetic and store
+ * phases, which a workgroup that holds a whole pair of rows (512 or 1024 threads, one or two per compute
+ * unit) cannot.  Same arguments and conventions as dl_div_dense, same results to fp32 rounding (the sums are
+ * taken part by part), bit-reproducible from call to call.
+ * workspace   at least dl_div_dense_workspace_bytes(...) bytes, 16-byte aligned, contents irrelevant on entry
+ *             and on return; NULL or too small: exactly dl_div_dense.  Launches that may overlap in time must
+ *             not share a workspace.  dl_div_dense_workspace_bytes returns 0 where rows are not cut (JSD,
+ *             narrow or very wide rows, V not a multiple of 8, dtype pairs without a register kernel).
+ * flags       DL_TOPK_NO_WAIT: the parts never wait for their partners (test hook, as for dl_div_topk).
+ */
+int dl_div_dense_ws(int kind,
+                    const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                    const int32_t* row_map,
+                    const void* t_logits, int t_dtype, int64_t t_stride, int64_t n_teacher_rows,
+                    float inv_T_student, float inv_T_teacher, float grad_scale,
+                    float* row_loss, void* grad, int64_t grad_stride,
+                    void* workspace, int64_t workspace_bytes, int flags, void* stream);
+
+/* Scratch size dl_div_dense_ws can make use of for this problem (0 = none: rows are not cut).  Host-only. */
+int64_t dl_div_dense_workspace_bytes(int kind, int logits_dtype, int t_dtype, int64_t n_rows, int64_t V);
+
+/*
  * Phase 1 of the general (two-phase) path: per valid row r with teacher row t = row_map[r],
  *   lse[t]   = logsumexp_j(logits[r, j] * inv_T)                       (fp32, natural log)
  *   zk[t, k] = logits[r, t_idx[t, k]] * inv_T                          (fp32; 0 for ids outside [0, V))

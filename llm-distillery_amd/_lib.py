@@ -36,6 +36,9 @@ _SIGNATURES = {
                                    c_float, c_float, c_float, _P, _P, c_int64, c_int, _P]),
     "dl_div_dense": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int64, c_int64,
                              c_float, c_float, c_float, _P, _P, c_int64, _P]),
+    "dl_div_dense_ws": (c_int, [c_int, _P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int64, c_int64,
+                                c_float, c_float, c_float, _P, _P, c_int64, _P, c_int64, c_int, _P]),
+    "dl_div_dense_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int64, c_int64]),
     "dl_rowstats_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int, c_int64, c_float,
                                  _P, _P, _P]),
     "dl_rowcoef_grad_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int, c_int64, c_float,

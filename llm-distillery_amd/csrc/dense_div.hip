@@ -1,5 +1,6 @@
 // Kernels and C entry point for divergences against a dense teacher stored in memory.
 #include "dense_div.hpp"
+#include <algorithm>
 
 namespace dl {
 
@@ -15,13 +16,26 @@ struct DenseParams {
 // Both rows in registers: NU units of 8 columns per thread.  ANY: rows of V columns that may start
 // anywhere and end inside a unit (unaligned 16-byte accesses; columns beyond the row read as -inf, which
 // adds nothing to any statistic, and are not stored).
+// BLOCKED (two fp32 rows on the grid): which 8 columns make up a unit is free as long as student, teacher and
+// gradient agree, and nothing but the loads and stores ever asks.  A unit of 8 consecutive fp32 columns is two
+// chunks side by side, so that a wave's load instruction touches every other 16 bytes: half of each line, and the
+// next instruction the other half.  Instead the 128 chunks of 64 consecutive units (one wave's worth) are dealt
+// chunk c to lane c % 64, first and second chunk of a unit 64 chunks apart (n apart in a last block of n < 64
+// units): every load and store instruction of a wave then covers 1 KiB in one piece.
 template <class TagS, class TagT, int NT, int NU, bool ANY = false>
 struct RegRows {
   static constexpr bool ONLINE = false;      // sweeps cost no memory traffic: maxima first, then sums
+  static constexpr bool BLOCKED = !ANY && TagS::bytes == 4 && TagT::bytes == 4;
   Unit<TagS> s[NU];
   Unit<TagT> t[NU];
   int64_t nunits;
   int64_t V;
+  // byte offset of chunk k of unit u in a BLOCKED row
+  __device__ __forceinline__ int64_t blocked_at(int64_t u, int k) const {
+    const int64_t b = u >> 6;
+    const int64_t nb = min((int64_t)64, nunits - (b << 6));
+    return ((b << 7) + k * nb + (u & 63)) * 16;
+  }
   __device__ __forceinline__ void load(const char* srow, const char* trow, int64_t nu, int64_t n_cols = 0) {
     nunits = nu;
     V = n_cols;
@@ -30,6 +44,14 @@ struct RegRows {
       const int64_t u = (int64_t)i * NT + threadIdx.x;
       if (u < nunits) {
         if constexpr (ANY) { s[i].load_any(srow, u, V); t[i].load_any(trow, u, V); }
+        else if constexpr (BLOCKED) {
+#pragma unroll
+          for (int k = 0; k < 2; ++k) {
+            const int64_t at = blocked_at(u, k);
+            s[i].c[k] = load16_stream(srow + at);
+            t[i].c[k] = load16_stream(trow + at);
+          }
+        }
         else { s[i].load(srow, u); t[i].load(trow, u); }
       } else {
         s[i].fill_neg_inf(); t[i].fill_neg_inf();
@@ -38,6 +60,10 @@ struct RegRows {
   }
   __device__ __forceinline__ void store(char* grow, int64_t u, const float* g) const {
     if constexpr (ANY) Unit<TagS>::store_any(grow, u, V, g);
+    else if constexpr (BLOCKED) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) store16_stream(grow + blocked_at(u, k), Chunk<TagS>::pack(g + k * 4));
+    }
     else Unit<TagS>::store(grow, u, g);
   }
   template <class F>
@@ -140,6 +166,261 @@ __global__ __launch_bounds__(NT) void dense_reg_kernel(const DenseParams p) {
     if (tid == 0 && p.row_loss) p.row_loss[r] = st.loss;
     if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
   }
+}
+
+// ---------------------------------------------------------------------------------------
+// Forward / reverse KL on rows cut into column parts.  A workgroup that holds a whole pair of rows is
+// 512 or 1024 threads wide, so one or two of them fill a CU and nothing overlaps their load,
+// arithmetic and store phases.  Here a row pair is cut into P <= 8 parts of 256 (or 512) threads x NU units
+// instead; four (two) parts of different rows share a CU and hide each other's phases, and each part still
+// reads its columns once.  The parts of a row exchange (maxima, sums of exponentials, divergence sum on the part's
+// own biases) through a 32-byte record per part in a caller-provided workspace: relaxed device-scope stores
+// and loads, validated by a tag over the five words; the wait is bounded, and a part that gives up -- it has
+// written nothing yet, also when the gradient goes over the logits -- puts itself on a list that a second
+// launch finishes from the then complete records.  Every part combines the records in part order: all parts
+// of a row arrive at the same bits, and so does the second launch.  Parts of a row sit 8 workgroup ids
+// apart, i.e. on one XCD back to back.  JSD is not cut: its divergence needs the row's normalisers inside a
+// logarithm, which would take a second exchange.
+// ---------------------------------------------------------------------------------------
+struct DenseRecord { unsigned ms, mt, ss, st, w, tag, pad0, pad1; };
+constexpr int DENSE_MAX_PARTS = 8;
+constexpr int DENSE_SPIN_LIMIT = 20000;
+
+struct DenseSplit {
+  DenseRecord* records;      // n_rows * parts
+  unsigned* retry_count;     // then a counter (16 bytes) and n_rows * parts list slots
+  unsigned* retry_list;
+  int parts;
+  int spin_limit;
+  __host__ __device__ static int64_t bytes(int64_t n_rows, int parts) { return n_rows * parts * (int64_t)(sizeof(DenseRecord) + 4) + 16; }
+  __host__ DenseSplit(void* ws, int64_t n_rows, int parts_, int spin) {
+    records = reinterpret_cast<DenseRecord*>(ws);
+    char* base = reinterpret_cast<char*>(ws) + n_rows * parts_ * (int64_t)sizeof(DenseRecord);
+    retry_count = reinterpret_cast<unsigned*>(base);
+    retry_list = reinterpret_cast<unsigned*>(base + 16);
+    parts = parts_;
+    spin_limit = spin;
+  }
+};
+
+__device__ __forceinline__ unsigned dense_record_tag(unsigned a, unsigned b, unsigned c, unsigned d, unsigned e) {
+  return a ^ ((b << 5) | (b >> 27)) ^ ((c << 11) | (c >> 21)) ^ ((d << 17) | (d >> 15)) ^ ((e << 23) | (e >> 9)) ^ 0x5eed4321u;
+}
+__device__ __forceinline__ void dense_record_publish(DenseRecord* w, float ms, float mt, float ss, float st, float wv) {
+  const unsigned a = __float_as_uint(ms), b = __float_as_uint(mt), c = __float_as_uint(ss), d = __float_as_uint(st),
+                 e = __float_as_uint(wv);
+  __hip_atomic_store(&w->ms, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->mt, b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->ss, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->st, d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->w, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&w->tag, dense_record_tag(a, b, c, d, e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Bounded wait for a partner's record; false = gave up after `limit` polls.  A cleared record is invalid.
+__device__ __forceinline__ bool dense_record_collect(DenseRecord* w, int limit, float* out) {
+  for (int spins = 0; spins < limit; ++spins) {
+    const unsigned a = __hip_atomic_load(&w->ms, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned b = __hip_atomic_load(&w->mt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned c = __hip_atomic_load(&w->ss, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned d = __hip_atomic_load(&w->st, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned e = __hip_atomic_load(&w->w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned t = __hip_atomic_load(&w->tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (t == dense_record_tag(a, b, c, d, e)) {
+      out[0] = __uint_as_float(a); out[1] = __uint_as_float(b); out[2] = __uint_as_float(c);
+      out[3] = __uint_as_float(d); out[4] = __uint_as_float(e);
+      return true;
+    }
+    __builtin_amdgcn_s_sleep(4);
+  }
+  return false;
+}
+
+template <int KIND, class TagS, class TagT, int NT, int NU, bool RETRY>
+__device__ __forceinline__ void dense_split_part(const DenseParams& p, const DenseSplit& x, int64_t r, int h, float* red,
+                                                 float (*xch)[DENSE_MAX_PARTS], int* xok) {
+  static_assert(KIND == DL_FKL || KIND == DL_RKL, "JSD rows are not cut into parts");
+  const int tid = threadIdx.x;
+  const int P = x.parts;
+  const int64_t u0 = (int64_t)h * NT * NU;                             // first unit of this part
+  const int64_t nu = min((int64_t)NT * NU, p.V / 8 - u0);               // its units
+  char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + (r * p.grad_stride + u0 * 8) * TagS::bytes : nullptr;
+  const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
+  if (trow < 0) {
+    if (grow) zero_row<TagS, NT>(grow, nu * 8 / TagS::epc);
+    if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = 0.f;
+    return;
+  }
+  using Rows = RegRows<TagS, TagT, NT, NU>;
+  Rows rows;
+  rows.load(reinterpret_cast<const char*>(p.logits) + (r * p.row_stride + u0 * 8) * TagS::bytes,
+            reinterpret_cast<const char*>(p.t_logits) + (trow * p.t_stride + u0 * 8) * TagT::bytes, nu);
+  const float a_s = p.inv_T_s * LOG2E, a_t = p.inv_T_t * LOG2E;
+  float ms = -INFINITY, mt = -INFINITY;
+  bool have = false;
+  if constexpr (KIND != DL_RKL && Rows::RAW_MAXIMA) have = rows.raw_maxima(ms, mt, red);
+  if (!have) {
+    rows.sweep([&](int64_t, const float* s, const float* t) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        mt = fmaxf(mt, t[e]);
+        ms = fmaxf(ms, (KIND == DL_RKL && t[e] == -INFINITY) ? -INFINITY : s[e]);
+      }
+    });
+    block_max2<NT>(ms, mt, red);
+  }
+  // a part that holds no finite logit (a masked stretch of the vocabulary): bias 0 keeps 2^(-inf - bias) = 0
+  const float bs = ms == -INFINITY ? 0.f : ms * a_s, bt = mt == -INFINITY ? 0.f : mt * a_t;
+  float ss = 0.f, stt = 0.f, w = 0.f;
+  rows.sweep([&](int64_t, const float* s, const float* t) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float xs = fmaf(s[e], a_s, -bs), xt = fmaf(t[e], a_t, -bt);
+      const float es = fast_exp2(xs), et = fast_exp2(xt);
+      stt += et;
+      if (KIND == DL_RKL) {
+        const bool on = t[e] != -INFINITY;
+        ss += on ? es : 0.f;
+        w += (on && es > 0.f) ? es * (xs - xt) : 0.f;
+      } else {
+        ss += es;
+        w += et > 0.f ? et * (xt - xs) : 0.f;
+      }
+    }
+  });
+  block_sum3<NT>(ss, stt, w, red);
+
+  DenseRecord* ws = x.records + r * P;
+  if (tid == 0 && !RETRY) dense_record_publish(ws + h, ms, mt, ss, stt, w);
+  if (tid < P) {
+    float rec[5] = {ms, mt, ss, stt, w};
+    const int ok = (tid == h) || dense_record_collect(ws + tid, RETRY ? 0x7fffffff : x.spin_limit, rec);
+#pragma unroll
+    for (int k = 0; k < 5; ++k) xch[k][tid] = rec[k];
+    xok[tid] = ok;
+  }
+  __syncthreads();
+  bool all_ok = true;
+  for (int j = 0; j < P; ++j) all_ok = all_ok && (xok[j] != 0);
+  if (!all_ok) {
+    if (tid == 0) x.retry_list[atomicAdd(x.retry_count, 1u)] = (unsigned)(r * P + h);
+    return;
+  }
+  // the row's statistics from the parts', in part order (the same bits in every part)
+  float Ms = xch[0][0], Mt = xch[1][0];
+  for (int j = 1; j < P; ++j) { Ms = fmaxf(Ms, xch[0][j]); Mt = fmaxf(Mt, xch[1][j]); }
+  float S = 0.f, T = 0.f, W = 0.f;
+  for (int j = 0; j < P; ++j) {
+    const float pms = xch[0][j], pmt = xch[1][j], pss = xch[2][j], pst = xch[3][j], pw = xch[4][j];
+    // shifts of the part's biases to the row's (log2 domain, >= 0); a part without a finite maximum summed nothing on that side
+    const float ds = pms == -INFINITY ? 0.f : (Ms - pms) * a_s, dt = pmt == -INFINITY ? 0.f : (Mt - pmt) * a_t;
+    const float fs = fast_exp2(-ds), ft = fast_exp2(-dt);
+    if (KIND == DL_FKL) W += ft * (pw - (dt - ds) * pst);
+    else W += fs * (pw - (ds - dt) * pss);
+    S += pss * fs;
+    T += pst * ft;
+  }
+  DenseStats st;
+  st.a_s = a_s; st.a_t = a_t;
+  const float l2s = fast_log2(S), l2t = fast_log2(T);
+  st.ls = (Ms == -INFINITY ? 0.f : Ms * a_s) + l2s;
+  st.lt = (Mt == -INFINITY ? 0.f : Mt * a_t) + l2t;
+  st.loss = (KIND == DL_FKL ? W / T - l2t + l2s : W / S - l2s + l2t) * LN2;
+  st.aux = st.loss;
+  st.tmax = Mt;
+  if (tid == 0 && h == 0 && p.row_loss) p.row_loss[r] = st.loss;
+  if (grow) dense_grad_sweep<KIND, TagS>(rows, st, p.inv_T_s * p.grad_scale, grow);
+}
+
+template <int KIND, class TagS, class TagT, int NT, int NU>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+void dense_split_kernel(const DenseParams p, const DenseSplit x) {
+  __shared__ float red[64];
+  __shared__ float xch[5][DENSE_MAX_PARTS];
+  __shared__ int xok[DENSE_MAX_PARTS];
+  const unsigned P = (unsigned)x.parts;
+  const unsigned grp = blockIdx.x / (8u * P), t_in = blockIdx.x % (8u * P);
+  const int64_t r = (int64_t)grp * 8 + (t_in & 7u);
+  if (r >= p.n_rows) return;
+  dense_split_part<KIND, TagS, TagT, NT, NU, false>(p, x, r, (int)(t_in >> 3), red, xch, xok);
+}
+
+// One listed part, as a real call: the loop around it then costs the body no registers.
+template <int KIND, class TagS, class TagT, int NT, int NU>
+__device__ __attribute__((noinline)) void dense_split_part_again(const DenseParams& p, const DenseSplit& x, unsigned at, float* red,
+                                                                 float (*xch)[DENSE_MAX_PARTS], int* xok) {
+  dense_split_part<KIND, TagS, TagT, NT, NU, true>(p, x, (int64_t)(at / (unsigned)x.parts), (int)(at % (unsigned)x.parts), red, xch, xok);
+}
+
+// The parts that gave up waiting, a fixed grid striding over their list (normally empty).
+template <int KIND, class TagS, class TagT, int NT, int NU>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+void dense_split_retry_kernel(const DenseParams p, const DenseSplit x) {
+  __shared__ float red[64];
+  __shared__ float xch[5][DENSE_MAX_PARTS];
+  __shared__ int xok[DENSE_MAX_PARTS];
+  const unsigned n = *x.retry_count;
+#pragma unroll 1
+  for (unsigned e = blockIdx.x; e < n; e += gridDim.x) {
+    dense_split_part_again<KIND, TagS, TagT, NT, NU>(p, x, x.retry_list[e], red, xch, xok);
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(256) void dense_clear_kernel(u32x4* ws, int64_t n16) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) ws[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
+// Units per thread of the split kernels for a dtype pair (0: the pair has no register kernel).
+static int dense_split_units(int s_dtype, int t_dtype) {
+  if (s_dtype == t_dtype) return s_dtype == F32 ? 4 : 8;
+  return t_dtype == F32 ? 4 : 0;
+}
+// How a row of V columns is cut: threads per part and parts (parts == 0: not cut).  Parts of 512 threads:
+// measured (forward KL, 512 and 8192 rows, fp32 pairs of 32000 to 131072 and bf16 pairs of 65536 to 262144
+// columns) they are level with or ahead of twice as many parts of 256 threads (half as many partners to wait
+// for; 8 parts of 256 lose even against one workgroup per row), and ahead of one workgroup per row except for
+// two parts on a few hundred rows.  `forced_nt` (256 / 512, a tuning hook) fixes the thread count and cuts
+// wherever two parts or more come out.
+struct DenseCut { int nt, parts; };
+static DenseCut dense_split_cut(int kind, int s_dtype, int t_dtype, int64_t n_rows, int64_t V, int forced_nt = 0) {
+  const int nu = dense_split_units(s_dtype, t_dtype);
+  if (kind == DL_JSD || nu == 0 || V % 8 != 0) return {0, 0};
+  const int64_t units = V / 8;
+  const int64_t p256 = (units + 256 * nu - 1) / (256 * nu), p512 = (units + 512 * nu - 1) / (512 * nu);
+  if (forced_nt == 256) return p256 >= 2 && p256 <= DENSE_MAX_PARTS ? DenseCut{256, (int)p256} : DenseCut{0, 0};
+  if (forced_nt == 512) return p512 >= 2 && p512 <= DENSE_MAX_PARTS ? DenseCut{512, (int)p512} : DenseCut{0, 0};
+  if (p512 < 2 || p512 > DENSE_MAX_PARTS) return {0, 0};
+  if (p512 == 2 && n_rows < 1024) return {0, 0};
+  return {512, (int)p512};
+}
+
+template <int KIND, class TagS, class TagT, int NT, int NU>
+static void launch_dense_split_kind(const DenseParams& p, const DenseSplit& x, hipStream_t st) {
+  const int64_t n16 = p.n_rows * x.parts * 2 + 1;      // records, then the retry counter
+  hipLaunchKernelGGL(dense_clear_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, st,
+                     reinterpret_cast<u32x4*>(x.records), n16);
+  hipLaunchKernelGGL((dense_split_kernel<KIND, TagS, TagT, NT, NU>), dim3((unsigned)((p.n_rows + 7) / 8 * 8 * x.parts)),
+                     dim3(NT), 0, st, p, x);
+  hipLaunchKernelGGL((dense_split_retry_kernel<KIND, TagS, TagT, NT, NU>),
+                     dim3((unsigned)std::min<int64_t>(p.n_rows * x.parts, 256)), dim3(NT), 0, st, p, x);
+}
+template <class TagS, class TagT, int NU>
+static void launch_dense_split(const DenseParams& p, const DenseSplit& x, int nt, hipStream_t st) {
+  if (nt == 256) {
+    if (p.kind == DL_FKL) launch_dense_split_kind<DL_FKL, TagS, TagT, 256, NU>(p, x, st);
+    else launch_dense_split_kind<DL_RKL, TagS, TagT, 256, NU>(p, x, st);
+  } else {
+    if (p.kind == DL_FKL) launch_dense_split_kind<DL_FKL, TagS, TagT, 512, NU>(p, x, st);
+    else launch_dense_split_kind<DL_RKL, TagS, TagT, 512, NU>(p, x, st);
+  }
+}
+static void launch_dense_split_pair(const DenseParams& p, const DenseSplit& x, int nt, hipStream_t st) {
+  if (p.s_dtype == F32 && p.t_dtype == F32) launch_dense_split<TagF32, TagF32, 4>(p, x, nt, st);
+  else if (p.s_dtype == BF16 && p.t_dtype == BF16) launch_dense_split<TagBF16, TagBF16, 8>(p, x, nt, st);
+  else if (p.s_dtype == F16 && p.t_dtype == F16) launch_dense_split<TagF16, TagF16, 8>(p, x, nt, st);
+  else if (p.s_dtype == BF16 && p.t_dtype == F32) launch_dense_split<TagBF16, TagF32, 4>(p, x, nt, st);
+  else launch_dense_split<TagF16, TagF32, 4>(p, x, nt, st);
 }
 
 // Rows too wide for the registers, 16-byte aligned: the same sweeps, every one of them over global
@@ -424,10 +705,28 @@ static bool launch_dense_pair(const DenseParams& p, hipStream_t st) {
 
 }  // namespace dl
 
+extern "C" int64_t dl_div_dense_workspace_bytes(int kind, int logits_dtype, int t_dtype, int64_t n_rows, int64_t V) {
+  if (n_rows <= 0 || V <= 0) return 0;
+  // enough for every cut the flags of dl_div_dense_ws may ask for
+  int parts = 0;
+  for (int nt : {0, 256, 512}) parts = std::max(parts, dl::dense_split_cut(kind, logits_dtype, t_dtype, n_rows, V, nt).parts);
+  return parts ? dl::DenseSplit::bytes(n_rows, parts) : 0;
+}
+
 extern "C" int dl_div_dense(int kind, const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
                             int64_t V, const int32_t* row_map, const void* t_logits, int t_dtype, int64_t t_stride,
                             int64_t n_teacher_rows, float inv_T_student, float inv_T_teacher, float grad_scale,
                             float* row_loss, void* grad, int64_t grad_stride, void* stream) {
+  return dl_div_dense_ws(kind, logits, logits_dtype, row_stride, n_rows, V, row_map, t_logits, t_dtype, t_stride,
+                         n_teacher_rows, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride, nullptr, 0, 0,
+                         stream);
+}
+
+extern "C" int dl_div_dense_ws(int kind, const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
+                               int64_t V, const int32_t* row_map, const void* t_logits, int t_dtype, int64_t t_stride,
+                               int64_t n_teacher_rows, float inv_T_student, float inv_T_teacher, float grad_scale,
+                               float* row_loss, void* grad, int64_t grad_stride, void* workspace, int64_t workspace_bytes,
+                               int flags, void* stream) {
   using namespace dl;
   if (!logits || (!t_logits && n_teacher_rows > 0)) return DL_ERR_NULL;      // no teacher rows: every row is masked
   if (kind < DL_FKL || kind > DL_JSD || logits_dtype < DL_F32 || logits_dtype > DL_F16 || t_dtype < DL_F32 ||
@@ -449,6 +748,15 @@ extern "C" int dl_div_dense(int kind, const void* logits, int logits_dtype, int6
   const bool elem = reinterpret_cast<uintptr_t>(logits) % sb == 0 && reinterpret_cast<uintptr_t>(t_logits) % tb == 0 &&
                     (!grad || reinterpret_cast<uintptr_t>(grad) % sb == 0);
   if (!elem) return DL_ERR_ALIGN;
+  // rows cut into column parts, where a workspace for their exchange came along
+  const int hook = (flags >> DL_TOPK_PARTS_SHIFT) & 15;      // 1 / 2: parts of 256 / 512 threads wherever the row can be cut
+  const DenseCut cut = vec ? dense_split_cut(kind, logits_dtype, t_dtype, n_rows, V, hook == 1 ? 256 : hook == 2 ? 512 : 0) : DenseCut{0, 0};
+  if (cut.parts && workspace && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+      workspace_bytes >= DenseSplit::bytes(n_rows, cut.parts) && n_rows * cut.parts <= 0x7fffffffLL) {
+    const DenseSplit x(workspace, n_rows, cut.parts, (flags & DL_TOPK_NO_WAIT) ? 0 : DENSE_SPIN_LIMIT);
+    launch_dense_split_pair(p, x, cut.nt, st);
+    return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+  }
   if (!(vec ? launch_dense_pair(p, st) : launch_dense_any_pair(p, st)))
     hipLaunchKernelGGL((dense_stream_kernel<1024>), dim3((unsigned)n_rows), dim3(1024), 0, st, p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;

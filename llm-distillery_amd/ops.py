@@ -184,9 +184,12 @@ def div_topk_static(kind: str, logits: torch.Tensor, t_val: torch.Tensor, t_idx:
 
 def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_map: torch.Tensor | None = None,
               T: float = 1.0, teacher_T: float | None = None, grad_scale: float = 1.0, want_grad: bool = True,
-              grad_out: torch.Tensor | None = None):
+              grad_out: torch.Tensor | None = None, split: bool = True, no_wait: bool = False, part_threads: int = 0):
     """Per-token "fkl", "rkl" or "jsd" against a dense teacher [N, V] and, in the same launch,
-    d(sum of row losses)/d(logits) * grad_scale.  Returns (row_loss fp32 [rows], grad or None)."""
+    d(sum of row losses)/d(logits) * grad_scale.  Returns (row_loss fp32 [rows], grad or None).
+    `split=False` withholds the workspace that lets wide forward / reverse-KL rows be cut into column parts
+    (dl_div_dense_ws); `no_wait` and `part_threads` (256 / 512) are the library's test hooks for those parts
+    (DL_TOPK_NO_WAIT, DL_TOPK_PARTS)."""
     if kind not in KINDS:
         raise ValueError("kind must be 'fkl', 'rkl' or 'jsd'")
     _dev(logits, "logits")
@@ -208,12 +211,17 @@ def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_ma
     if want_grad:
         grad = _grad_target(grad_out, R, V, x.dtype, dev)
         g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
+    lib = _lib.load()
+    ws_bytes = lib.dl_div_dense_workspace_bytes(KINDS[kind], _DT[x.dtype], _DT[t.dtype], R, V) if split else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     with torch.cuda.device(dev):
-        st = _lib.load().dl_div_dense(KINDS[kind], x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr,
-                                      t.data_ptr(), _DT[t.dtype], t.stride(0), N, 1.0 / T,
-                                      1.0 / (T if teacher_T is None else teacher_T), grad_scale,
-                                      row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
-    _lib.check(st, "dl_div_dense")
+        st = lib.dl_div_dense_ws(KINDS[kind], x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr,
+                                 t.data_ptr(), _DT[t.dtype], t.stride(0), N, 1.0 / T,
+                                 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
+                                 row_loss.data_ptr(), g_ptr, g_stride, ws.data_ptr() if ws is not None else 0, ws_bytes,
+                                 (_lib.DL_TOPK_NO_WAIT if no_wait else 0) |
+                                 ({0: 0, 256: 1, 512: 2}[part_threads] << _lib.DL_TOPK_PARTS_SHIFT), _stream_ptr(dev))
+    _lib.check(st, "dl_div_dense_ws")
     if grad is not None and logits.dim() != 2 and grad_out is None:
         grad = grad.view(logits.shape)
     return row_loss, grad

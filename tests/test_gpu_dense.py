@@ -17,7 +17,7 @@ def D():
     return d
 
 
-def _check(D, kind, logits, t_logits, T, valid=None, teacher_T=None):
+def _check(D, kind, logits, t_logits, T, valid=None, teacher_T=None, **hooks):
     R, V = logits.shape
     n_valid = R if valid is None else int(valid.sum())
     loss64, rows64, grad64 = O.mean_loss_and_grad(kind, logits, T, t_logits=t_logits, valid=valid, t_T=teacher_T,
@@ -28,7 +28,7 @@ def _check(D, kind, logits, t_logits, T, valid=None, teacher_T=None):
         rm[valid] = torch.arange(n_valid, dtype=torch.int32)
         row_map = rm.to(DEV)
     rl, grad = D.div_dense(kind, logits.to(DEV), t_logits.to(DEV), row_map=row_map, T=T, teacher_T=teacher_T,
-                           grad_scale=1.0 / n_valid)
+                           grad_scale=1.0 / n_valid, **hooks)
     loss = D.reduce_sum(rl, 1.0 / n_valid).item()
     rows = rl.cpu()
     g = grad.cpu()
@@ -274,6 +274,67 @@ def test_reverse_kl_with_student_logits_of_minus_infinity(D, dtype, V):
         fd = (O.rev_kl_dense_rows(hi[None] / 1.5, t[r:r + 1].double()) - O.rev_kl_dense_rows(lo[None] / 1.5, t[r:r + 1].double())).item() / (2 * eps)
         tol = (1e-4 if dtype == torch.float32 else 2e-3 + 2.0 ** -8) * abs(fd) + 2e-9
         assert abs(g[r, j].item() - fd) <= tol, (r, j, g[r, j].item(), fd)
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl"])
+@pytest.mark.parametrize("dtype,t_dtype,V,threads", [
+    (torch.float32, torch.float32, 32000, 256),      # 4 parts of 256 x 4 units (the last one partly filled)
+    (torch.float32, torch.float32, 32000, 512),      # 2 parts of 512 x 4
+    (torch.bfloat16, torch.bfloat16, 32000, 256),    # 2 parts of 256 x 8
+    (torch.bfloat16, torch.bfloat16, 128256, 0),     # the library's choice: 4 parts of 512 x 8
+    (torch.bfloat16, torch.bfloat16, 128256, 256),   # 8 parts
+    (torch.float16, torch.float16, 65536, 256),      # 4 full parts
+    (torch.float16, torch.float16, 262144, 0),       # 8 full parts of 512 x 8
+    (torch.bfloat16, torch.float32, 50264, 256),     # mixed pair: 7 parts of 8192 columns
+    (torch.float16, torch.float32, 8200, 256),       # one column chunk more than a part holds
+    (torch.float16, torch.float32, 40000, 0),        # mixed pair, 3 parts of 512 x 4
+    (torch.float32, torch.float32, 65536, 0)])       # 4 full parts of 512 x 4
+def test_rows_cut_into_column_parts(D, kind, dtype, t_dtype, V, threads):
+    """dl_div_dense_ws: wide forward / reverse-KL rows cut into parts of 256 threads that exchange their maxima
+    and sums through the workspace.  Both forms against the oracle, the row losses of the two against each other
+    (the same numbers to fp32 rounding), with parts that do
+    not wait for their partners (the second launch finishes them: the same bits), twice (the same bits), with
+    masked rows, and with the gradient written over the logits."""
+    s, t = _pair(13, V, dtype, 31, t_dtype, noise=1.5, std=3.0)
+    valid = torch.ones(13, dtype=torch.bool)
+    valid[[0, 6]] = False
+    _check(D, kind, s, t[valid], 1.3, valid=valid, teacher_T=1.0, part_threads=threads)
+    _check(D, kind, s, t[valid], 1.3, valid=valid, teacher_T=1.0, split=False)
+    rm = torch.full((13,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(11, dtype=torch.int32)
+    xs, xt, rm = s.to(DEV), t[valid].to(DEV), rm.to(DEV)
+    kw = dict(row_map=rm, T=1.3, teacher_T=1.0, grad_scale=1.0 / 11, part_threads=threads)
+    assert D._lib.load().dl_div_dense_workspace_bytes(D.ops.KINDS[kind], D.ops._DT[dtype], D.ops._DT[t_dtype], 13, V) > 0
+    rl, g = D.div_dense(kind, xs, xt, **kw)
+    rl2, g2 = D.div_dense(kind, xs, xt, **kw)
+    rl3, g3 = D.div_dense(kind, xs, xt, no_wait=True, **kw)
+    assert torch.equal(rl, rl2) and torch.equal(g, g2) and torch.equal(rl, rl3) and torch.equal(g, g3)
+    rl1, _ = D.div_dense(kind, xs, xt, split=False, row_map=rm, T=1.3, teacher_T=1.0, grad_scale=1.0 / 11)
+    np.testing.assert_allclose(rl.cpu().numpy(), rl1.cpu().numpy(), rtol=2e-6, atol=1e-7)
+    for no_wait in (False, True):
+        y = xs.clone()
+        rl4, g4 = D.div_dense(kind, y, xt, grad_out=y, no_wait=no_wait, **kw)
+        assert g4.data_ptr() == y.data_ptr() and torch.equal(rl, rl4) and torch.equal(g, y)
+
+
+@pytest.mark.parametrize("kind", ["fkl", "rkl"])
+def test_a_column_part_without_teacher_mass_or_without_student_mass(D, kind):
+    """Whole column parts of -inf: a teacher that masks a stretch of the vocabulary as wide as a part (no
+    support there for reverse KL, no mass for forward KL), and a student that masks another one where the
+    teacher has none either.  The parts' records then carry -inf maxima; the row's statistics come from the
+    other parts and the masked columns get zero gradient."""
+    R, V = 5, 32768                                          # four parts of 8192 fp32 columns
+    s, t = _pair(R, V, torch.float32, 41, noise=1.5, std=3.0)
+    t[:, 8192:16384] = -float("inf")                          # part 1: no teacher mass
+    t[:, 24576:] = -float("inf")
+    s[:, 24576:] = -float("inf")                              # part 3: neither
+    _check(D, kind, s, t, 1.1, part_threads=256)
+    rl, g = D.div_dense(kind, s.to(DEV), t.to(DEV), T=1.1, part_threads=256)
+    rl2, g2 = D.div_dense(kind, s.to(DEV), t.to(DEV), T=1.1, no_wait=True, part_threads=256)
+    assert torch.isfinite(rl).all() and torch.isfinite(g).all() and torch.equal(rl, rl2) and torch.equal(g, g2)
+    assert torch.count_nonzero(g[:, 24576:]) == 0
+    if kind == "rkl":
+        assert torch.count_nonzero(g[:, 8192:16384]) == 0
 
 
 def test_synthetic_configs_1_and_2_at_reduced_rows(D):
