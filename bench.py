@@ -380,13 +380,32 @@ def cpu_baseline(workload: str, rows: int, reps: int):
                       f"os.cpu_count()={os.cpu_count()})"}
 
 
+def kernel_source_hash() -> str:
+    """sha256 over the kernel sources and the C header, in path order: what the counter summaries were taken on."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(ROOT, "llm-distillery_amd", "csrc", "*")) + glob.glob(os.path.join(ROOT, "include", "*.h")))
+    for path in files:
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(workload: str):
-    """HBM bytes per launch from the committed rocprofv3 counter summary, if present."""
+    """HBM bytes per launch of this workload from the committed rocprofv3 counter summary -- a figure measured
+    in an earlier profiled run of this same command, not in this run (the counters need the profiler) -- and
+    only while the kernel sources are still the ones it was measured on (their hash is stored beside it):
+    after any change to the kernels it reads null until the counter runs are repeated."""
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            return json.load(f).get(f"{workload}_bytes_per_launch")
+            rec = json.load(f)
     except (OSError, ValueError):
         return None
+    if rec.get("kernel_source_hash") != kernel_source_hash():
+        return None
+    return rec.get(f"{workload}_bytes_per_launch")
 
 
 def main():
@@ -413,11 +432,16 @@ def main():
     ap.add_argument("--pitch", type=int, default=0, help="c3: columns per stored row, >= --vocab: the logits are the crop "
                     "[:, :vocab] of such rows")
     ap.add_argument("--no-split", action="store_true", help="c1 / dense: one workgroup per row pair (no workspace)")
+    ap.add_argument("--source-hash", action="store_true", help="print the hash of the kernel sources (the value "
+                    "profiles/traffic.json carries as kernel_source_hash) and exit")
     ap.add_argument("--inplace", action="store_true",
                     help="c3 only: write the gradient over the logits (same DRAM pages: about 4 %% faster).  After the "
                          "first step the buffer holds gradients, not logits, so the printed loss means nothing; the "
                          "traffic and the arithmetic per step are unchanged.  Not the default for that reason")
     args = ap.parse_args()
+    if args.source_hash:
+        print(kernel_source_hash())
+        return
     global INPLACE, PARTS
     global VOCAB, PITCH, NO_SPLIT
     NO_SPLIT = args.no_split
@@ -474,6 +498,8 @@ def main():
         "loss": loss.item(),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload),
+                     "traffic_from": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, committed; "
+                                     "null when the kernel sources have changed since)",
                      "kernel": kernel, "kernel_ms": kern_ms, "algorithmic_bytes": algo_bytes},
         "cpu_baseline": cpu_baseline(args.workload, cpu_rows, 7 if args.workload == "c3" else 3) if cpu_rows > 0 else None,
     }

@@ -346,44 +346,89 @@ def _offsets_arg(offsets):
     return (arr(*offsets[0]), arr(*offsets[1]), arr(*offsets[2])), 1, C
 
 
+def _composite_forward_raw(logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T, inv_T_teacher, alpha, crop, need_grad):
+    """Phase 1 over the logits + the K-wide epilogue: (nine values [C, 9], lse, zk, rec, coef or None)."""
+    x = _cropped(logits, crop)
+    dev = x.device
+    R, V = x.shape
+    N, K = t_idx.shape
+    lib = _lib.load()
+    offs, on_host, C = _offsets_arg(offsets)
+    if not on_host:      # with offsets on the device the library cannot see that a list is empty and wants both pointers
+        labels = labels if labels.numel() else torch.zeros(1, dtype=torch.int64, device=dev)
+        avoid = avoid if avoid.numel() else torch.zeros(1, dtype=avoid.dtype, device=dev)
+    # every teacher row is written by phase 1 unless a row map leaves some out or teacher rows outnumber the logits rows
+    make = torch.empty if row_map is None and N == R else torch.zeros
+    lse = make(N, dtype=torch.float32, device=dev)
+    zk = make((N, K), dtype=torch.float32, device=dev)
+    rec = torch.empty((N, 8), dtype=torch.float32, device=dev)
+    coef = torch.empty((N, 4), dtype=torch.float32, device=dev) if need_grad else None
+    out = torch.empty((C, 9), dtype=torch.float32, device=dev)
+    rm_ptr = row_map.data_ptr() if row_map is not None else 0
+    stream = _stream_ptr(dev)
+    with torch.cuda.device(dev):
+        st = lib.dl_rowstats_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(), _IT[t_idx.dtype],
+                                  K, N, inv_T, lse.data_ptr(), zk.data_ptr(), stream)
+        _lib.check(st, "dl_rowstats_topk")
+        st = lib.dl_composite_forward(
+            lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
+            _IT[t_idx.dtype], K, labels.data_ptr() if labels.numel() else 0, avoid.data_ptr() if avoid.numel() else 0,
+            _IT[avoid.dtype], offs[0], offs[1], offs[2], on_host, C, N, alpha, rec.data_ptr(),
+            coef.data_ptr() if need_grad else 0, out.data_ptr(), stream)
+        _lib.check(st, "dl_composite_forward")
+    return out, lse, zk, rec, coef
+
+
+def _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, offsets, row_map, inv_T, inv_T_teacher, crop):
+    """The epilogue's backward + phase 2: d(sum_c g_train[c] * train_loss[c]) / d logits, full width."""
+    x = _cropped(logits, crop)
+    dev = x.device
+    R, V = x.shape
+    N, K = t_idx.shape
+    lib = _lib.load()
+    offs, on_host, C = _offsets_arg(offsets)
+    g = g_train.to(torch.float32).contiguous()
+    g_lse = torch.empty_like(lse)
+    g_zk = torch.empty_like(zk)
+    grad = torch.empty_like(logits)                      # full width; the kernel fills [:, :crop]
+    if x is not logits:
+        grad[:, crop:].zero_()
+    gx = _cropped(grad, crop)
+    stream = _stream_ptr(dev)
+    with torch.cuda.device(dev):
+        st = lib.dl_composite_backward(
+            lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
+            _IT[t_idx.dtype], K, offs[0], on_host, C, N, rec.data_ptr(), coef.data_ptr(), g.data_ptr(),
+            g_lse.data_ptr(), g_zk.data_ptr(), stream)
+        _lib.check(st, "dl_composite_backward")
+        st = lib.dl_rowcoef_grad_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V,
+                                      row_map.data_ptr() if row_map is not None else 0, t_idx.data_ptr(),
+                                      _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), g_lse.data_ptr(), g_zk.data_ptr(),
+                                      gx.data_ptr(), gx.stride(0), stream)
+        _lib.check(st, "dl_rowcoef_grad_topk")
+    return grad
+
+
 class _CompositeLoss(torch.autograd.Function):
     """The reference's composite loss of C conversations as ONE autograd node: phase 1 over the logits
     (dl_rowstats_topk), the K-wide epilogue (dl_composite_forward), and in backward their two
     counterparts (dl_composite_backward, dl_rowcoef_grad_topk).  Returns (train_loss [C], the nine
-    values [C, 9]); only train_loss is differentiable, and only with respect to the logits."""
+    values [C, 9]); only train_loss is differentiable, and only with respect to the logits.
+    The eager path goes through this class rather than through the registered ops below (which run the
+    same launches): a call through the dispatcher costs tens of microseconds of host time more, which at
+    the reference's default shape (one conversation of 2048 x 32000 logits: 0.17 ms of kernels) is what
+    decides whether the host keeps ahead of the device."""
 
     @staticmethod
     def forward(ctx, logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T: float, inv_T_teacher: float,
                 alpha: float, crop: int):
-        x = _cropped(logits, crop)
-        dev = x.device
-        R, V = x.shape
-        N, K = t_idx.shape
-        lib = _lib.load()
-        offs, on_host, C = _offsets_arg(offsets)
         need_grad = ctx.needs_input_grad[0]          # False under torch.no_grad() (the validation loop) and for detached logits
-        # every teacher row is written by phase 1 unless a row map leaves some out or teacher rows outnumber the logits rows
-        make = torch.empty if row_map is None and N == R else torch.zeros
-        lse = make(N, dtype=torch.float32, device=dev)
-        zk = make((N, K), dtype=torch.float32, device=dev)
-        rec = torch.empty((N, 8), dtype=torch.float32, device=dev)
-        coef = torch.empty((N, 4), dtype=torch.float32, device=dev) if need_grad else None
-        out = torch.empty((C, 9), dtype=torch.float32, device=dev)
-        rm_ptr = row_map.data_ptr() if row_map is not None else 0
-        stream = _stream_ptr(dev)
-        with torch.cuda.device(dev):
-            st = lib.dl_rowstats_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(), _IT[t_idx.dtype],
-                                      K, N, inv_T, lse.data_ptr(), zk.data_ptr(), stream)
-            _lib.check(st, "dl_rowstats_topk")
-            st = lib.dl_composite_forward(
-                lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
-                _IT[t_idx.dtype], K, labels.data_ptr() if labels.numel() else 0, avoid.data_ptr() if avoid.numel() else 0,
-                _IT[avoid.dtype], offs[0], offs[1], offs[2], on_host, C, N, alpha, rec.data_ptr(),
-                coef.data_ptr() if need_grad else 0, out.data_ptr(), stream)
-            _lib.check(st, "dl_composite_forward")
+        out, lse, zk, rec, coef = _composite_forward_raw(logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T,
+                                                         inv_T_teacher, alpha, crop, need_grad)
         if need_grad:
+            on_host = not isinstance(offsets, torch.Tensor)
             ctx.save_for_backward(logits, t_val, t_idx, lse, zk, rec, coef, *([row_map] if row_map is not None else []),
-                                  *([offsets] if on_host == 0 else []))
+                                  *([] if on_host else [offsets]))
             ctx.host_offsets = offsets if on_host else None
             ctx.has_map = row_map is not None
             ctx.scalars = (inv_T, inv_T_teacher, crop)
@@ -398,32 +443,65 @@ class _CompositeLoss(torch.autograd.Function):
         row_map = saved[7] if ctx.has_map else None
         offsets = ctx.host_offsets if ctx.host_offsets is not None else saved[-1]
         inv_T, inv_T_teacher, crop = ctx.scalars
-        x = _cropped(logits, crop)
-        dev = x.device
-        R, V = x.shape
-        N, K = t_idx.shape
-        lib = _lib.load()
-        offs, on_host, C = _offsets_arg(offsets)
-        g = g_train.to(torch.float32).contiguous()
-        g_lse = torch.empty_like(lse)
-        g_zk = torch.empty_like(zk)
-        grad = torch.empty_like(logits)                      # full width; the kernel fills [:, :crop]
-        if x is not logits:
-            grad[:, crop:].zero_()
-        gx = _cropped(grad, crop)
-        stream = _stream_ptr(dev)
-        with torch.cuda.device(dev):
-            st = lib.dl_composite_backward(
-                lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
-                _IT[t_idx.dtype], K, offs[0], on_host, C, N, rec.data_ptr(), coef.data_ptr(), g.data_ptr(),
-                g_lse.data_ptr(), g_zk.data_ptr(), stream)
-            _lib.check(st, "dl_composite_backward")
-            st = lib.dl_rowcoef_grad_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V,
-                                          row_map.data_ptr() if row_map is not None else 0, t_idx.data_ptr(),
-                                          _IT[t_idx.dtype], K, N, inv_T, lse.data_ptr(), g_lse.data_ptr(), g_zk.data_ptr(),
-                                          gx.data_ptr(), gx.stride(0), stream)
-            _lib.check(st, "dl_rowcoef_grad_topk")
+        grad = _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, offsets, row_map, inv_T,
+                                       inv_T_teacher, crop)
         return (grad,) + (None,) * 10
+
+
+# The same two halves as registered operators (torch.library): visible to torch.compile, FakeTensor tracing and
+# torch.library.opcheck.  The forward returns what its backward needs as extra outputs; offsets are the device form.
+@torch.library.custom_op("distillery_amd::composite_forward", mutates_args=())
+def composite_forward_op(logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor, labels: torch.Tensor,
+                         avoid: torch.Tensor, offsets: torch.Tensor, row_map: Optional[torch.Tensor], inv_T: float,
+                         inv_T_teacher: float, alpha: float, crop: int = 0
+                         ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(train_loss [C], nine values [C, 9], lse [N], zk [N, K], per-row records [N, 8], per-row coefficients [N, 4])."""
+    out, lse, zk, rec, coef = _composite_forward_raw(logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T,
+                                                     inv_T_teacher, alpha, crop, True)
+    return out[:, 0].clone(), out, lse, zk, rec, coef
+
+
+@composite_forward_op.register_fake
+def _(logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T, inv_T_teacher, alpha, crop=0):
+    N, K = t_idx.shape
+    C = offsets.shape[1] - 1
+    f32 = dict(dtype=torch.float32)
+    return (logits.new_empty((C,), **f32), logits.new_empty((C, 9), **f32), logits.new_empty((N,), **f32),
+            logits.new_empty((N, K), **f32), logits.new_empty((N, 8), **f32), logits.new_empty((N, 4), **f32))
+
+
+@torch.library.custom_op("distillery_amd::composite_backward", mutates_args=())
+def composite_backward_op(logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor, lse: torch.Tensor, zk: torch.Tensor,
+                          rec: torch.Tensor, coef: torch.Tensor, g_train: torch.Tensor, offsets: torch.Tensor,
+                          row_map: Optional[torch.Tensor], inv_T: float, inv_T_teacher: float, crop: int = 0) -> torch.Tensor:
+    return _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, offsets, row_map, inv_T, inv_T_teacher, crop)
+
+
+@composite_backward_op.register_fake
+def _(logits, t_val, t_idx, lse, zk, rec, coef, g_train, offsets, row_map, inv_T, inv_T_teacher, crop=0):
+    return torch.empty_like(logits)
+
+
+def _composite_op_setup(ctx, inputs, output):
+    logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T, inv_T_teacher, alpha, crop = inputs
+    _, _, lse, zk, rec, coef = output
+    ctx.save_for_backward(logits, t_val, t_idx, lse, zk, rec, coef, offsets, *([row_map] if row_map is not None else []))
+    ctx.has_map = row_map is not None
+    ctx.scalars = (inv_T, inv_T_teacher, crop)
+
+
+def _composite_op_backward(ctx, g_train, *_unused):
+    saved = ctx.saved_tensors
+    logits, t_val, t_idx, lse, zk, rec, coef, offsets = saved[:8]
+    row_map = saved[8] if ctx.has_map else None
+    inv_T, inv_T_teacher, crop = ctx.scalars
+    if g_train is None:
+        g_train = torch.zeros(offsets.shape[1] - 1, dtype=torch.float32, device=logits.device)
+    grad = composite_backward_op(logits, t_val, t_idx, lse, zk, rec, coef, g_train, offsets, row_map, inv_T, inv_T_teacher, crop)
+    return (grad,) + (None,) * 10
+
+
+composite_forward_op.register_autograd(_composite_op_backward, setup_context=_composite_op_setup)
 
 
 def composite_loss(logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tensor, labels: torch.Tensor,
@@ -456,6 +534,12 @@ def composite_loss(logits: torch.Tensor, t_val: torch.Tensor, t_idx: torch.Tenso
             raise RuntimeError("device offsets must be a contiguous int32 [3, C + 1] tensor")
     elif len(offsets) != 3 or len(offsets[0]) - 1 > _lib.DL_MAX_HOST_CONVOS or offsets[0][-1] != N:
         raise RuntimeError("host offsets: three lists of C + 1 entries, C <= DL_MAX_HOST_CONVOS, rows ending at N")
+    if torch.compiler.is_compiling():      # traced: the registered operators (device offsets only)
+        if not isinstance(offsets, torch.Tensor):
+            offsets = torch.tensor(offsets, dtype=torch.int32, device=dev)
+        res = composite_forward_op(logits, t_val, t_idx, labels, avoid, offsets, row_map, float(inv_T), float(inv_T_teacher),
+                                   float(alpha), int(crop))
+        return res[0], res[1].detach()
     return _CompositeLoss.apply(logits, t_val, t_idx, labels, avoid, offsets, row_map, float(inv_T), float(inv_T_teacher),
                                 float(alpha), int(crop))
 

@@ -357,6 +357,37 @@ def test_fused_epilogue_equals_the_torch_epilogue(D, alpha):
     assert torch.count_nonzero(g_fused[3]) == 0
 
 
+def test_registered_composite_operators_equal_the_eager_node(D):
+    """distillery_amd::composite_forward / composite_backward (torch.library operators with fake implementations and a
+    registered autograd formula) run the launches of the eager autograd node: the same bits forward and backward;
+    torch.library.opcheck accepts schema, fake tensors and autograd registration."""
+    from llm_distillery_amd import ops
+    g = torch.Generator().manual_seed(31)
+    S, V, K = 40, 4096, 16
+    specs, lens = [[(2, 17)], [(20, 38)]], [17, 38]
+    logits = (torch.randn(S, V, generator=g) * 2).to(torch.bfloat16).to(DEV)
+    convos = [_ranged_convo(g, S, V, K, specs[b], lens[b]) for b in range(2)]
+    rows = torch.cat([c[0] for c in convos])
+    rm = torch.full((S,), -1, dtype=torch.int32)
+    rm[rows] = torch.arange(rows.numel(), dtype=torch.int32)
+    t_val = torch.cat([c[1] for c in convos]).to(DEV)
+    t_idx = torch.cat([c[2] for c in convos]).to(torch.int32).to(DEV)
+    labels = torch.cat([c[3] for c in convos]).to(DEV)
+    avoid = torch.cat([c[4] for c in convos]).to(DEV)
+    counts = [c[0].numel() for c in convos]
+    offs = [[0, counts[0], sum(counts)], [0, convos[0][3].numel(), labels.numel()], [0, convos[0][4].numel(), avoid.numel()]]
+    offs_dev = torch.tensor(offs, dtype=torch.int32, device=DEV)
+    x1 = logits.clone().requires_grad_(True)
+    train1, nine1 = ops.composite_loss(x1, t_val, t_idx, labels, avoid, offs, rm.to(DEV), 1 / 1.3, 1 / 1.3, 2.0, 0)
+    train1.sum().backward()
+    x2 = logits.clone().requires_grad_(True)
+    res = ops.composite_forward_op(x2, t_val, t_idx, labels, avoid, offs_dev, rm.to(DEV), 1 / 1.3, 1 / 1.3, 2.0, 0)
+    res[0].sum().backward()
+    assert torch.equal(train1, res[0]) and torch.equal(nine1, res[1]) and torch.equal(x1.grad, x2.grad)
+    torch.library.opcheck(ops.composite_forward_op, (x2.detach(), t_val, t_idx, labels, avoid, offs_dev, rm.to(DEV), 1 / 1.3, 1 / 1.3, 2.0, 0),
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+
+
 def test_fused_epilogue_under_no_grad_and_label_count_mismatch(D):
     g = torch.Generator().manual_seed(5)
     rows, tv, ti, labels, avoid = _ranged_convo(g, 40, 1024, 8, [(3, 19)], 19)

@@ -160,6 +160,28 @@ def test_losses_loss_dict_is_a_plain_writable_dict_also_after_packed_additions()
         P.backward()
 
 
+def test_registered_operators_trace_with_fake_tensors():
+    """The V-wide launches are registered torch.library operators with fake (shape-only) implementations, so that
+    FakeTensor tracing / torch.compile see through them without touching a GPU."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from llm_distillery_amd import ops
+    with FakeTensorMode():
+        logits = torch.empty(10, 64, dtype=torch.bfloat16)
+        t_val = torch.empty(7, 5, dtype=torch.float16)
+        t_idx = torch.empty(7, 5, dtype=torch.int32)
+        labels = torch.empty(5, dtype=torch.int64)
+        avoid = torch.empty(1, dtype=torch.int64)
+        offsets = torch.empty(3, 3, dtype=torch.int32)                  # two conversations
+        row_map = torch.empty(10, dtype=torch.int32)
+        train, nine, lse, zk, rec, coef = ops.composite_forward_op(logits, t_val, t_idx, labels, avoid, offsets, row_map, 1.0, 1.0, 2.0, 48)
+        assert train.shape == (2,) and nine.shape == (2, 9) and lse.shape == (7,) and zk.shape == (7, 5)
+        assert rec.shape == (7, 8) and coef.shape == (7, 4) and train.dtype == torch.float32
+        grad = ops.composite_backward_op(logits, t_val, t_idx, lse, zk, rec, coef, train, offsets, row_map, 1.0, 1.0, 48)
+        assert grad.shape == logits.shape and grad.dtype == logits.dtype
+        lse2, zk2 = ops.rowstats_topk(logits, t_idx, row_map, 1.0, 48)
+        assert lse2.shape == (7,) and zk2.shape == (7, 5)
+
+
 def test_library_exports_every_symbol_the_header_declares():
     header = open(os.path.join(ROOT, "include", "distill_hip.h")).read()
     declared = set(re.findall(r"\b(dl_[a-z0-9_]+)\s*\(", header))
