@@ -139,22 +139,41 @@ def _wl_dense(kind_name):
     return build
 
 
+ALPHABET = 256         # --alphabet: byte alphabet of C5's random vocabularies (256: nearly all teacher ids fall back to the
+                       # 256 single-byte student tokens; 4-16: a flat map, thousands of student ids in use)
+STUDENT_VOCAB = 0      # --student-vocab: C5's student vocabulary (default 32000)
+UNFUSED = False        # --unfused: C5 as two launches, the marginal through memory
+
+
 def _wl_c5(D, S, dev, rows):
     import torch
     rows = rows or 2 * 4096
-    Vs, Vt = 32000, 152064
-    c = S.config5(dev, rows=rows, Vs=Vs, Vt=Vt)
+    Vs, Vt = STUDENT_VOCAB or 32000, 152064
+    c = S.config5(dev, rows=rows, Vs=Vs, Vt=Vt, alphabet=ALPHABET)
     grad = torch.empty_like(c["logits"])
     scale = 1.0 / rows
     plan = D.vocab_utils.MarginalPlan(c["t2s_host"], Vs, dev)       # built once per tokenizer pair
+    used = int(torch.unique(c["t2s"][c["t2s"] >= 0]).numel())
+    fused = not UNFUSED and plan.ent is not None
+    what = (f"C5 byte-trie marginalisation ({Vt}->{Vs}, alphabet {ALPHABET}: {used} student ids in use) + reverse-KL fwd+bwd, "
+            f"{rows} tokens, fp32 teacher softmax, bf16 student, T=1.5")
 
-    def main():
-        return D.vocab_utils.rkl_marginalised(c["logits"], c["t_probs"], plan, T=c["T"], grad_scale=scale,
-                                              grad_out=grad)[0]
+    if fused:
+        def main():
+            return D.vocab_utils.rkl_marginalised(c["logits"], c["t_probs"], plan, T=c["T"], grad_scale=scale,
+                                                  grad_out=grad)[0]
+        kernel = "rkl_marginalised_kernel<bf16> (planned marginal)"
+    else:
+        # the marginal's logarithm through memory (fp32 [rows, Vs]), then the dense reverse KL on it: what student
+        # vocabularies beyond the fused kernel's 36864 ids take
+        def main():
+            lm = D.vocab_utils.marginalise(c["t_probs"], plan=plan if plan.ent is not None else None, t2s=c["t2s"],
+                                           n_student=Vs, log=True)
+            return D.div_dense("rkl", c["logits"], lm, T=c["T"], grad_scale=scale, grad_out=grad)[0]
+        kernel = "marginalise_map_kernel + dense reverse-KL kernel (the marginal through memory)"
+        what += "; in two launches"
 
-    return (lambda: D.reduce_sum(main(), scale), main, rows * (Vt * 4 + Vs * 2 + Vs * 2) + Vt * 4, rows,
-            f"C5 byte-trie marginalisation ({Vt}->{Vs}) + reverse-KL fwd+bwd, {rows} tokens, fp32 teacher softmax, "
-            "bf16 student, T=1.5", "rkl_marginalised_kernel<bf16> (planned marginal)", c, grad)
+    return (lambda: D.reduce_sum(main(), scale), main, rows * (Vt * 4 + Vs * 2 + Vs * 2) + Vt * 4, rows, what, kernel, c, grad)
 
 
 def _wl_producer(D, S, dev, rows):
@@ -431,6 +450,9 @@ def main():
     ap.add_argument("--vocab", type=int, default=0, help="c3: vocabulary size (default 128256)")
     ap.add_argument("--pitch", type=int, default=0, help="c3: columns per stored row, >= --vocab: the logits are the crop "
                     "[:, :vocab] of such rows")
+    ap.add_argument("--alphabet", type=int, default=256, help="c5: byte alphabet of the random vocabularies (256 / 4..16)")
+    ap.add_argument("--student-vocab", type=int, default=0, help="c5: student vocabulary size (default 32000)")
+    ap.add_argument("--unfused", action="store_true", help="c5: marginalise and reverse KL as two launches")
     ap.add_argument("--no-split", action="store_true", help="c1 / dense: one workgroup per row pair (no workspace)")
     ap.add_argument("--source-hash", action="store_true", help="print the hash of the kernel sources (the value "
                     "profiles/traffic.json carries as kernel_source_hash) and exit")
@@ -443,8 +465,9 @@ def main():
         print(kernel_source_hash())
         return
     global INPLACE, PARTS
-    global VOCAB, PITCH, NO_SPLIT
+    global VOCAB, PITCH, NO_SPLIT, ALPHABET, STUDENT_VOCAB, UNFUSED
     NO_SPLIT = args.no_split
+    ALPHABET, STUDENT_VOCAB, UNFUSED = args.alphabet, args.student_vocab, args.unfused
     VOCAB, PITCH = (args.vocab, args.pitch) if args.workload == "c3" else (0, 0)
     PARTS = args.parts if args.workload == "c3" else 0
     INPLACE = bool(args.inplace and args.workload == "c3")

@@ -424,6 +424,22 @@ int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t
                        const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
                        float* marg, int64_t marg_stride, int out_log, void* stream);
 
+/*
+ * Column subsets, for student vocabularies wider than the marginal that dl_rkl_marginalised can hold (36864 ids):
+ * a teacher -> student map only ever reaches the student ids in its image, all other columns of a row lie off
+ * the marginal's support (no loss term, zero gradient), so the fused kernel can run on the image alone.
+ *   dl_gather_columns   dst[r, c] = src[r, cols[c]] for c < n_cols; cols[c] < 0 (padding) gives -inf.
+ *   dl_expand_columns   dst[r, j] = src[r, col_src[j]] for j < V; col_src[j] < 0 (a column outside the subset) gives 0.
+ * Raw 2- or 4-byte elements of `dtype`, no conversion.  cols int32 [n_cols], col_src int32 [V], both 16-byte
+ * aligned; dst rows on the 16-byte grid, n_cols (gather) / V (expand) whole 16-byte chunks (else DL_ERR_ALIGN);
+ * src rows of any stride.  n_rows <= 65535 per call.  Reference: none (serves BASELINE configuration 5 at the
+ * student vocabulary of configurations 3 and 4).
+ */
+int dl_gather_columns(const void* src, int dtype, int64_t src_stride, int64_t n_rows, int64_t V, const int32_t* cols,
+                      int64_t n_cols, void* dst, int64_t dst_stride, void* stream);
+int dl_expand_columns(const void* src, int dtype, int64_t src_stride, int64_t n_rows, int64_t n_cols,
+                      const int32_t* col_src, int64_t V, void* dst, int64_t dst_stride, void* stream);
+
 /* The same marginal from the CSR form, each segment added in ascending teacher-id order (bit-reproducible). */
 int dl_marginalise_csr(const void* probs, int p_dtype, int64_t p_stride, int64_t n_rows, int64_t Vt,
                        const int32_t* offsets, const int32_t* indices, int64_t Vs, float* marg,
@@ -445,6 +461,31 @@ int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride
                         const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
                         float inv_T_student, float inv_T_teacher, float grad_scale,
                         float* row_loss, void* grad, int64_t grad_stride, void* stream);
+
+/*
+ * dl_rkl_marginalised for a student vocabulary wider than the marginal the kernel can hold (Vs_full columns per
+ * logits / gradient row, any width): a teacher -> student map only ever reaches the student ids in its image, and
+ * every other column of a row lies off the marginal's support -- no loss term, zero gradient -- so the kernel
+ * works on the image alone.  cols int32 [n_compact] names the image's columns, ascending, padded with -1 to a
+ * multiple of 8 (n_compact <= 36864); col_src16 uint16 [Vs_full] gives every column its position in `cols`
+ * (0xffff: outside the image); t2c int32 [Vt] maps teacher ids onto positions in `cols` (negative: dropped), and the
+ * plan arrays are dl_marginal_plan_build's for (t2c, n_compact).  The kernel gathers the row's logits at `cols`
+ * while the teacher row streams in, and writes the full-width gradient row from the compact one it holds in LDS:
+ * every 16-byte chunk once.  Other arguments, conventions and results as dl_rkl_marginalised (the loss and the
+ * gradient are those of the full vocabulary).  cols / col_src16 16-byte aligned, gradient rows on the 16-byte grid,
+ * Vs_full a multiple of 8; the logits rows need element alignment only.  No counterpart in the reference
+ * (BASELINE configuration 5 at the student vocabulary of configurations 3 and 4).
+ */
+int dl_rkl_marginalised_compact(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs_full,
+                                const int32_t* cols, const uint16_t* col_src16, int64_t n_compact,
+                                const int32_t* row_map,
+                                const void* t_probs, int p_dtype, int64_t p_stride, int64_t n_teacher_rows, int64_t Vt,
+                                const int32_t* t2c,
+                                const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                                const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
+                                float inv_T_student, float inv_T_teacher, float grad_scale,
+                                float* row_loss, void* grad, int64_t grad_stride, void* stream);
+
 
 /*
  * Deterministic sum of n fp32 values times `scale` into out[0] (fixed reduction tree,

@@ -55,8 +55,13 @@ _SIGNATURES = {
     "dl_marginalise_map": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, _P, _P, c_int, _P, c_int, c_int, _P,
                                    c_int64, c_int, _P]),
     "dl_marginalise_csr": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int64, _P, c_int64, c_int, _P]),
+    "dl_gather_columns": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, _P, c_int64, _P]),
+    "dl_expand_columns": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, _P, c_int64, _P]),
     "dl_rkl_marginalised": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int, c_int64, c_int64, c_int64, _P,
                                     _P, _P, c_int, _P, c_int, c_int, c_float, c_float, c_float, _P, _P, c_int64, _P]),
+    "dl_rkl_marginalised_compact": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, c_int64, _P, _P, c_int, c_int64,
+                                            c_int64, c_int64, _P, _P, _P, c_int, _P, c_int, c_int, c_float, c_float, c_float,
+                                            _P, _P, c_int64, _P]),
     "dl_composite_forward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, _P, c_int, _P, _P, _P, c_int, c_int,
                                      c_int64, c_float, _P, _P, _P, _P]),
     "dl_composite_backward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, c_int, c_int, c_int64, _P, _P, _P, _P,

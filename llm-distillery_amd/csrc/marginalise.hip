@@ -40,6 +40,10 @@ struct MargParams {
   // plan (all NULL/0: accumulate with LDS atomics along t2s instead)
   const int32_t* plan_row_off; const uint32_t* plan_ent; int plan_tile;
   const int32_t* plan_fold; int plan_n_fold; int plan_n_extra;       // replica slots behind the marginal and how they fold
+  // compact form of the fused reverse KL (Vs_full > 0): Vs counts the student ids the map reaches, `cols` [Vs] names
+  // their columns in the logits rows of Vs_full columns (-1: padding), col_src16 [Vs_full] the compact id of every
+  // column (0xffff: none); logits and gradient rows are full-width
+  const int32_t* cols; const unsigned short* col_src16; int64_t Vs_full;
 };
 
 // LDS words of the planned form behind the tile: the marginal and the replica slots, both padded to
@@ -336,6 +340,25 @@ __global__ __launch_bounds__(256) void marginalise_csr_kernel(const void* probs,
 
 // ---- fused: marginal in LDS -> reverse KL against the student row in registers -----------------
 // The student row of the fused kernel: NU units of 8 columns per thread, in registers.
+// Unit u of a compacted student row: the raw elements at columns cols[8u .. 8u + 7] of the full-width row.
+template <class TagS>
+__device__ __forceinline__ void gather_unit(Unit<TagS>& x, const char* srow, const int32_t* cols, int64_t u) {
+  const int4 a = *reinterpret_cast<const int4*>(cols + u * 8), b = *reinterpret_cast<const int4*>(cols + u * 8 + 4);
+  const int id[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  if constexpr (TagS::bytes == 4) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x.c[e >> 2][e & 3] = id[e] >= 0 ? reinterpret_cast<const unsigned*>(srow)[id[e]] : 0xff800000u;
+  } else {
+    const u32x4 ninf = Chunk<TagS>::neg_inf();
+    unsigned h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      h[e] = id[e] >= 0 ? (unsigned)reinterpret_cast<const unsigned short*>(srow)[id[e]] : (ninf[0] & 0xffffu);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) x.c[0][d] = h[2 * d] | (h[2 * d + 1] << 16);
+  }
+}
+
 template <class TagS, int NU>
 struct StudentRow {
   Unit<TagS> s[NU];
@@ -346,6 +369,15 @@ struct StudentRow {
     for (int i = 0; i < NU; ++i) {
       const int64_t u = (int64_t)i * MARG_NT + threadIdx.x;
       if (u < nunits) s[i].load(srow, u); else s[i].fill_neg_inf();
+    }
+  }
+  // The same from a full-width row, unit u = the logits at columns cols[8u .. 8u + 7] (-inf for a column of -1).
+  __device__ __forceinline__ void load_gathered(const char* srow, const int32_t* cols, int64_t nu) {
+    nunits = nu;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int64_t u = (int64_t)i * MARG_NT + threadIdx.x;
+      if (u < nunits) gather_unit<TagS>(s[i], srow, cols, u); else s[i].fill_neg_inf();
     }
   }
 };
@@ -455,9 +487,21 @@ __device__ __forceinline__ void rkl_sums_stash(Unit<TagS> (&s)[NU], int64_t nuni
 // The gradient from what rkl_sums_stash left: 2^(xs + B) * (k1 (xs - xt) - k1 wbar), k1 over the sum
 // that carries the same 2^B.  The factor is held finite (a column off the support stores 1e30 for its
 // difference), so that 0 * factor is 0.
+// COMPACT rows leave the gradient of unit u, as fp32, where its differences stood (marg[8u .. 8u + 7], the thread's
+// own slots); the caller expands it into the full-width row afterwards.
+template <class TagS>
+__device__ __forceinline__ void put_gradient_unit(char* grow, float* marg, int64_t u, const float* g, bool to_lds) {
+  if (to_lds) {
+    *reinterpret_cast<float4*>(marg + u * 8) = float4{g[0], g[1], g[2], g[3]};
+    *reinterpret_cast<float4*>(marg + u * 8 + 4) = float4{g[4], g[5], g[6], g[7]};
+  } else {
+    Unit<TagS>::store(grow, u, g);
+  }
+}
+
 template <class TagS, int NU>
-__device__ __forceinline__ void rkl_gradient_from_stash(Unit<TagS> (&s)[NU], int64_t nunits, const float* marg, float k1,
-                                                        float wbar, char* grow) {
+__device__ __forceinline__ void rkl_gradient_from_stash(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float k1,
+                                                        float wbar, char* grow, bool to_lds) {
   const int tid = threadIdx.x;
   const float k0 = -k1 * wbar;
 #pragma unroll
@@ -471,15 +515,15 @@ __device__ __forceinline__ void rkl_gradient_from_stash(Unit<TagS> (&s)[NU], int
       d[0] = m0.x; d[1] = m0.y; d[2] = m0.z; d[3] = m0.w; d[4] = m1.x; d[5] = m1.y; d[6] = m1.z; d[7] = m1.w;
 #pragma unroll
       for (int e = 0; e < 8; ++e) g[e] = es[e] * __builtin_amdgcn_fmed3f(fmaf(d[e], k1, k0), -3e38f, 3e38f);
-      Unit<TagS>::store(grow, u, g);
+      put_gradient_unit<TagS>(grow, marg, u, g, to_lds);
     }
   }
 }
 
 // Pass C on the stored xt (rows whose sums were redone on their maxima).
 template <class TagS, int NU>
-__device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t nunits, const float* marg, float a_s, float bs,
-                                                  float k1, float wbar, char* grow) {
+__device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float a_s, float bs,
+                                                  float k1, float wbar, char* grow, bool to_lds) {
   const int tid = threadIdx.x;
 #pragma unroll
   for (int i = 0; i < NU; ++i) {
@@ -494,7 +538,7 @@ __device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t n
         const float xs = fmaxf(fmaf(sv[e], a_s, -bs), XT_OFF);     // finite for a logit of -inf: 0 * difference is 0
         g[e] = xt[e] > 0.5f * XT_OFF ? fast_exp2(xs) * k1 * ((xs - xt[e]) - wbar) : 0.f;
       }
-      Unit<TagS>::store(grow, u, g);
+      put_gradient_unit<TagS>(grow, marg, u, g, to_lds);
     }
   }
 }
@@ -503,10 +547,13 @@ __device__ __forceinline__ void rkl_gradient_pass(Unit<TagS> (&s)[NU], int64_t n
 // then turn out to be out of range, the row is put back -- logits read again (nothing of the row has
 // been written yet, also when the gradient goes over the logits), xt from the stored differences --
 // and takes the passes on its maxima like a row without a gradient.
+// Compact rows (p.Vs_full > 0): returns true when the gradient of the compact columns was left in marg for the
+// caller to expand; false when there is none to expand (no gradient asked for, or the row was zero-filled here).
 template <class TagS, int NU>
-__device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float* red,
+__device__ __forceinline__ bool rkl_against_marginal(Unit<TagS> (&s)[NU], int64_t nunits, float* marg, float* red,
                                                      const MargParams& p, int64_t r, char* grow, const char* srow) {
   const int tid = threadIdx.x;
+  const bool compact = p.Vs_full > 0;
   const float a_s = p.inv_T_s * LOG2E;
   const auto stored_of = [&](int64_t u, float (&m)[8]) {
     const float4 m0 = *reinterpret_cast<const float4*>(marg + u * 8), m1 = *reinterpret_cast<const float4*>(marg + u * 8 + 4);
@@ -568,14 +615,15 @@ __device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_
     if (stash_ok && in_range(ss1) && in_range(stt1)) {      // the same for every thread
       const float wbar = w / ss;
       if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - fast_log2(ss1) + fast_log2(stt1)) * LN2;
-      if (grow) rkl_gradient_from_stash<TagS, NU>(s, nunits, marg, p.inv_T_s * p.grad_scale * LN2 / ss, wbar, grow);
-      return;
+      if (grow) rkl_gradient_from_stash<TagS, NU>(s, nunits, marg, p.inv_T_s * p.grad_scale * LN2 / ss, wbar, grow, compact);
+      return compact && grow;
     }
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int64_t u = (int64_t)i * MARG_NT + tid;
       if (u < nunits) {
-        s[i].load(srow, u);
+        if (compact) gather_unit<TagS>(s[i], srow, p.cols, u);
+        else s[i].load(srow, u);
         float sv[8], d[8];
         s[i].unpack(sv);
         stored_of(u, d);
@@ -615,8 +663,8 @@ __device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_
     block_max2<MARG_NT>(tmax, ms, red);
     if (!(tmax > 0.5f * XT_OFF)) {                    // the teacher row carried no mass at all
       if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
-      if (grow) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
-      return;
+      if (grow) zero_row<TagS, MARG_NT>(grow, (compact ? p.Vs_full : p.Vs) / TagS::epc);
+      return false;
     }
     bs = ms * a_s;
     ss = 0.f, stt = 0.f, w = 0.f;
@@ -645,7 +693,43 @@ __device__ __forceinline__ void rkl_against_marginal(Unit<TagS> (&s)[NU], int64_
   }
   const float wbar = w / ss;
   if (tid == 0 && p.row_loss) p.row_loss[r] = (wbar - fast_log2(ss) + fast_log2(stt)) * LN2;
-  if (grow) rkl_gradient_pass<TagS, NU>(s, nunits, marg, a_s, bs, p.inv_T_s * p.grad_scale * LN2 / ss, wbar, grow);
+  if (grow) rkl_gradient_pass<TagS, NU>(s, nunits, marg, a_s, bs, p.inv_T_s * p.grad_scale * LN2 / ss, wbar, grow, compact);
+  return compact && grow;
+}
+
+// The gradient of a compact row (fp32 in marg, one value per compact id) into the full-width row: column j takes the
+// value of compact id col_src16[j], or 0; every chunk of the row is written once, by a 16-byte store.
+template <class TagS>
+__device__ __forceinline__ void expand_gradient_row(const float* marg, const unsigned short* col_src16, int64_t Vs_full, char* grow) {
+  using C = Chunk<TagS>;
+  constexpr int U = 8;                                   // chunks in flight per thread: their table loads are issued together
+  const int64_t nch = Vs_full / C::N;
+  for (int64_t c0 = threadIdx.x; c0 < nch; c0 += (int64_t)U * MARG_NT) {
+    u32x4 t[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const int64_t ch = c0 + (int64_t)j * MARG_NT;
+      if constexpr (C::N == 8) {
+        t[j] = ch < nch ? *reinterpret_cast<const u32x4*>(col_src16 + ch * 8) : u32x4{~0u, ~0u, ~0u, ~0u};
+      } else {
+        const uint2 h = ch < nch ? *reinterpret_cast<const uint2*>(col_src16 + ch * 4) : uint2{~0u, ~0u};
+        t[j] = u32x4{h.x, h.y, ~0u, ~0u};
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const int64_t ch = c0 + (int64_t)j * MARG_NT;
+      if (ch < nch) {
+        float g[C::N];
+#pragma unroll
+        for (int e = 0; e < C::N; ++e) {
+          const unsigned id = (t[j][e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+          g[e] = id != 0xffffu ? marg[id] : 0.f;
+        }
+        store16_stream(grow + ch * 16, C::pack(g));
+      }
+    }
+  }
 }
 
 template <class TagS, int NU, bool VEC>
@@ -657,8 +741,9 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
   const int tid = threadIdx.x;
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + r * p.grad_stride * TagS::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_rows);
+  const bool compact = p.Vs_full > 0;
   if (trow < 0) {
-    if (grow) zero_row<TagS, MARG_NT>(grow, p.Vs / TagS::epc);
+    if (grow) zero_row<TagS, MARG_NT>(grow, (compact ? p.Vs_full : p.Vs) / TagS::epc);
     if (tid == 0 && p.row_loss) p.row_loss[r] = 0.f;
     return;
   }
@@ -667,15 +752,19 @@ __global__ __launch_bounds__(MARG_NT) void rkl_marginalised_kernel(const MargPar
   const int pb = p.p_dtype == F32 ? 4 : 2;
   const char* prow = reinterpret_cast<const char*>(p.probs) + trow * p.p_stride * pb;
   float* marg = acc;
+  // the student row is in flight during the accumulation
   if (VEC && p.plan_ent) {
     marg = acc + p.plan_tile + PLAN_ZERO_WORDS;  // the tile sits first: its addresses are then plain offsets
-    rows.load(srow, p.Vs / 8);                   // in flight during the accumulation
+    if (compact) rows.load_gathered(srow, p.cols, p.Vs / 8); else rows.load(srow, p.Vs / 8);
     accumulate_marginal_planned(p, prow, marg, acc);
   } else {
-    rows.load(srow, p.Vs / 8);                   // in flight during the scatter
+    if (compact) rows.load_gathered(srow, p.cols, p.Vs / 8); else rows.load(srow, p.Vs / 8);
     accumulate_marginal<VEC>(p, prow, acc, 0, (int)p.Vs);
   }
-  rkl_against_marginal<TagS, NU>(rows.s, rows.nunits, marg, red, p, r, grow, srow);
+  if (rkl_against_marginal<TagS, NU>(rows.s, rows.nunits, marg, red, p, r, grow, srow)) {      // the same for every thread
+    __syncthreads();                             // the gradient of every compact column is in LDS
+    expand_gradient_row<TagS>(marg, p.col_src16, p.Vs_full, grow);
+  }
 }
 
 static bool ok16(const void* ptr, int64_t stride, int eb) {
@@ -763,24 +852,33 @@ extern "C" int dl_marginalise_csr(const void* probs, int p_dtype, int64_t p_stri
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
-extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs,
+// Shared by dl_rkl_marginalised (cols == NULL: the rows are Vs wide) and dl_rkl_marginalised_compact (logits and
+// gradient rows Vs_full wide, the kernel works on the Vs columns `cols` names).
+static int rkl_marginalised_launch(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs,
                                    const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
                                    int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s,
                                    const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
                                    const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
                                    float inv_T_student, float inv_T_teacher, float grad_scale, float* row_loss,
-                                   void* grad, int64_t grad_stride, void* stream) {
+                                   void* grad, int64_t grad_stride, const int32_t* cols, const unsigned short* col_src16,
+                                   int64_t Vs_full, void* stream) {
   using namespace dl;
   if (!logits || !t_probs || !t2s) return DL_ERR_NULL;
   if (logits_dtype < DL_F32 || logits_dtype > DL_F16 || p_dtype < DL_F32 || p_dtype > DL_F16) return DL_ERR_DTYPE;
-  if (n_rows < 0 || Vs <= 0 || Vt <= 0 || n_teacher_rows < 0 || row_stride < Vs || p_stride < Vt ||
-      (grad && grad_stride < Vs))
+  const int64_t width = cols ? Vs_full : Vs;      // columns of a logits / gradient row
+  if (n_rows < 0 || Vs <= 0 || Vt <= 0 || n_teacher_rows < 0 || width < Vs || row_stride < width || p_stride < Vt ||
+      (grad && grad_stride < width))
     return DL_ERR_SHAPE;
-  if (Vs > MARG_MAX_VS || n_rows > 0x7fffffffLL || Vt > 0x7fffffffLL) return DL_ERR_LIMIT;
+  if (Vs > MARG_MAX_VS || n_rows > 0x7fffffffLL || Vt > 0x7fffffffLL || width > 0x7fffffffLL) return DL_ERR_LIMIT;
   const int sb = logits_dtype == DL_F32 ? 4 : 2;
-  if (Vs % 8 != 0 || !ok16(logits, row_stride, sb) || (grad && !ok16(grad, grad_stride, sb))) return DL_ERR_ALIGN;
+  if (Vs % 8 != 0 || width % 8 != 0 || (grad && !ok16(grad, grad_stride, sb))) return DL_ERR_ALIGN;
+  if (cols ? (reinterpret_cast<uintptr_t>(logits) % sb != 0 || reinterpret_cast<uintptr_t>(cols) % 16 != 0 ||
+              reinterpret_cast<uintptr_t>(col_src16) % 16 != 0)
+           : !ok16(logits, row_stride, sb))
+    return DL_ERR_ALIGN;
   if (n_rows == 0) return DL_OK;
   MargParams p{};
+  p.cols = cols; p.col_src16 = col_src16; p.Vs_full = cols ? Vs_full : 0;
   p.probs = t_probs; p.p_dtype = p_dtype; p.p_stride = p_stride; p.n_rows = n_teacher_rows; p.Vt = Vt; p.t2s = t2s;
   p.Vs = Vs; p.logits = logits; p.s_dtype = logits_dtype; p.row_stride = row_stride; p.n_srows = n_rows;
   p.row_map = row_map; p.inv_T_s = inv_T_student; p.inv_T_t = inv_T_teacher; p.grad_scale = grad_scale;
@@ -800,4 +898,32 @@ extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t
   else DL_LAUNCH_RKLM(TagF16);
 #undef DL_LAUNCH_RKLM
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}
+
+extern "C" int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs,
+                                   const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
+                                   int64_t n_teacher_rows, int64_t Vt, const int32_t* t2s,
+                                   const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                                   const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
+                                   float inv_T_student, float inv_T_teacher, float grad_scale, float* row_loss,
+                                   void* grad, int64_t grad_stride, void* stream) {
+  return rkl_marginalised_launch(logits, logits_dtype, row_stride, n_rows, Vs, row_map, t_probs, p_dtype, p_stride,
+                                 n_teacher_rows, Vt, t2s, plan_row_off, plan_ent, plan_tile, plan_fold, plan_n_fold,
+                                 plan_n_extra, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride, nullptr,
+                                 nullptr, 0, stream);
+}
+
+extern "C" int dl_rkl_marginalised_compact(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
+                                           int64_t Vs_full, const int32_t* cols, const uint16_t* col_src16, int64_t n_compact,
+                                           const int32_t* row_map, const void* t_probs, int p_dtype, int64_t p_stride,
+                                           int64_t n_teacher_rows, int64_t Vt, const int32_t* t2c,
+                                           const int32_t* plan_row_off, const uint32_t* plan_ent, int plan_tile,
+                                           const int32_t* plan_fold, int plan_n_fold, int plan_n_extra,
+                                           float inv_T_student, float inv_T_teacher, float grad_scale, float* row_loss,
+                                           void* grad, int64_t grad_stride, void* stream) {
+  if (!cols || !col_src16) return DL_ERR_NULL;
+  return rkl_marginalised_launch(logits, logits_dtype, row_stride, n_rows, n_compact, row_map, t_probs, p_dtype, p_stride,
+                                 n_teacher_rows, Vt, t2c, plan_row_off, plan_ent, plan_tile, plan_fold, plan_n_fold,
+                                 plan_n_extra, inv_T_student, inv_T_teacher, grad_scale, row_loss, grad, grad_stride, cols,
+                                 reinterpret_cast<const unsigned short*>(col_src16), Vs_full, stream);
 }

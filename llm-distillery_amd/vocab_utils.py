@@ -65,21 +65,53 @@ def csr_from_map(t2s: np.ndarray, n_student: int) -> tuple[np.ndarray, np.ndarra
 class MarginalPlan:
     """A teacher->student id map laid out for the planned marginalisation kernels (fixed summation
     order, no atomics): build once per tokenizer pair, reuse for every batch.  Holds the device
-    copies of the map and of the plan arrays."""
+    copies of the map and of the plan arrays.
 
-    def __init__(self, t2s: np.ndarray, n_student: int, device):
+    A student vocabulary too wide for the kernels' marginal (more than 36864 ids) is compacted to the map's
+    image -- the student ids some teacher id maps to, ascending, `cols` -- when that fits: every other column
+    lies off the marginal's support in every row.  The plan is then built over the compact ids (`t2c`), and
+    `rkl_marginalised` gathers the logits' columns, runs the fused kernel on them and expands the gradient
+    (`col_src`: compact column of every student id, -1 outside the image).  `compact=True` asks for that form
+    also where the full vocabulary would fit."""
+
+    def __init__(self, t2s: np.ndarray, n_student: int, device, compact: bool | None = None):
         t2s = np.ascontiguousarray(np.asarray(t2s, dtype=np.int32))
         self.n_student = int(n_student)
         self.n_teacher = int(t2s.size)
         self.t2s = torch.as_tensor(t2s, device=device)
         self.row_off = self.ent = self.fold = None
         self.tile = self.n_fold = self.n_extra = 0
+        self.cols = self.col_src = self.col_src16 = self.t2c = None
+        self.n_compact = 0
+        if not compact and self._build(t2s, self.n_student, device):
+            return
+        if compact is False:
+            return
+        used = np.unique(t2s[(t2s >= 0) & (t2s < self.n_student)])
+        n_compact = max(8, -(-used.size // 8) * 8)
+        t2c = np.full(t2s.size, -1, dtype=np.int32)
+        ok = (t2s >= 0) & (t2s < self.n_student)
+        t2c[ok] = np.searchsorted(used, t2s[ok]).astype(np.int32)
+        if not self._build(t2c, n_compact, device):
+            return                                      # the image itself is too wide: no plan (the atomic path still works)
+        cols = np.full(n_compact, -1, dtype=np.int32)
+        cols[:used.size] = used
+        col_src = np.full(-(-self.n_student // 8) * 8, -1, dtype=np.int32)
+        col_src[used] = np.arange(used.size, dtype=np.int32)
+        self.n_compact = n_compact
+        self.cols = torch.as_tensor(cols, device=device)
+        self.col_src = torch.as_tensor(col_src, device=device)
+        self.col_src16 = torch.as_tensor(col_src.astype(np.uint16).view(np.int16), device=device)      # -1 reads 0xffff
+        self.t2c = torch.as_tensor(t2c, device=device)
+
+    def _build(self, t2s: np.ndarray, n_student: int, device) -> bool:
+        """dl_marginal_plan_build for `t2s` onto `n_student` ids; False where the library says too wide."""
         lib = _lib.load()
         tile, rows, n_fold, n_extra = ctypes.c_int(0), ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int(0)
         st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), None, None, 0, ctypes.byref(rows),
                                         None, 0, ctypes.byref(n_fold), ctypes.byref(n_extra))
-        if st == -4:          # DL_ERR_LIMIT: student vocabulary too wide for a plan; the atomic path still works
-            return
+        if st == -4:          # DL_ERR_LIMIT: student vocabulary too wide for a plan
+            return False
         _lib.check(st, "dl_marginal_plan_build")
         ntiles = -(-t2s.size // tile.value)
         row_off = np.zeros(16 * ntiles + 1, dtype=np.int32)
@@ -93,6 +125,7 @@ class MarginalPlan:
         self.row_off = torch.as_tensor(row_off, device=device)
         self.ent = torch.as_tensor(ent.view(np.int32), device=device)     # same bits; torch has no uint32 arithmetic need
         self.fold = torch.as_tensor(fold, device=device)
+        return True
 
     def check(self, n_student: int, n_teacher: int, device) -> None:
         """Raises unless the plan was built for these vocabulary sizes and lives on `device`: the
@@ -142,11 +175,48 @@ def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=Non
             if plan is not None:
                 plan.check(n_student, Vt, x.device)
                 t2s = plan.t2s
-                plan_args = plan._args()
+                if plan.cols is None:                   # a plan over compact ids does not describe the full-width marginal
+                    plan_args = plan._args()
             _, _ = _opt_i32(t2s, Vt, "t2s", x.device)
             st = lib.dl_marginalise_map(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vt, t2s.data_ptr(), n_student,
                                         *plan_args, out.data_ptr(), out.stride(0), int(log), _stream_ptr(x.device))
             _lib.check(st, "dl_marginalise_map")
+    return out
+
+
+class _CompactView:
+    """A compact MarginalPlan seen from the compact side: the map onto compact ids and the plan over them."""
+
+    def __init__(self, plan: "MarginalPlan"):
+        self.plan = plan
+
+
+def gather_columns(x: torch.Tensor, cols: torch.Tensor) -> torch.Tensor:
+    """out[r, c] = x[r, cols[c]] (-inf where cols[c] < 0): dl_gather_columns."""
+    R, V = x.shape
+    out = torch.empty((R, cols.numel()), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        for a in range(0, R, 65535):
+            n = min(65535, R - a)
+            st = lib.dl_gather_columns(x[a:].data_ptr(), _DT[x.dtype], x.stride(0), n, V, cols.data_ptr(), cols.numel(),
+                                       out[a:].data_ptr(), out.stride(0), _stream_ptr(x.device))
+            _lib.check(st, "dl_gather_columns")
+    return out
+
+
+def expand_columns(xc: torch.Tensor, col_src: torch.Tensor, V: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r, j] = xc[r, col_src[j]] for j < V (0 where col_src[j] < 0): dl_expand_columns."""
+    R, n = xc.shape
+    if out is None:
+        out = torch.empty((R, V), dtype=xc.dtype, device=xc.device)
+    lib = _lib.load()
+    with torch.cuda.device(xc.device):
+        for a in range(0, R, 65535):
+            m = min(65535, R - a)
+            st = lib.dl_expand_columns(xc[a:].data_ptr(), _DT[xc.dtype], xc.stride(0), m, n, col_src.data_ptr(), V,
+                                       out[a:].data_ptr(), out.stride(0), _stream_ptr(xc.device))
+            _lib.check(st, "dl_expand_columns")
     return out
 
 
@@ -164,12 +234,36 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
     dev = x.device
     _dev(teacher_probs, "teacher_probs", dev)
     plan_args = (0, 0, 0, 0, 0, 0)
-    if isinstance(t2s, MarginalPlan):
-        t2s.check(Vs, Vt, dev)
-        plan_args = t2s._args()
-        t2s = t2s.t2s
     if x.dtype not in _DT or tp.dtype not in _DT:
         raise RuntimeError("unsupported dtype")
+    if isinstance(t2s, MarginalPlan):
+        t2s.check(Vs, Vt, dev)
+        if t2s.cols is not None and Vs % (16 // x.element_size()) == 0:
+            # the student vocabulary compacted to the map's image (dl_rkl_marginalised_compact)
+            plan = t2s
+            if row_map is None and N < R:
+                raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
+            _, rm_ptr = _opt_i32(row_map, R, "row_map", dev)
+            row_loss = torch.empty(R, dtype=torch.float32, device=dev)
+            grad, g_ptr, g_stride = None, 0, Vs
+            if want_grad:
+                grad = _grad_target(grad_out, R, Vs, x.dtype, dev)
+                g_ptr, g_stride = grad.data_ptr(), grad.stride(0)
+            with torch.cuda.device(dev):
+                st = _lib.load().dl_rkl_marginalised_compact(
+                    x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vs, plan.cols.data_ptr(), plan.col_src16.data_ptr(),
+                    plan.n_compact, rm_ptr, tp.data_ptr(), _DT[tp.dtype], tp.stride(0), N, Vt, plan.t2c.data_ptr(),
+                    *plan._args(), 1.0 / T, 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
+                    row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
+            _lib.check(st, "dl_rkl_marginalised_compact")
+            if grad is not None and logits.dim() != 2 and grad_out is None:
+                grad = grad.view(logits.shape)
+            return row_loss, grad
+        plan_args = t2s._args()
+        t2s = t2s.t2s
+    elif isinstance(t2s, _CompactView):
+        plan_args = t2s.plan._args()
+        t2s = t2s.plan.t2c
     if row_map is None and N < R:
         raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")
     _, rm_ptr = _opt_i32(row_map, R, "row_map", dev)

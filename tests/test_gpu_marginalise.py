@@ -295,3 +295,63 @@ def test_fused_path_limits_are_reported(D):
     with pytest.raises(RuntimeError, match="exceeds"):
         D.vocab_utils.rkl_marginalised(torch.zeros(2, 40000, device=DEV), torch.zeros(2, 64, device=DEV),
                                        torch.zeros(64, dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_column_gather_and_expansion(D, dtype):
+    """dl_gather_columns / dl_expand_columns move raw elements: a subset of the columns out (padding reads -inf)
+    and back in (columns outside the subset read 0), every bit as it was."""
+    g = torch.Generator().manual_seed(3)
+    R, V = 7, 4104
+    x = (torch.randn(R, V + 8, generator=g) * 3).to(dtype).to(DEV)[:, :V]           # rows of another pitch
+    used = torch.sort(torch.randperm(V, generator=g)[:1001]).values
+    cols = torch.full((1008,), -1, dtype=torch.int32)
+    cols[:1001] = used.to(torch.int32)
+    col_src = torch.full((V,), -1, dtype=torch.int32)
+    col_src[used] = torch.arange(1001, dtype=torch.int32)
+    xc = D.vocab_utils.gather_columns(x, cols.to(DEV))
+    assert torch.equal(xc[:, :1001], x[:, used.to(DEV)]) and torch.isneginf(xc[:, 1001:].float()).all()
+    back = D.vocab_utils.expand_columns(xc, col_src.to(DEV), V)
+    want = torch.zeros_like(x)
+    want[:, used.to(DEV)] = x[:, used.to(DEV)]
+    assert torch.equal(back, want)
+
+
+@pytest.mark.parametrize("dtype,Vs,Vt,alphabet", [(torch.bfloat16, 128256, 152064, 256), (torch.float32, 50000, 60000, 8),
+                                                  (torch.float16, 8192, 30000, 16)])
+def test_fused_reverse_kl_on_a_student_vocabulary_compacted_to_the_map_s_image(D, dtype, Vs, Vt, alphabet):
+    """Student vocabularies wider than the fused kernel's marginal (and, on request, narrower ones): the plan is
+    built over the student ids the map reaches, the logits' columns are gathered, the gradient expanded.  Loss
+    and gradient against the oracle on the full vocabulary; columns outside the image get exactly 0; masked
+    rows; bit-reproducible."""
+    R = 9
+    t2s, probs = _case(R, Vs, Vt, 5, alphabet, drop=0.01)
+    g = torch.Generator().manual_seed(11)
+    logits = (torch.randn(R + 2, Vs, generator=g) * 2).to(dtype)
+    valid = torch.ones(R + 2, dtype=torch.bool)
+    valid[[1, 7]] = False
+    rm = torch.full((R + 2,), -1, dtype=torch.int32)
+    rm[valid] = torch.arange(R, dtype=torch.int32)
+    plan = D.vocab_utils.MarginalPlan(t2s, Vs, DEV, compact=True)
+    assert plan.cols is not None and plan.n_compact % 8 == 0 and plan.n_compact < Vs
+    T = 1.5
+    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), plan, row_map=rm.to(DEV), T=T, grad_scale=1.0 / R)
+    rl2, grad2 = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), plan, row_map=rm.to(DEV), T=T, grad_scale=1.0 / R)
+    assert torch.equal(rl, rl2) and torch.equal(grad, grad2) and grad.shape == logits.shape and grad.dtype == dtype
+    marg = torch.tensor(O.marginalise_map(probs.numpy(), t2s, Vs))
+    with np.errstate(divide="ignore"):
+        t_logits = O.marginal_to_teacher_logits(marg)
+    loss64, rows64, grad64 = O.mean_loss_and_grad("rkl", logits, T, t_logits=t_logits, valid=valid, dtype=torch.float64)
+    np.testing.assert_allclose(rl.cpu()[valid].double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    assert torch.count_nonzero(grad.cpu()[~valid]) == 0 and torch.count_nonzero(rl.cpu()[~valid]) == 0
+    rtol = 1e-4 if dtype == torch.float32 else 2e-3
+    bound = O.storage_tolerance(grad64, dtype, rtol)
+    sel = torch.nonzero(valid).squeeze(-1)
+    bound[sel] = O.marginal_rkl_gradient_tolerance(grad64[sel], logits[sel], t_logits, rows64, T, T, 1.0 / R, dtype, rtol)
+    err = (grad.cpu().double() - grad64).abs()
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+    outside = torch.ones(Vs, dtype=torch.bool)
+    outside[torch.as_tensor(np.unique(t2s[t2s >= 0])).long()] = False
+    assert torch.count_nonzero(grad.cpu()[:, outside]) == 0
+    rl3, _ = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), plan, row_map=rm.to(DEV), T=T, want_grad=False)
+    np.testing.assert_allclose(rl3.cpu().numpy(), rl.cpu().numpy(), rtol=2e-5, atol=1e-6)

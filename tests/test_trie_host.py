@@ -161,9 +161,20 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     assert n_packed >= 4 * ntiles                 # one-run threads are gathered in the low waves: half the entries sit on 8 ids
     # half of the entries sit on 8 ids: without replicas one thread would hold > 1200 entries of a tile
     assert max(longest) <= 4 * (tile // 1024)
-    # too wide a student vocabulary: no plan, the atomic form remains
-    wide = D.vocab_utils.MarginalPlan(np.zeros(100, dtype=np.int32), 40000, "cpu")
-    assert wide.ent is None and wide.tile == 0
+    # too wide a student vocabulary: the plan is built over the map's image (the student ids it reaches) ...
+    wide_map = rng.integers(-1, 90000, 5000).astype(np.int32)
+    wide = D.vocab_utils.MarginalPlan(wide_map, 90000, "cpu")
+    used = np.unique(wide_map[wide_map >= 0])
+    assert wide.ent is not None and wide.n_compact == -(-used.size // 8) * 8
+    cols, col_src, t2c = wide.cols.numpy(), wide.col_src.numpy(), wide.t2c.numpy()
+    assert np.array_equal(cols[:used.size], used) and (cols[used.size:] == -1).all()
+    assert np.array_equal(np.nonzero(col_src >= 0)[0], used) and np.array_equal(col_src[used], np.arange(used.size))
+    assert np.array_equal(t2c >= 0, wide_map >= 0) and np.array_equal(cols[t2c[wide_map >= 0]], wide_map[wide_map >= 0])
+    # ... unless the caller rules that out, or the image itself is too wide: no plan, the atomic form remains
+    none = D.vocab_utils.MarginalPlan(np.zeros(100, dtype=np.int32), 40000, "cpu", compact=False)
+    assert none.ent is None and none.tile == 0 and none.cols is None
+    huge = D.vocab_utils.MarginalPlan(np.arange(60000, dtype=np.int32), 60000, "cpu")
+    assert huge.ent is None and huge.cols is None
 
 
 def _apply_plan(plan, probs, Vs):
