@@ -341,10 +341,16 @@ __global__ __launch_bounds__(256) void marginalise_csr_kernel(const void* probs,
 // ---- fused: marginal in LDS -> reverse KL against the student row in registers -----------------
 // The student row of the fused kernel: NU units of 8 columns per thread, in registers.
 // Unit u of a compacted student row: the raw elements at columns cols[8u .. 8u + 7] of the full-width row.
+// Unit u of a full-width row seen through `cols`: the logits at columns cols[8u .. 8u + 7] (-inf for a column of -1).
+// The ids are fetched apart from the elements, so that a caller with several units has all ids in flight together
+// before the first element load waits for them.
+struct UnitIds { int4 a, b; };
+__device__ __forceinline__ UnitIds unit_ids(const int32_t* cols, int64_t u) {
+  return UnitIds{*reinterpret_cast<const int4*>(cols + u * 8), *reinterpret_cast<const int4*>(cols + u * 8 + 4)};
+}
 template <class TagS>
-__device__ __forceinline__ void gather_unit(Unit<TagS>& x, const char* srow, const int32_t* cols, int64_t u) {
-  const int4 a = *reinterpret_cast<const int4*>(cols + u * 8), b = *reinterpret_cast<const int4*>(cols + u * 8 + 4);
-  const int id[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+__device__ __forceinline__ void gather_unit(Unit<TagS>& x, const char* srow, const UnitIds& ids) {
+  const int id[8] = {ids.a.x, ids.a.y, ids.a.z, ids.a.w, ids.b.x, ids.b.y, ids.b.z, ids.b.w};
   if constexpr (TagS::bytes == 4) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) x.c[e >> 2][e & 3] = id[e] >= 0 ? reinterpret_cast<const unsigned*>(srow)[id[e]] : 0xff800000u;
@@ -357,6 +363,10 @@ __device__ __forceinline__ void gather_unit(Unit<TagS>& x, const char* srow, con
 #pragma unroll
     for (int d = 0; d < 4; ++d) x.c[0][d] = h[2 * d] | (h[2 * d + 1] << 16);
   }
+}
+template <class TagS>
+__device__ __forceinline__ void gather_unit(Unit<TagS>& x, const char* srow, const int32_t* cols, int64_t u) {
+  gather_unit<TagS>(x, srow, unit_ids(cols, u));
 }
 
 template <class TagS, int NU>
@@ -374,11 +384,14 @@ struct StudentRow {
   // The same from a full-width row, unit u = the logits at columns cols[8u .. 8u + 7] (-inf for a column of -1).
   __device__ __forceinline__ void load_gathered(const char* srow, const int32_t* cols, int64_t nu) {
     nunits = nu;
+    UnitIds ids[NU];
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int64_t u = (int64_t)i * MARG_NT + threadIdx.x;
-      if (u < nunits) gather_unit<TagS>(s[i], srow, cols, u); else s[i].fill_neg_inf();
+      ids[i] = u < nunits ? unit_ids(cols, u) : UnitIds{int4{-1, -1, -1, -1}, int4{-1, -1, -1, -1}};
     }
+#pragma unroll
+    for (int i = 0; i < NU; ++i) gather_unit<TagS>(s[i], srow, ids[i]);
   }
 };
 

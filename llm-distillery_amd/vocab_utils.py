@@ -62,70 +62,94 @@ def csr_from_map(t2s: np.ndarray, n_student: int) -> tuple[np.ndarray, np.ndarra
     return offsets, indices[:n.value].copy()
 
 
+class _PlanArrays:
+    """Device copies of what dl_marginal_plan_build lays out for one map: list offsets, entries, fold table."""
+
+    def __init__(self, row_off, ent, fold, tile: int, n_fold: int, n_extra: int, device):
+        self.tile, self.n_fold, self.n_extra = tile, n_fold, n_extra
+        self.row_off = torch.as_tensor(row_off, device=device)
+        self.ent = torch.as_tensor(ent.view(np.int32), device=device)     # same bits; torch has no uint32 arithmetic need
+        self.fold = torch.as_tensor(fold, device=device)
+
+    def args(self):
+        """(row_off, ent, tile, fold, n_fold, n_extra) as the C ABI takes them."""
+        return self.row_off.data_ptr(), self.ent.data_ptr(), self.tile, self.fold.data_ptr(), self.n_fold, self.n_extra
+
+
+def _build_plan(t2s: np.ndarray, n_student: int, device) -> "_PlanArrays | None":
+    """dl_marginal_plan_build for `t2s` onto `n_student` ids; None where the library says too wide."""
+    lib = _lib.load()
+    tile, rows, n_fold, n_extra = ctypes.c_int(0), ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int(0)
+    st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), None, None, 0, ctypes.byref(rows),
+                                    None, 0, ctypes.byref(n_fold), ctypes.byref(n_extra))
+    if st == -4:          # DL_ERR_LIMIT: student vocabulary too wide for a plan
+        return None
+    _lib.check(st, "dl_marginal_plan_build")
+    ntiles = -(-t2s.size // tile.value)
+    row_off = np.zeros(16 * ntiles + 1, dtype=np.int32)
+    ent = np.empty((max(rows.value, 1), 64), dtype=np.uint32)
+    fold = np.zeros((max(n_fold.value, 1), 3), dtype=np.int32)
+    st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), _p(row_off), _p(ent), rows.value,
+                                    ctypes.byref(rows), _p(fold), n_fold.value, ctypes.byref(n_fold),
+                                    ctypes.byref(n_extra))
+    _lib.check(st, "dl_marginal_plan_build")
+    return _PlanArrays(row_off, ent, fold, tile.value, int(n_fold.value), int(n_extra.value), device)
+
+
 class MarginalPlan:
     """A teacher->student id map laid out for the planned marginalisation kernels (fixed summation
     order, no atomics): build once per tokenizer pair, reuse for every batch.  Holds the device
-    copies of the map and of the plan arrays.
+    copies of the map and of the plan arrays.  Up to two plans are built:
 
-    A student vocabulary too wide for the kernels' marginal (more than 36864 ids) is compacted to the map's
-    image -- the student ids some teacher id maps to, ascending, `cols` -- when that fits: every other column
-    lies off the marginal's support in every row.  The plan is then built over the compact ids (`t2c`), and
-    `rkl_marginalised` gathers the logits' columns, runs the fused kernel on them and expands the gradient
-    (`col_src`: compact column of every student id, -1 outside the image).  `compact=True` asks for that form
-    also where the full vocabulary would fit."""
+    * `full`: over the student ids themselves, where the kernels' marginal can hold them all (at most
+      36864 ids).  `marginalise` uses it, and `rkl_marginalised` where there is no compact one.
+    * `compact`: over the map's image -- the student ids some teacher id maps to, ascending, `cols`; every
+      other column lies off the marginal's support in every row.  `rkl_marginalised` then gathers those
+      columns of the logits inside the kernel, runs the passes behind the marginal on them alone and
+      expands the gradient row (`col_src`: compact column of every student id, -1 outside the image).
+      The passes behind the marginal cost time in proportion to the marginal's width, the expansion in
+      proportion to the full vocabulary (about 0.45 of a pass column per column); the compact plan is
+      therefore built where the image holds at most half of the student ids (and the vocabulary is a
+      multiple of 8 ids, the compact kernel's alignment), or where the full width does not fit.
+
+    `compact=True` builds the compact plan only, `compact=False` the full one only.  `row_off`, `ent`, `fold`,
+    `tile`, `n_fold` and `n_extra` describe the full plan, or the compact one where that is the only one."""
+
+    COMPACT_AT_MOST = 0.5          # image size / student vocabulary below which the compact plan pays
 
     def __init__(self, t2s: np.ndarray, n_student: int, device, compact: bool | None = None):
         t2s = np.ascontiguousarray(np.asarray(t2s, dtype=np.int32))
         self.n_student = int(n_student)
         self.n_teacher = int(t2s.size)
         self.t2s = torch.as_tensor(t2s, device=device)
-        self.row_off = self.ent = self.fold = None
-        self.tile = self.n_fold = self.n_extra = 0
+        self.full = self.compact = None
         self.cols = self.col_src = self.col_src16 = self.t2c = None
         self.n_compact = 0
-        if not compact and self._build(t2s, self.n_student, device):
-            return
-        if compact is False:
-            return
-        used = np.unique(t2s[(t2s >= 0) & (t2s < self.n_student)])
-        n_compact = max(8, -(-used.size // 8) * 8)
-        t2c = np.full(t2s.size, -1, dtype=np.int32)
+        if compact is not True:
+            self.full = _build_plan(t2s, self.n_student, device)
         ok = (t2s >= 0) & (t2s < self.n_student)
-        t2c[ok] = np.searchsorted(used, t2s[ok]).astype(np.int32)
-        if not self._build(t2c, n_compact, device):
-            return                                      # the image itself is too wide: no plan (the atomic path still works)
-        cols = np.full(n_compact, -1, dtype=np.int32)
-        cols[:used.size] = used
-        col_src = np.full(-(-self.n_student // 8) * 8, -1, dtype=np.int32)
-        col_src[used] = np.arange(used.size, dtype=np.int32)
-        self.n_compact = n_compact
-        self.cols = torch.as_tensor(cols, device=device)
-        self.col_src = torch.as_tensor(col_src, device=device)
-        self.col_src16 = torch.as_tensor(col_src.astype(np.uint16).view(np.int16), device=device)      # -1 reads 0xffff
-        self.t2c = torch.as_tensor(t2c, device=device)
-
-    def _build(self, t2s: np.ndarray, n_student: int, device) -> bool:
-        """dl_marginal_plan_build for `t2s` onto `n_student` ids; False where the library says too wide."""
-        lib = _lib.load()
-        tile, rows, n_fold, n_extra = ctypes.c_int(0), ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int(0)
-        st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), None, None, 0, ctypes.byref(rows),
-                                        None, 0, ctypes.byref(n_fold), ctypes.byref(n_extra))
-        if st == -4:          # DL_ERR_LIMIT: student vocabulary too wide for a plan
-            return False
-        _lib.check(st, "dl_marginal_plan_build")
-        ntiles = -(-t2s.size // tile.value)
-        row_off = np.zeros(16 * ntiles + 1, dtype=np.int32)
-        ent = np.empty((max(rows.value, 1), 64), dtype=np.uint32)
-        fold = np.zeros((max(n_fold.value, 1), 3), dtype=np.int32)
-        st = lib.dl_marginal_plan_build(_p(t2s), t2s.size, n_student, ctypes.byref(tile), _p(row_off), _p(ent), rows.value,
-                                        ctypes.byref(rows), _p(fold), n_fold.value, ctypes.byref(n_fold),
-                                        ctypes.byref(n_extra))
-        _lib.check(st, "dl_marginal_plan_build")
-        self.tile, self.n_fold, self.n_extra = tile.value, int(n_fold.value), int(n_extra.value)
-        self.row_off = torch.as_tensor(row_off, device=device)
-        self.ent = torch.as_tensor(ent.view(np.int32), device=device)     # same bits; torch has no uint32 arithmetic need
-        self.fold = torch.as_tensor(fold, device=device)
-        return True
+        used = np.unique(t2s[ok])
+        if compact is None:
+            compact = self.full is None or (self.n_student % 8 == 0 and
+                                            used.size <= self.COMPACT_AT_MOST * self.n_student)
+        if compact:
+            n_compact = max(8, -(-used.size // 8) * 8)
+            t2c = np.full(t2s.size, -1, dtype=np.int32)
+            t2c[ok] = np.searchsorted(used, t2s[ok]).astype(np.int32)
+            self.compact = _build_plan(t2c, n_compact, device)     # None: the image itself is too wide (the atomic path still works)
+            if self.compact is not None:
+                cols = np.full(n_compact, -1, dtype=np.int32)
+                cols[:used.size] = used
+                col_src = np.full(-(-self.n_student // 8) * 8, -1, dtype=np.int32)
+                col_src[used] = np.arange(used.size, dtype=np.int32)
+                self.n_compact = n_compact
+                self.cols = torch.as_tensor(cols, device=device)
+                self.col_src = torch.as_tensor(col_src, device=device)
+                self.col_src16 = torch.as_tensor(col_src.astype(np.uint16).view(np.int16), device=device)      # -1 reads 0xffff
+                self.t2c = torch.as_tensor(t2c, device=device)
+        main = self.full if self.full is not None else self.compact
+        self.row_off, self.ent, self.fold = (main.row_off, main.ent, main.fold) if main else (None, None, None)
+        self.tile, self.n_fold, self.n_extra = (main.tile, main.n_fold, main.n_extra) if main else (0, 0, 0)
 
     def check(self, n_student: int, n_teacher: int, device) -> None:
         """Raises unless the plan was built for these vocabulary sizes and lives on `device`: the
@@ -137,10 +161,8 @@ class MarginalPlan:
             raise RuntimeError(f"the plan lives on {self.t2s.device}, the call runs on {device}")
 
     def _args(self):
-        """(row_off, ent, tile, fold, n_fold, n_extra) as the C ABI takes them."""
-        if self.ent is None:
-            return 0, 0, 0, 0, 0, 0
-        return self.row_off.data_ptr(), self.ent.data_ptr(), self.tile, self.fold.data_ptr(), self.n_fold, self.n_extra
+        """The full plan's (row_off, ent, tile, fold, n_fold, n_extra) as the C ABI takes them; zeros without one."""
+        return self.full.args() if self.full is not None else (0, 0, 0, 0, 0, 0)
 
 
 def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=None, plan: MarginalPlan | None = None,
@@ -175,8 +197,7 @@ def marginalise(probs: torch.Tensor, *, t2s: torch.Tensor | None = None, csr=Non
             if plan is not None:
                 plan.check(n_student, Vt, x.device)
                 t2s = plan.t2s
-                if plan.cols is None:                   # a plan over compact ids does not describe the full-width marginal
-                    plan_args = plan._args()
+                plan_args = plan._args()                # the full plan; without one the LDS-atomic form runs
             _, _ = _opt_i32(t2s, Vt, "t2s", x.device)
             st = lib.dl_marginalise_map(x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vt, t2s.data_ptr(), n_student,
                                         *plan_args, out.data_ptr(), out.stride(0), int(log), _stream_ptr(x.device))
@@ -238,7 +259,7 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
         raise RuntimeError("unsupported dtype")
     if isinstance(t2s, MarginalPlan):
         t2s.check(Vs, Vt, dev)
-        if t2s.cols is not None and Vs % (16 // x.element_size()) == 0:
+        if t2s.compact is not None:
             # the student vocabulary compacted to the map's image (dl_rkl_marginalised_compact)
             plan = t2s
             if row_map is None and N < R:
@@ -253,7 +274,7 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
                 st = _lib.load().dl_rkl_marginalised_compact(
                     x.data_ptr(), _DT[x.dtype], x.stride(0), R, Vs, plan.cols.data_ptr(), plan.col_src16.data_ptr(),
                     plan.n_compact, rm_ptr, tp.data_ptr(), _DT[tp.dtype], tp.stride(0), N, Vt, plan.t2c.data_ptr(),
-                    *plan._args(), 1.0 / T, 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
+                    *plan.compact.args(), 1.0 / T, 1.0 / (T if teacher_T is None else teacher_T), grad_scale,
                     row_loss.data_ptr(), g_ptr, g_stride, _stream_ptr(dev))
             _lib.check(st, "dl_rkl_marginalised_compact")
             if grad is not None and logits.dim() != 2 and grad_out is None:
@@ -262,7 +283,7 @@ def rkl_marginalised(logits: torch.Tensor, teacher_probs: torch.Tensor, t2s: "to
         plan_args = t2s._args()
         t2s = t2s.t2s
     elif isinstance(t2s, _CompactView):
-        plan_args = t2s.plan._args()
+        plan_args = t2s.plan.compact.args()
         t2s = t2s.plan.t2c
     if row_map is None and N < R:
         raise RuntimeError(f"{R} logits rows but only {N} teacher rows and no row_map")

@@ -6,7 +6,7 @@ run is reproducible; a failure names its case.  What the draws are chosen to rea
     16-byte grid (odd vocabularies), the streaming kernel, parts that do not wait for their partners (the
     second launch finishes them), ids that repeat and crowd a few chunks, masked rows;
   * dense kernels: the three divergences, mixed dtypes, offsets that move the maxima, zero-mass teacher columns;
-  * fused marginal + reverse KL: the planned and the atomic accumulation, and all three ways a row is finished --
+  * fused marginal + reverse KL: the planned (full-width and compact) and the atomic accumulation, and all three ways a row is finished --
     from the values kept between the passes, put back and redone on its maxima (sums that leave the range: teachers
     scaled by 1e+-30; a student whose largest logits sit off the support), and without a gradient;
   * weighted merge + remap: ids bit-exact; the bucketed multi-teacher loss with maps that crowd every entry of a row
@@ -123,7 +123,7 @@ def test_fused_marginal_reverse_kl(D):
         dtype = DTYPES[int(rng.integers(0, 3))]
         T = float(rng.choice([0.5, 0.7, 1.0, 1.5, 2.0]))
         tT = float(rng.choice([T, T, 1.0, 0.25, 3.0]))
-        planned = bool(rng.integers(0, 2))
+        planned = (False, "full", "auto")[int(rng.integers(0, 3))]
         vocab_seed = int(rng.integers(0, 6))                      # a handful of tokenizer pairs, built once each
         key = (Vs, Vt, alphabet, vocab_seed)
         if key not in maps:
@@ -131,8 +131,9 @@ def test_fused_marginal_reverse_kl(D):
             teacher = S.random_byte_vocab(Vt, vocab_seed + 1, alphabet=alphabet, max_len=8)
             t2s = D.vocab_utils.longest_prefix_map(student, teacher).copy()
             t2s[np.random.default_rng(vocab_seed).random(Vt) < 0.02] = -1
-            maps[key] = (t2s, D.vocab_utils.MarginalPlan(t2s, Vs, DEV), torch.tensor(t2s, device=DEV))
-        t2s, plan, t2s_dev = maps[key]
+            maps[key] = (t2s, {"full": D.vocab_utils.MarginalPlan(t2s, Vs, DEV, compact=False),
+                               "auto": D.vocab_utils.MarginalPlan(t2s, Vs, DEV)}, torch.tensor(t2s, device=DEV))
+        t2s, plans, t2s_dev = maps[key]
         g = torch.Generator().manual_seed(case)
         probs = torch.softmax(torch.randn(R, Vt, generator=g) * float(rng.choice([1, 3, 8])), -1)
         # unnormalised teachers: the sums of such rows leave the range the optimistic pass covers
@@ -147,7 +148,7 @@ def test_fused_marginal_reverse_kl(D):
                 logits[:, dead[:2]] += float(rng.choice([10, 25, 60]))
         logits = logits.to(dtype)
         what = f"case {case}: Vs={Vs} Vt={Vt} alphabet={alphabet} R={R} {dtype} T={T} teacher T={tT} planned={planned}"
-        tmap = plan if planned else t2s_dev
+        tmap = plans[planned] if planned else t2s_dev
         rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, T=T, teacher_T=tT, grad_scale=1.0 / R)
         rl0, _ = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, T=T, teacher_T=tT, want_grad=False)
         with np.errstate(divide="ignore"):

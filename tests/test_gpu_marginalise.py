@@ -30,6 +30,15 @@ def _case(R, Vs, Vt, seed, alphabet=4, drop=0.0):
     return t2s, probs
 
 
+def _map_in_the_form(D, planned, t2s, Vs):
+    """False: the bare map on the GPU (LDS atomics); "full": the plan over the student ids only; "auto": what
+    MarginalPlan builds by itself (the compact plan beside the full one where the map's image is small)."""
+    if not planned:
+        return torch.tensor(t2s, device=DEV)
+    return D.vocab_utils.MarginalPlan(t2s, Vs, DEV, compact=False if planned == "full" else None)
+
+
+
 @pytest.mark.parametrize("Vs,Vt,alphabet", [(1000, 5000, 4), (32000, 152064, 256), (40000, 50001, 16)])
 def test_marginal_map_and_csr_forms(D, Vs, Vt, alphabet):
     t2s, probs = _case(6, Vs, Vt, 1, alphabet, drop=0.02)
@@ -122,7 +131,7 @@ def test_marginal_of_16bit_probabilities(D):
     np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=2e-6, atol=1e-9)
 
 
-@pytest.mark.parametrize("planned", [False, True])
+@pytest.mark.parametrize("planned", [False, "full", "auto"])
 @pytest.mark.parametrize("dtype,Vs,Vt,alphabet,T", [(torch.bfloat16, 32000, 152064, 256, 1.5), (torch.float32, 2048, 9000, 4, 1.0),
                                                     (torch.float16, 8192, 30000, 8, 0.8)])
 def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T, planned):
@@ -134,7 +143,7 @@ def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T, planne
     valid[[2, 5, 14]] = False
     rm = torch.full((R + 3,), -1, dtype=torch.int32)
     rm[valid] = torch.arange(R, dtype=torch.int32)
-    tmap = D.vocab_utils.MarginalPlan(t2s, Vs, DEV) if planned else torch.tensor(t2s, device=DEV)
+    tmap = _map_in_the_form(D, planned, t2s, Vs)
     rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, row_map=rm.to(DEV), T=T,
                                               grad_scale=1.0 / R)
     if planned:       # fixed summation order: bit-reproducible
@@ -158,7 +167,7 @@ def test_fused_reverse_kl_against_marginal(D, dtype, Vs, Vt, alphabet, T, planne
     assert torch.count_nonzero(grad.cpu()[valid][:, (marg.sum(0) == 0)]) == 0
 
 
-@pytest.mark.parametrize("planned", [False, True])
+@pytest.mark.parametrize("planned", [False, "full", "auto"])
 @pytest.mark.parametrize("T", [1.0, 2.0, 0.5])
 def test_fused_reverse_kl_on_rows_whose_sums_leave_the_range(D, T, planned):
     """Rows for which a bias of 0 for the teacher and the row's largest logit for the student do not keep
@@ -177,7 +186,7 @@ def test_fused_reverse_kl_on_rows_whose_sums_leave_the_range(D, T, planned):
     probs[2, torch.tensor(t2s == off)] = 0.0
     logits[2, off] = 300.0
     probs[3] = 0.0
-    tmap = D.vocab_utils.MarginalPlan(t2s, Vs, DEV) if planned else torch.tensor(t2s, device=DEV)
+    tmap = _map_in_the_form(D, planned, t2s, Vs)
     with_mass = torch.tensor([0, 1, 2, 4, 5])
     rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), tmap, T=T, grad_scale=1.0 / len(with_mass))
     rl, grad = rl.cpu(), grad.cpu()
@@ -261,7 +270,7 @@ def test_fused_reverse_kl_16bit_rows_whose_maximum_is_negative_zero_or_towering(
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("planned", [False, True])
+@pytest.mark.parametrize("planned", [False, "full", "auto"])
 def test_fused_reverse_kl_gradient_may_overwrite_the_logits(D, dtype, planned):
     """The gradient written over the logits, also for rows that are put back and redone (their logits are
     read a second time before anything of the row is written): the same bits as into a buffer of its own."""
@@ -276,7 +285,7 @@ def test_fused_reverse_kl_gradient_may_overwrite_the_logits(D, dtype, planned):
     logits[1::2, off_cols] += 40.0                   # every other row has its mass off the support
     probs[4] *= 1e-30                                # and one hardly any teacher mass
     x = logits.to(dtype).to(DEV)
-    tmap = D.vocab_utils.MarginalPlan(t2s, Vs, DEV) if planned else torch.tensor(t2s, device=DEV)
+    tmap = _map_in_the_form(D, planned, t2s, Vs)
     rl, grad = D.vocab_utils.rkl_marginalised(x, probs.to(DEV), tmap, T=1.3, grad_scale=0.5)
     y = x.clone()
     rl2, g2 = D.vocab_utils.rkl_marginalised(y, probs.to(DEV), tmap, T=1.3, grad_scale=0.5, grad_out=y)
@@ -355,3 +364,26 @@ def test_fused_reverse_kl_on_a_student_vocabulary_compacted_to_the_map_s_image(D
     assert torch.count_nonzero(grad.cpu()[:, outside]) == 0
     rl3, _ = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), plan, row_map=rm.to(DEV), T=T, want_grad=False)
     np.testing.assert_allclose(rl3.cpu().numpy(), rl.cpu().numpy(), rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("Vs,dtype", [(4008, torch.float32), (4000, torch.bfloat16)])
+def test_a_plan_that_holds_the_compact_form_only(D, Vs, dtype):
+    """No full plan to fall back to: the fused kernel runs on the compact ids, and `marginalise` gives the full-width marginal from the bare map."""
+    R, Vt = 5, 9000
+    t2s, probs = _case(R, Vs, Vt, 9, 16)
+    plan = D.vocab_utils.MarginalPlan(t2s, Vs, DEV, compact=True)
+    assert plan.full is None and plan.compact is not None
+    g = torch.Generator().manual_seed(4)
+    logits = (torch.randn(R, Vs, generator=g) * 2).to(dtype)
+    rl, grad = D.vocab_utils.rkl_marginalised(logits.to(DEV), probs.to(DEV), plan, T=1.2, grad_scale=1.0 / R)
+    marg = torch.tensor(O.marginalise_map(probs.numpy(), t2s, Vs))
+    with np.errstate(divide="ignore"):
+        t_logits = O.marginal_to_teacher_logits(marg)
+    _, rows64, grad64 = O.mean_loss_and_grad("rkl", logits, 1.2, t_logits=t_logits, dtype=torch.float64)
+    np.testing.assert_allclose(rl.cpu().double().numpy(), rows64.numpy(), rtol=3e-5, atol=3e-6)
+    bound = O.marginal_rkl_gradient_tolerance(grad64, logits, t_logits, rows64, 1.2, 1.2, 1.0 / R, dtype,
+                                              1e-4 if dtype == torch.float32 else 2e-3)
+    err = (grad.cpu().double() - grad64).abs()
+    assert (err <= bound).all(), f"worst ratio {(err / bound).max():.2f}"
+    m = D.vocab_utils.marginalise(probs.to(DEV), plan=plan, n_student=Vs).cpu().numpy()
+    np.testing.assert_allclose(m, marg.numpy(), rtol=2e-6, atol=1e-9)

@@ -165,7 +165,8 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     wide_map = rng.integers(-1, 90000, 5000).astype(np.int32)
     wide = D.vocab_utils.MarginalPlan(wide_map, 90000, "cpu")
     used = np.unique(wide_map[wide_map >= 0])
-    assert wide.ent is not None and wide.n_compact == -(-used.size // 8) * 8
+    assert wide.full is None and wide.compact is not None and wide.ent is wide.compact.ent
+    assert wide.n_compact == -(-used.size // 8) * 8
     cols, col_src, t2c = wide.cols.numpy(), wide.col_src.numpy(), wide.t2c.numpy()
     assert np.array_equal(cols[:used.size], used) and (cols[used.size:] == -1).all()
     assert np.array_equal(np.nonzero(col_src >= 0)[0], used) and np.array_equal(col_src[used], np.arange(used.size))
@@ -175,6 +176,15 @@ def test_marginal_plan_covers_every_mapped_id_once_with_single_owner_slots():
     assert none.ent is None and none.tile == 0 and none.cols is None
     huge = D.vocab_utils.MarginalPlan(np.arange(60000, dtype=np.int32), 60000, "cpu")
     assert huge.ent is None and huge.cols is None
+    # a vocabulary that fits gets the full plan, and the compact one beside it where the image is at most half of it
+    narrow = rng.integers(-1, 3000, 9000).astype(np.int32)
+    both = D.vocab_utils.MarginalPlan(narrow, 8000, "cpu")
+    assert both.full is not None and both.compact is not None and both.ent is both.full.ent and both.n_compact <= 3000
+    assert D.vocab_utils.MarginalPlan(narrow, 8004, "cpu").compact is None          # not a multiple of 8 ids
+    assert D.vocab_utils.MarginalPlan(narrow, 4000, "cpu").compact is None          # image above half of the vocabulary
+    assert D.vocab_utils.MarginalPlan(narrow, 8000, "cpu", compact=False).compact is None
+    only = D.vocab_utils.MarginalPlan(narrow, 4000, "cpu", compact=True)
+    assert only.full is None and only.compact is not None and only._args() == (0, 0, 0, 0, 0, 0)
 
 
 def _apply_plan(plan, probs, Vs):
