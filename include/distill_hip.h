@@ -175,19 +175,20 @@ int dl_div_dense(int kind,
                  float* row_loss, void* grad, int64_t grad_stride, void* stream);
 
 /*
- * dl_div_dense with a workspace: forward and reverse KL on rows that one 256-thread workgroup's registers do
- * not hold (more than 16384 columns of two 16-bit rows, 8192 with an fp32 row; up to 8 times that) are then
- * cut into column parts of that size, one workgroup each, which exchange their maxima and sums through the
- * workspace -- the split of dl_div_topk applied to the dense pair (same reference lines as dl_div_dense).
- * Four parts of different rows share a compute unit and hide each other's load, arithmetic and store
- * phases, which a workgroup that holds a whole pair of rows (512 or 1024 threads, one or two per compute
- * unit) cannot.  Same arguments and conventions as dl_div_dense, same results to fp32 rounding (the sums are
- * taken part by part), bit-reproducible from call to call.
+ * dl_div_dense with a workspace: forward and reverse KL on rows that the registers of 512 threads do not hold
+ * (more than 32768 columns of two 16-bit rows, 24576 of a 16-bit row against an fp32 one, 16384 of two fp32
+ * rows) are cut evenly into 2 to 8 column parts, one workgroup of 256, 512 or 1024 threads each, which exchange
+ * their maxima and sums through the workspace -- the split of dl_div_topk applied to the dense pair (same
+ * reference lines as dl_div_dense).  Parts of different rows share a compute unit and hide each other's load,
+ * arithmetic and store phases, which a workgroup that holds a whole pair of rows cannot.  Same arguments and
+ * conventions as dl_div_dense, same results to fp32 rounding (the sums are taken part by part),
+ * bit-reproducible from call to call.
  * workspace   at least dl_div_dense_workspace_bytes(...) bytes, 16-byte aligned, contents irrelevant on entry
  *             and on return; NULL or too small: exactly dl_div_dense.  Launches that may overlap in time must
  *             not share a workspace.  dl_div_dense_workspace_bytes returns 0 where rows are not cut (JSD,
  *             narrow or very wide rows, V not a multiple of 8, dtype pairs without a register kernel).
- * flags       DL_TOPK_NO_WAIT: the parts never wait for their partners (test hook, as for dl_div_topk).
+ * flags       DL_TOPK_NO_WAIT: the parts never wait for their partners; DL_TOPK_PARTS(1 / 2 / 3): parts of
+ *             256 / 512 / 1024 threads wherever two or more come out (test and tuning hooks).
  */
 int dl_div_dense_ws(int kind,
                     const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,

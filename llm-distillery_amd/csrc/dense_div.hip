@@ -192,8 +192,13 @@ struct DenseSplit {
   unsigned* retry_list;
   int parts;
   int spin_limit;
+  int64_t part_units;        // units of 8 columns per part (the last part takes what is left)
   __host__ __device__ static int64_t bytes(int64_t n_rows, int parts) { return n_rows * parts * (int64_t)(sizeof(DenseRecord) + 4) + 16; }
-  __host__ DenseSplit(void* ws, int64_t n_rows, int parts_, int spin) {
+  // The row is cut evenly, in whole waves of units: a last part that holds a few columns would still take a
+  // workgroup, and its partners would wait for it like for a full one.
+  __host__ DenseSplit(void* ws, int64_t n_rows, int parts_, int spin, int64_t units, int64_t most_units) {
+    part_units = ((units + parts_ - 1) / parts_ + 63) / 64 * 64;
+    if (part_units > most_units || (parts_ - 1) * part_units >= units) part_units = most_units;
     records = reinterpret_cast<DenseRecord*>(ws);
     char* base = reinterpret_cast<char*>(ws) + n_rows * parts_ * (int64_t)sizeof(DenseRecord);
     retry_count = reinterpret_cast<unsigned*>(base);
@@ -241,8 +246,8 @@ __device__ __forceinline__ void dense_split_part(const DenseParams& p, const Den
   static_assert(KIND == DL_FKL || KIND == DL_RKL, "JSD rows are not cut into parts");
   const int tid = threadIdx.x;
   const int P = x.parts;
-  const int64_t u0 = (int64_t)h * NT * NU;                             // first unit of this part
-  const int64_t nu = min((int64_t)NT * NU, p.V / 8 - u0);               // its units
+  const int64_t u0 = (int64_t)h * x.part_units;                        // first unit of this part
+  const int64_t nu = min(x.part_units, p.V / 8 - u0);                   // its units
   char* grow = p.grad ? reinterpret_cast<char*>(p.grad) + (r * p.grad_stride + u0 * 8) * TagS::bytes : nullptr;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   if (trow < 0) {
@@ -374,25 +379,35 @@ __global__ __launch_bounds__(256) void dense_clear_kernel(u32x4* ws, int64_t n16
 // Units per thread of the split kernels for a dtype pair (0: the pair has no register kernel).
 static int dense_split_units(int s_dtype, int t_dtype) {
   if (s_dtype == t_dtype) return s_dtype == F32 ? 4 : 8;
-  return t_dtype == F32 ? 4 : 0;
+  return t_dtype == F32 ? 6 : 0;
 }
-// How a row of V columns is cut: threads per part and parts (parts == 0: not cut).  Parts of 512 threads:
-// measured (forward KL, 512 and 8192 rows, fp32 pairs of 32000 to 131072 and bf16 pairs of 65536 to 262144
-// columns) they are level with or ahead of twice as many parts of 256 threads (half as many partners to wait
-// for; 8 parts of 256 lose even against one workgroup per row), and ahead of one workgroup per row except for
-// two parts on a few hundred rows.  `forced_nt` (256 / 512, a tuning hook) fixes the thread count and cuts
-// wherever two parts or more come out.
+// How a row of V columns is cut: threads per part and parts (parts == 0: not cut).  Measured (forward KL, 512 and
+// 8192 rows, 32000 to 262144 columns, fp32 pairs, 16-bit pairs and a 16-bit student against an fp32 teacher):
+//   * a row that half a workgroup's registers hold (512 threads) stays whole;
+//   * up to four parts of 256 threads beat half as many of 512 (more workgroups per CU to hide the exchange
+//     behind), beyond that the partners to wait for cost more than they bring: parts of 512 threads, at most 8;
+//   * wider still, rows against an fp32 teacher take parts of 1024 threads (beyond 8 of those, and beyond 262144
+//     columns of a 16-bit pair, one workgroup per row streams the row from the caches);
+//   * on fewer than 1024 rows the cut pays only from 256 KiB of row pair upwards (one workgroup per row keeps
+//     the CUs busy by itself below that, and has no partners to wait for).
+// `forced_nt` (256 / 512 / 1024, a tuning hook) fixes the thread count and cuts wherever two parts or more come out.
 struct DenseCut { int nt, parts; };
 static DenseCut dense_split_cut(int kind, int s_dtype, int t_dtype, int64_t n_rows, int64_t V, int forced_nt = 0) {
   const int nu = dense_split_units(s_dtype, t_dtype);
   if (kind == DL_JSD || nu == 0 || V % 8 != 0) return {0, 0};
   const int64_t units = V / 8;
-  const int64_t p256 = (units + 256 * nu - 1) / (256 * nu), p512 = (units + 512 * nu - 1) / (512 * nu);
-  if (forced_nt == 256) return p256 >= 2 && p256 <= DENSE_MAX_PARTS ? DenseCut{256, (int)p256} : DenseCut{0, 0};
-  if (forced_nt == 512) return p512 >= 2 && p512 <= DENSE_MAX_PARTS ? DenseCut{512, (int)p512} : DenseCut{0, 0};
-  if (p512 < 2 || p512 > DENSE_MAX_PARTS) return {0, 0};
-  if (p512 == 2 && n_rows < 1024) return {0, 0};
-  return {512, (int)p512};
+  const auto parts_of = [&](int nt) { return (units + (int64_t)nt * nu - 1) / ((int64_t)nt * nu); };
+  const auto cut_of = [&](int nt) {
+    const int64_t parts = parts_of(nt);
+    return parts >= 2 && parts <= DENSE_MAX_PARTS && (nt != 1024 || t_dtype == F32) ? DenseCut{nt, (int)parts} : DenseCut{0, 0};
+  };
+  if (forced_nt) return cut_of(forced_nt);
+  if (parts_of(512) < 2) return {0, 0};
+  const int64_t pair_bytes = V * ((s_dtype == F32 ? 4 : 2) + (t_dtype == F32 ? 4 : 2));
+  if (n_rows < 1024 && pair_bytes < 256 * 1024) return {0, 0};
+  if (parts_of(256) <= 4) return cut_of(256);
+  if (parts_of(512) <= DENSE_MAX_PARTS) return cut_of(512);
+  return cut_of(1024);
 }
 
 template <int KIND, class TagS, class TagT, int NT, int NU>
@@ -410,6 +425,11 @@ static void launch_dense_split(const DenseParams& p, const DenseSplit& x, int nt
   if (nt == 256) {
     if (p.kind == DL_FKL) launch_dense_split_kind<DL_FKL, TagS, TagT, 256, NU>(p, x, st);
     else launch_dense_split_kind<DL_RKL, TagS, TagT, 256, NU>(p, x, st);
+  } else if (nt == 1024) {
+    if constexpr (TagT::bytes == 4) {                  // 16-bit pairs reach 262144 columns with parts of 512 threads
+      if (p.kind == DL_FKL) launch_dense_split_kind<DL_FKL, TagS, TagT, 1024, NU>(p, x, st);
+      else launch_dense_split_kind<DL_RKL, TagS, TagT, 1024, NU>(p, x, st);
+    }
   } else {
     if (p.kind == DL_FKL) launch_dense_split_kind<DL_FKL, TagS, TagT, 512, NU>(p, x, st);
     else launch_dense_split_kind<DL_RKL, TagS, TagT, 512, NU>(p, x, st);
@@ -419,8 +439,8 @@ static void launch_dense_split_pair(const DenseParams& p, const DenseSplit& x, i
   if (p.s_dtype == F32 && p.t_dtype == F32) launch_dense_split<TagF32, TagF32, 4>(p, x, nt, st);
   else if (p.s_dtype == BF16 && p.t_dtype == BF16) launch_dense_split<TagBF16, TagBF16, 8>(p, x, nt, st);
   else if (p.s_dtype == F16 && p.t_dtype == F16) launch_dense_split<TagF16, TagF16, 8>(p, x, nt, st);
-  else if (p.s_dtype == BF16 && p.t_dtype == F32) launch_dense_split<TagBF16, TagF32, 4>(p, x, nt, st);
-  else launch_dense_split<TagF16, TagF32, 4>(p, x, nt, st);
+  else if (p.s_dtype == BF16 && p.t_dtype == F32) launch_dense_split<TagBF16, TagF32, 6>(p, x, nt, st);
+  else launch_dense_split<TagF16, TagF32, 6>(p, x, nt, st);
 }
 
 // Rows too wide for the registers, 16-byte aligned: the same sweeps, every one of them over global
@@ -709,7 +729,7 @@ extern "C" int64_t dl_div_dense_workspace_bytes(int kind, int logits_dtype, int 
   if (n_rows <= 0 || V <= 0) return 0;
   // enough for every cut the flags of dl_div_dense_ws may ask for
   int parts = 0;
-  for (int nt : {0, 256, 512}) parts = std::max(parts, dl::dense_split_cut(kind, logits_dtype, t_dtype, n_rows, V, nt).parts);
+  for (int nt : {0, 256, 512, 1024}) parts = std::max(parts, dl::dense_split_cut(kind, logits_dtype, t_dtype, n_rows, V, nt).parts);
   return parts ? dl::DenseSplit::bytes(n_rows, parts) : 0;
 }
 
@@ -750,10 +770,11 @@ extern "C" int dl_div_dense_ws(int kind, const void* logits, int logits_dtype, i
   if (!elem) return DL_ERR_ALIGN;
   // rows cut into column parts, where a workspace for their exchange came along
   const int hook = (flags >> DL_TOPK_PARTS_SHIFT) & 15;      // 1 / 2: parts of 256 / 512 threads wherever the row can be cut
-  const DenseCut cut = vec ? dense_split_cut(kind, logits_dtype, t_dtype, n_rows, V, hook == 1 ? 256 : hook == 2 ? 512 : 0) : DenseCut{0, 0};
+  const DenseCut cut = vec ? dense_split_cut(kind, logits_dtype, t_dtype, n_rows, V, hook == 1 ? 256 : hook == 2 ? 512 : hook == 3 ? 1024 : 0) : DenseCut{0, 0};
   if (cut.parts && workspace && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
       workspace_bytes >= DenseSplit::bytes(n_rows, cut.parts) && n_rows * cut.parts <= 0x7fffffffLL) {
-    const DenseSplit x(workspace, n_rows, cut.parts, (flags & DL_TOPK_NO_WAIT) ? 0 : DENSE_SPIN_LIMIT);
+    const DenseSplit x(workspace, n_rows, cut.parts, (flags & DL_TOPK_NO_WAIT) ? 0 : DENSE_SPIN_LIMIT, V / 8,
+                       (int64_t)cut.nt * dense_split_units(logits_dtype, t_dtype));
     launch_dense_split_pair(p, x, cut.nt, st);
     return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
   }

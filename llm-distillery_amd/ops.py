@@ -188,7 +188,7 @@ def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_ma
     """Per-token "fkl", "rkl" or "jsd" against a dense teacher [N, V] and, in the same launch,
     d(sum of row losses)/d(logits) * grad_scale.  Returns (row_loss fp32 [rows], grad or None).
     `split=False` withholds the workspace that lets wide forward / reverse-KL rows be cut into column parts
-    (dl_div_dense_ws); `no_wait` and `part_threads` (256 / 512) are the library's test hooks for those parts
+    (dl_div_dense_ws); `no_wait` and `part_threads` (256 / 512 / 1024) are the library's test hooks for those parts
     (DL_TOPK_NO_WAIT, DL_TOPK_PARTS)."""
     if kind not in KINDS:
         raise ValueError("kind must be 'fkl', 'rkl' or 'jsd'")
@@ -220,7 +220,7 @@ def div_dense(kind: str, logits: torch.Tensor, t_logits: torch.Tensor, *, row_ma
                                  1.0 / (T if teacher_T is None else teacher_T), grad_scale,
                                  row_loss.data_ptr(), g_ptr, g_stride, ws.data_ptr() if ws is not None else 0, ws_bytes,
                                  (_lib.DL_TOPK_NO_WAIT if no_wait else 0) |
-                                 ({0: 0, 256: 1, 512: 2}[part_threads] << _lib.DL_TOPK_PARTS_SHIFT), _stream_ptr(dev))
+                                 ({0: 0, 256: 1, 512: 2, 1024: 3}[part_threads] << _lib.DL_TOPK_PARTS_SHIFT), _stream_ptr(dev))
     _lib.check(st, "dl_div_dense_ws")
     if grad is not None and logits.dim() != 2 and grad_out is None:
         grad = grad.view(logits.shape)

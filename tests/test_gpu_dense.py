@@ -278,20 +278,24 @@ def test_reverse_kl_with_student_logits_of_minus_infinity(D, dtype, V):
 
 @pytest.mark.parametrize("kind", ["fkl", "rkl"])
 @pytest.mark.parametrize("dtype,t_dtype,V,threads", [
-    (torch.float32, torch.float32, 32000, 256),      # 4 parts of 256 x 4 units (the last one partly filled)
+    (torch.float32, torch.float32, 32000, 256),      # 4 parts of 256 threads x 4 units of 8 columns, cut evenly: 3 x 1024 + 928 units
     (torch.float32, torch.float32, 32000, 512),      # 2 parts of 512 x 4
     (torch.bfloat16, torch.bfloat16, 32000, 256),    # 2 parts of 256 x 8
     (torch.bfloat16, torch.bfloat16, 128256, 0),     # the library's choice: 4 parts of 512 x 8
     (torch.bfloat16, torch.bfloat16, 128256, 256),   # 8 parts
     (torch.float16, torch.float16, 65536, 256),      # 4 full parts
     (torch.float16, torch.float16, 262144, 0),       # 8 full parts of 512 x 8
-    (torch.bfloat16, torch.float32, 50264, 256),     # mixed pair: 7 parts of 8192 columns
-    (torch.float16, torch.float32, 8200, 256),       # one column chunk more than a part holds
-    (torch.float16, torch.float32, 40000, 0),        # mixed pair, 3 parts of 512 x 4
+    (torch.bfloat16, torch.float32, 50264, 256),     # mixed pair (6 units per thread): 5 parts, the last one shorter
+    (torch.bfloat16, torch.float32, 50304, 0),       # the library's choice: 3 parts of 512 x 6
+    (torch.float16, torch.float32, 12296, 256),      # one unit more than a part holds: 2 parts of 832 and 705 units
+    (torch.float16, torch.float32, 40000, 0),        # mixed pair, 4 parts of 256 x 6
+    (torch.bfloat16, torch.float32, 200064, 0),      # too wide for 8 parts of 512 x 6: 5 parts of 1024 threads
+    (torch.float32, torch.float32, 151936, 0),       # the same for an fp32 pair: 5 parts of 1024 x 4
+    (torch.float32, torch.float32, 40000, 1024),     # 2 parts of 1024 x 4
     (torch.float32, torch.float32, 65536, 0)])       # 4 full parts of 512 x 4
 def test_rows_cut_into_column_parts(D, kind, dtype, t_dtype, V, threads):
-    """dl_div_dense_ws: wide forward / reverse-KL rows cut into parts of 256 threads that exchange their maxima
-    and sums through the workspace.  Both forms against the oracle, the row losses of the two against each other
+    """dl_div_dense_ws: wide forward / reverse-KL rows cut into parts of 256, 512 or 1024 threads that exchange their
+    maxima and sums through the workspace.  Both forms against the oracle, the row losses of the two against each other
     (the same numbers to fp32 rounding), with parts that do
     not wait for their partners (the second launch finishes them: the same bits), twice (the same bits), with
     masked rows, and with the gradient written over the logits."""
