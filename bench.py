@@ -242,7 +242,8 @@ def _wl_dropin(batched):
     save_topK 400, batch 4): per conversation `calculate_divergence` on fp32 logits + `Losses.add_losses`,
     then one `Losses.backward` for the batch (classes/student/model.py:415-441) -- or, `batched`, the same
     batch through `distill_loss_batch` + `Losses.add_batch`.  The dominant-kernel figure is the library's
-    launches alone (phase 1, epilogue, its backward, phase 2 per conversation) on preallocated buffers."""
+    launches alone (phase 1, the epilogue, phase 2 with the rows' coefficients made in it, per conversation) on
+    preallocated buffers."""
     def build(D, S, dev, rows):
         import torch
         from llm_distillery_amd import ops
@@ -276,7 +277,7 @@ def _wl_dropin(batched):
         lib = D._lib.load()
         bufs = [dict(lse=torch.empty(N, device=dev), zk=torch.empty(N, K, device=dev), rec=torch.empty(N, 8, device=dev),
                      coef=torch.empty(N, 4, device=dev), out=torch.empty(1, 9, device=dev), g=torch.ones(1, device=dev),
-                     g_lse=torch.empty(N, device=dev), g_zk=torch.empty(N, K, device=dev), grad=torch.empty(N, V, device=dev))
+                     grad=torch.empty(N, V, device=dev))
                 for _ in range(B)]
         import ctypes
         arr = ctypes.c_int32 * 2
@@ -293,18 +294,16 @@ def _wl_dropin(batched):
                                          b["rec"].data_ptr(), b["coef"].data_ptr(), b["out"].data_ptr(), st)
             for i in range(B):
                 x, b = xs[i].detach(), bufs[i]
-                lib.dl_composite_backward(b["lse"].data_ptr(), b["zk"].data_ptr(), tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
-                                          offs[0], 1, 1, N, b["rec"].data_ptr(), b["coef"].data_ptr(), b["g"].data_ptr(),
-                                          b["g_lse"].data_ptr(), b["g_zk"].data_ptr(), st)
-                lib.dl_rowcoef_grad_topk(x.data_ptr(), 0, V, N, V, 0, tis[i].data_ptr(), 1, K, N, 1.0, b["lse"].data_ptr(),
-                                         b["g_lse"].data_ptr(), b["g_zk"].data_ptr(), b["grad"].data_ptr(), V, st)
+                lib.dl_composite_backward_fused(x.data_ptr(), 0, V, N, V, 1.0, tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
+                                                offs[0], 1, 1, b["lse"].data_ptr(), b["zk"].data_ptr(), b["rec"].data_ptr(),
+                                                b["coef"].data_ptr(), b["g"].data_ptr(), b["grad"].data_ptr(), V, st)
             return bufs[0]["out"]
 
         algo = B * (N * V * 4 * 3 + N * K * (4 + 8 + 4 + 4 + 4))
         return (step, launches, algo, B * N,
                 f"the reference's call pattern at its default shape: {B} conversations x {N} tokens x {V} vocab fp32, K={K}: "
                 + ("distill_loss_batch + Losses.add_batch" if batched else "calculate_divergence + Losses.add_losses per conversation")
-                + " + Losses.backward", "library launches alone: rowstats + composite epilogue + its backward + rowcoef_grad, per conversation",
+                + " + Losses.backward", "library launches alone: rowstats with the rows' records + conversation epilogue + rowcoef_grad with the rows' coefficients, per conversation",
                 {"logits": xb.detach()}, torch.empty_like(xb))
     return build
 

@@ -12,164 +12,21 @@
 // A conversation's rows couple through max(kl), the valid-mean of the cross entropy and the means,
 // which is why the middle launch exists.  Sums over a conversation are accumulated in double in a
 // fixed order: bit-reproducible.
-#include "distill_common.hpp"
-#include "distill_hip.h"
+#include "composite.hpp"
 
 namespace dl {
 
 constexpr int CMP_ROWS_PER_WG = 4;            // one wave each
 constexpr int CMP_NT = 256;
 
-// per-row record written by the forward row kernel, read by the other two
-struct RowRec { float kl, rkl, own_s, own_t, t_lse, s_lse; int kstar; int valid; };       // 32 bytes
-// per-row coefficients for a unit upstream gradient on the conversation's train loss
-struct RowCoef { float g_kl, g_rkl, g_own; float pad; };                                  // 16 bytes
-
-// First row / label / ignore entry of every conversation, [C + 1] each: device arrays, or -- for up to
-// DL_MAX_HOST_CONVOS conversations -- copies that travel with the launch (a caller with one
-// conversation, or a handful, then needs no upload of three tiny arrays per call).
-struct ConvoOffsets {
-  const int32_t* dev[3];                          // row, label, avoid; NULL = use `inl`
-  int32_t inl[3][DL_MAX_HOST_CONVOS + 1];
-  __device__ __forceinline__ int row(int c) const { return dev[0] ? dev[0][c] : inl[0][c]; }
-  __device__ __forceinline__ int label(int c) const { return dev[1] ? dev[1][c] : inl[1][c]; }
-  __device__ __forceinline__ int avoid(int c) const { return dev[2] ? dev[2][c] : inl[2][c]; }
-};
-
-struct CompositeParams {
-  const float* lse; const float* zk;
-  const void* t_val; int t_val_dtype; float inv_T_t;
-  const void* t_idx; int t_idx_itype; int K;
-  const int64_t* labels; const void* avoid; int avoid_itype;
-  ConvoOffsets off;
-  int n_convos; int64_t n_rows; float alpha;
-  RowRec* rec; RowCoef* coef; float* out;         // out [C, 9]
-  const float* g_train; float* g_lse; float* g_zk;
-};
-
-__device__ __forceinline__ int wave_min_int(int v) {
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, WAVE));
-  return v;
-}
-
-// conversation that holds row i: last c whose first row is <= i
-__device__ __forceinline__ int convo_of_row(const ConvoOffsets& off, int n_convos, int64_t i) {
-  int lo = 0, hi = n_convos - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (off.row(mid) <= i) lo = mid; else hi = mid - 1;
-  }
-  return lo;
-}
-
 // ---- rows, forward ---------------------------------------------------------------------------------
-// One wave per token row.  R > 0: K <= 64 * R and the storage types are known at compile time: the
-// row's teacher values, ids and gathered logits are fetched once, all loads in flight together, and
-// stay in registers for the three passes (maxima, sums, divergences).  R == 0: any K, any types,
-// three passes over memory.
+// One wave per token row (composite_row_record).
 template <int VD, int IT, int R>
 __global__ __launch_bounds__(CMP_NT) void composite_rows_fwd_kernel(const CompositeParams p) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int64_t i = (int64_t)blockIdx.x * CMP_ROWS_PER_WG + threadIdx.x / WAVE;
   if (i >= p.n_rows) return;
-  const int K = p.K;
-  const float* z = p.zk + i * K;
-  const float lse = p.lse[i];
-  constexpr int RR = R > 0 ? R : 1;
-  float tv[RR], zv[RR];
-  int64_t id[RR];
-  if constexpr (R > 0) {
-#pragma unroll
-    for (int j = 0; j < R; ++j) {
-      const int k = lane + j * WAVE;
-      const int64_t at = i * K + (k < K ? k : 0);      // lanes beyond K read entry 0 and discard it: no branch between the loads
-      float t;
-      if constexpr (VD == F32) t = reinterpret_cast<const float*>(p.t_val)[at];
-      else if constexpr (VD == BF16) t = __uint_as_float((unsigned)reinterpret_cast<const unsigned short*>(p.t_val)[at] << 16);
-      else t = (float)reinterpret_cast<const _Float16*>(p.t_val)[at];
-      if constexpr (IT == I32) id[j] = reinterpret_cast<const int32_t*>(p.t_idx)[at];
-      else id[j] = reinterpret_cast<const int64_t*>(p.t_idx)[at];
-      const float zz = z[k < K ? k : 0];
-      tv[j] = k < K ? t * p.inv_T_t : -INFINITY;
-      zv[j] = k < K ? zz : -INFINITY;
-      id[j] = k < K ? id[j] : -1;
-    }
-  }
-  // maxima
-  float tmax = -INFINITY, zmax = -INFINITY;
-  if constexpr (R > 0) {
-#pragma unroll
-    for (int j = 0; j < R; ++j) { tmax = fmaxf(tmax, tv[j]); zmax = fmaxf(zmax, zv[j]); }
-  } else {
-    for (int k = lane; k < K; k += WAVE) {
-      tmax = fmaxf(tmax, load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t);
-      zmax = fmaxf(zmax, z[k]);
-    }
-  }
-  tmax = wave_max(tmax);
-  zmax = wave_max(zmax);
-  float tsum = 0.f, zsum = 0.f;
-  if constexpr (R > 0) {
-#pragma unroll
-    for (int j = 0; j < R; ++j) { tsum += expf(tv[j] - tmax); zsum += expf(zv[j] - zmax); }      // exp(-inf) = 0 beyond K
-  } else {
-    for (int k = lane; k < K; k += WAVE) {
-      tsum += expf(load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t - tmax);
-      zsum += expf(z[k] - zmax);
-    }
-  }
-  const float t_lse = tmax + logf(wave_sum(tsum));          // teacher renormalised over its K entries
-  const float z_lse = zmax + logf(wave_sum(zsum));          // log-sum-exp of the student over the support
-  const float s_lse = z_lse - lse;                          // = logsumexp_k(s_k), s_k = z_k - lse
-
-  // label of this row, if it has one: conversation-local row li carries label li, for li < #labels
-  const int c = convo_of_row(p.off, p.n_convos, i);
-  const int li = (int)(i - p.off.row(c));
-  const int n_lab = p.off.label(c + 1) - p.off.label(c);
-  bool want = li < n_lab;
-  int64_t label = -1;
-  if (want) {
-    label = p.labels[p.off.label(c) + li];
-    for (int a = p.off.avoid(c); a < p.off.avoid(c + 1); ++a) want = want && (load_index(p.avoid, p.avoid_itype, a) != li);
-  }
-  float kl = 0.f, rkl = 0.f;
-  int kfound = 0x7fffffff;
-  if constexpr (R > 0) {
-#pragma unroll
-    for (int j = 0; j < R; ++j) {
-      const int k = lane + j * WAVE;
-      if (k < K) {
-        const float t = tv[j] - t_lse;
-        const float s = zv[j] - lse;
-        const float s2 = s - s_lse;
-        kl += expf(t) * (t - s);
-        rkl += expf(s2) * (s2 - t);
-        if (want && id[j] == label) kfound = min(kfound, k);
-      }
-    }
-  } else {
-    for (int k = lane; k < K; k += WAVE) {
-      const float t = load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t - t_lse;
-      const float s = z[k] - lse;
-      const float s2 = s - s_lse;
-      kl += expf(t) * (t - s);
-      rkl += expf(s2) * (s2 - t);
-      if (want && load_index(p.t_idx, p.t_idx_itype, i * K + k) == label) kfound = min(kfound, k);
-    }
-  }
-  kl = wave_sum(kl);
-  rkl = wave_sum(rkl);
-  kfound = wave_min_int(kfound);
-  if (lane == 0) {
-    RowRec r;
-    r.kl = kl; r.rkl = rkl; r.t_lse = t_lse; r.s_lse = s_lse;
-    r.valid = kfound != 0x7fffffff ? 1 : 0;
-    r.kstar = r.valid ? kfound : -1;
-    r.own_s = r.valid ? z[kfound] - lse : 0.f;
-    r.own_t = r.valid ? load_as_float(p.t_val, p.t_val_dtype, i * K + kfound) * p.inv_T_t - t_lse : 0.f;
-    p.rec[i] = r;
-  }
+  composite_row_record<VD, IT, R>(p, i, p.zk + i * p.K, p.lse[i], lane);
 }
 
 // ---- conversations -----------------------------------------------------------------------------------
@@ -178,11 +35,19 @@ template <int NT, int N>
 __device__ __forceinline__ void block_sums_f64(double (&v)[N], double* scratch) {
   constexpr int NW = NT / WAVE;
   const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  // step by step for all N sums together: the N exchanges of a step are in flight at once (sum by sum, every
+  // exchange would wait for the one before it: N times the latency for the same additions in the same order)
 #pragma unroll
-  for (int k = 0; k < N; ++k) {
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    double t[N];
 #pragma unroll
-    for (int o = WAVE / 2; o > 0; o >>= 1) v[k] += __shfl_xor(v[k], o, WAVE);
-    if (lane == 0) scratch[k * NW + w] = v[k];
+    for (int k = 0; k < N; ++k) t[k] = __shfl_xor(v[k], o, WAVE);
+#pragma unroll
+    for (int k = 0; k < N; ++k) v[k] += t[k];
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) scratch[k * NW + w] = v[k];
   }
   __syncthreads();
 #pragma unroll
@@ -258,6 +123,7 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
   double a_wkl = 0.0, a_wrkl = 0.0, a_kl = 0.0, a_rkl = 0.0, a_ces = 0.0, a_cet = 0.0, a_d = 0.0;
   double a_gmk = 0.0, a_gmr = 0.0, a_ginv = 0.0;
   const float inv_n = 1.f / (float)n;
+  const float inv_mk2 = 1.f / (mk * mk), inv_mr2 = 1.f / (mr * mr), inv_mk = 1.f / mk, inv_mr = 1.f / mr;      // for the gradient's terms; the weights themselves divide
   convo_rows(mine, rec, n, [&](int i, const RowRec& r) {
     float cpos = 0.f;
     if (i < m) {
@@ -275,8 +141,8 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
     const float wk = pk + cpos, wr = pr + cpos;
     a_wkl += (double)(r.kl * wk); a_wrkl += (double)(r.rkl * wr);
     a_kl += (double)r.kl; a_rkl += (double)r.rkl;
-    a_gmk += (double)(r.kl * alpha * pk1 * (-r.kl / (mk * mk)));
-    a_gmr += (double)(r.rkl * alpha * pr1 * (-r.rkl / (mr * mr)));
+    a_gmk += (double)(r.kl * alpha * pk1 * (-r.kl * inv_mk2));
+    a_gmr += (double)(r.rkl * alpha * pr1 * (-r.rkl * inv_mr2));
   });
   {
     double v[10] = {a_wkl, a_wrkl, a_kl, a_rkl, a_ces, a_cet, a_d, a_gmk, a_gmr, a_ginv};
@@ -317,8 +183,8 @@ __global__ __launch_bounds__(CONVO_NT) void composite_convo_kernel(const Composi
     weight_powers(Ak, alpha, pk, pk1);
     weight_powers(Ar, alpha, pr, pr1);
     RowCoef o;
-    o.g_kl = 0.5f * inv_n * (pk + cpos + r.kl * alpha * pk1 / mk) + (r.kl == mk ? gmk : 0.f);
-    o.g_rkl = 0.5f * inv_n * (pr + cpos + r.rkl * alpha * pr1 / mr) + (r.rkl == mr ? gmr : 0.f);
+    o.g_kl = 0.5f * inv_n * (pk + cpos + r.kl * alpha * pk1 * inv_mk) + (r.kl == mk ? gmk : 0.f);
+    o.g_rkl = 0.5f * inv_n * (pr + cpos + r.rkl * alpha * pr1 * inv_mr) + (r.rkl == mr ? gmr : 0.f);
     o.g_own = g_own;
     o.pad = 0.f;
     coef[i] = o;
@@ -340,12 +206,7 @@ __global__ __launch_bounds__(CMP_NT) void composite_rows_bwd_kernel(const Compos
   float* gz = p.g_zk + i * K;
   float acc = 0.f;
   for (int k = lane; k < K; k += WAVE) {
-    const float t = load_as_float(p.t_val, p.t_val_dtype, i * K + k) * p.inv_T_t - r.t_lse;
-    const float s2 = z[k] - lse - r.s_lse;
-    // d kl / d s_k = -q_k ;  d rkl / d s_k = r_k ((s'_k - t_k) - rkl)
-    float gs = g.g_kl * (-expf(t)) + g.g_rkl * expf(s2) * ((s2 - t) - r.rkl);
-    if (k == r.kstar) gs += g.g_own;
-    gs = up == 0.f ? 0.f : gs * up;             // a conversation that is not part of the loss gets exact zeros, NaN or not
+    const float gs = composite_entry_grad(p, r, g, up, lse, i, k, z[k]);
     gz[k] = gs;
     acc += gs;
   }
@@ -402,13 +263,13 @@ static void set_offsets(dl::ConvoOffsets& off, const int32_t* row_off, const int
   }
 }
 
-extern "C" int dl_composite_forward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
-                                    float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
-                                    const int64_t* labels, const void* avoid, int avoid_itype, const int32_t* row_off,
-                                    const int32_t* label_off, const int32_t* avoid_off, int offsets_on_host, int n_convos,
-                                    int64_t n_rows, float alpha, void* row_records, void* row_coef, float* out,
-                                    void* stream) {
-  using namespace dl;
+namespace dl {
+
+int composite_forward_params(CompositeParams& p, const float* lse, const float* zk, const void* t_val, int t_val_dtype,
+                             float inv_T_teacher, const void* t_idx, int t_idx_itype, int K, const int64_t* labels,
+                             const void* avoid, int avoid_itype, const int32_t* row_off, const int32_t* label_off,
+                             const int32_t* avoid_off, int offsets_on_host, int n_convos, int64_t n_rows, float alpha,
+                             void* row_records, void* row_coef, float* out) {
   const int st0 = composite_check(lse, zk, t_val, t_val_dtype, t_idx, t_idx_itype, K, row_off, label_off, avoid_off,
                                   offsets_on_host, n_convos, n_rows, row_records);
   if (st0 != DL_OK) return st0;
@@ -417,16 +278,55 @@ extern "C" int dl_composite_forward(const float* lse, const float* zk, const voi
   if (offsets_on_host && ((label_off[n_convos] > label_off[0] && !labels) || (avoid_off[n_convos] > avoid_off[0] && !avoid)))
     return DL_ERR_NULL;                       // without labels / ignore entries the pointers may be NULL
   if (!offsets_on_host && (!labels || !avoid)) return DL_ERR_NULL;
-  CompositeParams p{};
+  p = CompositeParams{};
   p.lse = lse; p.zk = zk; p.t_val = t_val; p.t_val_dtype = t_val_dtype; p.inv_T_t = inv_T_teacher;
   p.t_idx = t_idx; p.t_idx_itype = t_idx_itype; p.K = K; p.labels = labels; p.avoid = avoid; p.avoid_itype = avoid_itype;
   set_offsets(p.off, row_off, label_off, avoid_off, offsets_on_host, n_convos);
   p.n_convos = n_convos; p.n_rows = n_rows;
   p.alpha = alpha; p.rec = reinterpret_cast<RowRec*>(row_records); p.coef = reinterpret_cast<RowCoef*>(row_coef);
   p.out = out;
+  return DL_OK;
+}
+
+int composite_backward_params(CompositeParams& p, const float* lse, const float* zk, const void* t_val, int t_val_dtype,
+                              float inv_T_teacher, const void* t_idx, int t_idx_itype, int K, const int32_t* row_off,
+                              int offsets_on_host, int n_convos, int64_t n_rows, const void* row_records,
+                              const void* row_coef, const float* g_train) {
+  const int st0 = composite_check(lse, zk, t_val, t_val_dtype, t_idx, t_idx_itype, K, row_off, row_off, row_off,
+                                  offsets_on_host, n_convos, n_rows, row_records);
+  if (st0 != DL_OK) return st0;
+  if (!row_coef || !g_train) return DL_ERR_NULL;
+  p = CompositeParams{};
+  p.lse = lse; p.zk = zk; p.t_val = t_val; p.t_val_dtype = t_val_dtype; p.inv_T_t = inv_T_teacher;
+  p.t_idx = t_idx; p.t_idx_itype = t_idx_itype; p.K = K; p.n_convos = n_convos; p.n_rows = n_rows;
+  set_offsets(p.off, row_off, row_off, row_off, offsets_on_host, n_convos);
+  p.rec = reinterpret_cast<RowRec*>(const_cast<void*>(row_records));
+  p.coef = reinterpret_cast<RowCoef*>(const_cast<void*>(row_coef));
+  p.g_train = g_train;
+  return DL_OK;
+}
+
+void launch_composite_convo(const CompositeParams& p, hipStream_t st) {
+  hipLaunchKernelGGL(composite_convo_kernel, dim3((unsigned)p.n_convos), dim3(CONVO_NT), 0, st, p);
+}
+
+}  // namespace dl
+
+extern "C" int dl_composite_forward(const float* lse, const float* zk, const void* t_val, int t_val_dtype,
+                                    float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
+                                    const int64_t* labels, const void* avoid, int avoid_itype, const int32_t* row_off,
+                                    const int32_t* label_off, const int32_t* avoid_off, int offsets_on_host, int n_convos,
+                                    int64_t n_rows, float alpha, void* row_records, void* row_coef, float* out,
+                                    void* stream) {
+  using namespace dl;
+  CompositeParams p;
+  const int st0 = composite_forward_params(p, lse, zk, t_val, t_val_dtype, inv_T_teacher, t_idx, t_idx_itype, K, labels, avoid,
+                                           avoid_itype, row_off, label_off, avoid_off, offsets_on_host, n_convos, n_rows,
+                                           alpha, row_records, row_coef, out);
+  if (st0 != DL_OK) return st0;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (n_rows > 0) launch_rows_fwd(p, st);
-  hipLaunchKernelGGL(composite_convo_kernel, dim3((unsigned)n_convos), dim3(CONVO_NT), 0, st, p);
+  launch_composite_convo(p, st);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
@@ -436,18 +336,13 @@ extern "C" int dl_composite_backward(const float* lse, const float* zk, const vo
                                      const void* row_records, const void* row_coef, const float* g_train, float* g_lse,
                                      float* g_zk, void* stream) {
   using namespace dl;
-  const int st0 = composite_check(lse, zk, t_val, t_val_dtype, t_idx, t_idx_itype, K, row_off, row_off, row_off,
-                                  offsets_on_host, n_convos, n_rows, row_records);
+  CompositeParams p;
+  const int st0 = composite_backward_params(p, lse, zk, t_val, t_val_dtype, inv_T_teacher, t_idx, t_idx_itype, K, row_off,
+                                            offsets_on_host, n_convos, n_rows, row_records, row_coef, g_train);
   if (st0 != DL_OK) return st0;
-  if (!row_coef || !g_train || !g_lse || !g_zk) return DL_ERR_NULL;
+  if (!g_lse || !g_zk) return DL_ERR_NULL;
   if (n_rows == 0) return DL_OK;
-  CompositeParams p{};
-  p.lse = lse; p.zk = zk; p.t_val = t_val; p.t_val_dtype = t_val_dtype; p.inv_T_t = inv_T_teacher;
-  p.t_idx = t_idx; p.t_idx_itype = t_idx_itype; p.K = K; p.n_convos = n_convos; p.n_rows = n_rows;
-  set_offsets(p.off, row_off, row_off, row_off, offsets_on_host, n_convos);
-  p.rec = reinterpret_cast<RowRec*>(const_cast<void*>(row_records));
-  p.coef = reinterpret_cast<RowCoef*>(const_cast<void*>(row_coef));
-  p.g_train = g_train; p.g_lse = g_lse; p.g_zk = g_zk;
+  p.g_lse = g_lse; p.g_zk = g_zk;
   hipLaunchKernelGGL(composite_rows_bwd_kernel, dim3((unsigned)((n_rows + CMP_ROWS_PER_WG - 1) / CMP_ROWS_PER_WG)),
                      dim3(CMP_NT), 0, reinterpret_cast<hipStream_t>(stream), p);
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;

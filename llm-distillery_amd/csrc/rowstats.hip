@@ -4,8 +4,7 @@
 //     grad[r, j] = ( a_r * softmax(z_r)_j + sum_k c_rk [j == idx_rk] ) * inv_T
 // where a_r = dL/d lse_r and c_rk = dL/d zk_rk.  Phase 1 is a read-only streaming reduction,
 // phase 2 an element-wise sweep (read row, write gradient) plus K sparse additions.
-#include "distill_common.hpp"
-#include "distill_hip.h"
+#include "composite.hpp"
 
 namespace dl {
 
@@ -50,8 +49,9 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int64_t ch = c0 + (int64_t)u * NT + tid;
-        // streamed, not cached: the K gathers above then fetch their lines a second time, but also where they are
-        // a fifth of the row (K = 400 on 32000 fp32 columns) the cached form is slower (53.5 against 50.5 us on 2048 rows)
+        // streamed, not cached: the K gathers above then fetch their lines a second time (9 of the kernel's 50 us on 2048
+        // rows of 32000 fp32 columns, K = 400), but the cached form is slower (53.5 us), and so is handing every id to the
+        // thread that sweeps its chunk, to be fetched right behind the chunk's own load (60 us)
         v[u] = ch < nch ? load16_stream(body + ch * 16) : C::neg_inf();
       }
       float cm = -INFINITY;
@@ -106,10 +106,13 @@ __device__ __forceinline__ float coef_on_id(const int* s_idx, const float* s_c, 
 // rows): the ragged chunk is loaded and converted like the others -- its 16 bytes start inside the row and,
 // aligned as they are, end inside the row's pitch or at least inside the page of the row's last column; what
 // lies behind the row is computed on and dropped -- and stored element by element.
-template <class Tag, int NT, int NCH, int MODE>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
-void rowcoef_grad_kernel(const StatsParams p, int parts) {
+// COMPOSITE: the coefficients are not read but made here, from the row's record and its conversation's
+// coefficients (composite_entry_grad; every part of a row makes all K of them, in the same order: the same bits),
+// which saves the launch that would write them and the row's coefficient on the log-sum-exp, their sum.
+template <class Tag, int NT, int NCH, int MODE, bool COMPOSITE>
+__device__ __forceinline__ void rowcoef_grad_part(const StatsParams& p, int parts, const CompositeParams* cp) {
   constexpr bool VEC = MODE != 0;
+  __shared__ float red[64];
   extern __shared__ __align__(16) unsigned char smem[];
   using C = Chunk<Tag>;
   const int Kp = (p.K + 15) & ~15;
@@ -151,8 +154,17 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     return;
   }
   const float a = p.inv_T * LOG2E;
-  const float b = p.lse[trow] * LOG2E;
-  const float w = p.coef_lse[trow] * p.inv_T;
+  const float lse = p.lse[trow];
+  const float b = lse * LOG2E;
+  float w = COMPOSITE ? 0.f : p.coef_lse[trow] * p.inv_T;
+  RowRec rec{};
+  RowCoef rc{};
+  float up = 0.f, acc = 0.f;
+  if constexpr (COMPOSITE) {
+    rec = cp->rec[trow];
+    rc = cp->coef[trow];
+    up = cp->g_train[convo_of_row(cp->off, cp->n_convos, trow)];
+  }
   // Teacher ids, their coefficients and the logits at the ids of this part go to LDS; issued behind
   // the row's own loads so that their latencies overlap instead of trailing the dense sweep.
   auto stage = [&]() {
@@ -164,7 +176,12 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
         id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
         in_row = id >= 0 && id < p.V;
         id -= shift;
-        cv = p.coef_zk[trow * p.K + k];
+        if constexpr (COMPOSITE) {
+          cv = composite_entry_grad(*cp, rec, rc, up, lse, trow, k, cp->zk[trow * p.K + k]);
+          acc += cv;
+        } else {
+          cv = p.coef_zk[trow * p.K + k];
+        }
       }
       const bool mine = in_row && id >= lo && id < hi;
       if (MODE == 2 && h == 0 && in_row && (id < 0 || id >= V)) {
@@ -192,6 +209,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     }
     correction_clear<NT>(s_head, s_own);
     stage();
+    if constexpr (COMPOSITE) w = -block_sum<NT>(acc, red) * p.inv_T;      // s_k = z_k - lse: d / d lse = -sum_k
     __syncthreads();
     // dense part of the columns that carry a teacher entry, handed to the threads that hold them
     for (int k = tid; k < Kp; k += NT) {
@@ -231,6 +249,7 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     return;
   } else {
     stage();
+    if constexpr (COMPOSITE) w = -block_sum<NT>(acc, red) * p.inv_T;
     for (int64_t j = lo + tid; j < hi; j += NT)
       store_from_float(grow, Tag::id, j, fast_exp2(fmaf(load_as_float(row, Tag::id, j), a, -b)) * w);
   }
@@ -241,6 +260,17 @@ void rowcoef_grad_kernel(const StatsParams p, int parts) {
     const float dense = fast_exp2(fmaf(s_z[k], a, -b)) * w;
     store_from_float(grow, Tag::id, id, dense + coef_on_id(s_idx, s_c, Kp, k, id) * p.inv_T);
   }
+}
+
+template <class Tag, int NT, int NCH, int MODE>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+void rowcoef_grad_kernel(const StatsParams p, int parts) {
+  rowcoef_grad_part<Tag, NT, NCH, MODE, false>(p, parts, nullptr);
+}
+template <class Tag, int NT, int NCH, int MODE>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+void rowcoef_composite_kernel(const StatsParams p, int parts, const CompositeParams cp) {
+  rowcoef_grad_part<Tag, NT, NCH, MODE, true>(p, parts, &cp);
 }
 
 static bool aligned16(const void* ptr, int64_t stride, int eb) {
@@ -262,7 +292,7 @@ static hipError_t launch_stats(const StatsParams& p, int mode, hipStream_t st) {
 }
 
 template <class Tag>
-static hipError_t launch_coef(const StatsParams& p, int mode, hipStream_t st) {
+static hipError_t launch_coef(const StatsParams& p, int mode, hipStream_t st, const CompositeParams* cp = nullptr) {
   // 4 chunks per thread: this kernel keeps nothing of the row beyond the chunk it is converting, and a
   // stream that moves few chunks per thread between its loads and its stores runs 6-9 % faster on this
   // device than one that moves 16 (measured on a plain copy as well: 78 % against 70 % of peak)
@@ -271,6 +301,13 @@ static hipError_t launch_coef(const StatsParams& p, int mode, hipStream_t st) {
   const int parts = (int)((p.V + per_part - 1) / per_part);
   const size_t lds = (size_t)((p.K + 15) & ~15) * 20 + (size_t)CORRECTION_HEADS * 4 + (size_t)NT * 4;   // ids, coefficients, logits, values, links; list heads, chunk masks
   const dim3 grid((unsigned)((p.n_rows + 7) / 8 * 8 * parts));
+  if (cp) {
+    if (mode == 1) hipLaunchKernelGGL((rowcoef_composite_kernel<Tag, NT, NCH, 1>), grid, dim3(NT), lds, st, p, parts, *cp);
+    else if (mode == 2) hipLaunchKernelGGL((rowcoef_composite_kernel<Tag, NT, NCH, 2>), grid, dim3(NT), lds, st, p, parts, *cp);
+    else if (mode == 3) hipLaunchKernelGGL((rowcoef_composite_kernel<Tag, NT, NCH, 3>), grid, dim3(NT), lds, st, p, parts, *cp);
+    else hipLaunchKernelGGL((rowcoef_composite_kernel<Tag, NT, NCH, 0>), grid, dim3(NT), lds, st, p, parts, *cp);
+    return hipGetLastError();
+  }
   if (mode == 1) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 1>), grid, dim3(NT), lds, st, p, parts);
   else if (mode == 2) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 2>), grid, dim3(NT), lds, st, p, parts);
   else if (mode == 3) hipLaunchKernelGGL((rowcoef_grad_kernel<Tag, NT, NCH, 3>), grid, dim3(NT), lds, st, p, parts);
@@ -329,5 +366,34 @@ extern "C" int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_
   const hipError_t e = logits_dtype == DL_F32 ? launch_coef<TagF32>(p, vec, st)
                        : logits_dtype == DL_BF16 ? launch_coef<TagBF16>(p, vec, st)
                                                  : launch_coef<TagF16>(p, vec, st);
+  return e == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}
+
+extern "C" int dl_composite_backward_fused(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
+                                           int64_t V, float inv_T, const void* t_val, int t_val_dtype,
+                                           float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
+                                           const int32_t* row_off, int offsets_on_host, int n_convos, const float* lse,
+                                           const float* zk, const void* row_records, const void* row_coef,
+                                           const float* g_train, void* grad, int64_t grad_stride, void* stream) {
+  using namespace dl;
+  const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_rows);
+  if (rc != DL_OK) return rc;
+  CompositeParams cp;
+  const int st0 = composite_backward_params(cp, lse, zk, t_val, t_val_dtype, inv_T_teacher, t_idx, t_idx_itype, K, row_off,
+                                            offsets_on_host, n_convos, n_rows, row_records, row_coef, g_train);
+  if (st0 != DL_OK) return st0;
+  if (!grad) return DL_ERR_NULL;
+  if (grad_stride < V) return DL_ERR_SHAPE;
+  if (n_rows == 0) return DL_OK;
+  const int eb = logits_dtype == DL_F32 ? 4 : 2;
+  if (reinterpret_cast<uintptr_t>(logits) % eb != 0 || reinterpret_cast<uintptr_t>(grad) % eb != 0) return DL_ERR_ALIGN;
+  const bool on_grid = aligned16(logits, row_stride, eb) && aligned16(grad, grad_stride, eb);
+  const int vec = on_grid ? (V % (16 / eb) == 0 ? 1 : 3) : same_phase16(logits, row_stride, grad, grad_stride, eb) ? 2 : 0;
+  StatsParams p{logits, row_stride, n_rows, V, nullptr, t_idx, t_idx_itype, K, n_rows, inv_T,
+                const_cast<float*>(lse), nullptr, nullptr, nullptr, grad, grad_stride};
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const hipError_t e = logits_dtype == DL_F32 ? launch_coef<TagF32>(p, vec, st, &cp)
+                       : logits_dtype == DL_BF16 ? launch_coef<TagBF16>(p, vec, st, &cp)
+                                                 : launch_coef<TagF16>(p, vec, st, &cp);
   return e == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }

@@ -388,13 +388,21 @@ def _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, o
     lib = _lib.load()
     offs, on_host, C = _offsets_arg(offsets)
     g = g_train.to(torch.float32).contiguous()
-    g_lse = torch.empty_like(lse)
-    g_zk = torch.empty_like(zk)
     grad = torch.empty_like(logits)                      # full width; the kernel fills [:, :crop]
     if x is not logits:
         grad[:, crop:].zero_()
     gx = _cropped(grad, crop)
     stream = _stream_ptr(dev)
+    if row_map is None and N == R:                       # teacher row i belongs to logits row i: one launch
+        with torch.cuda.device(dev):
+            st = lib.dl_composite_backward_fused(
+                x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, inv_T, t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher,
+                t_idx.data_ptr(), _IT[t_idx.dtype], K, offs[0], on_host, C, lse.data_ptr(), zk.data_ptr(), rec.data_ptr(),
+                coef.data_ptr(), g.data_ptr(), gx.data_ptr(), gx.stride(0), stream)
+            _lib.check(st, "dl_composite_backward_fused")
+        return grad
+    g_lse = torch.empty_like(lse)
+    g_zk = torch.empty_like(zk)
     with torch.cuda.device(dev):
         st = lib.dl_composite_backward(
             lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),

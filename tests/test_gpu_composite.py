@@ -400,3 +400,77 @@ def test_fused_epilogue_under_no_grad_and_label_count_mismatch(D):
     # as many labels as rows: the reference raises (empty crop); so does the drop-in, from the same torch ops
     with pytest.raises(RuntimeError):
         D.calculate_divergence(z, tv.float().to(DEV), ti.to(DEV), torch.cat([labels, labels[:1]]).to(DEV), 2.0, avoid.to(DEV))
+
+
+@pytest.mark.parametrize("dtype,V,pitch,K,lens,host_offsets", [
+    (torch.float32, 32000, 32000, 400, [130], True),            # the reference's default width and K, one conversation
+    (torch.bfloat16, 5001, 5120, 37, [20, 1, 33], False),       # a crop of padded rows, K off the wave size, device offsets
+    (torch.float16, 1003, 1003, 16, [9, 40], True),             # rows off the 16-byte grid
+    (torch.bfloat16, 128256, 128256, 200, [5, 6], True),
+    (torch.float32, 4096, 4096, 600, [12, 7], True)])
+def test_coefficients_made_inside_phase_two_equal_the_separate_launches(D, dtype, V, pitch, K, lens, host_offsets):
+    """Without a row map phase 2 makes the K coefficients of a row itself (dl_composite_backward_fused); an identity
+    row map sends the same problem through the separate launches.  Forward: the same launches, the same bits.
+    Backward: the sum of the K coefficients is taken in another order, so the gradients agree to fp32 rounding of
+    the dense term."""
+    from llm_distillery_amd import ops
+    N = sum(lens)
+    g = torch.Generator().manual_seed(V + K)
+    xs = (torch.randn(N, V, generator=g) * 2).to(dtype)
+    tfull = torch.log_softmax(xs.float() + torch.randn(N, V, generator=g), -1)
+    tv, ti = torch.topk(tfull, K)
+    tv = tv.to(torch.float16).contiguous()
+    labels, row_off, label_off, avoid_off, avoid = [], [0], [0], [0], []
+    for n in lens:
+        r0 = row_off[-1]
+        lab = ti[r0:r0 + n - 1, 0].clone()
+        miss = torch.rand(max(n - 1, 0), generator=g) < 0.3
+        lab[miss] = torch.randint(0, V, (int(miss.sum()),), generator=g)
+        labels.append(lab)
+        row_off.append(r0 + n)
+        label_off.append(label_off[-1] + n - 1)
+        if n > 4:
+            avoid.append(n // 2)
+        avoid_off.append(len(avoid))
+    labels = torch.cat(labels).to(DEV)
+    avoid = torch.tensor(avoid, dtype=torch.int64, device=DEV)
+    offsets = [row_off, label_off, avoid_off]
+    if not host_offsets:
+        offsets = torch.tensor(offsets, dtype=torch.int32, device=DEV)
+    full = torch.zeros(N, pitch, dtype=dtype, device=DEV)
+    full[:, :V] = xs.to(DEV)
+    ident = torch.arange(N, dtype=torch.int32, device=DEV)
+    res = {}
+    for name, rm in (("fused", None), ("separate", ident)):
+        x = full.clone().requires_grad_(True)
+        train, nine = ops.composite_loss(x, tv.to(DEV), ti.to(DEV), labels, avoid, offsets, rm, 1.0 / 1.3, 1.0, 2.0, crop=V if pitch != V else 0)
+        w = torch.arange(1, len(lens) + 1, dtype=torch.float32, device=DEV)
+        (train * w).sum().backward()
+        res[name] = (train.detach(), nine, x.grad)
+    same = lambda a, b: torch.equal(a.nan_to_num(nan=-7.0), b.nan_to_num(nan=-7.0))      # a conversation of one row has no labels: its CE means are 0 / 0
+    assert same(res["fused"][0], res["separate"][0]) and same(res["fused"][1], res["separate"][1])
+    gf, gs = res["fused"][2].float(), res["separate"][2].float()
+    assert torch.count_nonzero(gf[:, V:]) == 0
+    tol = gs.abs() * (2e-5 if dtype == torch.float32 else 2.0 ** -7) + gs.abs().amax(-1, keepdim=True) * 1e-6
+    assert ((gf - gs).abs() <= tol).all(), ((gf - gs).abs() / tol).max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_phase_one_logits_at_clustered_repeated_and_outlying_teacher_ids(D, dtype):
+    """Rows whose ids all fall on every 256th chunk, rows with one id K times, ids in the first and the last column
+    and ids outside the row: zk bit for bit the gathered logits times 1/T, zeros for ids outside."""
+    from llm_distillery_amd import ops
+    R, V, K = 6, 32768, 40
+    n = 16 // torch.empty(0, dtype=dtype).element_size()           # columns per 16-byte chunk
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(R, V, generator=g) * 3).to(dtype)
+    idx = torch.randint(0, V, (R, K), generator=g, dtype=torch.int64)
+    idx[0] = (torch.arange(K) % (V // (256 * n))) * 256 * n + 5 * n + 1      # every 256th chunk (some ids twice)
+    idx[1] = idx[1, 0]                                                      # one id K times
+    idx[2, :4] = torch.tensor([0, V - 1, -1, V])                            # first and last column, two ids outside the row
+    idx[3] = torch.arange(K) * n                                           # consecutive chunks, one id each
+    lse, zk = ops._rowstats_raw(x.to(DEV), idx.to(DEV), None, 0.7)
+    inside = (idx >= 0) & (idx < V)
+    want = torch.where(inside, torch.gather(x.float(), 1, idx.clamp(0, V - 1)) * 0.7, torch.zeros(()))
+    assert torch.equal(zk.cpu(), want)
+    np.testing.assert_allclose(lse.cpu().double().numpy(), torch.logsumexp(x.double() * 0.7, -1).numpy(), rtol=2e-6, atol=2e-6)
