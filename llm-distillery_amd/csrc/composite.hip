@@ -35,16 +35,8 @@ template <int NT, int N>
 __device__ __forceinline__ void block_sums_f64(double (&v)[N], double* scratch) {
   constexpr int NW = NT / WAVE;
   const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
-  // step by step for all N sums together: the N exchanges of a step are in flight at once (sum by sum, every
-  // exchange would wait for the one before it: N times the latency for the same additions in the same order)
 #pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) {
-    double t[N];
-#pragma unroll
-    for (int k = 0; k < N; ++k) t[k] = __shfl_xor(v[k], o, WAVE);
-#pragma unroll
-    for (int k = 0; k < N; ++k) v[k] += t[k];
-  }
+  for (int k = 0; k < N; ++k) v[k] = wave_sum(v[k]);
   if (lane == 0) {
 #pragma unroll
     for (int k = 0; k < N; ++k) scratch[k * NW + w] = v[k];

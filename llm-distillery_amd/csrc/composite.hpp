@@ -34,11 +34,7 @@ struct CompositeParams {
   const float* g_train; float* g_lse; float* g_zk;
 };
 
-__device__ __forceinline__ int wave_min_int(int v) {
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, WAVE));
-  return v;
-}
+__device__ __forceinline__ int wave_min_int(int v) { return wave_min(v); }
 
 // conversation that holds row i: last c whose first row is <= i
 __device__ __forceinline__ int convo_of_row(const ConvoOffsets& off, int n_convos, int64_t i) {

@@ -301,16 +301,85 @@ __device__ __forceinline__ int64_t xcd_banded_row(unsigned b) {
 }
 static inline unsigned xcd_banded_grid(int64_t n_rows) { return (unsigned)((n_rows + 63) / 64 * 64); }
 
-// ---- reductions: fixed butterfly order => bit-reproducible ----------------------
+// ---- reductions: fixed order => bit-reproducible ---------------------------------
+// Over the 64 lanes of a wave (all of them active), result in every lane.  Data-parallel-primitive moves
+// instead of lane exchanges through the LDS crossbar (six round trips of ~100 cycles each for a butterfly): the
+// operand of each step comes through the ALU's own lane permutation -- neighbours inside a quad, quads inside
+// half a row of 16, halves, then lane 15 of a row into the next row and lane 31 into the upper half -- after
+// which lane 63 holds the total, read out as a scalar.  The order of the additions is fixed by the pattern.
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_move(float old, float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+constexpr int DPP_QUAD_XOR1 = 0xB1, DPP_QUAD_XOR2 = 0x4E, DPP_ROW_HALF_MIRROR = 0x141, DPP_ROW_MIRROR = 0x140,
+              DPP_ROW_BCAST15 = 0x142, DPP_ROW_BCAST31 = 0x143;
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
-  return v;
+  v = fmaxf(v, dpp_move<DPP_QUAD_XOR1>(v, v));
+  v = fmaxf(v, dpp_move<DPP_QUAD_XOR2>(v, v));
+  v = fmaxf(v, dpp_move<DPP_ROW_HALF_MIRROR>(v, v));
+  v = fmaxf(v, dpp_move<DPP_ROW_MIRROR>(v, v));
+  v = fmaxf(v, dpp_move<DPP_ROW_BCAST15, 0xa>(v, v));      // rows 1 and 3 take in rows 0 and 2 (the others keep their own)
+  v = fmaxf(v, dpp_move<DPP_ROW_BCAST31, 0xc>(v, v));      // rows 2 and 3 take in rows 0-1
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), WAVE - 1));
+}
+// The same moves for other types: `from(old, v)` = v of the lane the step reads, or `old` where the step leaves the lane out.
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ int dpp_move(int old, int v) { return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, 0xf, false); }
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ double dpp_move(double old, double v) {
+  const unsigned long long o = __builtin_bit_cast(unsigned long long, old), x = __builtin_bit_cast(unsigned long long, v);
+  const unsigned lo = (unsigned)__builtin_amdgcn_update_dpp((int)(unsigned)o, (int)(unsigned)x, CTRL, ROW_MASK, 0xf, false);
+  const unsigned hi = (unsigned)__builtin_amdgcn_update_dpp((int)(unsigned)(o >> 32), (int)(unsigned)(x >> 32), CTRL, ROW_MASK, 0xf, false);
+  return __builtin_bit_cast(double, ((unsigned long long)hi << 32) | lo);
+}
+// The six steps with any commutative op; lanes that a step leaves out combine with their own value (`self`: min,
+// max) or with `neutral` (sums).
+template <class T, class Op>
+__device__ __forceinline__ T wave_reduce_lane63(T v, T neutral, bool self, Op op) {
+  v = op(v, dpp_move<DPP_QUAD_XOR1>(self ? v : neutral, v));
+  v = op(v, dpp_move<DPP_QUAD_XOR2>(self ? v : neutral, v));
+  v = op(v, dpp_move<DPP_ROW_HALF_MIRROR>(self ? v : neutral, v));
+  v = op(v, dpp_move<DPP_ROW_MIRROR>(self ? v : neutral, v));
+  v = op(v, dpp_move<DPP_ROW_BCAST15, 0xa>(self ? v : neutral, v));
+  v = op(v, dpp_move<DPP_ROW_BCAST31, 0xc>(self ? v : neutral, v));
+  return v;                                    // lane 63 holds the result
+}
+__device__ __forceinline__ int wave_min(int v) {
+  v = wave_reduce_lane63(v, 0, true, [](int a, int b) { return a < b ? a : b; });
+  return __builtin_amdgcn_readlane(v, WAVE - 1);
+}
+__device__ __forceinline__ int wave_max(int v) {
+  v = wave_reduce_lane63(v, 0, true, [](int a, int b) { return a > b ? a : b; });
+  return __builtin_amdgcn_readlane(v, WAVE - 1);
+}
+__device__ __forceinline__ unsigned wave_max(unsigned v) {
+  int x = (int)v;
+  x = wave_reduce_lane63(x, 0, true, [](int a, int b) { return (unsigned)a > (unsigned)b ? a : b; });
+  return (unsigned)__builtin_amdgcn_readlane(x, WAVE - 1);
+}
+__device__ __forceinline__ unsigned wave_min(unsigned v) {
+  int x = (int)v;
+  x = wave_reduce_lane63(x, 0, true, [](int a, int b) { return (unsigned)a < (unsigned)b ? a : b; });
+  return (unsigned)__builtin_amdgcn_readlane(x, WAVE - 1);
+}
+__device__ __forceinline__ int wave_sum(int v) {
+  v = wave_reduce_lane63(v, 0, false, [](int a, int b) { return a + b; });
+  return __builtin_amdgcn_readlane(v, WAVE - 1);
+}
+__device__ __forceinline__ double wave_sum(double v) {
+  v = wave_reduce_lane63(v, 0.0, false, [](double a, double b) { return a + b; });
+  const unsigned long long x = __builtin_bit_cast(unsigned long long, v);
+  const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)x, WAVE - 1), hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(x >> 32), WAVE - 1);
+  return __builtin_bit_cast(double, ((unsigned long long)hi << 32) | lo);
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
+  v += dpp_move<DPP_QUAD_XOR1>(0.f, v);
+  v += dpp_move<DPP_QUAD_XOR2>(0.f, v);
+  v += dpp_move<DPP_ROW_HALF_MIRROR>(0.f, v);
+  v += dpp_move<DPP_ROW_MIRROR>(0.f, v);
+  v += dpp_move<DPP_ROW_BCAST15, 0xa>(0.f, v);
+  v += dpp_move<DPP_ROW_BCAST31, 0xc>(0.f, v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), WAVE - 1));
 }
 
 // All threads of the workgroup receive the result.  `scratch` holds NT/64 floats;

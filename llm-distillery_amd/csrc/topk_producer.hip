@@ -123,8 +123,7 @@ template <> struct Keys<TagF16> : Keys16<false> {};
 template <int NT>
 __device__ __forceinline__ int block_sum_int(int v, int* scratch) {
   constexpr int NW = NT / WAVE;
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  v = wave_sum(v);
   const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
   if (lane == 0) scratch[w] = v;
   __syncthreads();
@@ -139,8 +138,7 @@ __device__ __forceinline__ int block_sum_int(int v, int* scratch) {
 template <int NT>
 __device__ __forceinline__ int block_max_int(int v, int* scratch) {
   constexpr int NW = NT / WAVE;
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, WAVE));
+  v = wave_max(v);
   const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
   if (lane == 0) scratch[w] = v;
   __syncthreads();
@@ -416,8 +414,7 @@ void topk_part_kernel(const ProducerParams p) {
         unsigned top = 0u;
 #pragma unroll
         for (int j = 0; j < G * NW; ++j) top = max(top, v[j]);
-#pragma unroll
-        for (int o = WAVE / 2; o > 0; o >>= 1) top = max(top, (unsigned)__shfl_xor((int)top, o, WAVE));
+        top = wave_max(top);
         const unsigned pre = top & ~((1u << (KY::BITS - 6)) - 1u);
         int cpre = 0;
 #pragma unroll
@@ -637,8 +634,7 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p)
   };
   unsigned best = 0xffffffffu;
   for (int a = tid; a < total; a += 256) best = min(best, (unsigned)(all[a] >> 32));
-#pragma unroll
-  for (int o = WAVE / 2; o > 0; o >>= 1) best = min(best, (unsigned)__shfl_xor((int)best, o, WAVE));
+  best = wave_min(best);
   if (lane == 0) s_best[w] = best;
   __syncthreads();
   best = min(min(s_best[0], s_best[1]), min(s_best[2], s_best[3]));
