@@ -43,6 +43,7 @@ struct ProducerParams {
   int K; int parts;
   char* ws; int64_t part_stride;            // bytes per (row, part) record
   void* out_val; int out_dtype; void* out_idx; int out_itype;
+  unsigned* redo_count; int32_t* redo_rows; // behind the records: output rows the row-level selection hands back
 };
 
 // Entries a part record can hold: a part with no more candidates than this hands all of them,
@@ -68,8 +69,13 @@ __host__ __device__ inline int producer_merge_slots(int K, int parts) {
   while (n2 < parts * producer_record_cap(K, parts)) n2 <<= 1;
   return n2;
 }
-__host__ __device__ inline int64_t producer_part_stride(int K, int parts) {
-  return 16 + (((int64_t)producer_record_cap(K, parts) * 8 + 15) & ~15LL);
+// Chunk groups per thread of the part kernel: 1024 groups per part for K <= 256, else one per chunk (4096).
+__host__ __device__ inline int producer_groups(int K) { return K <= 256 ? PROD_G_SMALL : PROD_G_LARGE; }
+// A (row, part) record: 16-byte header, then either the part's candidates (8 bytes each) or the largest key of
+// each of its chunk groups (key_bytes each).
+__host__ __device__ inline int64_t producer_part_stride(int K, int parts, int key_bytes) {
+  const int64_t cands = (int64_t)producer_record_cap(K, parts) * 8, maxima = (int64_t)producer_groups(K) * PROD_NT * key_bytes;
+  return 16 + (((cands > maxima ? cands : maxima) + 15) & ~15LL);
 }
 
 // ---- order-preserving keys ---------------------------------------------------------------------
@@ -77,6 +83,7 @@ __host__ __device__ inline int64_t producer_part_stride(int K, int parts) {
 template <class Tag> struct Keys;
 
 template <> struct Keys<TagF32> {
+  typedef unsigned Stored;
   static constexpr int BITS = 32;
   static constexpr int PER_DWORD = 1;
   __device__ static __forceinline__ unsigned encode(unsigned u) {      // dword of raw bits -> dword of keys
@@ -93,6 +100,7 @@ template <> struct Keys<TagF32> {
 };
 
 template <bool IS_BF16> struct Keys16 {
+  typedef unsigned short Stored;
   static constexpr int BITS = 16;
   static constexpr int PER_DWORD = 2;
   __device__ static __forceinline__ unsigned encode(unsigned u) {
@@ -270,15 +278,35 @@ __device__ __forceinline__ int64_t producer_row(const ProducerParams& p, int64_t
   return (r >= 0 && r < p.n_rows) ? r : -1;
 }
 
+// Chunk c of a part that starts at rpart and holds n_elems columns in nch chunks (beyond them: -inf).  ALIGNED: rows
+// on the 16-byte grid that hold a whole number of chunks.  Otherwise only a last chunk that the row does not fill is put
+// together element by element; the others come by 16-byte loads, from rows off the grid (`on_grid` false) by unaligned
+// ones (which the device takes).
+template <class Tag, bool ALIGNED>
+__device__ __forceinline__ u32x4 producer_load_chunk(const char* rpart, int c, int nch, int n_elems, bool on_grid) {
+  using C = Chunk<Tag>;
+  if constexpr (ALIGNED) {
+    return c < nch ? load16_stream(rpart + (int64_t)c * 16) : C::neg_inf();
+  } else {
+    const bool whole = (c + 1) * C::N <= n_elems;
+    return c >= nch ? C::neg_inf()
+           : !whole ? load_chunk_elementwise<Tag>(rpart, c, n_elems)
+           : on_grid ? load16_stream(rpart + (int64_t)c * 16) : load16_unaligned(rpart + (int64_t)c * 16);
+  }
+}
+
+constexpr int PART_FULL = 0;    // threshold, candidates and record of the part: all the part kernel's stages
+constexpr int PART_LIGHT = 1;   // statistics and chunk-group maxima only: the candidates are picked per row (topk_select_kernel)
+constexpr int PART_REDO = 2;    // PART_FULL for the rows the row-level selection handed back
+
 // G = chunk groups per thread whose maxima feed the threshold search: 256 * G groups per part must
 // be a few times K for the candidate set to stay close to K (4 for K <= 256, else 16).
 // ALIGNED: rows start on 16-byte boundaries and hold a whole number of chunks (16-byte loads);
 // otherwise the chunks are assembled element by element and the last one is padded with -inf,
 // which the collection leaves out (a padding entry has the lowest key and the highest columns of
 // its part, so the threshold searches, which only count, need no such test).
-template <class Tag, int G, bool ALIGNED>
-__global__ __launch_bounds__(PROD_NT) __attribute__((amdgpu_waves_per_eu(PROD_NT / 64, 8)))
-void topk_part_kernel(const ProducerParams p) {
+template <class Tag, int G, bool ALIGNED, int MODE>
+__device__ __forceinline__ void topk_part(const ProducerParams& p, int64_t ro, int h_part) {
   constexpr int NT = PROD_NT, NCH = PROD_NCH, NW = NT / WAVE, CPG = NCH / G;
   using C = Chunk<Tag>;
   using KY = Keys<Tag>;
@@ -293,12 +321,6 @@ void topk_part_kernel(const ProducerParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), w = tid / WAVE;
   const int P = p.parts;
-  // Workgroup ids are dealt round-robin to the 8 XCDs: within a group of 8 * P ids, id t serves
-  // row 8 * group + t % 8, part t / 8, so the parts of a row run on one XCD back to back.
-  const unsigned grp = blockIdx.x / (8u * P), t_in = blockIdx.x % (8u * P);
-  const int64_t ro = (int64_t)grp * 8 + (t_in & 7u);
-  const int h_part = (int)(t_in >> 3);
-  if (ro >= p.n_out) return;
   const int64_t r = producer_row(p, ro);
   if (r < 0) return;                                                 // masked output row: the merge kernel fills it
   const int64_t c0 = (int64_t)h_part * NT * NCH;
@@ -314,19 +336,7 @@ void topk_part_kernel(const ProducerParams p) {
   u32x4 reg[NCH];
   const bool on_grid = (reinterpret_cast<uintptr_t>(rpart) & 15) == 0;      // the same for the whole workgroup
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = i * NT + tid;
-    if constexpr (ALIGNED) {
-      reg[i] = c < nch ? load16_stream(rpart + (int64_t)c * 16) : C::neg_inf();
-    } else {
-      // only a last chunk that the row does not fill is put together element by element; the others
-      // come by 16-byte loads, from rows off the 16-byte grid by unaligned ones (which the device takes)
-      const bool whole = (c + 1) * C::N <= n_elems;
-      reg[i] = c >= nch ? C::neg_inf()
-               : !whole ? load_chunk_elementwise<Tag>(rpart, c, n_elems)
-               : on_grid ? load16_stream(rpart + (int64_t)c * 16) : load16_unaligned(rpart + (int64_t)c * 16);
-    }
-  }
+  for (int i = 0; i < NCH; ++i) reg[i] = producer_load_chunk<Tag, ALIGNED>(rpart, i * NT + tid, nch, n_elems, on_grid);
   if (tid == 0) s_n = 0;
 
   // max and sum-exp of the part (natural log-softmax; no temperature at collection time)
@@ -375,8 +385,36 @@ void topk_part_kernel(const ProducerParams p) {
   }
   sm = block_sum<NT>(sm, red);
 
-  // raw bits -> ordered keys, in place; largest key of every chunk group
   const int my_chunks = (nch - tid + NT - 1) / NT;                  // chunks i < my_chunks are inside the part
+  if constexpr (MODE == PART_LIGHT) {
+    // Largest key of every chunk group, nothing else.  A group here is what the selection reads again: with four
+    // chunks per group, the chunks that four neighbouring threads hold in the same register (64 contiguous bytes of
+    // the row: one access); the group's maximum is taken across the quad.  One chunk per group: the thread's own.
+    if (tid == 0) {
+      PartHeader hd{mx, sm, -1, 0};
+      *reinterpret_cast<PartHeader*>(rec) = hd;
+    }
+    typedef typename KY::Stored KS;
+    KS* gout = reinterpret_cast<KS*>(rec + 16);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      forget(reg[i]);
+      unsigned e[4];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) e[d] = KY::encode(reg[i][d]);
+      unsigned k = i < my_chunks ? KY::top_key(KY::dword_max(KY::dword_max(e[0], e[1]), KY::dword_max(e[2], e[3]))) : 0u;      // 0: no chunk of the part
+      if constexpr (CPG == 4) {
+        k = max(k, (unsigned)dpp_move<DPP_QUAD_XOR1>((int)k, (int)k));
+        k = max(k, (unsigned)dpp_move<DPP_QUAD_XOR2>((int)k, (int)k));
+        if ((tid & 3) == (i & 3)) gout[i * (NT / 4) + (tid >> 2)] = (KS)k;
+      } else {
+        static_assert(CPG == 1 || CPG == 4, "chunk groups: a thread's chunk, or a quad's four");
+        gout[i * NT + tid] = (KS)k;
+      }
+    }
+    return;
+  }
+  // raw bits -> ordered keys, in place; largest key of every chunk group
   unsigned gm[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
@@ -553,6 +591,29 @@ void topk_part_kernel(const ProducerParams p) {
   }
 }
 
+// Workgroup ids are dealt round-robin to the 8 XCDs: within a group of 8 * P ids, id t serves row (or, PART_REDO,
+// entry of the list of rows handed back) 8 * group + t % 8, part t / 8, so the parts of a row run on one XCD back to
+// back.  PART_REDO: a small grid whose workgroups walk the list, which is empty as a rule.
+template <class Tag, int G, bool ALIGNED, int MODE>
+__global__ __launch_bounds__(PROD_NT) __attribute__((amdgpu_waves_per_eu(PROD_NT / 64, 8)))
+void topk_part_kernel(const ProducerParams p) {
+  const unsigned P = (unsigned)p.parts;
+  const unsigned grp = blockIdx.x / (8u * P), t_in = blockIdx.x % (8u * P);
+  const int64_t slot = (int64_t)grp * 8 + (t_in & 7u);
+  const int h_part = (int)(t_in >> 3);
+  if constexpr (MODE == PART_REDO) {
+    const int64_t n = min((int64_t)*p.redo_count, p.n_out), step = (int64_t)(gridDim.x / (8u * P)) * 8;
+    for (int64_t e = slot; e < n; e += step) {
+      topk_part<Tag, G, ALIGNED, MODE>(p, p.redo_rows[e], h_part);
+      __syncthreads();                                               // the next row reuses the workgroup's LDS
+    }
+  } else {
+    if (slot >= p.n_out) return;
+    if (MODE == PART_LIGHT && blockIdx.x == 0 && threadIdx.x == 0) *p.redo_count = 0u;      // the selection, the next launch, appends to the list
+    topk_part<Tag, G, ALIGNED, MODE>(p, slot, h_part);
+  }
+}
+
 // Emits sorted words [0, K) held as element e = lane * EPL + j of one wave.
 template <class Tag, int EPL>
 __device__ __forceinline__ void emit_sorted(const ProducerParams& p, int64_t ro, float lse, const u64 (&c)[EPL]) {
@@ -570,51 +631,39 @@ __device__ __forceinline__ void emit_sorted(const ProducerParams& p, int64_t ro,
   }
 }
 
-// Merge of the parts of one row: log-sum-exp from the part statistics, and the K best of the parts'
-// candidates.  Words sort ascending = key descending, column ascending, and no two are equal (the
-// column is part of the word).  The K-th smallest high word (= K-th largest key) is found bit by
-// bit; the words at or below it (K plus ties) are compacted and sorted by one wave in registers.
-// More than 512 of them (a tie plateau): everything is sorted in LDS instead.
+// The K best of `total` candidate words (LDS) to the output row.  Words sort ascending = key descending, column
+// ascending, and no two are equal (the column is part of the word).  The K-th smallest high word (= K-th
+// largest key) is found bit by bit; the words at or below it (K plus ties) are compacted and sorted by one wave in
+// registers.  More than 512 of them (a tie plateau): everything is sorted in LDS instead.  256 threads, all of
+// them; s_nsel zero and `all` complete behind a barrier on entry.
+struct SelectLds { int slots[2 * 4]; unsigned best[4]; int nsel; };
 template <class Tag>
-__global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p) {
-  extern __shared__ __align__(16) unsigned char smem_raw[];
-  u64* all = reinterpret_cast<u64*>(smem_raw);                      // the parts' records; producer_merge_slots words
-  __shared__ int slots[2 * 4];
-  __shared__ unsigned s_best[4];
-  __shared__ int s_nsel;
+__device__ __forceinline__ void select_and_emit(const ProducerParams& p, int64_t ro, float lse, u64* all, u64* sel, int total,
+                                                int sel_cap, SelectLds& sh) {
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), w = tid / WAVE;
-  const int64_t ro = blockIdx.x;
-  const int P = p.parts, K = p.K;
-  const int capw = producer_record_cap(K, P);
-  const int sel_cap = producer_sel_cap(K);
-  u64* sel = all + producer_merge_slots(K, P);                      // the selected words; sel_cap words
-  const char* rec0 = p.ws + ro * P * p.part_stride;
-  if (producer_row(p, ro) < 0) {                                    // the row list names no logits row: masked output row
-    for (int k = tid; k < K; k += 256) {
-      store_from_float(p.out_val, p.out_dtype, ro * K + k, -INFINITY);
-      if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * K + k] = -1;
-      else reinterpret_cast<int64_t*>(p.out_idx)[ro * K + k] = -1;
+  const int K = p.K;
+  int* slots = sh.slots;
+  unsigned* s_best = sh.best;
+  int& s_nsel = sh.nsel;
+  if (total <= 512) {            // few enough for one wave's registers: sorted as they are (the same for every thread)
+    if (w == 0) {
+      if (total <= 256) {
+        u64 c[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = lane * 4 + j < total ? all[lane * 4 + j] : ~0ull;
+        wave_sort<u64, 4>(c);
+        emit_sorted<Tag, 4>(p, ro, lse, c);
+      } else {
+        u64 c[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c[j] = lane * 8 + j < total ? all[lane * 8 + j] : ~0ull;
+        wave_sort<u64, 8>(c);
+        emit_sorted<Tag, 8>(p, ro, lse, c);
+      }
     }
     return;
   }
-
-  float M = -INFINITY;
-  for (int q = 0; q < P; ++q) M = fmaxf(M, reinterpret_cast<const PartHeader*>(rec0 + q * p.part_stride)->mx);
-  float S = 0.f;
-  int total = 0;
-  for (int q = 0; q < P; ++q) {
-    const PartHeader hd = *reinterpret_cast<const PartHeader*>(rec0 + q * p.part_stride);
-    if (hd.mx != -INFINITY) S += hd.sm * fast_exp2((hd.mx - M) * LOG2E);
-    const int cnt = min(max(hd.cnt, 0), capw);
-    const u64* lst = reinterpret_cast<const u64*>(rec0 + q * p.part_stride + 16);
-    for (int j = tid; j < cnt; j += 256) all[total + j] = lst[j];
-    total += cnt;
-  }
-  const float lse = (M * LOG2E + fast_log2(S)) * LN2;
-  if (tid == 0) s_nsel = 0;
-  __syncthreads();
-
   // U = smallest high word with at least K words at or below it; only the low Keys::BITS bits vary.
   // Counting is ballot + popcount per wave, one barrier per probe; the first probe tries the six
   // leading bits of the best word, which the K-th almost always shares.
@@ -703,24 +752,320 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p)
   }
 }
 
+// Merge of the parts of one row: log-sum-exp from the part statistics, and the K best of the parts'
+// candidates (select_and_emit).  REDO: only the rows on the list of rows handed back.
+template <class Tag, bool REDO>
+__device__ __forceinline__ void topk_merge_row(const ProducerParams& p, int64_t redo_entry) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  u64* all = reinterpret_cast<u64*>(smem_raw);                      // the parts' records; producer_merge_slots words
+  __shared__ SelectLds sh;
+  const int tid = threadIdx.x;
+  const int P = p.parts, K = p.K;
+  int64_t ro = blockIdx.x;
+  if constexpr (REDO) {                       // launched as workgroups of one round; see topk_merge_redo_kernel
+    ro = p.redo_rows[redo_entry];
+  }
+  const int capw = producer_record_cap(K, P);
+  const int sel_cap = producer_sel_cap(K);
+  u64* sel = all + producer_merge_slots(K, P);                      // the selected words; sel_cap words
+  const char* rec0 = p.ws + ro * P * p.part_stride;
+  if (producer_row(p, ro) < 0) {                                    // the row list names no logits row: masked output row
+    for (int k = tid; k < K; k += 256) {
+      store_from_float(p.out_val, p.out_dtype, ro * K + k, -INFINITY);
+      if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * K + k] = -1;
+      else reinterpret_cast<int64_t*>(p.out_idx)[ro * K + k] = -1;
+    }
+    return;
+  }
+
+  float M = -INFINITY;
+  for (int q = 0; q < P; ++q) M = fmaxf(M, reinterpret_cast<const PartHeader*>(rec0 + q * p.part_stride)->mx);
+  float S = 0.f;
+  int total = 0;
+  for (int q = 0; q < P; ++q) {
+    const PartHeader hd = *reinterpret_cast<const PartHeader*>(rec0 + q * p.part_stride);
+    if (hd.mx != -INFINITY) S += hd.sm * fast_exp2((hd.mx - M) * LOG2E);
+    const int cnt = min(max(hd.cnt, 0), capw);
+    const u64* lst = reinterpret_cast<const u64*>(rec0 + q * p.part_stride + 16);
+    for (int j = tid; j < cnt; j += 256) all[total + j] = lst[j];
+    total += cnt;
+  }
+  const float lse = (M * LOG2E + fast_log2(S)) * LN2;
+  if (tid == 0) sh.nsel = 0;
+  __syncthreads();
+  select_and_emit<Tag>(p, ro, lse, all, sel, total, sel_cap, sh);
+}
+
+template <class Tag>
+__global__ __launch_bounds__(256) void topk_merge_kernel(const ProducerParams p) { topk_merge_row<Tag, false>(p, 0); }
+// The rows handed back: a small grid whose workgroups walk the list.
+template <class Tag>
+__global__ __launch_bounds__(256) void topk_merge_redo_kernel(const ProducerParams p) {
+  const int64_t n = min((int64_t)*p.redo_count, p.n_out);
+  for (int64_t e = blockIdx.x; e < n; e += gridDim.x) {
+    topk_merge_row<Tag, true>(p, e);
+    __syncthreads();
+  }
+}
+
+// ---- row-level selection behind the light part kernel ----------------------------------------------
+// Candidate words the selection keeps in LDS, and chunk groups it opens, for a given K; a row with more (a tie
+// plateau, a constant row) is handed back to the part kernel's own, exact selection.
+__host__ __device__ inline int producer_select_cands(int K) {
+  int c = 1024;
+  while (c < 4 * K) c <<= 1;
+  return c;
+}
+__host__ __device__ inline int producer_select_groups(int K) { return 2 * K > 512 ? 2 * K : 512; }
+// Dynamic LDS of topk_select_kernel: the group maxima of all parts, later the candidate words; the selected
+// words; the list of groups to open.
+__host__ __device__ inline size_t producer_select_lds(int K, int parts, int key_bytes) {
+  const size_t maxima = (size_t)parts * producer_groups(K) * PROD_NT * key_bytes, cands = (size_t)producer_select_cands(K) * 8;
+  return ((maxima > cands ? maxima : cands) + 15) / 16 * 16 + (size_t)producer_sel_cap(K) * 8 + (size_t)producer_select_groups(K) * 4;
+}
+
+// One workgroup per output row.  The K-th largest of the row's chunk-group maxima, L, is a lower bound of the
+// row's K-th largest key (K groups reach it, so K entries do), so every entry of the best K -- ties at the K-th
+// key included -- lies in a group whose maximum reaches L.  Those groups (about K of them, out of thousands) are read
+// again from the logits, the entries at or above L become the candidate words, and select_and_emit picks the best K.
+// Against thresholds per part this opens a quarter of the groups when a row has four parts, and the part kernel,
+// bound by vector-ALU issue, sheds its collection stage (a third of its instructions) for 20 % more bytes fetched.
+template <class Tag, int G, bool ALIGNED>
+__global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  using KY = Keys<Tag>;
+  using C = Chunk<Tag>;
+  typedef typename KY::Stored KS;
+  constexpr int NT = PROD_NT, NCH = PROD_NCH, CPG = NCH / G, GPP = G * NT;      // chunks per group, groups per part
+  __shared__ SelectLds sh;
+  __shared__ int s_sum[2 * 4];
+  __shared__ int s_nq, s_total;
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1), w = tid / WAVE;
+  const int64_t ro = blockIdx.x;
+  const int P = p.parts, K = p.K;
+  const int n_g = P * GPP;
+  const int acap = producer_select_cands(K), qcap = producer_select_groups(K), sel_cap = producer_sel_cap(K);
+  const size_t region = (((size_t)n_g * sizeof(KS) > (size_t)acap * 8 ? (size_t)n_g * sizeof(KS) : (size_t)acap * 8) + 15) / 16 * 16;
+  KS* gmax = reinterpret_cast<KS*>(smem_raw);
+  u64* all = reinterpret_cast<u64*>(smem_raw);                      // takes the place of the maxima
+  u64* sel = reinterpret_cast<u64*>(smem_raw + region);
+  int* glist = reinterpret_cast<int*>(smem_raw + region + (size_t)sel_cap * 8);
+  const int64_t r = producer_row(p, ro);
+  if (r < 0) {                                                      // the row list names no logits row: masked output row
+    for (int k = tid; k < K; k += 256) {
+      store_from_float(p.out_val, p.out_dtype, ro * K + k, -INFINITY);
+      if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * K + k] = -1;
+      else reinterpret_cast<int64_t*>(p.out_idx)[ro * K + k] = -1;
+    }
+    return;
+  }
+  const char* rec0 = p.ws + ro * P * p.part_stride;
+  // all loads of the row's records first: the headers of the parts, then the group maxima, a few per thread and round
+  PartHeader hd[PROD_MAX_PARTS];
+#pragma unroll
+  for (int q = 0; q < PROD_MAX_PARTS; ++q)
+    hd[q] = *reinterpret_cast<const PartHeader*>(rec0 + (q < P ? q : 0) * p.part_stride);
+  constexpr int RND = 16;
+  for (int a0 = 0; a0 < n_g; a0 += RND * 256) {
+    KS v[RND];
+#pragma unroll
+    for (int j = 0; j < RND; ++j) {
+      const int a = a0 + j * 256 + tid, aa = a < n_g ? a : 0;
+      v[j] = reinterpret_cast<const KS*>(rec0 + (aa / GPP) * p.part_stride + 16)[aa % GPP];
+    }
+#pragma unroll
+    for (int j = 0; j < RND; ++j) {
+      const int a = a0 + j * 256 + tid;
+      if (a < n_g) gmax[a] = v[j];
+    }
+  }
+  float M = -INFINITY;
+#pragma unroll
+  for (int q = 0; q < PROD_MAX_PARTS; ++q) M = fmaxf(M, q < P ? hd[q].mx : -INFINITY);
+  float S = 0.f;
+#pragma unroll
+  for (int q = 0; q < PROD_MAX_PARTS; ++q)
+    if (q < P && hd[q].mx != -INFINITY) S += hd[q].sm * fast_exp2((hd[q].mx - M) * LOG2E);
+  const float lse = (M * LOG2E + fast_log2(S)) * LN2;
+  int* hist = reinterpret_cast<int*>(sel);                          // 256 counters, in the list of selected words (unused so far)
+  if (tid == 0) { s_nq = 0; s_total = 0; sh.nsel = 0; }
+  hist[tid] = 0;
+  __syncthreads();
+
+  // L: a lower bound of the K-th largest group maximum, as tight as a few steps make it.  (Any bound at or below the
+  // K-th largest key of the row gives the same result; a looser one costs candidates.)
+  int probe = 0;
+  const auto count_ge = [&](unsigned t) {
+    int c = 0;
+    for (int a = tid; a < n_g; a += 256) c += (unsigned)gmax[a] >= t ? 1 : 0;
+    c = wave_sum(c);
+    int* sl = s_sum + (probe++ & 1) * 4;
+    if (lane == 0) sl[w] = c;
+    __syncthreads();
+    return sl[0] + sl[1] + sl[2] + sl[3];
+  };
+  // the answer nearly always shares the six leading bits of the largest maximum
+  unsigned top = 0u;
+  for (int a = tid; a < n_g; a += 256) top = max(top, (unsigned)gmax[a]);
+  top = wave_max(top);
+  if (lane == 0) sh.best[w] = top;
+  __syncthreads();
+  top = max(max(sh.best[0], sh.best[1]), max(sh.best[2], sh.best[3]));
+  constexpr int TAIL = KY::BITS - 6;                                // bits below the prefix
+  const unsigned prefix = top & ~((1u << TAIL) - 1u);
+  unsigned L = 0;
+  if (count_ge(prefix) >= K) {
+    // histogram of the next eight bits of the maxima that share the prefix; the bin that holds the K-th largest,
+    // counted from the top, gives eight more bits of L (its lowest key: at most the bins' width below the true one)
+    constexpr int SH = TAIL - 8;
+    for (int a = tid; a < n_g; a += 256) {
+      const unsigned v = (unsigned)gmax[a];
+      if (v >= prefix) atomicAdd(&hist[(v >> SH) & 255u], 1);
+    }
+    __syncthreads();
+    if (w == 0) {
+      // lane l holds bins 4l .. 4l + 3; suffix sums from the top bin down
+      int c[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) c[j] = hist[lane * 4 + j];
+      const int mine = c[0] + c[1] + c[2] + c[3];
+      int incl = mine;                                               // inclusive scan over the lanes
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const int t = __shfl_up(incl, o, WAVE);
+        incl += lane >= o ? t : 0;
+      }
+      const int above = __shfl(incl, WAVE - 1, WAVE) - incl;         // entries in the bins of the lanes above this one
+      int run = above, bin = -1;
+#pragma unroll
+      for (int j = 3; j >= 0; --j) {
+        if (bin < 0 && run + c[j] >= K && run < K) bin = lane * 4 + j;
+        run += c[j];
+      }
+      if (bin >= 0) s_sum[0] = bin;                                 // exactly one lane finds it
+    }
+    __syncthreads();
+    L = prefix | ((unsigned)s_sum[0] << SH);
+    __syncthreads();
+  } else {
+#pragma unroll 1
+    for (int b = KY::BITS - 1; b >= 0; --b) {
+      const unsigned t = L | (1u << b);
+      if (count_ge(t) >= K) L = t;
+    }
+  }
+  // the groups to open
+  for (int a = tid; a < n_g; a += 256) {
+    if ((unsigned)gmax[a] >= L) {
+      const int slot = atomicAdd(&s_nq, 1);
+      if (slot < qcap) glist[slot] = a;
+    }
+  }
+  __syncthreads();                                                  // the maxima are done with: their LDS takes the candidates
+  const int n_q = s_nq;
+  bool redo = n_q > qcap || L == 0;                                 // L == 0: fewer than K groups hold anything; the part kernel's own selection takes every entry then
+  if (!redo) {
+    const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
+    // four chunks per thread and round: their loads are in flight together
+    constexpr int U = 4;
+    for (int idx0 = 0; idx0 < n_q * CPG; idx0 += U * 256) {
+      u32x4 v[U];
+      int base[U], left[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int idx = idx0 + u * 256 + tid;
+        base[u] = 0;
+        left[u] = 0;                                                // columns of the part from the chunk's first on: 0 = nothing to test
+        v[u] = C::neg_inf();
+        if (idx < n_q * CPG) {
+          const int a = glist[idx / CPG], j = idx % CPG;
+          const int q = a / GPP, gi = a % GPP;
+          // chunk of the part: the j-th of the quad's four neighbours, or the thread's own
+          const int c = CPG == 4 ? (gi / (NT / 4)) * NT + 4 * (gi % (NT / 4)) + j : gi;
+          const int64_t c0 = (int64_t)q * NT * NCH;
+          const int lo = (int)(c0 * C::N);
+          const int n_elems = (int)min((int64_t)NT * NCH * C::N, p.V - lo);
+          const int nch = (n_elems + C::N - 1) / C::N;
+          const char* rpart = row + c0 * 16;
+          v[u] = producer_load_chunk<Tag, ALIGNED>(rpart, c, nch, n_elems, (reinterpret_cast<uintptr_t>(rpart) & 15) == 0);
+          base[u] = lo + c * C::N;
+          left[u] = n_elems - c * C::N;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const unsigned kd = KY::encode(v[u][d]);
+#pragma unroll
+          for (int h = 0; h < KY::PER_DWORD; ++h) {
+            const unsigned k = KY::key(kd, h);
+            const int e = d * KY::PER_DWORD + h;
+            if (k >= L && e < left[u]) {
+              const int slot = atomicAdd(&s_total, 1);
+              if (slot < acap)
+                all[slot] = ((u64)(KY::BITS == 32 ? ~k : (0xffff0000u | (~k & 0xffffu))) << 32) | (unsigned)(base[u] + e);
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();
+    redo = s_total > acap;
+  }
+  if (redo) {                                                       // the same for every thread
+    if (tid == 0) p.redo_rows[atomicAdd(p.redo_count, 1u)] = (int32_t)ro;
+    return;
+  }
+  select_and_emit<Tag>(p, ro, lse, all, sel, s_total, sel_cap, sh);
+}
+
 static int producer_parts(int64_t V, int logits_dtype) {
   const int epc = logits_dtype == DL_F32 ? 4 : 8;
   const int64_t nch = (V + epc - 1) / epc;
   return (int)((nch + PROD_NT * PROD_NCH - 1) / (PROD_NT * PROD_NCH));
 }
 
+template <class Tag, int G, bool ALIGNED>
+static void launch_producer_shape(const ProducerParams& p, hipStream_t st) {
+  const dim3 grid((unsigned)((p.n_out + 7) / 8 * 8 * p.parts));
+  const size_t lds_merge = (size_t)(producer_merge_slots(p.K, p.parts) + producer_sel_cap(p.K)) * 8;      // <= 48 KiB
+  const size_t lds_select = producer_select_lds(p.K, p.parts, Tag::bytes == 4 ? 4 : 2);
+  // chunk groups of a row that hold anything: with fewer than 4 K of them the group maxima bound the K-th key too
+  // loosely (or not at all) for opening groups a second time to pay
+  const int64_t chunks = (p.V + Chunk<Tag>::N - 1) / Chunk<Tag>::N, groups = (chunks + (PROD_NCH / G) - 1) / (PROD_NCH / G);
+  if (lds_select > 64 * 1024 || groups < 4 * (int64_t)p.K) {      // (or too many groups for the selection's LDS): thresholds per part
+    hipLaunchKernelGGL((topk_part_kernel<Tag, G, ALIGNED, PART_FULL>), grid, dim3(PROD_NT), 0, st, p);
+    hipLaunchKernelGGL((topk_merge_kernel<Tag>), dim3((unsigned)p.n_out), dim3(256), lds_merge, st, p);
+    return;
+  }
+  hipLaunchKernelGGL((topk_part_kernel<Tag, G, ALIGNED, PART_LIGHT>), grid, dim3(PROD_NT), 0, st, p);
+  hipLaunchKernelGGL((topk_select_kernel<Tag, G, ALIGNED>), dim3((unsigned)p.n_out), dim3(256), lds_select, st, p);
+  // the rows handed back (none, as a rule: the workgroups then leave at once)
+  const unsigned redo_rows = (unsigned)std::min<int64_t>((p.n_out + 7) / 8 * 8, 256);
+  hipLaunchKernelGGL((topk_part_kernel<Tag, G, ALIGNED, PART_REDO>), dim3(redo_rows * p.parts), dim3(PROD_NT), 0, st, p);
+  hipLaunchKernelGGL((topk_merge_redo_kernel<Tag>), dim3(redo_rows), dim3(256), lds_merge, st, p);
+}
+
 template <class Tag>
 static int launch_producer(const ProducerParams& p, bool aligned, hipStream_t st) {
-  const dim3 grid((unsigned)((p.n_out + 7) / 8 * 8 * p.parts));
-  if (aligned) {
-    if (p.K <= 256) hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_SMALL, true>), grid, dim3(PROD_NT), 0, st, p);
-    else hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_LARGE, true>), grid, dim3(PROD_NT), 0, st, p);
-  } else {
-    if (p.K <= 256) hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_SMALL, false>), grid, dim3(PROD_NT), 0, st, p);
-    else hipLaunchKernelGGL((topk_part_kernel<Tag, PROD_G_LARGE, false>), grid, dim3(PROD_NT), 0, st, p);
+  static bool lds_allowed = false;
+  if (!lds_allowed) {
+    // (up to 64 KiB of dynamic LDS for the selection: above the default limit of a launch)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_SMALL, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_SMALL, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_LARGE, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_LARGE, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    lds_allowed = true;
   }
-  const size_t lds = (size_t)(producer_merge_slots(p.K, p.parts) + producer_sel_cap(p.K)) * 8;      // <= 48 KiB
-  hipLaunchKernelGGL((topk_merge_kernel<Tag>), dim3((unsigned)p.n_out), dim3(256), lds, st, p);
+  if (aligned) {
+    if (p.K <= 256) launch_producer_shape<Tag, PROD_G_SMALL, true>(p, st);
+    else launch_producer_shape<Tag, PROD_G_LARGE, true>(p, st);
+  } else {
+    if (p.K <= 256) launch_producer_shape<Tag, PROD_G_SMALL, false>(p, st);
+    else launch_producer_shape<Tag, PROD_G_LARGE, false>(p, st);
+  }
   return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
@@ -730,7 +1075,8 @@ extern "C" int64_t dl_teacher_topk_workspace_bytes(int logits_dtype, int64_t n_o
   if (n_out <= 0 || V <= 0 || K <= 0) return 0;
   const int parts = dl::producer_parts(V, logits_dtype);
   if (parts > dl::PROD_MAX_PARTS || K > dl::PROD_MAX_K || (int64_t)parts * K > 4096) return 0;
-  return n_out * parts * dl::producer_part_stride(K, parts);
+  const int64_t records = n_out * parts * dl::producer_part_stride(K, parts, logits_dtype == DL_F32 ? 4 : 2);
+  return records + 16 + ((n_out * 4 + 15) & ~15LL);                 // then the counter and the list of rows handed back
 }
 
 extern "C" int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
@@ -754,8 +1100,11 @@ extern "C" int dl_teacher_topk(const void* logits, int logits_dtype, int64_t row
   if (!workspace) return DL_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return DL_ERR_ALIGN;
   if (workspace_bytes < dl_teacher_topk_workspace_bytes(logits_dtype, n_out, V, K)) return DL_ERR_WORKSPACE;
+  const int64_t stride = producer_part_stride(K, parts, eb == 4 ? 4 : 2);
+  char* redo = reinterpret_cast<char*>(workspace) + n_out * parts * stride;
   ProducerParams p{logits, row_stride, n_rows, V, row_list, n_out, K, parts, reinterpret_cast<char*>(workspace),
-                   producer_part_stride(K, parts), out_val, out_dtype, out_idx, out_itype};
+                   stride, out_val, out_dtype, out_idx, out_itype, reinterpret_cast<unsigned*>(redo),
+                   reinterpret_cast<int32_t*>(redo + 16)};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   return logits_dtype == DL_F32 ? launch_producer<TagF32>(p, aligned, st)
          : logits_dtype == DL_BF16 ? launch_producer<TagBF16>(p, aligned, st)
