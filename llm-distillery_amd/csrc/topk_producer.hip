@@ -339,6 +339,62 @@ __device__ __forceinline__ void topk_part(const ProducerParams& p, int64_t ro, i
   for (int i = 0; i < NCH; ++i) reg[i] = producer_load_chunk<Tag, ALIGNED>(rpart, i * NT + tid, nch, n_elems, on_grid);
   if (tid == 0) s_n = 0;
 
+  if constexpr (MODE == PART_LIGHT) {
+    // Statistics and the largest key of every chunk group, nothing else, and no barrier before the end: every
+    // thread sums its exponentials against the largest of its own 64 entries, which it knows from the chunk keys it
+    // makes anyway; the workgroup's maximum and the rescaled sums are combined once at the end.
+    // A group is what the selection reads again: with four chunks per group, the chunks that four neighbouring
+    // threads hold in the same register (64 contiguous bytes of the row: one access); the group's maximum is taken
+    // across the quad.  One chunk per group: the thread's own.
+    typedef typename KY::Stored KS;
+    KS* gout = reinterpret_cast<KS*>(rec + 16);
+    const int mine = (nch - tid + NT - 1) / NT;                       // chunks i < mine are inside the part
+    unsigned tk = 0u;                                                 // largest key of the thread (0: none)
+    unsigned gk[NCH];                                                 // group maxima; stored at the end: a store between the
+                                                                      // loads' waits would make each of them a wait for everything
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      unsigned e[4];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) e[d] = KY::encode(reg[i][d]);
+      unsigned k = i < mine ? KY::top_key(KY::dword_max(KY::dword_max(e[0], e[1]), KY::dword_max(e[2], e[3]))) : 0u;
+      tk = max(tk, k);
+      if constexpr (CPG == 4) {
+        k = max(k, (unsigned)dpp_move<DPP_QUAD_XOR1>((int)k, (int)k));
+        k = max(k, (unsigned)dpp_move<DPP_QUAD_XOR2>((int)k, (int)k));
+      } else {
+        static_assert(CPG == 1 || CPG == 4, "chunk groups: a thread's chunk, or a quad's four");
+      }
+      gk[i] = k;
+    }
+    const float mt = tk ? KY::value(tk) : -INFINITY;
+    const float mbt = (mt == -INFINITY) ? 0.f : mt * LOG2E;
+    float st = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      float f[C::N];
+      forget(reg[i]);
+      C::unpack(reg[i], f);
+#pragma unroll
+      for (int e = 0; e < C::N; ++e) st += fast_exp2(fmaf(f[e], LOG2E, -mbt));
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      if constexpr (CPG == 4) {
+        if ((tid & 3) == (i & 3)) gout[i * (NT / 4) + (tid >> 2)] = (KS)gk[i];
+      } else {
+        gout[i * NT + tid] = (KS)gk[i];
+      }
+    }
+    const float M = block_max<NT>(mt, red);
+    st = (mt == -INFINITY) ? 0.f : st * fast_exp2((mt - M) * LOG2E);
+    st = block_sum<NT>(st, red);
+    if (tid == 0) {
+      PartHeader hd{M, st, -1, 0};
+      *reinterpret_cast<PartHeader*>(rec) = hd;
+    }
+    return;
+  }
   // max and sum-exp of the part (natural log-softmax; no temperature at collection time)
   float mx = -INFINITY;
   bool have_max = false;
@@ -386,34 +442,6 @@ __device__ __forceinline__ void topk_part(const ProducerParams& p, int64_t ro, i
   sm = block_sum<NT>(sm, red);
 
   const int my_chunks = (nch - tid + NT - 1) / NT;                  // chunks i < my_chunks are inside the part
-  if constexpr (MODE == PART_LIGHT) {
-    // Largest key of every chunk group, nothing else.  A group here is what the selection reads again: with four
-    // chunks per group, the chunks that four neighbouring threads hold in the same register (64 contiguous bytes of
-    // the row: one access); the group's maximum is taken across the quad.  One chunk per group: the thread's own.
-    if (tid == 0) {
-      PartHeader hd{mx, sm, -1, 0};
-      *reinterpret_cast<PartHeader*>(rec) = hd;
-    }
-    typedef typename KY::Stored KS;
-    KS* gout = reinterpret_cast<KS*>(rec + 16);
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      forget(reg[i]);
-      unsigned e[4];
-#pragma unroll
-      for (int d = 0; d < 4; ++d) e[d] = KY::encode(reg[i][d]);
-      unsigned k = i < my_chunks ? KY::top_key(KY::dword_max(KY::dword_max(e[0], e[1]), KY::dword_max(e[2], e[3]))) : 0u;      // 0: no chunk of the part
-      if constexpr (CPG == 4) {
-        k = max(k, (unsigned)dpp_move<DPP_QUAD_XOR1>((int)k, (int)k));
-        k = max(k, (unsigned)dpp_move<DPP_QUAD_XOR2>((int)k, (int)k));
-        if ((tid & 3) == (i & 3)) gout[i * (NT / 4) + (tid >> 2)] = (KS)k;
-      } else {
-        static_assert(CPG == 1 || CPG == 4, "chunk groups: a thread's chunk, or a quad's four");
-        gout[i * NT + tid] = (KS)k;
-      }
-    }
-    return;
-  }
   // raw bits -> ordered keys, in place; largest key of every chunk group
   unsigned gm[G];
 #pragma unroll
