@@ -426,6 +426,19 @@ def measured_traffic(workload: str):
     return rec.get(f"{workload}_bytes_per_launch")
 
 
+def measured_valu_busy(workload: str):
+    """Share of the dominant kernel's time its vector ALUs were busy, from the committed SQ counter summary (same
+    rule as measured_traffic: null once the kernel sources have changed)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if rec.get("kernel_source_hash") != kernel_source_hash():
+        return None
+    return rec.get(f"{workload}_valu_busy")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -525,6 +538,11 @@ def main():
                      "kernel": kernel, "kernel_ms": kern_ms, "algorithmic_bytes": algo_bytes},
         "cpu_baseline": cpu_baseline(args.workload, cpu_rows, 7 if args.workload == "c3" else 3) if cpu_rows > 0 else None,
     }
+    busy = measured_valu_busy(args.workload)
+    if busy is not None and busy >= 0.6:
+        # a kernel whose vector ALUs are busy most of its time is held by instruction issue before it is held by memory
+        out["roofline"]["bound_secondary"] = {"bound": "valu", "busy": busy,
+                                              "from": "profiles/traffic.json (rocprofv3 --pmc SQ_ACTIVE_INST_VALU of this command, committed)"}
     if args.workload.startswith("dropin"):
         out["step_over_launches"] = ms_per_step / kern_ms
     print(json.dumps(out))
