@@ -384,8 +384,9 @@ static int dense_split_units(int s_dtype, int t_dtype) {
 // How a row of V columns is cut: threads per part and parts (parts == 0: not cut).  Measured (forward KL, 512 and
 // 8192 rows, 32000 to 262144 columns, fp32 pairs, 16-bit pairs and a 16-bit student against an fp32 teacher):
 //   * a row that half a workgroup's registers hold (512 threads) stays whole;
-//   * up to four parts of 256 threads beat half as many of 512 (more workgroups per CU to hide the exchange
-//     behind), beyond that the partners to wait for cost more than they bring: parts of 512 threads, at most 8;
+//   * with a 16-bit student up to four parts of 256 threads beat half as many of 512 (more workgroups per CU to
+//     hide the exchange behind), beyond that the partners to wait for cost more than they bring: parts of 512
+//     threads, at most 8; fp32 pairs (a part of 256 threads holds 8192 columns only) take parts of 512 from the start;
 //   * wider still, rows against an fp32 teacher take parts of 1024 threads (beyond 8 of those, and beyond 262144
 //     columns of a 16-bit pair, one workgroup per row streams the row from the caches);
 //   * on fewer than 1024 rows the cut pays only from 256 KiB of row pair upwards (one workgroup per row keeps
@@ -405,7 +406,7 @@ static DenseCut dense_split_cut(int kind, int s_dtype, int t_dtype, int64_t n_ro
   if (parts_of(512) < 2) return {0, 0};
   const int64_t pair_bytes = V * ((s_dtype == F32 ? 4 : 2) + (t_dtype == F32 ? 4 : 2));
   if (n_rows < 1024 && pair_bytes < 256 * 1024) return {0, 0};
-  if (parts_of(256) <= 4) return cut_of(256);
+  if (parts_of(256) <= 4 && s_dtype != F32) return cut_of(256);
   if (parts_of(512) <= DENSE_MAX_PARTS) return cut_of(512);
   return cut_of(1024);
 }

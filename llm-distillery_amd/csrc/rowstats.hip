@@ -21,37 +21,82 @@ struct StatsParams {
 // MODE 0: element-wise loads (rows that are not even element-aligned never get here; kept for reference
 // and for rows shorter than a chunk).  MODE 1: rows on the 16-byte grid, a whole number of chunks long.
 // MODE 2: any other row: its 16-byte chunks by vector loads, the elements before and behind them one by one.
-template <class Tag, int NT, int MODE>
+//
+// STASH: the logits at the teacher's ids are not fetched by loads of their own (K random reads of cold lines per
+// row, which the sweep then fetches a second time: a quarter more traffic and 9 of the kernel's 50 us on 2048
+// rows of 32000 fp32 columns with K = 400) but taken from the sweep itself.  Chunk c of the body belongs to
+// thread c % NT in its round c / NT; the ids set one bit per (thread, round) in LDS, a scan over the threads'
+// bit counts gives every marked chunk a slot, the sweep drops the marked chunks (16 bytes, as loaded) into their
+// slots on its way, and behind the sweep every entry reads its element from its chunk's slot.  At most 64 rounds
+// (64 * NT chunks per row) and one slot per entry (K * 16 bytes of LDS from the launch).
+constexpr int STASH_ROUNDS = 64;
+constexpr int STASH_MAX_K = 1024;
+
+template <class Tag, int NT, int MODE, bool STASH>
 __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
   __shared__ float red[64];
+  __shared__ unsigned long long s_bits[STASH ? NT : 1];
+  __shared__ int s_pre[STASH ? NT : 1];
+  __shared__ int s_wave[STASH ? NT / 64 : 1];
+  extern __shared__ __align__(16) unsigned char smem[];        // STASH: K slots of 16 bytes
   using C = Chunk<Tag>;
   const int64_t r = blockIdx.x;
   const int tid = threadIdx.x;
   const int64_t trow = teacher_row(p.row_map, r, p.n_trows);
   if (trow < 0) return;
   const char* row = reinterpret_cast<const char*>(p.logits) + r * p.row_stride * Tag::bytes;
-  for (int k = tid; k < p.K; k += NT) {
-    const int64_t id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
-    p.zk[trow * p.K + k] = (id >= 0 && id < p.V) ? load_as_float(row, Tag::id, id) * p.inv_T : 0.f;
-  }
   const float a = p.inv_T * LOG2E;
   float m = -INFINITY, sm = 0.f;
   const auto one = [&](float f) {
     if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
     if (f > -INFINITY) sm += fast_exp2(fmaf(f, a, -m * a));
   };
+  if constexpr (!STASH) {
+    for (int k = tid; k < p.K; k += NT) {
+      const int64_t id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
+      p.zk[trow * p.K + k] = (id >= 0 && id < p.V) ? load_as_float(row, Tag::id, id) * p.inv_T : 0.f;
+    }
+  }
   if (MODE != 0) {
     const RowSplit<Tag> sp(row, p.V, MODE == 2);
     const char* body = row + (int64_t)sp.head * Tag::bytes;
     const int64_t nch = sp.nbody;
+    u32x4* stash = reinterpret_cast<u32x4*>(smem);
+    unsigned long long mybits = 0;
+    int slot = 0;
+    if constexpr (STASH) {
+      s_bits[tid] = 0;
+      __syncthreads();
+      for (int k = tid; k < p.K; k += NT) {
+        const int64_t rel = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k) - sp.head;
+        if (rel >= 0 && rel < nch * C::N) {
+          const int ch = (int)(rel / C::N);
+          atomicOr(&s_bits[ch % NT], 1ull << (ch / NT));
+        }
+      }
+      __syncthreads();
+      mybits = s_bits[tid];
+      const int cnt = __popcll(mybits);
+      int inc = cnt;                                         // inclusive scan over the wave, then over the waves
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(inc, d, 64);
+        if ((tid & 63) >= d) inc += up;
+      }
+      if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
+      __syncthreads();
+      int before = 0;
+#pragma unroll
+      for (int w = 0; w < NT / 64; ++w) before += (w < (tid >> 6)) ? s_wave[w] : 0;
+      slot = before + inc - cnt;
+      s_pre[tid] = slot;
+    }
     for (int64_t c0 = 0; c0 < nch; c0 += 4 * NT) {          // four 16-byte loads in flight per thread
       u32x4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int64_t ch = c0 + (int64_t)u * NT + tid;
-        // streamed, not cached: the K gathers above then fetch their lines a second time (9 of the kernel's 50 us on 2048
-        // rows of 32000 fp32 columns, K = 400), but the cached form is slower (53.5 us), and so is handing every id to the
-        // thread that sweeps its chunk, to be fetched right behind the chunk's own load (60 us)
+        // streamed, not cached: with cached loads the kernel is slower, whether or not gathers follow that could hit
         v[u] = ch < nch ? load16_stream(body + ch * 16) : C::neg_inf();
       }
       float cm = -INFINITY;
@@ -61,6 +106,12 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
         C::unpack(v[u], f[u]);
 #pragma unroll
         for (int e = 0; e < C::N; ++e) cm = fmaxf(cm, f[u][e]);
+      }
+      if constexpr (STASH) {
+        const unsigned four = (unsigned)(mybits >> (c0 / NT)) & 15u;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (four >> u & 1) stash[slot++] = v[u];
       }
       if (cm > m) { sm *= fast_exp2((m - cm) * a); m = cm; }
       const float mb = m * a;
@@ -72,6 +123,24 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
       }
     }
     if (MODE == 2 && tid < sp.leftovers()) one(load_as_float(row, Tag::id, sp.column(tid)));
+    if constexpr (STASH) {
+      __syncthreads();
+      for (int k = tid; k < p.K; k += NT) {
+        const int64_t id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
+        const int64_t rel = id - sp.head;
+        float z = 0.f;
+        if (rel >= 0 && rel < nch * C::N) {
+          const int ch = (int)(rel / C::N), t = ch % NT, j = ch / NT;
+          const int at = s_pre[t] + __popcll(s_bits[t] & ((1ull << j) - 1ull));
+          const int e = at * C::N + (int)(rel % C::N);
+          if constexpr (Tag::bytes == 4) z = reinterpret_cast<const float*>(smem)[e];
+          else z = load_as_float(reinterpret_cast<const unsigned short*>(smem) + e, Tag::id, 0);
+        } else if (id >= 0 && id < p.V) {
+          z = load_as_float(row, Tag::id, id);               // the few columns before and behind the body
+        }
+        p.zk[trow * p.K + k] = z * p.inv_T;
+      }
+    }
   } else {
     for (int64_t j = tid; j < p.V; j += NT) one(load_as_float(row, Tag::id, j));
   }
@@ -99,6 +168,29 @@ __device__ __forceinline__ float coef_on_id(const int* s_idx, const float* s_c, 
   return cs;
 }
 
+// correction_apply for a correction that is added to the dense value: element e of chunk i becomes
+// dense + coef(k) * scale for the entry k that names it; true if some element is named more than once.
+template <class Tag, int NT, class Coef>
+__device__ __forceinline__ bool correction_add(const int* head, const int* next, const int* col, int lo, int i,
+                                               float (&f)[Chunk<Tag>::N], float scale, Coef coef) {
+  using C = Chunk<Tag>;
+  unsigned seen = 0u, again = 0u;
+  float dense[C::N];
+#pragma unroll
+  for (int j = 0; j < C::N; ++j) dense[j] = f[j];
+  for (int k = head[(i % (CORRECTION_HEADS / NT)) * NT + threadIdx.x]; k >= 0; k = next[k]) {
+    const int off = col[k] - lo;
+    if (ChunkMap<NT, 0>::reg(off / C::N) != i) continue;
+    const int e = off % C::N;
+    again |= seen & (1u << e);
+    seen |= 1u << e;
+    const float c = coef(k) * scale;
+#pragma unroll
+    for (int j = 0; j < C::N; ++j) f[j] = (j == e) ? dense[j] + c : f[j];
+  }
+  return again != 0u;
+}
+
 // MODE as for phase 1.  MODE 2 needs the gradient row to sit on the 16-byte grid exactly as the logits row does
 // (same address modulo 16): the kernel then works on the rows' bodies, with the teacher ids counted
 // from the body's first column, and part 0 adds the few columns before and behind the body one by one.
@@ -119,7 +211,7 @@ __device__ __forceinline__ void rowcoef_grad_part(const StatsParams& p, int part
   int* s_idx = reinterpret_cast<int*>(smem);
   float* s_c = reinterpret_cast<float*>(s_idx + Kp);
   float* s_z = s_c + Kp;
-  float* s_val = s_z + Kp;                         // VEC: final value at the entry's column, owner lists
+  float* s_val = s_z + Kp;                         // (spare)
   int* s_next = reinterpret_cast<int*>(s_val + Kp);
   int* s_head = s_next + Kp;
   unsigned* s_own = reinterpret_cast<unsigned*>(s_head + CORRECTION_HEADS);
@@ -194,7 +286,7 @@ __device__ __forceinline__ void rowcoef_grad_part(const StatsParams& p, int part
       }
       s_idx[k] = mine ? (int)id : -1;
       s_c[k] = cv;
-      s_z[k] = mine ? load_as_float(row, Tag::id, id) : 0.f;
+      if (!VEC) s_z[k] = mine ? load_as_float(row, Tag::id, id) : 0.f;      // VEC: the column's owner has it in its registers
     }
   };
   if (VEC) {
@@ -203,25 +295,25 @@ __device__ __forceinline__ void rowcoef_grad_part(const StatsParams& p, int part
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int64_t ch = c_lo + (int64_t)i * NT + tid;
-      // cached, not streaming, loads: the gather of the logits at the teacher ids that follows then
-      // finds its lines in L2 instead of fetching them a second time
-      v[i] = ch < c_hi ? *reinterpret_cast<const u32x4*>(row + ch * 16) : C::neg_inf();
+      v[i] = ch < c_hi ? load16_stream(row + ch * 16) : C::neg_inf();
     }
     correction_clear<NT>(s_head, s_own);
     stage();
     if constexpr (COMPOSITE) w = -block_sum<NT>(acc, red) * p.inv_T;      // s_k = z_k - lse: d / d lse = -sum_k
     __syncthreads();
-    // dense part of the columns that carry a teacher entry, handed to the threads that hold them
+    // the columns that carry a teacher entry, handed to the threads that hold them: those add the entry's coefficient
+    // to the dense value they have just made
     for (int k = tid; k < Kp; k += NT) {
       const int id = s_idx[k];
-      if (id < 0) continue;
-      s_val[k] = fast_exp2(fmaf(s_z[k], a, -b)) * w;
-      correction_link<Tag, NT>(s_head, s_own, s_next, k, id - (int)lo);
+      if (id >= 0) correction_link<Tag, NT>(s_head, s_own, s_next, k, id - (int)lo);
     }
     __syncthreads();
     const unsigned mine = s_own[tid];
     const auto coef = [&](int k) { return s_c[k]; };
-    const auto value = [&](int k, float cs) { return s_val[k] + cs * p.inv_T; };
+    // a column named by several entries (the rare path behind the sweep): its dense value made again, the same bits
+    const auto value = [&](int k, float cs) {
+      return fast_exp2(fmaf(load_as_float(row, Tag::id, s_idx[k]), a, -b)) * w + cs * p.inv_T;
+    };
     unsigned repeats = 0u;            // chunks in which an id occurs more than once
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -232,7 +324,7 @@ __device__ __forceinline__ void rowcoef_grad_part(const StatsParams& p, int part
 #pragma unroll
         for (int e = 0; e < C::N; ++e) f[e] = fast_exp2(fmaf(f[e], a, -b)) * w;
         if (mine & (1u << i))
-          if (correction_apply<Tag, NT>(s_head, s_next, s_idx, (int)lo, i, f, coef, value)) repeats |= 1u << i;
+          if (correction_add<Tag, NT>(s_head, s_next, s_idx, (int)lo, i, f, p.inv_T, coef)) repeats |= 1u << i;
         put(ch, C::pack(f));
       }
     }
@@ -285,9 +377,16 @@ static bool same_phase16(const void* a, int64_t stride_a, const void* b, int64_t
 
 template <class Tag>
 static hipError_t launch_stats(const StatsParams& p, int mode, hipStream_t st) {
-  if (mode == 1) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 1>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
-  else if (mode == 2) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 2>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 0>), dim3((unsigned)p.n_rows), dim3(256), 0, st, p);
+  // the logits at the teacher's ids out of the sweep where the row's chunks fit the threads' 64 rounds (the bound holds
+  // for every row: a peeled head only shortens the body)
+  const bool stash = mode != 0 && p.K <= STASH_MAX_K && (p.V + Tag::epc - 1) / Tag::epc <= (int64_t)STASH_ROUNDS * 256;
+  const size_t lds = stash ? (size_t)p.K * 16 : 0;
+  const dim3 grid((unsigned)p.n_rows), block(256);
+  if (mode == 1 && stash) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 1, true>), grid, block, lds, st, p);
+  else if (mode == 2 && stash) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 2, true>), grid, block, lds, st, p);
+  else if (mode == 1) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 1, false>), grid, block, 0, st, p);
+  else if (mode == 2) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 2, false>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 0, false>), grid, block, 0, st, p);
   return hipGetLastError();
 }
 
