@@ -659,6 +659,26 @@ __device__ __forceinline__ void emit_sorted(const ProducerParams& p, int64_t ro,
   }
 }
 
+// The same for narrow words (16-bit keys that share their leading bits `prefix`): the complement of the key's low
+// TAIL bits above CB bits of column.
+template <class Tag, int EPL>
+__device__ __forceinline__ void emit_sorted_narrow(const ProducerParams& p, int64_t ro, float lse, const unsigned (&c)[EPL],
+                                                   unsigned prefix, int tail, int cb) {
+  const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const int k = lane * EPL + j;
+    if (k < p.K) {
+      const unsigned key = prefix | (~(c[j] >> cb) & ((1u << tail) - 1u));
+      const float logp = Keys<Tag>::value(key) - lse;
+      const int col = (int)(c[j] & ((1u << cb) - 1u));
+      store_from_float(p.out_val, p.out_dtype, ro * p.K + k, logp);
+      if (p.out_itype == I32) reinterpret_cast<int32_t*>(p.out_idx)[ro * p.K + k] = col;
+      else reinterpret_cast<int64_t*>(p.out_idx)[ro * p.K + k] = col;
+    }
+  }
+}
+
 // The K best of `total` candidate words (LDS) to the output row.  Words sort ascending = key descending, column
 // ascending, and no two are equal (the column is part of the word).  The K-th smallest high word (= K-th
 // largest key) is found bit by bit; the words at or below it (K plus ties) are compacted and sorted by one wave in
@@ -858,7 +878,9 @@ __host__ __device__ inline size_t producer_select_lds(int K, int parts, int key_
 // again from the logits, the entries at or above L become the candidate words, and select_and_emit picks the best K.
 // Against thresholds per part this opens a quarter of the groups when a row has four parts, and the part kernel,
 // bound by vector-ALU issue, sheds its collection stage (a third of its instructions) for 20 % more bytes fetched.
-template <class Tag, int G, bool ALIGNED>
+// MAXR > 0: the group maxima stay in the threads' registers (MAXR rounds of 16 bytes per thread: every pass over them
+// then costs no LDS access and no address arithmetic); MAXR == 0: any number of them, in LDS.
+template <class Tag, int G, bool ALIGNED, int MAXR>
 __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   using KY = Keys<Tag>;
@@ -877,6 +899,7 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
   const size_t region = (((size_t)n_g * sizeof(KS) > (size_t)acap * 8 ? (size_t)n_g * sizeof(KS) : (size_t)acap * 8) + 15) / 16 * 16;
   KS* gmax = reinterpret_cast<KS*>(smem_raw);
   u64* all = reinterpret_cast<u64*>(smem_raw);                      // takes the place of the maxima
+  unsigned* all32 = reinterpret_cast<unsigned*>(smem_raw);          // the same list in narrow words
   u64* sel = reinterpret_cast<u64*>(smem_raw + region);
   int* glist = reinterpret_cast<int*>(smem_raw + region + (size_t)sel_cap * 8);
   const int64_t r = producer_row(p, ro);
@@ -889,23 +912,35 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
     return;
   }
   const char* rec0 = p.ws + ro * P * p.part_stride;
-  // all loads of the row's records first: the headers of the parts, then the group maxima, a few per thread and round
+  // all loads of the row's records first: the headers of the parts, then the group maxima
   PartHeader hd[PROD_MAX_PARTS];
 #pragma unroll
   for (int q = 0; q < PROD_MAX_PARTS; ++q)
     hd[q] = *reinterpret_cast<const PartHeader*>(rec0 + (q < P ? q : 0) * p.part_stride);
-  constexpr int RND = 16;
-  for (int a0 = 0; a0 < n_g; a0 += RND * 256) {
-    KS v[RND];
+  constexpr int KPL = 16 / (int)sizeof(KS), DW = KY::PER_DWORD;      // maxima per 16 bytes, per dword
+  u32x4 mreg[MAXR > 0 ? MAXR : 1];
+  if constexpr (MAXR > 0) {
 #pragma unroll
-    for (int j = 0; j < RND; ++j) {
-      const int a = a0 + j * 256 + tid, aa = a < n_g ? a : 0;
-      v[j] = reinterpret_cast<const KS*>(rec0 + (aa / GPP) * p.part_stride + 16)[aa % GPP];
+    for (int rr = 0; rr < MAXR; ++rr) {
+      const int a0 = (rr * 256 + tid) * KPL;                          // groups a0 .. a0 + KPL - 1: one part's (GPP is a multiple of KPL)
+      mreg[rr] = u32x4{0u, 0u, 0u, 0u};                               // key 0: below every threshold but 0, which hands the row back
+      if (a0 < n_g)
+        mreg[rr] = *reinterpret_cast<const u32x4*>(rec0 + (int64_t)(a0 / GPP) * p.part_stride + 16 + (size_t)(a0 % GPP) * sizeof(KS));
     }
+  } else {
+    constexpr int RND = 16;
+    for (int a0 = 0; a0 < n_g; a0 += RND * 256) {
+      KS v[RND];
 #pragma unroll
-    for (int j = 0; j < RND; ++j) {
-      const int a = a0 + j * 256 + tid;
-      if (a < n_g) gmax[a] = v[j];
+      for (int j = 0; j < RND; ++j) {
+        const int a = a0 + j * 256 + tid, aa = a < n_g ? a : 0;
+        v[j] = reinterpret_cast<const KS*>(rec0 + (aa / GPP) * p.part_stride + 16)[aa % GPP];
+      }
+#pragma unroll
+      for (int j = 0; j < RND; ++j) {
+        const int a = a0 + j * 256 + tid;
+        if (a < n_g) gmax[a] = v[j];
+      }
     }
   }
   float M = -INFINITY;
@@ -921,73 +956,167 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
   hist[tid] = 0;
   __syncthreads();
 
-  // L: a lower bound of the K-th largest group maximum, as tight as a few steps make it.  (Any bound at or below the
-  // K-th largest key of the row gives the same result; a looser one costs candidates.)
-  int probe = 0;
-  const auto count_ge = [&](unsigned t) {
-    int c = 0;
-    for (int a = tid; a < n_g; a += 256) c += (unsigned)gmax[a] >= t ? 1 : 0;
-    c = wave_sum(c);
-    int* sl = s_sum + (probe++ & 1) * 4;
-    if (lane == 0) sl[w] = c;
-    __syncthreads();
-    return sl[0] + sl[1] + sl[2] + sl[3];
-  };
-  // the answer nearly always shares the six leading bits of the largest maximum
-  unsigned top = 0u;
-  for (int a = tid; a < n_g; a += 256) top = max(top, (unsigned)gmax[a]);
-  top = wave_max(top);
-  if (lane == 0) sh.best[w] = top;
-  __syncthreads();
-  top = max(max(sh.best[0], sh.best[1]), max(sh.best[2], sh.best[3]));
-  constexpr int TAIL = KY::BITS - 6;                                // bits below the prefix
-  const unsigned prefix = top & ~((1u << TAIL) - 1u);
+  // Candidate words of 32 bits where the keys have 16 and the bound comes from the histogram step: every candidate then
+  // shares the six leading bits of the largest maximum, so 10 key bits and 22 bits of column tell the words apart,
+  // and the wave that sorts them moves and compares half as many registers.
+  constexpr int TAIL_BITS = KY::BITS - 6, COL_BITS = 32 - TAIL_BITS;
+  bool narrow = false;
+  unsigned key_prefix = 0u;
   unsigned L = 0;
-  if (count_ge(prefix) >= K) {
-    // histogram of the next eight bits of the maxima that share the prefix; the bin that holds the K-th largest,
-    // counted from the top, gives eight more bits of L (its lowest key: at most the bins' width below the true one)
-    constexpr int SH = TAIL - 8;
-    for (int a = tid; a < n_g; a += 256) {
-      const unsigned v = (unsigned)gmax[a];
-      if (v >= prefix) atomicAdd(&hist[(v >> SH) & 255u], 1);
-    }
+  if constexpr (MAXR > 0) {
+    // every thread's maxima: `visit(key, group)` for each of them
+    const auto for_keys = [&](auto visit) {
+#pragma unroll
+      for (int rr = 0; rr < MAXR; ++rr)
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+          for (int h = 0; h < DW; ++h) visit(KY::key(mreg[rr][d], h), (rr * 256 + tid) * KPL + d * DW + h);
+    };
+    int probe = 0;
+    const auto count_ge = [&](unsigned t) {
+      int c = 0;
+      for_keys([&](unsigned k, int) { c += k >= t ? 1 : 0; });
+      c = wave_sum(c);
+      int* sl = s_sum + (probe++ & 1) * 4;
+      if (lane == 0) sl[w] = c;
+      __syncthreads();
+      return sl[0] + sl[1] + sl[2] + sl[3];
+    };
+    unsigned dm = 0u;
+#pragma unroll
+    for (int rr = 0; rr < MAXR; ++rr)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) dm = KY::dword_max(dm, mreg[rr][d]);
+    unsigned top = wave_max(KY::top_key(dm));
+    if (lane == 0) sh.best[w] = top;
     __syncthreads();
-    if (w == 0) {
-      // lane l holds bins 4l .. 4l + 3; suffix sums from the top bin down
-      int c[4];
+    top = max(max(sh.best[0], sh.best[1]), max(sh.best[2], sh.best[3]));
+    constexpr int TAIL = KY::BITS - 6;                                // bits below the prefix
+    const unsigned prefix = top & ~((1u << TAIL) - 1u);
+    // histogram of the next eight bits of the maxima that share the prefix (prefix 0: the padding keys would count);
+    // should fewer than K of them share it, no bin is found and the bisection below takes over
+    bool found = false;
+    if (prefix != 0u) {
+      constexpr int SH = TAIL - 8;
+      for_keys([&](unsigned k, int) { if (k >= prefix) atomicAdd(&hist[(k >> SH) & 255u], 1); });
+      __syncthreads();
+      if (w == 0) {
+        int c[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) c[j] = hist[lane * 4 + j];
-      const int mine = c[0] + c[1] + c[2] + c[3];
-      int incl = mine;                                               // inclusive scan over the lanes
+        for (int j = 0; j < 4; ++j) c[j] = hist[lane * 4 + j];
+        const int mine = c[0] + c[1] + c[2] + c[3];
+        int incl = mine;
 #pragma unroll
-      for (int o = 1; o < WAVE; o <<= 1) {
-        const int t = __shfl_up(incl, o, WAVE);
-        incl += lane >= o ? t : 0;
+        for (int o = 1; o < WAVE; o <<= 1) {
+          const int t = __shfl_up(incl, o, WAVE);
+          incl += lane >= o ? t : 0;
+        }
+        const int sharing = __shfl(incl, WAVE - 1, WAVE);
+        const int above = sharing - incl;
+        int run = above, bin = -1;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+          if (bin < 0 && run + c[j] >= K && run < K) bin = lane * 4 + j;
+          run += c[j];
+        }
+        if (lane == 0 && sharing < K) s_sum[0] = -1;
+        if (bin >= 0) s_sum[0] = bin;                                 // exactly one lane finds it when K or more share the prefix
       }
-      const int above = __shfl(incl, WAVE - 1, WAVE) - incl;         // entries in the bins of the lanes above this one
-      int run = above, bin = -1;
-#pragma unroll
-      for (int j = 3; j >= 0; --j) {
-        if (bin < 0 && run + c[j] >= K && run < K) bin = lane * 4 + j;
-        run += c[j];
+      __syncthreads();
+      const int bin = s_sum[0];
+      __syncthreads();
+      if (bin >= 0) {
+        L = prefix | ((unsigned)bin << SH);
+        narrow = KY::BITS == 16 && p.V <= (1ll << COL_BITS);
+        key_prefix = prefix;
+        found = true;
       }
-      if (bin >= 0) s_sum[0] = bin;                                 // exactly one lane finds it
     }
-    __syncthreads();
-    L = prefix | ((unsigned)s_sum[0] << SH);
-    __syncthreads();
-  } else {
+    if (!found) {
 #pragma unroll 1
-    for (int b = KY::BITS - 1; b >= 0; --b) {
-      const unsigned t = L | (1u << b);
-      if (count_ge(t) >= K) L = t;
+      for (int b = KY::BITS - 1; b >= 0; --b) {
+        const unsigned t = L | (1u << b);
+        if (count_ge(t) >= K) L = t;
+      }
     }
-  }
-  // the groups to open
-  for (int a = tid; a < n_g; a += 256) {
-    if ((unsigned)gmax[a] >= L) {
-      const int slot = atomicAdd(&s_nq, 1);
-      if (slot < qcap) glist[slot] = a;
+    if (L != 0u)
+      for_keys([&](unsigned k, int a) {
+        if (k >= L) {
+          const int slot = atomicAdd(&s_nq, 1);
+          if (slot < qcap) glist[slot] = a;
+        }
+      });
+  } else {
+    // L: a lower bound of the K-th largest group maximum, as tight as a few steps make it.  (Any bound at or below the
+    // K-th largest key of the row gives the same result; a looser one costs candidates.)
+    int probe = 0;
+    const auto count_ge = [&](unsigned t) {
+      int c = 0;
+      for (int a = tid; a < n_g; a += 256) c += (unsigned)gmax[a] >= t ? 1 : 0;
+      c = wave_sum(c);
+      int* sl = s_sum + (probe++ & 1) * 4;
+      if (lane == 0) sl[w] = c;
+      __syncthreads();
+      return sl[0] + sl[1] + sl[2] + sl[3];
+    };
+    // the answer nearly always shares the six leading bits of the largest maximum
+    unsigned top = 0u;
+    for (int a = tid; a < n_g; a += 256) top = max(top, (unsigned)gmax[a]);
+    top = wave_max(top);
+    if (lane == 0) sh.best[w] = top;
+    __syncthreads();
+    top = max(max(sh.best[0], sh.best[1]), max(sh.best[2], sh.best[3]));
+    constexpr int TAIL = KY::BITS - 6;                                // bits below the prefix
+    const unsigned prefix = top & ~((1u << TAIL) - 1u);
+    if (count_ge(prefix) >= K) {
+      // histogram of the next eight bits of the maxima that share the prefix; the bin that holds the K-th largest,
+      // counted from the top, gives eight more bits of L (its lowest key: at most the bins' width below the true one)
+      constexpr int SH = TAIL - 8;
+      for (int a = tid; a < n_g; a += 256) {
+        const unsigned v = (unsigned)gmax[a];
+        if (v >= prefix) atomicAdd(&hist[(v >> SH) & 255u], 1);
+      }
+      __syncthreads();
+      if (w == 0) {
+        // lane l holds bins 4l .. 4l + 3; suffix sums from the top bin down
+        int c[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = hist[lane * 4 + j];
+        const int mine = c[0] + c[1] + c[2] + c[3];
+        int incl = mine;                                               // inclusive scan over the lanes
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) {
+          const int t = __shfl_up(incl, o, WAVE);
+          incl += lane >= o ? t : 0;
+        }
+        const int above = __shfl(incl, WAVE - 1, WAVE) - incl;         // entries in the bins of the lanes above this one
+        int run = above, bin = -1;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+          if (bin < 0 && run + c[j] >= K && run < K) bin = lane * 4 + j;
+          run += c[j];
+        }
+        if (bin >= 0) s_sum[0] = bin;                                 // exactly one lane finds it
+      }
+      __syncthreads();
+      L = prefix | ((unsigned)s_sum[0] << SH);
+      narrow = KY::BITS == 16 && p.V <= (1ll << COL_BITS);
+      key_prefix = prefix;
+      __syncthreads();
+    } else {
+#pragma unroll 1
+      for (int b = KY::BITS - 1; b >= 0; --b) {
+        const unsigned t = L | (1u << b);
+        if (count_ge(t) >= K) L = t;
+      }
+    }
+    // the groups to open
+    for (int a = tid; a < n_g; a += 256) {
+      if ((unsigned)gmax[a] >= L) {
+        const int slot = atomicAdd(&s_nq, 1);
+        if (slot < qcap) glist[slot] = a;
+      }
     }
   }
   __syncthreads();                                                  // the maxima are done with: their LDS takes the candidates
@@ -1032,8 +1161,10 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
             const int e = d * KY::PER_DWORD + h;
             if (k >= L && e < left[u]) {
               const int slot = atomicAdd(&s_total, 1);
-              if (slot < acap)
-                all[slot] = ((u64)(KY::BITS == 32 ? ~k : (0xffff0000u | (~k & 0xffffu))) << 32) | (unsigned)(base[u] + e);
+              if (slot < acap) {
+                if (narrow) all32[slot] = ((~k & ((1u << TAIL_BITS) - 1u)) << COL_BITS) | (unsigned)(base[u] + e);
+                else all[slot] = ((u64)(KY::BITS == 32 ? ~k : (0xffff0000u | (~k & 0xffffu))) << 32) | (unsigned)(base[u] + e);
+              }
             }
           }
         }
@@ -1046,7 +1177,41 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
     if (tid == 0) p.redo_rows[atomicAdd(p.redo_count, 1u)] = (int32_t)ro;
     return;
   }
-  select_and_emit<Tag>(p, ro, lse, all, sel, s_total, sel_cap, sh);
+  const int total = s_total;
+  if (KY::BITS == 16 && narrow) {
+    if (total <= 512) {                                             // the rule: one wave sorts the narrow words as they are
+      if (w == 0) {
+        if (total <= 256) {
+          unsigned c[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) c[j] = lane * 4 + j < total ? all32[lane * 4 + j] : ~0u;
+          wave_sort<unsigned, 4>(c);
+          emit_sorted_narrow<Tag, 4>(p, ro, lse, c, key_prefix, TAIL_BITS, COL_BITS);
+        } else {
+          unsigned c[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) c[j] = lane * 8 + j < total ? all32[lane * 8 + j] : ~0u;
+          wave_sort<unsigned, 8>(c);
+          emit_sorted_narrow<Tag, 8>(p, ro, lse, c, key_prefix, TAIL_BITS, COL_BITS);
+        }
+      }
+      return;
+    }
+    // more of them (a tie plateau): widened in place, through registers, for the general selection
+    constexpr int PER = (4 * PROD_MAX_K + 255) / 256;                // acap <= 4 * PROD_MAX_K
+    unsigned wv[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) wv[j] = j * 256 + tid < total ? all32[j * 256 + tid] : 0u;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (j * 256 + tid < total) {
+        const unsigned key = key_prefix | (~(wv[j] >> COL_BITS) & ((1u << TAIL_BITS) - 1u));
+        all[j * 256 + tid] = ((u64)(0xffff0000u | (~key & 0xffffu)) << 32) | (wv[j] & ((1u << COL_BITS) - 1u));
+      }
+    __syncthreads();
+  }
+  select_and_emit<Tag>(p, ro, lse, all, sel, total, sel_cap, sh);
 }
 
 static int producer_parts(int64_t V, int logits_dtype) {
@@ -1069,7 +1234,11 @@ static void launch_producer_shape(const ProducerParams& p, hipStream_t st) {
     return;
   }
   hipLaunchKernelGGL((topk_part_kernel<Tag, G, ALIGNED, PART_LIGHT>), grid, dim3(PROD_NT), 0, st, p);
-  hipLaunchKernelGGL((topk_select_kernel<Tag, G, ALIGNED>), dim3((unsigned)p.n_out), dim3(256), lds_select, st, p);
+  // the maxima of a row in the selection's registers where four rounds of 16 bytes per thread hold them
+  if ((size_t)p.parts * G * PROD_NT * sizeof(typename Keys<Tag>::Stored) <= (size_t)4 * 256 * 16)
+    hipLaunchKernelGGL((topk_select_kernel<Tag, G, ALIGNED, 4>), dim3((unsigned)p.n_out), dim3(256), lds_select, st, p);
+  else
+    hipLaunchKernelGGL((topk_select_kernel<Tag, G, ALIGNED, 0>), dim3((unsigned)p.n_out), dim3(256), lds_select, st, p);
   // the rows handed back (none, as a rule: the workgroups then leave at once)
   const unsigned redo_rows = (unsigned)std::min<int64_t>((p.n_out + 7) / 8 * 8, 256);
   hipLaunchKernelGGL((topk_part_kernel<Tag, G, ALIGNED, PART_REDO>), dim3(redo_rows * p.parts), dim3(PROD_NT), 0, st, p);
@@ -1081,10 +1250,10 @@ static int launch_producer(const ProducerParams& p, bool aligned, hipStream_t st
   static bool lds_allowed = false;
   if (!lds_allowed) {
     // (up to 64 KiB of dynamic LDS for the selection: above the default limit of a launch)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_SMALL, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_SMALL, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_LARGE, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_LARGE, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_SMALL, true, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_SMALL, false, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_LARGE, true, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_select_kernel<Tag, PROD_G_LARGE, false, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
     lds_allowed = true;
   }
   if (aligned) {

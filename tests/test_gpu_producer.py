@@ -126,6 +126,28 @@ def test_tie_plateaus_of_every_size(D, dtype, n_tied):
     np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("n_blocks", [12, 20, 28])
+def test_a_plateau_packed_into_few_stretches_of_the_row(D, dtype, n_blocks):
+    """Hundreds of equal entries that fill a few contiguous stretches of the row: few chunk groups hold them, so the
+    bound taken from the group maxima lies below the plateau and the selection meets more candidates than one wave
+    sorts (between 512 and the list's size), all of them tied at the K-th value but a few."""
+    g = torch.Generator().manual_seed(n_blocks)
+    V, K = 128256, 200
+    logits = (torch.randn(6, V, generator=g) * 2).clamp(max=7.5)
+    for r in range(6):
+        starts = torch.randperm(V // 64 - 1, generator=g)[:n_blocks] * 64
+        for s0 in starts.tolist():
+            logits[r, s0:s0 + 32] = 8.0
+        above = torch.randperm(V, generator=g)[: 5 * r]
+        logits[r, above] = 9.0 + torch.rand(above.numel(), generator=g)
+    logits = logits.to(dtype)
+    val, idx = D.teacher_topk(logits.to(DEV), K, val_dtype=torch.float32, idx_dtype=torch.int32)
+    rv, ri = _ref(logits, V, K)
+    assert torch.equal(idx.cpu().long(), ri)
+    np.testing.assert_allclose(val.cpu().double().numpy(), rv.numpy(), atol=1e-5)
+
+
 @pytest.mark.parametrize("dtype,V,K", [(torch.bfloat16, 50257, 200), (torch.float32, 50257, 400), (torch.float16, 1001, 10),
                                        (torch.bfloat16, 131073, 64), (torch.float32, 7, 7)])
 def test_any_vocabulary_size(D, dtype, V, K):
