@@ -943,14 +943,17 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
       }
     }
   }
-  float M = -INFINITY;
+  // the row's log-sum-exp from the parts' statistics: worked out where it is used, by the threads that emit
+  const auto row_lse = [&]() {
+    float M = -INFINITY;
 #pragma unroll
-  for (int q = 0; q < PROD_MAX_PARTS; ++q) M = fmaxf(M, q < P ? hd[q].mx : -INFINITY);
-  float S = 0.f;
+    for (int q = 0; q < PROD_MAX_PARTS; ++q) M = fmaxf(M, q < P ? hd[q].mx : -INFINITY);
+    float S = 0.f;
 #pragma unroll
-  for (int q = 0; q < PROD_MAX_PARTS; ++q)
-    if (q < P && hd[q].mx != -INFINITY) S += hd[q].sm * fast_exp2((hd[q].mx - M) * LOG2E);
-  const float lse = (M * LOG2E + fast_log2(S)) * LN2;
+    for (int q = 0; q < PROD_MAX_PARTS; ++q)
+      if (q < P && hd[q].mx != -INFINITY) S += hd[q].sm * fast_exp2((hd[q].mx - M) * LOG2E);
+    return (M * LOG2E + fast_log2(S)) * LN2;
+  };
   int* hist = reinterpret_cast<int*>(sel);                          // 256 counters, in the list of selected words (unused so far)
   if (tid == 0) { s_nq = 0; s_total = 0; sh.nsel = 0; }
   hist[tid] = 0;
@@ -1135,7 +1138,19 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
         base[u] = 0;
         left[u] = 0;                                                // columns of the part from the chunk's first on: 0 = nothing to test
         v[u] = C::neg_inf();
-        if (idx < n_q * CPG) {
+        if constexpr (ALIGNED) {
+          // whole chunks on the grid: the chunk's number in the row gives address and column; a chunk that is not
+          // there reads as keys of 0, below every L
+          v[u] = u32x4{~0u, ~0u, ~0u, ~0u};
+          left[u] = C::N;
+          if (idx < n_q * CPG) {
+            const int a = glist[idx / CPG], j = idx % CPG;
+            const int q = a / GPP, gi = a % GPP;
+            const unsigned c = (unsigned)q * (NT * NCH) + (CPG == 4 ? (gi / (NT / 4)) * NT + 4 * (gi % (NT / 4)) + j : gi);
+            base[u] = (int)(c * C::N);
+            if ((int64_t)base[u] < p.V) v[u] = load16_stream(row + (uint64_t)c * 16);
+          }
+        } else if (idx < n_q * CPG) {
           const int a = glist[idx / CPG], j = idx % CPG;
           const int q = a / GPP, gi = a % GPP;
           // chunk of the part: the j-th of the quad's four neighbours, or the thread's own
@@ -1159,7 +1174,7 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
           for (int h = 0; h < KY::PER_DWORD; ++h) {
             const unsigned k = KY::key(kd, h);
             const int e = d * KY::PER_DWORD + h;
-            if (k >= L && e < left[u]) {
+            if (k >= L && (ALIGNED || e < left[u])) {
               const int slot = atomicAdd(&s_total, 1);
               if (slot < acap) {
                 if (narrow) all32[slot] = ((~k & ((1u << TAIL_BITS) - 1u)) << COL_BITS) | (unsigned)(base[u] + e);
@@ -1181,6 +1196,7 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
   if (KY::BITS == 16 && narrow) {
     if (total <= 512) {                                             // the rule: one wave sorts the narrow words as they are
       if (w == 0) {
+        const float lse = row_lse();
         if (total <= 256) {
           unsigned c[4];
 #pragma unroll
@@ -1211,7 +1227,7 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const ProducerParams p
       }
     __syncthreads();
   }
-  select_and_emit<Tag>(p, ro, lse, all, sel, total, sel_cap, sh);
+  select_and_emit<Tag>(p, ro, row_lse(), all, sel, total, sel_cap, sh);
 }
 
 static int producer_parts(int64_t V, int logits_dtype) {
