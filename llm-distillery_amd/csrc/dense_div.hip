@@ -379,15 +379,15 @@ __global__ __launch_bounds__(256) void dense_clear_kernel(u32x4* ws, int64_t n16
 // Units per thread of the split kernels for a dtype pair (0: the pair has no register kernel).
 static int dense_split_units(int s_dtype, int t_dtype) {
   if (s_dtype == t_dtype) return s_dtype == F32 ? 4 : 8;
-  return t_dtype == F32 ? 6 : 0;
+  return t_dtype == F32 ? 6 : s_dtype == F32 ? 4 : 0;
 }
 // How a row of V columns is cut: threads per part and parts (parts == 0: not cut).  Measured (forward KL, 512 and
 // 8192 rows, 32000 to 262144 columns, fp32 pairs, 16-bit pairs and a 16-bit student against an fp32 teacher):
 //   * a row that half a workgroup's registers hold (512 threads) stays whole;
 //   * with a 16-bit student up to four parts of 256 threads beat half as many of 512 (more workgroups per CU to
 //     hide the exchange behind), beyond that the partners to wait for cost more than they bring: parts of 512
-//     threads, at most 8; fp32 pairs (a part of 256 threads holds 8192 columns only) take parts of 512 from the start;
-//   * wider still, rows against an fp32 teacher take parts of 1024 threads (beyond 8 of those, and beyond 262144
+//     threads, at most 8; fp32 students (a part of 256 threads holds 8192 columns only) take parts of 512 from the start;
+//   * wider still, pairs with an fp32 row take parts of 1024 threads (beyond 8 of those, and beyond 262144
 //     columns of a 16-bit pair, one workgroup per row streams the row from the caches);
 //   * on fewer than 1024 rows the cut pays only from 256 KiB of row pair upwards (one workgroup per row keeps
 //     the CUs busy by itself below that, and has no partners to wait for).
@@ -400,13 +400,13 @@ static DenseCut dense_split_cut(int kind, int s_dtype, int t_dtype, int64_t n_ro
   const auto parts_of = [&](int nt) { return (units + (int64_t)nt * nu - 1) / ((int64_t)nt * nu); };
   const auto cut_of = [&](int nt) {
     const int64_t parts = parts_of(nt);
-    return parts >= 2 && parts <= DENSE_MAX_PARTS && (nt != 1024 || t_dtype == F32) ? DenseCut{nt, (int)parts} : DenseCut{0, 0};
+    return parts >= 2 && parts <= DENSE_MAX_PARTS && (nt != 1024 || t_dtype == F32 || s_dtype == F32) ? DenseCut{nt, (int)parts} : DenseCut{0, 0};
   };
   if (forced_nt) return cut_of(forced_nt);
   if (parts_of(512) < 2) return {0, 0};
   const int64_t pair_bytes = V * ((s_dtype == F32 ? 4 : 2) + (t_dtype == F32 ? 4 : 2));
   if (n_rows < 1024 && pair_bytes < 256 * 1024) return {0, 0};
-  if (parts_of(256) <= 4 && s_dtype != F32) return cut_of(256);
+  if (parts_of(256) <= 4 && s_dtype != F32) return cut_of(256);      // (fp32 students: 8192 columns per such part only)
   if (parts_of(512) <= DENSE_MAX_PARTS) return cut_of(512);
   return cut_of(1024);
 }
@@ -427,7 +427,7 @@ static void launch_dense_split(const DenseParams& p, const DenseSplit& x, int nt
     if (p.kind == DL_FKL) launch_dense_split_kind<DL_FKL, TagS, TagT, 256, NU>(p, x, st);
     else launch_dense_split_kind<DL_RKL, TagS, TagT, 256, NU>(p, x, st);
   } else if (nt == 1024) {
-    if constexpr (TagT::bytes == 4) {                  // 16-bit pairs reach 262144 columns with parts of 512 threads
+    if constexpr (TagT::bytes == 4 || TagS::bytes == 4) {      // 16-bit pairs reach 262144 columns with parts of 512 threads
       if (p.kind == DL_FKL) launch_dense_split_kind<DL_FKL, TagS, TagT, 1024, NU>(p, x, st);
       else launch_dense_split_kind<DL_RKL, TagS, TagT, 1024, NU>(p, x, st);
     }
@@ -441,7 +441,9 @@ static void launch_dense_split_pair(const DenseParams& p, const DenseSplit& x, i
   else if (p.s_dtype == BF16 && p.t_dtype == BF16) launch_dense_split<TagBF16, TagBF16, 8>(p, x, nt, st);
   else if (p.s_dtype == F16 && p.t_dtype == F16) launch_dense_split<TagF16, TagF16, 8>(p, x, nt, st);
   else if (p.s_dtype == BF16 && p.t_dtype == F32) launch_dense_split<TagBF16, TagF32, 6>(p, x, nt, st);
-  else launch_dense_split<TagF16, TagF32, 6>(p, x, nt, st);
+  else if (p.s_dtype == F16 && p.t_dtype == F32) launch_dense_split<TagF16, TagF32, 6>(p, x, nt, st);
+  else if (p.s_dtype == F32 && p.t_dtype == BF16) launch_dense_split<TagF32, TagBF16, 4>(p, x, nt, st);
+  else launch_dense_split<TagF32, TagF16, 4>(p, x, nt, st);
 }
 
 // Rows too wide for the registers, 16-byte aligned: the same sweeps, every one of them over global
@@ -714,13 +716,16 @@ static bool launch_dense_reg(const DenseParams& p, hipStream_t st) {
   return launch_dense_kind<DL_JSD, TagS, TagT, NU>(p, st);
 }
 
-// Register path for the dtype pairs that occur: teacher stored like the student, or in fp32.
+// Register path for the dtype pairs that occur: teacher stored like the student, or in fp32, or a 16-bit teacher
+// against a student that the caller has already cast to fp32 (as the reference does with its logits).
 static bool launch_dense_pair(const DenseParams& p, hipStream_t st) {
   if (p.s_dtype == F32 && p.t_dtype == F32) return launch_dense_reg<TagF32, TagF32, 4>(p, st);
   if (p.s_dtype == BF16 && p.t_dtype == BF16) return launch_dense_reg<TagBF16, TagBF16, 8>(p, st);
   if (p.s_dtype == F16 && p.t_dtype == F16) return launch_dense_reg<TagF16, TagF16, 8>(p, st);
   if (p.s_dtype == BF16 && p.t_dtype == F32) return launch_dense_reg<TagBF16, TagF32, 4>(p, st);
   if (p.s_dtype == F16 && p.t_dtype == F32) return launch_dense_reg<TagF16, TagF32, 4>(p, st);
+  if (p.s_dtype == F32 && p.t_dtype == BF16) return launch_dense_reg<TagF32, TagBF16, 4>(p, st);
+  if (p.s_dtype == F32 && p.t_dtype == F16) return launch_dense_reg<TagF32, TagF16, 4>(p, st);
   return false;
 }
 

@@ -55,7 +55,9 @@ def _pair(R, V, dtype, seed, t_dtype=None, noise=1.0, std=2.0):
 
 @pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
 @pytest.mark.parametrize("dtype,t_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
-                                           (torch.float16, torch.float16), (torch.bfloat16, torch.float32)])
+                                           (torch.float16, torch.float16), (torch.bfloat16, torch.float32),
+                                           (torch.float32, torch.bfloat16), (torch.float32, torch.float16),
+                                           (torch.bfloat16, torch.float16)])
 def test_dense_small(D, kind, dtype, t_dtype):
     s, t = _pair(21, 2048, dtype, 1, t_dtype)
     _check(D, kind, s, t, T=1.0)
@@ -190,6 +192,17 @@ def test_dense_wide_16bit_student_fp32_teacher_with_masked_rows(D, kind):
     _check(D, kind, s, t[valid], T=1.7, valid=valid, teacher_T=1.0)
 
 
+@pytest.mark.parametrize("kind", ["fkl", "rkl", "jsd"])
+@pytest.mark.parametrize("V,t_dtype", [(32000, torch.bfloat16), (70000, torch.float16), (151936, torch.bfloat16)])
+def test_dense_fp32_student_against_a_16bit_teacher(D, kind, V, t_dtype):
+    # the student already cast to fp32 by the caller, the teacher as its model left it: register kernels up to
+    # 1024 threads x 4 units, the student row on the CU beyond, both rows streamed beyond that
+    s, t = _pair(7, V, torch.float32, 12, t_dtype)
+    valid = torch.ones(7, dtype=torch.bool)
+    valid[3] = False
+    _check(D, kind, s, t[valid], T=1.2, valid=valid, teacher_T=0.9)
+
+
 def test_dense_identical_distributions_give_zero(D):
     s, _ = _pair(8, 8192, torch.float32, 6)
     for kind in ("fkl", "rkl", "jsd"):
@@ -292,7 +305,10 @@ def test_reverse_kl_with_student_logits_of_minus_infinity(D, dtype, V):
     (torch.bfloat16, torch.float32, 200064, 0),      # too wide for 8 parts of 512 x 6: 5 parts of 1024 threads
     (torch.float32, torch.float32, 151936, 0),       # the same for an fp32 pair: 5 parts of 1024 x 4
     (torch.float32, torch.float32, 40000, 1024),     # 2 parts of 1024 x 4
-    (torch.float32, torch.float32, 65536, 0)])       # 4 full parts of 512 x 4
+    (torch.float32, torch.float32, 65536, 0),        # 4 full parts of 512 x 4
+    (torch.float32, torch.bfloat16, 50304, 0),       # fp32 student against a 16-bit teacher: 4 parts of 512 x 4
+    (torch.float32, torch.float16, 32000, 256),      # 4 parts of 256 x 4
+    (torch.float32, torch.bfloat16, 151936, 0)])     # 5 parts of 1024 x 4
 def test_rows_cut_into_column_parts(D, kind, dtype, t_dtype, V, threads):
     """dl_div_dense_ws: wide forward / reverse-KL rows cut into parts of 256, 512 or 1024 threads that exchange their
     maxima and sums through the workspace.  Both forms against the oracle, the row losses of the two against each other
