@@ -474,3 +474,29 @@ def test_phase_one_logits_at_clustered_repeated_and_outlying_teacher_ids(D, dtyp
     want = torch.where(inside, torch.gather(x.float(), 1, idx.clamp(0, V - 1)) * 0.7, torch.zeros(()))
     assert torch.equal(zk.cpu(), want)
     np.testing.assert_allclose(lse.cpu().double().numpy(), torch.logsumexp(x.double() * 0.7, -1).numpy(), rtol=2e-6, atol=2e-6)
+
+
+@pytest.mark.parametrize("dtype,V,K", [(torch.bfloat16, 131072, 64),      # 64 rounds of 256 chunks: the widest row whose ids come out of the sweep
+                                       (torch.bfloat16, 131080, 64),      # one chunk more: gathered directly
+                                       (torch.float32, 65536, 300), (torch.float32, 65540, 300),
+                                       (torch.bfloat16, 50257, 200),      # rows off the 16-byte grid: ids before and behind the aligned body
+                                       (torch.float32, 32003, 1100),      # more entries than the sweep keeps slots for
+                                       (torch.float16, 4104, 1024)])
+def test_phase_one_ids_out_of_the_sweep_or_gathered(D, dtype, V, K):
+    """zk is the logit at the teacher's id times 1/T, bit for bit, whichever way phase 1 fetches it: out of its sweep
+    (rows of up to 64 rounds, up to 1024 entries), by loads of its own beyond, element by element in the columns before
+    and behind the aligned body of a row off the 16-byte grid."""
+    from llm_distillery_amd import ops
+    R = 5
+    g = torch.Generator().manual_seed(V + K)
+    x = (torch.randn(R, V, generator=g) * 3).to(dtype)
+    idx = torch.randint(0, V, (R, K), generator=g, dtype=torch.int64)
+    idx[0, :16] = torch.arange(16)                                         # the row's first columns
+    idx[1, :16] = V - 1 - torch.arange(16)                                 # and its last
+    idx[2, :8] = torch.tensor([-5, V, V + 7, 2 ** 31 - 1, -1, 0, V - 1, V // 2])
+    idx[3] = idx[3, 0] // 8 * 8 + torch.arange(K) % 8                      # every entry in one chunk or two
+    lse, zk = ops._rowstats_raw(x.to(DEV), idx.to(DEV), None, 1.0 / 1.3)
+    inside = (idx >= 0) & (idx < V)
+    want = torch.where(inside, torch.gather(x.float(), 1, idx.clamp(0, V - 1)) * np.float32(1.0 / 1.3), torch.zeros(()))
+    assert torch.equal(zk.cpu(), want)
+    np.testing.assert_allclose(lse.cpu().double().numpy(), torch.logsumexp(x.double() / 1.3, -1).numpy(), rtol=3e-6, atol=3e-6)
