@@ -450,8 +450,8 @@ int dl_marginalise_map(const void* probs, int p_dtype, int64_t p_stride, int64_t
  *   dl_expand_columns   dst[r, j] = src[r, col_src[j]] for j < V; col_src[j] < 0 (a column outside the subset) gives 0.
  * Raw 2- or 4-byte elements of `dtype`, no conversion.  cols int32 [n_cols], col_src int32 [V], both 16-byte
  * aligned; dst rows on the 16-byte grid, n_cols (gather) / V (expand) whole 16-byte chunks (else DL_ERR_ALIGN);
- * src rows of any stride.  n_rows <= 65535 per call.  Reference: none (serves BASELINE configuration 5 at the
- * student vocabulary of configurations 3 and 4).
+ * src rows of any stride.  n_rows <= 65535 per call.  Reference: none (serves the byte-trie reverse KL where the
+ * student vocabulary is too wide for a marginal in LDS: 128256 ids).
  */
 int dl_gather_columns(const void* src, int dtype, int64_t src_stride, int64_t n_rows, int64_t V, const int32_t* cols,
                       int64_t n_cols, void* dst, int64_t dst_stride, void* stream);
@@ -492,7 +492,7 @@ int dl_rkl_marginalised(const void* logits, int logits_dtype, int64_t row_stride
  * every 16-byte chunk once.  Other arguments, conventions and results as dl_rkl_marginalised (the loss and the
  * gradient are those of the full vocabulary).  cols / col_src16 16-byte aligned, gradient rows on the 16-byte grid,
  * Vs_full a multiple of 8; the logits rows need element alignment only.  No counterpart in the reference
- * (BASELINE configuration 5 at the student vocabulary of configurations 3 and 4).
+ * (the byte-trie reverse KL on maps that use few student ids, and on student vocabularies of 128256 ids).
  */
 int dl_rkl_marginalised_compact(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t Vs_full,
                                 const int32_t* cols, const uint16_t* col_src16, int64_t n_compact,
