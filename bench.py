@@ -294,7 +294,7 @@ def _wl_dropin(batched):
                                          b["rec"].data_ptr(), b["coef"].data_ptr(), b["out"].data_ptr(), st)
             for i in range(B):
                 x, b = xs[i].detach(), bufs[i]
-                lib.dl_composite_backward_fused(x.data_ptr(), 0, V, N, V, 1.0, tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
+                lib.dl_composite_backward_fused(x.data_ptr(), 0, V, N, V, 0, N, 1.0, tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
                                                 offs[0], 1, 1, b["lse"].data_ptr(), b["zk"].data_ptr(), b["rec"].data_ptr(),
                                                 b["coef"].data_ptr(), b["g"].data_ptr(), b["grad"].data_ptr(), V, st)
             return bufs[0]["out"]

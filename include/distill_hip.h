@@ -268,18 +268,18 @@ int dl_composite_backward(const float* lse, const float* zk, const void* t_val, 
                           float* g_zk, void* stream);
 
 /*
- * dl_composite_backward and dl_rowcoef_grad_topk in one launch, for the usual case that teacher row i belongs to
- * logits row i (no row map, as many teacher rows as logits rows): every column part of a row makes the row's K
+ * dl_composite_backward and dl_rowcoef_grad_topk in one launch: every column part of a row makes the row's K
  * coefficients and their sum itself (from the row's record, its conversation's coefficients and g_train) instead
  * of reading what a launch before it wrote (the reference's default shape, one conversation of 2048 x 32000
  * logits, is a few tens of microseconds of kernels per call: a launch saved counts there).  Same reference lines
- * and the same arguments with the same meaning as the two entry points it stands for.  grad [n_rows, V] =
+ * and the same arguments with the same meaning as the two entry points it stands for (row_map / n_teacher_rows as
+ * for dl_rowcoef_grad_topk: the K-wide arrays, the records and the offsets count teacher rows).  grad [n_rows, V] =
  * d(sum_c g_train[c] * train_loss[c]) / d logits, to fp32 rounding what the two entry points give (the sum over
  * the K coefficients is taken in another order); rows and alignment as for dl_rowcoef_grad_topk.
  */
 int dl_composite_backward_fused(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
-                                int64_t V, float inv_T, const void* t_val, int t_val_dtype,
-                                float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
+                                int64_t V, const int32_t* row_map, int64_t n_teacher_rows, float inv_T,
+                                const void* t_val, int t_val_dtype, float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
                                 const int32_t* row_off, int offsets_on_host, int n_convos, const float* lse,
                                 const float* zk, const void* row_records, const void* row_coef,
                                 const float* g_train, void* grad, int64_t grad_stride, void* stream);

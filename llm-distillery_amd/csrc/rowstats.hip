@@ -469,17 +469,18 @@ extern "C" int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_
 }
 
 extern "C" int dl_composite_backward_fused(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,
-                                           int64_t V, float inv_T, const void* t_val, int t_val_dtype,
+                                           int64_t V, const int32_t* row_map, int64_t n_teacher_rows, float inv_T,
+                                           const void* t_val, int t_val_dtype,
                                            float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
                                            const int32_t* row_off, int offsets_on_host, int n_convos, const float* lse,
                                            const float* zk, const void* row_records, const void* row_coef,
                                            const float* g_train, void* grad, int64_t grad_stride, void* stream) {
   using namespace dl;
-  const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_rows);
+  const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_teacher_rows);
   if (rc != DL_OK) return rc;
   CompositeParams cp;
   const int st0 = composite_backward_params(cp, lse, zk, t_val, t_val_dtype, inv_T_teacher, t_idx, t_idx_itype, K, row_off,
-                                            offsets_on_host, n_convos, n_rows, row_records, row_coef, g_train);
+                                            offsets_on_host, n_convos, n_teacher_rows, row_records, row_coef, g_train);
   if (st0 != DL_OK) return st0;
   if (!grad) return DL_ERR_NULL;
   if (grad_stride < V) return DL_ERR_SHAPE;
@@ -488,7 +489,7 @@ extern "C" int dl_composite_backward_fused(const void* logits, int logits_dtype,
   if (reinterpret_cast<uintptr_t>(logits) % eb != 0 || reinterpret_cast<uintptr_t>(grad) % eb != 0) return DL_ERR_ALIGN;
   const bool on_grid = aligned16(logits, row_stride, eb) && aligned16(grad, grad_stride, eb);
   const int vec = on_grid ? (V % (16 / eb) == 0 ? 1 : 3) : same_phase16(logits, row_stride, grad, grad_stride, eb) ? 2 : 0;
-  StatsParams p{logits, row_stride, n_rows, V, nullptr, t_idx, t_idx_itype, K, n_rows, inv_T,
+  StatsParams p{logits, row_stride, n_rows, V, row_map, t_idx, t_idx_itype, K, n_teacher_rows, inv_T,
                 const_cast<float*>(lse), nullptr, nullptr, nullptr, grad, grad_stride};
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const hipError_t e = logits_dtype == DL_F32 ? launch_coef<TagF32>(p, vec, st, &cp)

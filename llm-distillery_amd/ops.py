@@ -379,6 +379,11 @@ def _composite_forward_raw(logits, t_val, t_idx, labels, avoid, offsets, row_map
     return out, lse, zk, rec, coef
 
 
+# The composite loss's backward is one launch (dl_composite_backward_fused) or two (dl_composite_backward +
+# dl_rowcoef_grad_topk), chosen by the rows' width; "fused" / "separate" here fixes the form (the tests compare them).
+FORCE_COMPOSITE_BACKWARD = None
+
+
 def _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, offsets, row_map, inv_T, inv_T_teacher, crop):
     """The epilogue's backward + phase 2: d(sum_c g_train[c] * train_loss[c]) / d logits, full width."""
     x = _cropped(logits, crop)
@@ -393,10 +398,15 @@ def _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, o
         grad[:, crop:].zero_()
     gx = _cropped(grad, crop)
     stream = _stream_ptr(dev)
-    if row_map is None and N == R:                       # teacher row i belongs to logits row i: one launch
+    # Phase 2 making the rows' coefficients itself saves a launch and two K-wide arrays, but every column part of a row
+    # (32 KiB of logits) makes all K of them: it pays up to four parts per row (0.664 against 0.676 ms on 8192 x 32000
+    # fp32 rows, K = 400) and costs beyond (4.01 against 3.95 ms on 32768 x 128256 bf16 rows, K = 200: eight parts)
+    fused = V * x.element_size() <= 4 * 32768 if FORCE_COMPOSITE_BACKWARD is None else FORCE_COMPOSITE_BACKWARD == "fused"
+    if fused:
         with torch.cuda.device(dev):
             st = lib.dl_composite_backward_fused(
-                x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, inv_T, t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher,
+                x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, row_map.data_ptr() if row_map is not None else 0, N, inv_T,
+                t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher,
                 t_idx.data_ptr(), _IT[t_idx.dtype], K, offs[0], on_host, C, lse.data_ptr(), zk.data_ptr(), rec.data_ptr(),
                 coef.data_ptr(), g.data_ptr(), gx.data_ptr(), gx.stride(0), stream)
             _lib.check(st, "dl_composite_backward_fused")
@@ -419,8 +429,8 @@ def _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, o
 
 class _CompositeLoss(torch.autograd.Function):
     """The reference's composite loss of C conversations as ONE autograd node: phase 1 over the logits
-    (dl_rowstats_topk), the K-wide epilogue (dl_composite_forward), and in backward their two
-    counterparts (dl_composite_backward, dl_rowcoef_grad_topk).  Returns (train_loss [C], the nine
+    (dl_rowstats_topk), the K-wide epilogue (dl_composite_forward), and in backward their
+    counterpart (dl_composite_backward_fused: the epilogue's backward inside phase 2).  Returns (train_loss [C], the nine
     values [C, 9]); only train_loss is differentiable, and only with respect to the logits.
     The eager path goes through this class rather than through the registered ops below (which run the
     same launches): a call through the dispatcher costs tens of microseconds of host time more, which at

@@ -409,10 +409,11 @@ def test_fused_epilogue_under_no_grad_and_label_count_mismatch(D):
     (torch.bfloat16, 128256, 128256, 200, [5, 6], True),
     (torch.float32, 4096, 4096, 600, [12, 7], True)])
 def test_coefficients_made_inside_phase_two_equal_the_separate_launches(D, dtype, V, pitch, K, lens, host_offsets):
-    """Without a row map phase 2 makes the K coefficients of a row itself (dl_composite_backward_fused); an identity
-    row map sends the same problem through the separate launches.  Forward: the same launches, the same bits.
+    """Phase 2 makes the K coefficients of a row itself (dl_composite_backward_fused), or reads what
+    dl_composite_backward wrote: ops.FORCE_COMPOSITE_BACKWARD sends the same problem through either form.  With and without a row map (one that scatters
+    the teacher rows over more logits rows, some of them masked).  Forward: the same launches, the same bits.
     Backward: the sum of the K coefficients is taken in another order, so the gradients agree to fp32 rounding of
-    the dense term."""
+    the dense term; masked rows get zeros."""
     from llm_distillery_amd import ops
     N = sum(lens)
     g = torch.Generator().manual_seed(V + K)
@@ -437,22 +438,35 @@ def test_coefficients_made_inside_phase_two_equal_the_separate_launches(D, dtype
     offsets = [row_off, label_off, avoid_off]
     if not host_offsets:
         offsets = torch.tensor(offsets, dtype=torch.int32, device=DEV)
-    full = torch.zeros(N, pitch, dtype=dtype, device=DEV)
-    full[:, :V] = xs.to(DEV)
-    ident = torch.arange(N, dtype=torch.int32, device=DEV)
-    res = {}
-    for name, rm in (("fused", None), ("separate", ident)):
-        x = full.clone().requires_grad_(True)
-        train, nine = ops.composite_loss(x, tv.to(DEV), ti.to(DEV), labels, avoid, offsets, rm, 1.0 / 1.3, 1.0, 2.0, crop=V if pitch != V else 0)
-        w = torch.arange(1, len(lens) + 1, dtype=torch.float32, device=DEV)
-        (train * w).sum().backward()
-        res[name] = (train.detach(), nine, x.grad)
     same = lambda a, b: torch.equal(a.nan_to_num(nan=-7.0), b.nan_to_num(nan=-7.0))      # a conversation of one row has no labels: its CE means are 0 / 0
-    assert same(res["fused"][0], res["separate"][0]) and same(res["fused"][1], res["separate"][1])
-    gf, gs = res["fused"][2].float(), res["separate"][2].float()
-    assert torch.count_nonzero(gf[:, V:]) == 0
-    tol = gs.abs() * (2e-5 if dtype == torch.float32 else 2.0 ** -7) + gs.abs().amax(-1, keepdim=True) * 1e-6
-    assert ((gf - gs).abs() <= tol).all(), ((gf - gs).abs() / tol).max()
+    # logits rows: as many as teacher rows, or more of them with the teacher rows scattered over every third but one
+    R = N + N // 2 + 3
+    place = torch.sort(torch.randperm(R, generator=g)[:N]).values
+    scatter = torch.full((R,), -1, dtype=torch.int32)
+    scatter[place] = torch.arange(N, dtype=torch.int32)
+    for rm, rows in ((None, torch.arange(N)), (scatter.to(DEV), place)):
+        full = torch.randn(N if rm is None else R, pitch, generator=g).to(dtype).to(DEV)      # masked rows hold logits too
+        full[rows.to(DEV), :V] = xs.to(DEV)
+        res = {}
+        for name in ("fused", "separate"):
+            ops.FORCE_COMPOSITE_BACKWARD = name
+            try:
+                x = full.clone().requires_grad_(True)
+                train, nine = ops.composite_loss(x, tv.to(DEV), ti.to(DEV), labels, avoid, offsets, rm, 1.0 / 1.3, 1.0, 2.0, crop=V if pitch != V else 0)
+                w = torch.arange(1, len(lens) + 1, dtype=torch.float32, device=DEV)
+                (train * w).sum().backward()
+            finally:
+                ops.FORCE_COMPOSITE_BACKWARD = None
+            res[name] = (train.detach(), nine, x.grad)
+        assert same(res["fused"][0], res["separate"][0]) and same(res["fused"][1], res["separate"][1])
+        gf, gs = res["fused"][2].float(), res["separate"][2].float()
+        assert torch.count_nonzero(gf[:, V:]) == 0
+        if rm is not None:
+            masked = torch.ones(R, dtype=torch.bool)
+            masked[place] = False
+            assert torch.count_nonzero(gf[masked.to(DEV)]) == 0
+        tol = gs.abs() * (2e-5 if dtype == torch.float32 else 2.0 ** -7) + gs.abs().amax(-1, keepdim=True) * 1e-6
+        assert ((gf - gs).abs() <= tol).all(), ((gf - gs).abs() / tol).max()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
