@@ -7,7 +7,9 @@ extern "C" int64_t dl_div_topk_workspace_bytes(int kind, int logits_dtype, int64
   if (kind != DL_FKL || n_rows <= 0 || V <= 0) return 0;
   const int epc = logits_dtype == DL_F32 ? 4 : 8;
   const int64_t nch = (V + epc - 1) / epc;      // a row that ends inside a chunk holds that chunk too
-  if (nch <= 512 * 16 || nch > (int64_t)dl::MAX_COARSE_PARTS * 256 * 16) return 0;
+  if (nch <= 256 * 16 || nch > (int64_t)dl::MAX_COARSE_PARTS * 256 * 16) return 0;
+  // up to 512 x 16 chunks only rows that cannot lie on the 16-byte grid are cut (in two)
+  if (nch <= 512 * 16) return V % epc != 0 ? dl::RetryList::bytes(n_rows, 2) : 0;
   return dl::RetryList::bytes(n_rows, nch <= 1024 * 16 ? 4 : dl::MAX_COARSE_PARTS);
 }
 

@@ -510,7 +510,7 @@ __device__ __forceinline__ void zero_part(char* gpart, int64_t nch, int64_t ncol
 template <class Tag, int NT, int NCH, bool SPLIT, int J, bool RETRY, bool MULTI, int RAG = ROWS_WHOLE>
 __device__ __forceinline__ void fkl_topk_part(const TopkParams& p, const TopkLds& s, int64_t r, int h) {
   static_assert(!MULTI || J > 0, "the head of a bucket travels in registers");
-  static_assert(RAG != ROWS_ANY || (!SPLIT && !MULTI), "rows off the 16-byte grid: one workgroup per row, one stored teacher");
+  static_assert(RAG != ROWS_ANY || !MULTI, "rows off the 16-byte grid: one stored teacher");
   using C = Chunk<Tag>;
   const int tid = threadIdx.x;
   const int P = SPLIT ? p.parts : 1;
@@ -1033,13 +1033,17 @@ static int split_parts(int64_t nch, int forced, bool fine = false) {
 // workgroup, chunks per thread, column parts per row (parts > 1: the split kernels, which need the
 // exchange workspace: `split_ok`).  NT == 0: none (rows too wide: the streaming kernel).
 struct FklShape { int NT, NCH, parts; };
-static FklShape fkl_shape(int64_t nch, int bytes, int forced_parts, bool split_ok, bool fine = false) {
+static FklShape fkl_shape(int64_t nch, int bytes, int forced_parts, bool split_ok, bool fine = false, bool thirteen = false) {
   if (nch > (int64_t)MAX_COARSE_PARTS * 256 * 16) return {0, 0, 0};
   if (fine && split_ok && nch > 256 * 4 && nch <= (int64_t)MAX_PARTS * 256 * 4) return {256, 4, split_parts(nch, forced_parts, true)};
   if (nch <= 256 * 4) return {256, 4, 1};
   if (nch <= 256 * 8) return {256, 8, 1};
   // 4-byte logits: 8 chunks per thread from twice the threads keep the corrections in registers
   if (nch <= 256 * 16) return bytes == 4 ? FklShape{512, 8, 1} : FklShape{256, 16, 1};
+  // two-byte rows of up to 53248 columns (the 50k vocabularies): 13 chunks per thread.  A workgroup's waves are
+  // filled one after the other and the full ones set its time: 13 sweeps instead of 16
+  // (16384 x 50304 bf16: 64.6 -> 68.3 % of the HBM peak, 51200 columns: 69 %)
+  if (thirteen && bytes != 4 && nch <= 512 * 13) return {512, 13, 1};
   if (nch <= 512 * 16) return {512, 16, 1};
   const int parts = split_parts(nch, forced_parts);
   // The widest rows in half as many parts of 512 threads: fewer partners to wait for.  Measured at 8192
@@ -1063,9 +1067,9 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
   const bool fine = !MULTI && (p.flags & DL_TOPK_FINE_PARTS) != 0 &&
                     ws_bytes >= RetryList::bytes(p.n_rows, split_parts(nch, forced, true));
   // the shape a workspace would allow; without room for that shape's records, the shape that needs none
-  const FklShape wish = aligned ? fkl_shape(nch, Tag::bytes, forced, true, fine) : FklShape{0, 0, 0};
+  const FklShape wish = aligned ? fkl_shape(nch, Tag::bytes, forced, true, fine, !MULTI) : FklShape{0, 0, 0};
   const bool split_ok = p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, wish.parts) && p.n_rows * wish.parts <= 0x7fffffffLL;
-  const FklShape sh = !aligned || wish.parts <= 1 || split_ok ? wish : fkl_shape(nch, Tag::bytes, forced, false, fine);
+  const FklShape sh = !aligned || wish.parts <= 1 || split_ok ? wish : fkl_shape(nch, Tag::bytes, forced, false, fine, !MULTI);
   switch (sh.NT * 100 + sh.NCH) {
     case 256 * 100 + 4:
       if constexpr (!MULTI)
@@ -1078,6 +1082,9 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
     case 256 * 100 + 16:
       if (sh.parts > 1) return launch_split<Tag, 256, 16, MULTI, RAG>(p, sh.parts, st, ws_cleared);
       if constexpr (Tag::bytes != 4) return launch_reg<Tag, 256, 16, MULTI, RAG>(p, st);
+      break;
+    case 512 * 100 + 13:
+      if constexpr (Tag::bytes != 4 && !MULTI) return launch_reg<Tag, 512, 13, MULTI, RAG>(p, st);
       break;
     case 512 * 100 + 16:
       return sh.parts > 1 ? launch_split<Tag, 512, 16, MULTI, RAG>(p, sh.parts, st, ws_cleared) : launch_reg<Tag, 512, 16, MULTI, RAG>(p, st);
@@ -1096,7 +1103,14 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
       // (16384 x 32100 bf16: 0.47 ms against 0.75 ms streaming; 16384 x 50257: 1.27 against 0.92): up to
       // 256 x 16 chunks they win; the 512 x 16 shape spills under the extra addressing and only beats the
       // element-wise kernel, which rows on different phases would otherwise take.
-      const FklShape any = fkl_shape((p.V + Tag::epc - 1) / Tag::epc, Tag::bytes, 0, false);
+      // Beyond 256 x 16 chunks: column parts of that shape (parts of a row start a whole number of chunks behind the
+      // row's first element, wherever that lies), where a workspace for their exchange came along.
+      const int64_t nch_any = (p.V + Tag::epc - 1) / Tag::epc;
+      const int parts_any = (int)((nch_any + 256 * 16 - 1) / (256 * 16));
+      if (parts_any >= 2 && parts_any <= MAX_COARSE_PARTS && p.workspace && ws_bytes >= RetryList::bytes(p.n_rows, parts_any) &&
+          p.n_rows * parts_any <= 0x7fffffffLL)
+        return launch_split<Tag, 256, 16, false, ROWS_ANY>(p, parts_any, st, ws_cleared);
+      const FklShape any = fkl_shape(nch_any, Tag::bytes, 0, false);
       if (any.parts == 1) switch (any.NT * 100 + any.NCH) {
         case 256 * 100 + 4: return launch_reg_any<Tag, 256, 4>(p, st);
         case 256 * 100 + 8: return launch_reg_any<Tag, 256, 8>(p, st);

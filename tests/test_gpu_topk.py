@@ -66,7 +66,7 @@ def test_topk_small(D, dtype, kind):
 
 
 @pytest.mark.parametrize("V,K", [(32000, 200), (128256, 200), (50264, 64), (8192, 400), (32000, 2048), (128256, 1024),
-                                 (65536, 2048)])
+                                 (65536, 2048), (40968, 200), (49152, 1000), (53248, 400), (53256, 16)])      # 512 x 13 chunks up to 53248 columns
 def test_fkl_topk_register_path_sizes(D, V, K):
     logits, tv, ti = _case(24, V, K, torch.bfloat16, 2, std=3.0)
     _check(D, "fkl", logits, tv, ti, T=1.0)
@@ -99,7 +99,9 @@ def test_streaming_path_odd_vocab_and_int64_fp32_teacher(D, V):
                                                   (torch.bfloat16, 5001, 5120, 3),          # a column slice of aligned rows: one phase for all rows
                                                   (torch.float16, 7, 7, 0),                 # rows shorter than a chunk
                                                   (torch.float32, 4099, 4104, 2),
-                                                  (torch.bfloat16, 50257, 50257, 0),        # wider than 256 x 16 chunks: streaming, or 512 x 16 unaligned
+                                                  (torch.bfloat16, 50257, 50257, 0),        # wider than 256 x 16 chunks: two column parts
+                                                  (torch.float16, 151665, 151665, 0),       # five
+                                                  (torch.float32, 40003, 40003, 0),         # three, of four-byte chunks
                                                   (torch.float32, 10001, 10001, 0)])        # 512 threads x 8 chunks of fp32
 @pytest.mark.parametrize("grad_mode", ["fresh", "in_place", "other_phase"])
 @pytest.mark.parametrize("kind", ["fkl", "rkl"])
@@ -147,7 +149,7 @@ def test_rows_off_the_16_byte_grid(D, kind, dtype, V, pitch, offset, grad_mode):
         assert torch.count_nonzero(full[:, :offset]) == 0 and torch.count_nonzero(full[:, offset + V:]) == 0
 
 
-@pytest.mark.parametrize("dtype,V,pitch", [(torch.bfloat16, 50257, 50304),      # GPT-2's vocabulary in its padded rows: 512 x 16, one workgroup per row
+@pytest.mark.parametrize("dtype,V,pitch", [(torch.bfloat16, 50257, 50304),      # GPT-2's vocabulary in its padded rows: 512 x 13, one workgroup per row
                                            (torch.bfloat16, 151665, 151936),    # Qwen's: five column parts, the last one ragged
                                            (torch.float32, 32003, 32064),       # 512 x 16 of four-byte chunks
                                            (torch.float16, 4099, 4104),         # 256 x 4
