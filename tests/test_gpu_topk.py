@@ -151,6 +151,7 @@ def test_rows_off_the_16_byte_grid(D, kind, dtype, V, pitch, offset, grad_mode):
 
 @pytest.mark.parametrize("dtype,V,pitch", [(torch.bfloat16, 50257, 50304),      # GPT-2's vocabulary in its padded rows: 512 x 13, one workgroup per row
                                            (torch.bfloat16, 151665, 151936),    # Qwen's: five column parts, the last one ragged
+                                           (torch.float16, 100277, 100352),     # four parts of 13 chunks per thread
                                            (torch.float32, 32003, 32064),       # 512 x 16 of four-byte chunks
                                            (torch.float16, 4099, 4104),         # 256 x 4
                                            (torch.bfloat16, 65537, 65544),      # one column more than two parts hold: the third part is one ragged chunk
@@ -316,11 +317,13 @@ def test_gradient_may_overwrite_the_logits(D, kind, V, dtype):
 
 
 @pytest.mark.parametrize("V,dtype", [(152064, torch.bfloat16), (128256, torch.float32), (262144, torch.float16),
-                                     (100000, torch.float32), (98304, torch.float32), (229376, torch.bfloat16)])
+                                     (100000, torch.float32), (98304, torch.float32), (229376, torch.bfloat16),
+                                     (100352, torch.bfloat16), (114688, torch.float16), (200064, torch.bfloat16)])
 def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
     """Vocabularies beyond 131072 two-byte (65536 four-byte) entries are cut into 5..8 parts of 4096
-    chunks, or (four-byte rows of 6 parts and more, two-byte rows of 8) into 3..4 parts of 8192; with and
-    without waiting for the partners the oracle's numbers and the same bits."""
+    chunks, or (four-byte rows of 6 parts and more, two-byte rows of 8) into 3..4 parts of 8192; two-byte rows that do
+    not fill their parts into parts of 13 to 15 chunks per thread (100352 columns: 4 x 256 x 13, 114688: 4 x 14,
+    152064: 5 x 15, 200064: 7 x 14); with and without waiting for the partners the oracle's numbers and the same bits."""
     logits, tv, ti = _case(10, V, 48, dtype, 41, std=3.0)
     valid = torch.ones(10, dtype=torch.bool)
     valid[4] = False
