@@ -1052,10 +1052,10 @@ static FklShape fkl_shape(int64_t nch, int bytes, int forced_parts, bool split_o
   if (split_ok && nch > 1024 * 16 && (bytes == 4 ? parts >= 6 : parts == 8)) return {512, 16, (parts + 1) / 2};
   if (parts == 2 && split_ok) return {512, 16, 2};
   if (parts >= 3 && split_ok) {
-    // two-byte rows that do not fill their parts: as few chunks per thread as hold the row (13 to 15), the parts then
-    // equally full -- every wave of every part carries the same share, and that share sets the row's time
+    // rows that do not fill their parts: as few chunks per thread as hold the row (13 to 15), the parts then equally
+    // full -- every wave of every part carries the same share, and that share sets the row's time
     const int64_t per_thread = (nch + (int64_t)parts * 256 - 1) / ((int64_t)parts * 256);
-    if (thirteen && bytes != 4 && per_thread < 16) return {256, per_thread < 13 ? 13 : (int)per_thread, parts};
+    if (thirteen && per_thread < 16) return {256, per_thread < 13 ? 13 : (int)per_thread, parts};
     return {256, 16, parts};
   }
   if (nch <= 1024 * 16) return {1024, 16, 1};      // no workspace: one workgroup per row
@@ -1093,13 +1093,13 @@ static int launch_fkl(const TopkParams& p, bool aligned, int64_t ws_bytes, hipSt
       if constexpr (Tag::bytes != 4 && !MULTI) return launch_reg<Tag, 512, 13, MULTI, RAG>(p, st);
       break;
     case 256 * 100 + 13:
-      if constexpr (Tag::bytes != 4 && !MULTI) return launch_split<Tag, 256, 13, MULTI, RAG>(p, sh.parts, st, ws_cleared);
+      if constexpr (!MULTI) return launch_split<Tag, 256, 13, MULTI, RAG>(p, sh.parts, st, ws_cleared);
       break;
     case 256 * 100 + 14:
-      if constexpr (Tag::bytes != 4 && !MULTI) return launch_split<Tag, 256, 14, MULTI, RAG>(p, sh.parts, st, ws_cleared);
+      if constexpr (!MULTI) return launch_split<Tag, 256, 14, MULTI, RAG>(p, sh.parts, st, ws_cleared);
       break;
     case 256 * 100 + 15:
-      if constexpr (Tag::bytes != 4 && !MULTI) return launch_split<Tag, 256, 15, MULTI, RAG>(p, sh.parts, st, ws_cleared);
+      if constexpr (!MULTI) return launch_split<Tag, 256, 15, MULTI, RAG>(p, sh.parts, st, ws_cleared);
       break;
     case 512 * 100 + 16:
       return sh.parts > 1 ? launch_split<Tag, 512, 16, MULTI, RAG>(p, sh.parts, st, ws_cleared) : launch_reg<Tag, 512, 16, MULTI, RAG>(p, st);

@@ -318,12 +318,13 @@ def test_gradient_may_overwrite_the_logits(D, kind, V, dtype):
 
 @pytest.mark.parametrize("V,dtype", [(152064, torch.bfloat16), (128256, torch.float32), (262144, torch.float16),
                                      (100000, torch.float32), (98304, torch.float32), (229376, torch.bfloat16),
-                                     (100352, torch.bfloat16), (114688, torch.float16), (200064, torch.bfloat16)])
+                                     (100352, torch.bfloat16), (114688, torch.float16), (200064, torch.bfloat16),
+                                     (50304, torch.float32), (57344, torch.float32)])
 def test_rows_cut_into_five_to_eight_parts(D, V, dtype):
     """Vocabularies beyond 131072 two-byte (65536 four-byte) entries are cut into 5..8 parts of 4096
     chunks, or (four-byte rows of 6 parts and more, two-byte rows of 8) into 3..4 parts of 8192; two-byte rows that do
-    not fill their parts into parts of 13 to 15 chunks per thread (100352 columns: 4 x 256 x 13, 114688: 4 x 14,
-    152064: 5 x 15, 200064: 7 x 14); with and without waiting for the partners the oracle's numbers and the same bits."""
+    not fill their parts -- and four-byte rows of up to five -- into parts of 13 to 15 chunks per thread (100352
+    two-byte columns: 4 x 256 x 13, 114688: 4 x 14, 152064: 5 x 15, 200064: 7 x 14; 50304 four-byte columns: 4 x 13); with and without waiting for the partners the oracle's numbers and the same bits."""
     logits, tv, ti = _case(10, V, 48, dtype, 41, std=3.0)
     valid = torch.ones(10, dtype=torch.bool)
     valid[4] = False
