@@ -102,8 +102,10 @@ const char* dl_status_string(int status);
  * row's stride or at least inside the memory page of the row's last column, so the read cannot fault; what
  * it brings in from beyond column V is discarded.  The same holds for dl_rowcoef_grad_topk and
  * dl_fkl_multi_teacher.  Other rows (an odd row stride, a column slice that starts off the grid) are still
- * moved 16 bytes at a time: forward-KL rows of up to 4096 16-byte chunks by unaligned accesses in the
- * register kernels; wider ones, and dl_rowstats_topk / dl_rowcoef_grad_topk, by the aligned chunks inside
+ * moved 16 bytes at a time: forward-KL rows by unaligned accesses in the register kernels (one workgroup per
+ * row of up to 4096 16-byte chunks, column parts beyond where a workspace came along -- which
+ * dl_div_topk_workspace_bytes asks for from 4097 chunks on when V is not a whole number of chunks); wider ones
+ * without a workspace, and dl_rowstats_topk / dl_rowcoef_grad_topk, by the aligned chunks inside
  * each row, provided that logits and gradient rows share their address modulo 16 (the same stride from
  * 16-byte aligned bases, or the gradient written over the logits; reverse KL: any gradient row), and
  * element by element otherwise.
