@@ -38,7 +38,7 @@ def _masked_map(R, masked):
                                            (152064, torch.float16, {}), (40000, torch.float32, {"no_wait": True}),
                                            (32000, torch.bfloat16, {})])
 def test_static_scratch_entry_point_matches_the_workspace_one(D, V, dtype, hooks):
-    """Rows cut into 4 parts (128256 bf16), 3 (40000 fp32: 10000 chunks in parts of 4096) and 5 (152064 fp16)
+    """Rows cut into 4 parts (128256 bf16), 3 (40000 fp32: 10000 chunks in parts of 256 x 14) and 5 (152064 fp16)
     meet through the scratch; 32000-wide rows need none.  With `no_wait` every part also goes through the list of
     deferred parts that lives in the same array."""
     K = 200
