@@ -287,11 +287,10 @@ def _wl_dropin(batched):
             st = torch.cuda.current_stream().cuda_stream
             for i in range(B):
                 x, b = xs[i].detach(), bufs[i]
-                lib.dl_rowstats_topk(x.data_ptr(), 0, V, N, V, 0, tis[i].data_ptr(), 1, K, N, 1.0, b["lse"].data_ptr(),
-                                     b["zk"].data_ptr(), st)
-                lib.dl_composite_forward(b["lse"].data_ptr(), b["zk"].data_ptr(), tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
-                                         labs[i].data_ptr(), avoid.data_ptr(), 1, offs[0], offs[1], offs[2], 1, 1, N, alpha,
-                                         b["rec"].data_ptr(), b["coef"].data_ptr(), b["out"].data_ptr(), st)
+                lib.dl_composite_forward_fused(x.data_ptr(), 0, V, N, V, 0, N, 1.0, tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,
+                                               labs[i].data_ptr(), avoid.data_ptr(), 1, offs[0], offs[1], offs[2], 1, 1, alpha,
+                                               b["lse"].data_ptr(), b["zk"].data_ptr(), b["rec"].data_ptr(), b["coef"].data_ptr(),
+                                               b["out"].data_ptr(), st)
             for i in range(B):
                 x, b = xs[i].detach(), bufs[i]
                 lib.dl_composite_backward_fused(x.data_ptr(), 0, V, N, V, 0, N, 1.0, tvs[i].data_ptr(), 0, 1.0, tis[i].data_ptr(), 1, K,

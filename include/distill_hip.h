@@ -258,6 +258,22 @@ int dl_composite_forward(const float* lse, const float* zk, const void* t_val, i
                          void* stream);
 
 /*
+ * dl_rowstats_topk and dl_composite_forward in one call.  Where every teacher row has its logits row (no row map,
+ * n_teacher_rows == n_rows), K <= 1024 and a row holds at most 16384 16-byte chunks, phase 1 makes the rows'
+ * records at its own tail -- the logits at the teacher's ids are in LDS when its sweep ends -- and the call is two
+ * launches instead of three; otherwise it runs the launches of the two entry points it stands for.  Arguments,
+ * reference lines and results as theirs (lse, zk, row_records, row_coef, out are all written; the records agree
+ * with dl_composite_forward's to fp32 rounding: the sums over K are taken by a workgroup instead of a wave).
+ */
+int dl_composite_forward_fused(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                               const int32_t* row_map, int64_t n_teacher_rows, float inv_T, const void* t_val,
+                               int t_val_dtype, float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
+                               const int64_t* labels, const void* avoid, int avoid_itype, const int32_t* row_off,
+                               const int32_t* label_off, const int32_t* avoid_off, int offsets_on_host,
+                               int n_convos, float alpha, float* lse, float* zk, void* row_records,
+                               void* row_coef, float* out, void* stream);
+
+/*
  * Backward of dl_composite_forward for upstream gradients g_train [n_convos] on each conversation's
  * train_loss: g_lse [n_rows] = dL/dlse and g_zk [n_rows, K] = dL/dzk, the inputs of
  * dl_rowcoef_grad_topk.  Replaces the autograd replay started at classes/losses.py:77-78.

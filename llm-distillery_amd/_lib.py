@@ -66,6 +66,8 @@ _SIGNATURES = {
                                      c_int64, c_float, _P, _P, _P, _P]),
     "dl_composite_backward": (c_int, [_P, _P, _P, c_int, c_float, _P, c_int, c_int, _P, c_int, c_int, c_int64, _P, _P, _P, _P,
                                       _P, _P]),
+    "dl_composite_forward_fused": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, c_float, _P, c_int, c_float, _P, c_int, c_int,
+                                           _P, _P, c_int, _P, _P, _P, c_int, c_int, c_float, _P, _P, _P, _P, _P, _P]),
     "dl_composite_backward_fused": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, c_float, _P, c_int, c_float, _P, c_int, c_int,
                                             _P, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int64, _P]),
     "dl_teacher_topk": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int64, c_int, _P, c_int, _P, c_int, _P, c_int64, _P]),

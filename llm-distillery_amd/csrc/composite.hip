@@ -298,6 +298,8 @@ int composite_backward_params(CompositeParams& p, const float* lse, const float*
   return DL_OK;
 }
 
+void launch_composite_rows_fwd(const CompositeParams& p, hipStream_t st) { launch_rows_fwd(p, st); }
+
 void launch_composite_convo(const CompositeParams& p, hipStream_t st) {
   hipLaunchKernelGGL(composite_convo_kernel, dim3((unsigned)p.n_convos), dim3(CONVO_NT), 0, st, p);
 }

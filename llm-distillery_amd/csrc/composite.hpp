@@ -172,6 +172,7 @@ int composite_backward_params(CompositeParams& p, const float* lse, const float*
                               float inv_T_teacher, const void* t_idx, int t_idx_itype, int K, const int32_t* row_off,
                               int offsets_on_host, int n_convos, int64_t n_rows, const void* row_records,
                               const void* row_coef, const float* g_train);
+void launch_composite_rows_fwd(const CompositeParams& p, hipStream_t st);
 void launch_composite_convo(const CompositeParams& p, hipStream_t st);
 
 }  // namespace dl

@@ -32,8 +32,15 @@ struct StatsParams {
 constexpr int STASH_ROUNDS = 64;
 constexpr int STASH_MAX_K = 1024;
 
-template <class Tag, int NT, int MODE, bool STASH>
-__global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
+//
+// RECORD (with STASH): the row's record of the composite loss (composite_row_record, there by one wave of a launch
+// of its own) is made here, by the whole workgroup, behind the sweep: the teacher's K values are fetched before the
+// sweep, the logits at its ids are in LDS when the sweep ends, so the record costs three rounds of workgroup
+// reductions and no memory round trip.  K <= STASH_MAX_K: at most STASH_MAX_K / NT entries per thread.
+template <class Tag, int NT, int MODE, bool STASH, bool RECORD>
+__device__ __forceinline__ void rowstats_row(const StatsParams& p, const CompositeParams* cp) {
+  static_assert(!RECORD || STASH, "the record is made from the logits the sweep leaves in LDS");
+  constexpr int E = STASH_MAX_K / NT;
   __shared__ float red[64];
   __shared__ unsigned long long s_bits[STASH ? NT : 1];
   __shared__ int s_pre[STASH ? NT : 1];
@@ -51,6 +58,17 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
     if (f > m) { sm *= fast_exp2((m - f) * a); m = f; }
     if (f > -INFINITY) sm += fast_exp2(fmaf(f, a, -m * a));
   };
+  unsigned traw[RECORD ? E : 1];      // the teacher's values as stored, converted behind the sweep: all loads in flight together
+  if constexpr (RECORD) {
+    const int64_t at0 = trow * p.K;
+    if (cp->t_val_dtype == F32) {
+#pragma unroll
+      for (int j = 0; j < E; ++j) traw[j] = reinterpret_cast<const unsigned*>(cp->t_val)[at0 + (tid + j * NT < p.K ? tid + j * NT : 0)];
+    } else {
+#pragma unroll
+      for (int j = 0; j < E; ++j) traw[j] = reinterpret_cast<const unsigned short*>(cp->t_val)[at0 + (tid + j * NT < p.K ? tid + j * NT : 0)];
+    }
+  }
   if constexpr (!STASH) {
     for (int k = tid; k < p.K; k += NT) {
       const int64_t id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
@@ -64,15 +82,39 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
     u32x4* stash = reinterpret_cast<u32x4*>(smem);
     unsigned long long mybits = 0;
     int slot = 0;
+    int64_t idv[RECORD ? E : 1];      // RECORD: the thread's teacher ids, its row's label and whether that counts: known
+    bool want = false;                // before the sweep, so that the record behind it waits for no load
+    int64_t label = -1;
     if constexpr (STASH) {
       s_bits[tid] = 0;
       __syncthreads();
-      for (int k = tid; k < p.K; k += NT) {
-        const int64_t rel = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k) - sp.head;
+      const auto mark = [&](int64_t id) {
+        const int64_t rel = id - sp.head;
         if (rel >= 0 && rel < nch * C::N) {
           const int ch = (int)(rel / C::N);
           atomicOr(&s_bits[ch % NT], 1ull << (ch / NT));
         }
+      };
+      if constexpr (RECORD) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+          const int k = tid + j * NT;
+          idv[j] = load_index(p.t_idx, p.t_idx_itype, trow * p.K + (k < p.K ? k : 0));
+        }
+        const int c = convo_of_row(cp->off, cp->n_convos, trow);
+        const int li = (int)(trow - cp->off.row(c));
+        want = li < cp->off.label(c + 1) - cp->off.label(c);
+        if (want) {
+          label = cp->labels[cp->off.label(c) + li];
+          for (int av = cp->off.avoid(c); av < cp->off.avoid(c + 1); ++av) want = want && (load_index(cp->avoid, cp->avoid_itype, av) != li);
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+          if (tid + j * NT < p.K) mark(idv[j]);
+          else idv[j] = -1;
+        }
+      } else {
+        for (int k = tid; k < p.K; k += NT) mark(load_index(p.t_idx, p.t_idx_itype, trow * p.K + k));
       }
       __syncthreads();
       mybits = s_bits[tid];
@@ -123,10 +165,15 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
       }
     }
     if (MODE == 2 && tid < sp.leftovers()) one(load_as_float(row, Tag::id, sp.column(tid)));
+    const float mx = block_max<NT>(m, red);
+    sm = (m == -INFINITY) ? 0.f : sm * fast_exp2((m - mx) * a);
+    sm = block_sum<NT>(sm, red);
+    const float lse = (mx * a + fast_log2(sm)) * LN2;
+    if (tid == 0) p.lse[trow] = lse;
     if constexpr (STASH) {
       __syncthreads();
-      for (int k = tid; k < p.K; k += NT) {
-        const int64_t id = load_index(p.t_idx, p.t_idx_itype, trow * p.K + k);
+      // the logit at teacher entry k out of its chunk's slot (the few columns before and behind the body: from memory)
+      const auto logit_at = [&](int64_t id) {
         const int64_t rel = id - sp.head;
         float z = 0.f;
         if (rel >= 0 && rel < nch * C::N) {
@@ -136,11 +183,78 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
           if constexpr (Tag::bytes == 4) z = reinterpret_cast<const float*>(smem)[e];
           else z = load_as_float(reinterpret_cast<const unsigned short*>(smem) + e, Tag::id, 0);
         } else if (id >= 0 && id < p.V) {
-          z = load_as_float(row, Tag::id, id);               // the few columns before and behind the body
+          z = load_as_float(row, Tag::id, id);
         }
-        p.zk[trow * p.K + k] = z * p.inv_T;
+        return z * p.inv_T;
+      };
+      if constexpr (!RECORD) {
+        for (int k = tid; k < p.K; k += NT) p.zk[trow * p.K + k] = logit_at(load_index(p.t_idx, p.t_idx_itype, trow * p.K + k));
+      } else {
+        const int K = p.K;
+        float tv[E], zv[E];
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+          const int k = tid + j * NT;
+          tv[j] = zv[j] = -INFINITY;
+          if (j * NT >= K) continue;
+          if (k < K) {
+            zv[j] = logit_at(idv[j]);
+            p.zk[trow * K + k] = zv[j];
+            const float t = cp->t_val_dtype == F32 ? __uint_as_float(traw[j])
+                            : cp->t_val_dtype == BF16 ? __uint_as_float(traw[j] << 16)
+                                                      : (float)__builtin_bit_cast(_Float16, (unsigned short)traw[j]);
+            tv[j] = t * cp->inv_T_t;
+          }
+        }
+        // the arithmetic of composite_row_record, entry for entry, with the reductions over the workgroup
+        float tmax = -INFINITY, zmax = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < E; ++j) { tmax = fmaxf(tmax, tv[j]); zmax = fmaxf(zmax, zv[j]); }
+        block_max2<NT>(tmax, zmax, red);
+        // (rounds j that hold no entry at all are skipped by the whole workgroup; exponentials and logarithms by the
+        // hardware's base-2 instructions: a few units in the last place, against a record that is good to 1e-6)
+        const auto ex = [](float v) { return fast_exp2(v * LOG2E); };
+        float tsum = 0.f, zsum = 0.f;
+#pragma unroll
+        for (int j = 0; j < E; ++j)
+          if (j * NT < K) { tsum += ex(tv[j] - tmax); zsum += ex(zv[j] - zmax); }      // exp(-inf) = 0 beyond K
+        block_sum2<NT>(tsum, zsum, red);
+        const float t_lse = tmax + fast_log2(tsum) * LN2;
+        const float z_lse = zmax + fast_log2(zsum) * LN2;
+        const float s_lse = z_lse - lse;
+        float kl = 0.f, rkl = 0.f, found = -INFINITY;      // found: minus the first entry that carries the label
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+          const int k = tid + j * NT;
+          if (j * NT >= K) continue;
+          if (k < K) {
+            const float t = tv[j] - t_lse;
+            const float sk = zv[j] - lse;
+            const float s2 = sk - s_lse;
+            kl += ex(t) * (t - sk);
+            rkl += ex(s2) * (s2 - t);
+            if (want && idv[j] == label) found = fmaxf(found, -(float)k);
+          }
+        }
+        block_sum2<NT>(kl, rkl, red);
+        found = block_max<NT>(found, red);
+        const int kstar = found == -INFINITY ? -1 : (int)(-found);
+#pragma unroll
+        for (int j = 0; j < E; ++j)
+          if (kstar >= 0 && tid + j * NT == kstar) { red[0] = zv[j] - lse; red[1] = tv[j] - t_lse; }
+        __syncthreads();
+        if (tid == 0) {
+          RowRec rr;
+          rr.kl = kl; rr.rkl = rkl; rr.t_lse = t_lse; rr.s_lse = s_lse;
+          rr.valid = kstar >= 0 ? 1 : 0;
+          rr.kstar = kstar;
+          rr.own_s = kstar >= 0 ? red[0] : 0.f;
+          rr.own_t = kstar >= 0 ? red[1] : 0.f;
+          cp->rec[trow] = rr;
+        }
       }
     }
+    return;
   } else {
     for (int64_t j = tid; j < p.V; j += NT) one(load_as_float(row, Tag::id, j));
   }
@@ -148,6 +262,15 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
   sm = (m == -INFINITY) ? 0.f : sm * fast_exp2((m - mx) * a);
   sm = block_sum<NT>(sm, red);
   if (tid == 0) p.lse[trow] = (mx * a + fast_log2(sm)) * LN2;
+}
+
+template <class Tag, int NT, int MODE, bool STASH>
+__global__ __launch_bounds__(NT) void rowstats_kernel(const StatsParams p) {
+  rowstats_row<Tag, NT, MODE, STASH, false>(p, nullptr);
+}
+template <class Tag, int NT, int MODE>
+__global__ __launch_bounds__(NT) void rowstats_record_kernel(const StatsParams p, const CompositeParams cp) {
+  rowstats_row<Tag, NT, MODE, true, true>(p, &cp);
 }
 
 // ---- phase 2 -------------------------------------------------------------------------------
@@ -375,11 +498,24 @@ static bool same_phase16(const void* a, int64_t stride_a, const void* b, int64_t
   return reinterpret_cast<uintptr_t>(a) % 16 == reinterpret_cast<uintptr_t>(b) % 16 && ((stride_a - stride_b) * eb) % 16 == 0;
 }
 
+// phase 1 with the rows' records of the composite loss made at its tail (the caller has checked stash_fits)
+static bool stash_fits(int mode, int K, int64_t V, int epc) {
+  return mode != 0 && K <= STASH_MAX_K && (V + epc - 1) / epc <= (int64_t)STASH_ROUNDS * 256;
+}
+template <class Tag>
+static hipError_t launch_stats_record(const StatsParams& p, int mode, const CompositeParams& cp, hipStream_t st) {
+  const size_t lds = (size_t)p.K * 16;
+  const dim3 grid((unsigned)p.n_rows), block(256);
+  if (mode == 1) hipLaunchKernelGGL((rowstats_record_kernel<Tag, 256, 1>), grid, block, lds, st, p, cp);
+  else hipLaunchKernelGGL((rowstats_record_kernel<Tag, 256, 2>), grid, block, lds, st, p, cp);
+  return hipGetLastError();
+}
+
 template <class Tag>
 static hipError_t launch_stats(const StatsParams& p, int mode, hipStream_t st) {
   // the logits at the teacher's ids out of the sweep where the row's chunks fit the threads' 64 rounds (the bound holds
   // for every row: a peeled head only shortens the body)
-  const bool stash = mode != 0 && p.K <= STASH_MAX_K && (p.V + Tag::epc - 1) / Tag::epc <= (int64_t)STASH_ROUNDS * 256;
+  const bool stash = stash_fits(mode, p.K, p.V, Tag::epc);
   const size_t lds = stash ? (size_t)p.K * 16 : 0;
   const dim3 grid((unsigned)p.n_rows), block(256);
   if (mode == 1 && stash) hipLaunchKernelGGL((rowstats_kernel<Tag, 256, 1, true>), grid, block, lds, st, p);
@@ -443,6 +579,50 @@ extern "C" int dl_rowstats_topk(const void* logits, int logits_dtype, int64_t ro
                        : logits_dtype == DL_BF16 ? launch_stats<TagBF16>(p, vec, st)
                                                  : launch_stats<TagF16>(p, vec, st);
   return e == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
+}
+
+extern "C" int dl_composite_forward_fused(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows, int64_t V,
+                                          const int32_t* row_map, int64_t n_teacher_rows, float inv_T, const void* t_val,
+                                          int t_val_dtype, float inv_T_teacher, const void* t_idx, int t_idx_itype, int K,
+                                          const int64_t* labels, const void* avoid, int avoid_itype, const int32_t* row_off,
+                                          const int32_t* label_off, const int32_t* avoid_off, int offsets_on_host,
+                                          int n_convos, float alpha, float* lse, float* zk, void* row_records,
+                                          void* row_coef, float* out, void* stream) {
+  using namespace dl;
+  const int rc = check_common(logits, logits_dtype, row_stride, n_rows, V, t_idx, t_idx_itype, K, n_teacher_rows);
+  if (rc != DL_OK) return rc;
+  if ((!lse || !zk) && n_teacher_rows > 0) return DL_ERR_NULL;
+  CompositeParams cp;
+  const int st0 = composite_forward_params(cp, lse, zk, t_val, t_val_dtype, inv_T_teacher, t_idx, t_idx_itype, K, labels, avoid,
+                                           avoid_itype, row_off, label_off, avoid_off, offsets_on_host, n_convos,
+                                           n_teacher_rows, alpha, row_records, row_coef, out);
+  if (st0 != DL_OK) return st0;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int eb = logits_dtype == DL_F32 ? 4 : 2;
+  if (n_rows > 0) {
+    if (reinterpret_cast<uintptr_t>(logits) % eb != 0) return DL_ERR_ALIGN;
+    const int vec = V % (16 / eb) == 0 && aligned16(logits, row_stride, eb) ? 1 : 2;
+    StatsParams p{logits, row_stride, n_rows, V, row_map, t_idx, t_idx_itype, K, n_teacher_rows, inv_T, lse, zk,
+                  nullptr, nullptr, nullptr, 0};
+    // every teacher row has its logits row (no map, as many of the one as of the other): the rows' records at the
+    // tail of phase 1; else teacher rows without a logits row need records too: the launch of their own
+    if (!row_map && n_teacher_rows == n_rows && stash_fits(vec, K, V, 16 / eb)) {
+      const hipError_t e = logits_dtype == DL_F32 ? launch_stats_record<TagF32>(p, vec, cp, st)
+                           : logits_dtype == DL_BF16 ? launch_stats_record<TagBF16>(p, vec, cp, st)
+                                                     : launch_stats_record<TagF16>(p, vec, cp, st);
+      if (e != hipSuccess) return DL_ERR_LAUNCH;
+    } else {
+      const hipError_t e = logits_dtype == DL_F32 ? launch_stats<TagF32>(p, vec, st)
+                           : logits_dtype == DL_BF16 ? launch_stats<TagBF16>(p, vec, st)
+                                                     : launch_stats<TagF16>(p, vec, st);
+      if (e != hipSuccess) return DL_ERR_LAUNCH;
+      if (n_teacher_rows > 0) launch_composite_rows_fwd(cp, st);
+    }
+  } else if (n_teacher_rows > 0) {
+    launch_composite_rows_fwd(cp, st);
+  }
+  launch_composite_convo(cp, st);
+  return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH;
 }
 
 extern "C" int dl_rowcoef_grad_topk(const void* logits, int logits_dtype, int64_t row_stride, int64_t n_rows,

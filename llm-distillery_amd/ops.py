@@ -346,6 +346,11 @@ def _offsets_arg(offsets):
     return (arr(*offsets[0]), arr(*offsets[1]), arr(*offsets[2])), 1, C
 
 
+# True: phase 1 and the K-wide epilogue of the composite loss as the two entry points a caller with launches of its own
+# uses (dl_rowstats_topk, dl_composite_forward) instead of the one call that stands for them; the tests compare the two.
+SEPARATE_COMPOSITE_FORWARD = False
+
+
 def _composite_forward_raw(logits, t_val, t_idx, labels, avoid, offsets, row_map, inv_T, inv_T_teacher, alpha, crop, need_grad):
     """Phase 1 over the logits + the K-wide epilogue: (nine values [C, 9], lse, zk, rec, coef or None)."""
     x = _cropped(logits, crop)
@@ -367,15 +372,23 @@ def _composite_forward_raw(logits, t_val, t_idx, labels, avoid, offsets, row_map
     rm_ptr = row_map.data_ptr() if row_map is not None else 0
     stream = _stream_ptr(dev)
     with torch.cuda.device(dev):
-        st = lib.dl_rowstats_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(), _IT[t_idx.dtype],
-                                  K, N, inv_T, lse.data_ptr(), zk.data_ptr(), stream)
-        _lib.check(st, "dl_rowstats_topk")
-        st = lib.dl_composite_forward(
-            lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
-            _IT[t_idx.dtype], K, labels.data_ptr() if labels.numel() else 0, avoid.data_ptr() if avoid.numel() else 0,
-            _IT[avoid.dtype], offs[0], offs[1], offs[2], on_host, C, N, alpha, rec.data_ptr(),
-            coef.data_ptr() if need_grad else 0, out.data_ptr(), stream)
-        _lib.check(st, "dl_composite_forward")
+        if SEPARATE_COMPOSITE_FORWARD:
+            st = lib.dl_rowstats_topk(x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, t_idx.data_ptr(), _IT[t_idx.dtype],
+                                      K, N, inv_T, lse.data_ptr(), zk.data_ptr(), stream)
+            _lib.check(st, "dl_rowstats_topk")
+            st = lib.dl_composite_forward(
+                lse.data_ptr(), zk.data_ptr(), t_val.data_ptr(), _DT[t_val.dtype], inv_T_teacher, t_idx.data_ptr(),
+                _IT[t_idx.dtype], K, labels.data_ptr() if labels.numel() else 0, avoid.data_ptr() if avoid.numel() else 0,
+                _IT[avoid.dtype], offs[0], offs[1], offs[2], on_host, C, N, alpha, rec.data_ptr(),
+                coef.data_ptr() if need_grad else 0, out.data_ptr(), stream)
+            _lib.check(st, "dl_composite_forward")
+        else:
+            st = lib.dl_composite_forward_fused(
+                x.data_ptr(), _DT[x.dtype], x.stride(0), R, V, rm_ptr, N, inv_T, t_val.data_ptr(), _DT[t_val.dtype],
+                inv_T_teacher, t_idx.data_ptr(), _IT[t_idx.dtype], K, labels.data_ptr() if labels.numel() else 0,
+                avoid.data_ptr() if avoid.numel() else 0, _IT[avoid.dtype], offs[0], offs[1], offs[2], on_host, C, alpha,
+                lse.data_ptr(), zk.data_ptr(), rec.data_ptr(), coef.data_ptr() if need_grad else 0, out.data_ptr(), stream)
+            _lib.check(st, "dl_composite_forward_fused")
     return out, lse, zk, rec, coef
 
 

@@ -514,3 +514,66 @@ def test_phase_one_ids_out_of_the_sweep_or_gathered(D, dtype, V, K):
     want = torch.where(inside, torch.gather(x.float(), 1, idx.clamp(0, V - 1)) * np.float32(1.0 / 1.3), torch.zeros(()))
     assert torch.equal(zk.cpu(), want)
     np.testing.assert_allclose(lse.cpu().double().numpy(), torch.logsumexp(x.double() / 1.3, -1).numpy(), rtol=3e-6, atol=3e-6)
+
+
+@pytest.mark.parametrize("dtype,V,pitch,K,lens,host_offsets", [
+    (torch.float32, 32000, 32000, 400, [130], True),            # the reference's default width and K
+    (torch.bfloat16, 5001, 5120, 37, [20, 1, 33], False),       # a crop of padded rows, K off the wave size, device offsets
+    (torch.float16, 1003, 1003, 16, [9, 40], True),             # rows off the 16-byte grid
+    (torch.bfloat16, 128256, 128256, 200, [5, 6], True),
+    (torch.float32, 4096, 4096, 1024, [12, 7], True),           # four entries per thread
+    (torch.float32, 4096, 4096, 1100, [12, 7], True)])          # beyond what the tail of phase 1 takes: three launches
+def test_records_made_at_the_tail_of_phase_one_equal_the_separate_launches(D, dtype, V, pitch, K, lens, host_offsets):
+    """dl_composite_forward_fused against dl_rowstats_topk + dl_composite_forward (ops.SEPARATE_COMPOSITE_FORWARD):
+    lse and zk bit for bit, the nine values and the gradient to fp32 rounding (the sums over K are taken by a
+    workgroup instead of a wave); teacher values in every storage type, labels that hit and miss the support."""
+    from llm_distillery_amd import ops
+    N = sum(lens)
+    g = torch.Generator().manual_seed(V + K)
+    xs = (torch.randn(N, V, generator=g) * 2).to(dtype)
+    tfull = torch.log_softmax(xs.float() + torch.randn(N, V, generator=g), -1)
+    tv, ti = torch.topk(tfull, K)
+    labels, row_off, label_off, avoid_off, avoid = [], [0], [0], [0], []
+    for n in lens:
+        r0 = row_off[-1]
+        lab = ti[r0:r0 + n - 1, K // 3].clone()
+        miss = torch.rand(max(n - 1, 0), generator=g) < 0.3
+        lab[miss] = torch.randint(0, V, (int(miss.sum()),), generator=g)
+        labels.append(lab)
+        row_off.append(r0 + n)
+        label_off.append(label_off[-1] + n - 1)
+        if n > 4:
+            avoid.append(n // 2)
+        avoid_off.append(len(avoid))
+    labels = torch.cat(labels).to(DEV)
+    avoid = torch.tensor(avoid, dtype=torch.int64, device=DEV)
+    offsets = [row_off, label_off, avoid_off]
+    if not host_offsets:
+        offsets = torch.tensor(offsets, dtype=torch.int32, device=DEV)
+    full = torch.zeros(N, pitch, dtype=dtype, device=DEV)
+    full[:, :V] = xs.to(DEV)
+    same = lambda a, b: torch.equal(a.nan_to_num(nan=-7.0), b.nan_to_num(nan=-7.0))
+    for tdt, idt in ((torch.float32, torch.int64), (torch.float16, torch.int32), (torch.bfloat16, torch.int64)):
+        res = {}
+        for name in ("fused", "separate"):
+            ops.SEPARATE_COMPOSITE_FORWARD = name == "separate"
+            try:
+                x = full.clone().requires_grad_(True)
+                crop = V if pitch != V else 0
+                out, lse, zk, rec, coef = ops._composite_forward_raw(x.detach(), tv.to(tdt).to(DEV), ti.to(idt).to(DEV), labels, avoid,
+                                                                     offsets, None, 1.0 / 1.3, 1.0, 2.0, crop, True)
+                train, nine = ops.composite_loss(x, tv.to(tdt).to(DEV), ti.to(idt).to(DEV), labels, avoid, offsets, None, 1.0 / 1.3, 1.0, 2.0, crop=crop)
+                w = torch.arange(1, len(lens) + 1, dtype=torch.float32, device=DEV)
+                (train * w).sum().backward()
+            finally:
+                ops.SEPARATE_COMPOSITE_FORWARD = False
+            res[name] = (lse, zk, rec, out, nine, x.grad)
+        f, s_ = res["fused"], res["separate"]
+        assert torch.equal(f[0], s_[0]) and torch.equal(f[1], s_[1])                      # lse, zk
+        assert torch.equal(f[2].view(torch.int32)[:, 6:], s_[2].view(torch.int32)[:, 6:])  # kstar, valid
+        np.testing.assert_allclose(f[2][:, :6].cpu().numpy(), s_[2][:, :6].cpu().numpy(), rtol=2e-5, atol=2e-6)
+        np.testing.assert_allclose(f[3].nan_to_num(nan=-7.0).cpu().numpy(), s_[3].nan_to_num(nan=-7.0).cpu().numpy(), rtol=2e-5, atol=2e-6)
+        assert same(f[3], f[4])
+        gf, gs = f[5].float(), s_[5].float()
+        tol = gs.abs() * (1e-4 if dtype == torch.float32 else 2.0 ** -7) + gs.abs().amax(-1, keepdim=True) * 2e-6
+        assert ((gf - gs).abs() <= tol).all(), ((gf - gs).abs() / tol).max()
