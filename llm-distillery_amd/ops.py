@@ -441,9 +441,9 @@ def _composite_backward_raw(logits, t_val, t_idx, lse, zk, rec, coef, g_train, o
 
 
 class _CompositeLoss(torch.autograd.Function):
-    """The reference's composite loss of C conversations as ONE autograd node: phase 1 over the logits
-    (dl_rowstats_topk), the K-wide epilogue (dl_composite_forward), and in backward their
-    counterpart (dl_composite_backward_fused: the epilogue's backward inside phase 2).  Returns (train_loss [C], the nine
+    """The reference's composite loss of C conversations as ONE autograd node: phase 1 over the logits and the
+    K-wide epilogue (dl_composite_forward_fused), and in backward their counterpart (dl_composite_backward_fused:
+    the epilogue's backward inside phase 2, or dl_composite_backward + dl_rowcoef_grad_topk on wide rows).  Returns (train_loss [C], the nine
     values [C, 9]); only train_loss is differentiable, and only with respect to the logits.
     The eager path goes through this class rather than through the registered ops below (which run the
     same launches): a call through the dispatcher costs tens of microseconds of host time more, which at
